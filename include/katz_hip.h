@@ -1,0 +1,128 @@
+/*
+ * katz_hip -- C ABI of the MI355X (gfx950) kernels for the adapter-augmented SDXL UNet hot path.
+ *
+ * The reference binds its native ops through TORCH_LIBRARY(fast_kernel)
+ * (diffusers-hf/src/fast_kernel/fast_kernel/csrc/main.cpp:10-12, bind.cu:12-15) with torch::Tensor
+ * signatures; this library is the layer underneath such a binding: plain device pointers, sizes and a
+ * stream, no torch types, so it can be bound from torch (ctypes / TORCH_LIBRARY), from C++ or from a
+ * standalone benchmark.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless stated otherwise; bf16 tensors are raw 16-bit storage;
+ *   - tensors are dense row-major unless strides are explicit arguments;
+ *   - `stream` is a hipStream_t (NULL = default stream); every call only enqueues work, never
+ *     synchronises, never allocates, and is safe under HIP graph capture;
+ *   - return value: 0 = enqueued; < 0 = argument rejected before any launch (KH_ERR_*);
+ *     > 0 = the hipError_t reported by the launch.  The reference's GroupNorm swallows launch errors
+ *     (csrc/group_norm.cu:167-169, :219-221); this ABI never does.
+ */
+#ifndef KATZ_HIP_H
+#define KATZ_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define KH_OK 0
+#define KH_ERR_INVALID_ARG (-1) /* null pointer, non-positive size, inconsistent shape */
+#define KH_ERR_UNSUPPORTED (-2) /* shape outside what the kernels are built for (e.g. head_dim != 64) */
+#define KH_ERR_ALIGNMENT (-3)   /* a pointer or stride is not 16-byte aligned */
+#define KH_ERR_TOO_LARGE (-4)   /* size beyond a documented maximum */
+
+/* ABI version, bumped on any signature change. */
+int kh_version(void);
+/* Static string for a KH_ERR_* code or a hipError_t (host pointer, never NULL). */
+const char* kh_error_string(int code);
+
+/* ---- K1: LoRA-patched Linear ------------------------------------------------------------------
+ * y[M,N] = x[M,K] W[N,K]^T + bias[N] + ((x A_cat[R,K]^T) * col_scale[R]) B_cat[N,R]^T (+ residual[M,N])
+ * Replaces base Linear + per-adapter low-rank branch of the reference:
+ *   LoRACompatibleLinear.forward  diffusers-hf/src/diffusers/models/lora.py:451-457
+ *   LoRALinearLayer.forward       diffusers-hf/src/diffusers/models/lora.py:222-232
+ * (the peft Linear injected at diffusers-hf/src/diffusers/loaders/lora.py:409,475-476 computes the same
+ * sum over active adapters).  A_cat/B_cat: active adapters concatenated along the rank axis and padded
+ * with zero rows/columns to R % 32 == 0, R <= 128; col_scale[r] = weight_i * alpha_i / rank_i of the
+ * adapter that owns rank column r (what scale_lora_layers / set_adapters compute on the host,
+ * diffusers-hf/src/diffusers/utils/peft_utils.py:103-147,238-269).  R == 0 is a plain Linear.
+ * bias, residual may be NULL.  K % 8 == 0, N % 8 == 0.
+ * flags bit 0: GEGLU epilogue -- W/bias/B_cat rows are permuted so that every 64 consecutive rows are
+ *   32 value rows followed by their 32 gate rows; y is [M, N/2] = value * gelu_erf(gate)
+ *   (GEGLU.forward, diffusers-hf/src/diffusers/models/activations.py:139-149); N % 64 == 0, no residual.
+ * flags bits 8..15: tile override for tuning (0 = automatic). */
+int kh_lora_linear_bf16(const void* x, const void* w, const void* bias, const void* a_cat, const void* b_cat,
+                        const float* col_scale, const void* residual, void* y, int64_t M, int64_t N, int64_t K,
+                        int64_t R, int flags, void* stream);
+/* fp32 variant of the same formula (fp32 parity path); R <= 128, any M/N/K. */
+int kh_lora_linear_f32(const float* x, const float* w, const float* bias, const float* a_cat, const float* b_cat,
+                       const float* col_scale, const float* residual, float* y, int64_t M, int64_t N, int64_t K,
+                       int64_t R, void* stream);
+
+/* ---- K2: segmented multi-adapter shrink / expand ----------------------------------------------
+ * Per-request adapters in one batch: segment s = rows [seg_start[s], seg_start[s+1]) uses adapter
+ * seg_adapter[s] (< 0: none).  No counterpart in the reference; semantics = the LoRA linear above
+ * applied request by request (lora.py:222-232).  a_all [n_adapters, RP, K], b_all [n_adapters, N, RP],
+ * t [rows_total, RP]; adapter_rank[a] = rank rounded up to a multiple of 32 (zero padded), RP <= 128.
+ * seg_start (n_segments+1), seg_adapter, adapter_rank: device int32; adapter_scale: device float.
+ * max_seg_rows = longest segment (sizes the grid).
+ *   shrink: t[rows, 0:r] = x[rows,:] A_a^T          expand: y[rows,:] += scale_a * t[rows,0:r] B_a^T */
+int kh_sgmv_shrink_bf16(const void* x, const void* a_all, void* t, const int32_t* seg_start,
+                        const int32_t* seg_adapter, const int32_t* adapter_rank, int64_t n_segments,
+                        int64_t max_seg_rows, int64_t K, int64_t RP, void* stream);
+int kh_sgmv_expand_bf16(const void* t, const void* b_all, void* y, const int32_t* seg_start,
+                        const int32_t* seg_adapter, const int32_t* adapter_rank, const float* adapter_scale,
+                        int64_t n_segments, int64_t max_seg_rows, int64_t N, int64_t RP, void* stream);
+
+/* ---- K3: attention ----------------------------------------------------------------------------
+ * o = softmax(q k^T * scale) v per (batch, head); replaces F.scaled_dot_product_attention in
+ * AttnProcessor2_0.__call__ (diffusers-hf/src/diffusers/models/attention_processor.py:1269-1283).
+ * q,o: [B,T,H*64]; k,v: [B,S,H*64] addressed with row strides ld* and batch strides bs* (elements,
+ * multiples of 8), so q/k/v may be column slices of a fused projection.  head_dim must be 64. */
+int kh_attention_bf16(const void* q, const void* k, const void* v, void* o, int64_t B, int64_t H, int64_t T,
+                      int64_t S, int64_t head_dim, int64_t ldq, int64_t ldk, int64_t ldv, int64_t ldo, int64_t bsq,
+                      int64_t bsk, int64_t bsv, int64_t bso, float scale, void* stream);
+
+/* ---- K4: GroupNorm (+SiLU), LayerNorm -----------------------------------------------------------
+ * Replaces torch.ops.fast_kernel.group_norm_fp16(x, y, eps, num_groups, activation, weight, bias,
+ * affine, channels_last) (csrc/group_norm.cu:264-274, called at
+ * diffusers-hf/src/diffusers/models/normalization.py:90-91); y is caller-allocated as there.
+ * activation: 0 none, 1 silu.  channels_last: 1 = x,y are [N,HW,C] (NHWC), 0 = [N,C,HW] (NCHW).
+ * gamma/beta may be NULL (affine=False).  workspace: kh_group_norm_workspace_bytes(...) bytes of
+ * device memory owned by the caller (the reference allocates its mean/inv_variance tensors per call,
+ * group_norm.cu:240-242, which is not graph-capturable).  NHWC needs C % 8 == 0, C <= 4096, G <= 512;
+ * NCHW needs HW % 8 == 0. */
+int64_t kh_group_norm_workspace_bytes(int64_t N, int64_t C, int64_t HW, int64_t G, int channels_last);
+int kh_group_norm_bf16(const void* x, void* y, const void* gamma, const void* beta, float* workspace, int64_t N,
+                       int64_t C, int64_t HW, int64_t G, float eps, int activation, int channels_last, void* stream);
+/* nn.LayerNorm over the last axis (norm1/2/3 of BasicTransformerBlock,
+ * diffusers-hf/src/diffusers/models/attention.py:195,225,253); D % 8 == 0, D <= 2048. */
+int kh_layer_norm_bf16(const void* x, void* y, const void* gamma, const void* beta, int64_t M, int64_t D, float eps,
+                       void* stream);
+
+/* ---- K5: GEGLU -----------------------------------------------------------------------------------
+ * out[M,D] = proj[M, 0:D] * gelu(proj[M, D:2D])  (GEGLU.forward unfused branch, activations.py:148-149;
+ * approximate_tanh = 0 is F.gelu's exact erf form, 1 the tanh form of csrc/gelu.cuh:29-42). */
+int kh_geglu_bf16(const void* proj, void* out, int64_t M, int64_t D, int approximate_tanh, void* stream);
+/* out = gelu(x) * m, n elements: torch.ops.fast_kernel.fast_gelu_mul_fp16(x, m)
+ * (csrc/gelu.cuh:44-59, called at activations.py:145); the caller allocates out. */
+int kh_gelu_mul_bf16(const void* x, const void* m, void* out, int64_t n, int approximate_tanh, void* stream);
+
+/* ---- ControlNet residual injection -----------------------------------------------------------------
+ * dst[n] += (sum_k srcs[k][n]) * inv_count : skip_j + r_j and sample + r_mid
+ * (diffusers-hf/src/diffusers/models/unets/unet_2d_condition.py:1284-1292), with the multi-ControlNet
+ * sum then mean of :1418-1439 folded in (inv_count = 1/#ControlNets).  srcs: HOST array of n_srcs (<= 8)
+ * device pointers; n % 8 == 0. */
+int kh_residual_add_bf16(void* dst, const void* const* srcs, int n_srcs, float inv_count, int64_t n, void* stream);
+/* Channels-last concat with the residual add folded in:
+ * out[rows, 0:C1] = h[rows, C1]; out[rows, C1:C1+C2] = skip[rows, C2] + (sum_k residuals[k]) * inv_count.
+ * Replaces torch.cat([hidden_states, res_hidden_states], dim=1) of the up blocks
+ * (diffusers-hf/src/diffusers/models/unets/unet_2d_blocks.py:2512, :2645) plus the adds above.
+ * residuals: HOST array of n_residuals (0..8) device pointers; C1 % 8 == 0, C2 % 8 == 0. */
+int kh_concat_residual_bf16(const void* h, const void* skip, const void* const* residuals, int n_residuals,
+                            float inv_count, void* out, int64_t rows, int64_t C1, int64_t C2, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KATZ_HIP_H */

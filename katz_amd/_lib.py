@@ -1,0 +1,64 @@
+"""ctypes binding of libkatz_hip.so (the C ABI declared in include/katz_hip.h).
+
+There is no fallback: if the library is missing the import of any op fails with an error that says
+how to build it.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p
+from pathlib import Path
+
+LIB_PATH = Path(__file__).resolve().parent / "libkatz_hip.so"
+
+_P = c_void_p
+_I = c_int64
+
+# name -> (restype, argtypes); mirrors include/katz_hip.h one to one
+SIGNATURES = {
+    "kh_version": (c_int, []),
+    "kh_error_string": (c_char_p, [c_int]),
+    "kh_lora_linear_bf16": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, c_int, _P]),
+    "kh_lora_linear_f32": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
+    "kh_sgmv_shrink_bf16": (c_int, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
+    "kh_sgmv_expand_bf16": (c_int, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
+    "kh_attention_bf16": (c_int, [_P, _P, _P, _P] + [_I] * 13 + [c_float, _P]),
+    "kh_group_norm_workspace_bytes": (c_int64, [_I, _I, _I, _I, c_int]),
+    "kh_group_norm_bf16": (c_int, [_P, _P, _P, _P, _P, _I, _I, _I, _I, c_float, c_int, c_int, _P]),
+    "kh_layer_norm_bf16": (c_int, [_P, _P, _P, _P, _I, _I, c_float, _P]),
+    "kh_geglu_bf16": (c_int, [_P, _P, _I, _I, c_int, _P]),
+    "kh_gelu_mul_bf16": (c_int, [_P, _P, _P, _I, c_int, _P]),
+    "kh_residual_add_bf16": (c_int, [_P, _P, c_int, c_float, _I, _P]),
+    "kh_concat_residual_bf16": (c_int, [_P, _P, _P, c_int, c_float, _P, _I, _I, _I, _P]),
+}
+
+_lib = None
+
+
+class KatzHipError(RuntimeError):
+    """A katz_hip entry point rejected its arguments or the launch failed."""
+
+
+def load() -> ctypes.CDLL:
+    """Load libkatz_hip.so once and attach the prototypes. Raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not LIB_PATH.exists():
+        raise KatzHipError(
+            f"{LIB_PATH} is missing: build the HIP kernels with `python -m katz_amd.build` "
+            "(needs hipcc); there is no CPU fallback for these ops"
+        )
+    lib = ctypes.CDLL(str(LIB_PATH))
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError here means header and library disagree
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(code: int, what: str) -> None:
+    if code != 0:
+        msg = load().kh_error_string(int(code)).decode()
+        raise KatzHipError(f"{what} failed with code {code}: {msg}")

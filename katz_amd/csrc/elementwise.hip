@@ -1,0 +1,206 @@
+// K5 + ControlNet residual injection: HBM-bound elementwise kernels for gfx950, 16 bytes per lane.
+//
+// * kh_geglu_bf16: out = value * gelu(gate) with [value | gate] = proj(x) split along the last
+//   axis (diffusers-hf/src/diffusers/models/activations.py:139-149; erf-exact F.gelu by default).
+// * kh_gelu_mul_bf16: out = gelu(x) * m, the two-tensor form of the reference's fused op
+//   torch.ops.fast_kernel.fast_gelu_mul_fp16 (diffusers-hf/src/fast_kernel/fast_kernel/csrc/gelu.cuh:29-59,
+//   tanh approximation 0.5*x*(1+tanh(0.79788456*(x+0.044715*x^3)))).
+// * kh_residual_add_bf16: dst += (sum_k src_k) * inv_k -- the ControlNet residual injection
+//   skip_j + r_j / sample + r_mid (diffusers-hf/src/diffusers/models/unets/unet_2d_condition.py:1284-1292)
+//   including the multi-ControlNet sum-then-mean (:1418-1439).
+// * kh_concat_residual_bf16: out[..., :C1] = h, out[..., C1:] = skip + (sum_k r_k) * inv_k over
+//   channels-last rows: the up-block torch.cat([hidden, skip], dim=1) is a copy anyway, so the
+//   residual add rides on it for free.
+#include "kh_common.h"
+
+namespace {
+
+constexpr int EW_THREADS = 256;
+constexpr int KH_MAX_SRCS = 8;
+
+__device__ __forceinline__ float gelu_erf_f(float x) { return 0.5f * x * (1.f + erff(x * 0.70710678118654752f)); }
+__device__ __forceinline__ float gelu_tanh_f(float x) {
+  return 0.5f * x * (1.f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
+}
+// gelu is rounded to bf16 before the product, as the reference's separate gelu and mul ops do
+template <bool TANH>
+__device__ __forceinline__ uint32_t geglu_pair(uint32_t val, uint32_t gate) {
+  const float g0 = bf16_lo(gate), g1 = bf16_hi(gate);
+  const float a0 = TANH ? gelu_tanh_f(g0) : gelu_erf_f(g0);
+  const float a1 = TANH ? gelu_tanh_f(g1) : gelu_erf_f(g1);
+  const uint32_t ar = pack_bf16x2(a0, a1);
+  return pack_bf16x2(bf16_lo(val) * bf16_lo(ar), bf16_hi(val) * bf16_hi(ar));
+}
+
+template <bool TANH>
+__global__ __launch_bounds__(EW_THREADS) void geglu_kernel(const bf16_t* __restrict__ proj, bf16_t* __restrict__ out,
+                                                           long M, int D) {
+  const int cpr = D / 8;
+  const long total = M * cpr;
+  for (long i = (long)blockIdx.x * EW_THREADS + threadIdx.x; i < total; i += (long)gridDim.x * EW_THREADS) {
+    const long row = i / cpr;
+    const int c = (int)(i % cpr) * 8;
+    const u32x4 hv = *reinterpret_cast<const u32x4*>(proj + row * 2 * D + c);
+    const u32x4 gv = *reinterpret_cast<const u32x4*>(proj + row * 2 * D + D + c);
+    u32x4 o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = geglu_pair<TANH>(hv[e], gv[e]);
+    *reinterpret_cast<u32x4*>(out + row * D + c) = o;
+  }
+}
+
+template <bool TANH>
+__global__ __launch_bounds__(EW_THREADS) void gelu_mul_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ m,
+                                                              bf16_t* __restrict__ out, long n) {
+  const long chunks = n / 8;
+  for (long i = (long)blockIdx.x * EW_THREADS + threadIdx.x; i < chunks; i += (long)gridDim.x * EW_THREADS) {
+    const u32x4 xv = *reinterpret_cast<const u32x4*>(x + i * 8);
+    const u32x4 mv = *reinterpret_cast<const u32x4*>(m + i * 8);
+    u32x4 o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = geglu_pair<TANH>(mv[e], xv[e]);
+    *reinterpret_cast<u32x4*>(out + i * 8) = o;
+  }
+  // tail (n % 8 elements)
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    for (long j = chunks * 8; j < n; ++j) {
+      const float g = (float)x[j];
+      const float a = (float)(bf16_t)(TANH ? gelu_tanh_f(g) : gelu_erf_f(g));
+      out[j] = (bf16_t)((float)m[j] * a);
+    }
+  }
+}
+
+struct SrcList {
+  const bf16_t* p[KH_MAX_SRCS];
+  int n;
+  float inv;
+};
+
+__device__ __forceinline__ void accumulate_srcs(const SrcList& s, long off, float (&acc)[8]) {
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+  for (int k = 0; k < s.n; ++k) {
+    const u32x4 v = *reinterpret_cast<const u32x4*>(s.p[k] + off);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) { acc[2 * e] += bf16_lo(v[e]); acc[2 * e + 1] += bf16_hi(v[e]); }
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] *= s.inv;
+}
+
+__global__ __launch_bounds__(EW_THREADS) void residual_add_kernel(bf16_t* __restrict__ dst, const SrcList s, long n) {
+  const long chunks = n / 8;
+  for (long i = (long)blockIdx.x * EW_THREADS + threadIdx.x; i < chunks; i += (long)gridDim.x * EW_THREADS) {
+    float acc[8];
+    accumulate_srcs(s, i * 8, acc);
+    const u32x4 d = *reinterpret_cast<const u32x4*>(dst + i * 8);
+    u32x4 o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = pack_bf16x2(bf16_lo(d[e]) + acc[2 * e], bf16_hi(d[e]) + acc[2 * e + 1]);
+    *reinterpret_cast<u32x4*>(dst + i * 8) = o;
+  }
+}
+
+// rows = N*HW pixels; out row = [h row (C1) | skip row (C2) + residual]
+__global__ __launch_bounds__(EW_THREADS) void concat_residual_kernel(const bf16_t* __restrict__ h,
+                                                                     const bf16_t* __restrict__ skip, const SrcList s,
+                                                                     bf16_t* __restrict__ out, long rows, int C1,
+                                                                     int C2) {
+  const int cp1 = C1 / 8, cp = (C1 + C2) / 8;
+  const long total = rows * cp;
+  for (long i = (long)blockIdx.x * EW_THREADS + threadIdx.x; i < total; i += (long)gridDim.x * EW_THREADS) {
+    const long row = i / cp;
+    const int c = (int)(i % cp);
+    u32x4 o;
+    if (c < cp1) {
+      o = *reinterpret_cast<const u32x4*>(h + row * C1 + c * 8);
+    } else {
+      const long off = row * C2 + (long)(c - cp1) * 8;
+      o = *reinterpret_cast<const u32x4*>(skip + off);
+      if (s.n > 0) {
+        float acc[8];
+        accumulate_srcs(s, off, acc);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = pack_bf16x2(bf16_lo(o[e]) + acc[2 * e], bf16_hi(o[e]) + acc[2 * e + 1]);
+      }
+    }
+    *reinterpret_cast<u32x4*>(out + row * (C1 + C2) + c * 8) = o;
+  }
+}
+
+unsigned ew_grid(long work_items) {
+  long b = (work_items + EW_THREADS - 1) / EW_THREADS;
+  const long cap = 256L * 16;  // 16 workgroups per CU, grid-stride beyond that
+  if (b > cap) b = cap;
+  if (b < 1) b = 1;
+  return (unsigned)b;
+}
+
+int fill_srcs(SrcList& s, const void* const* srcs, int n_srcs, float inv) {
+  if (n_srcs < 0 || n_srcs > KH_MAX_SRCS) return KH_ERR_TOO_LARGE;
+  s.n = n_srcs; s.inv = inv;
+  for (int k = 0; k < KH_MAX_SRCS; ++k) s.p[k] = nullptr;
+  for (int k = 0; k < n_srcs; ++k) {
+    if (!srcs || !srcs[k]) return KH_ERR_INVALID_ARG;
+    if (!kh_aligned16(srcs[k])) return KH_ERR_ALIGNMENT;
+    s.p[k] = (const bf16_t*)srcs[k];
+  }
+  return KH_OK;
+}
+
+}  // namespace
+
+KH_EXPORT int kh_geglu_bf16(const void* proj, void* out, int64_t M, int64_t D, int approximate_tanh, void* stream) {
+  if (!proj || !out || M <= 0 || D <= 0) return KH_ERR_INVALID_ARG;
+  if (D % 8 != 0) return KH_ERR_UNSUPPORTED;
+  if (!kh_aligned16(proj) || !kh_aligned16(out)) return KH_ERR_ALIGNMENT;
+  const unsigned grid = ew_grid(M * (D / 8));
+  if (approximate_tanh)
+    hipLaunchKernelGGL(geglu_kernel<true>, dim3(grid), dim3(EW_THREADS), 0, (hipStream_t)stream, (const bf16_t*)proj,
+                       (bf16_t*)out, (long)M, (int)D);
+  else
+    hipLaunchKernelGGL(geglu_kernel<false>, dim3(grid), dim3(EW_THREADS), 0, (hipStream_t)stream, (const bf16_t*)proj,
+                       (bf16_t*)out, (long)M, (int)D);
+  KH_RETURN_LAST_ERROR();
+}
+
+KH_EXPORT int kh_gelu_mul_bf16(const void* x, const void* m, void* out, int64_t n, int approximate_tanh, void* stream) {
+  if (!x || !m || !out || n <= 0) return KH_ERR_INVALID_ARG;
+  if (!kh_aligned16(x) || !kh_aligned16(m) || !kh_aligned16(out)) return KH_ERR_ALIGNMENT;
+  const unsigned grid = ew_grid(n / 8 + 1);
+  if (approximate_tanh)
+    hipLaunchKernelGGL(gelu_mul_kernel<true>, dim3(grid), dim3(EW_THREADS), 0, (hipStream_t)stream, (const bf16_t*)x,
+                       (const bf16_t*)m, (bf16_t*)out, (long)n);
+  else
+    hipLaunchKernelGGL(gelu_mul_kernel<false>, dim3(grid), dim3(EW_THREADS), 0, (hipStream_t)stream, (const bf16_t*)x,
+                       (const bf16_t*)m, (bf16_t*)out, (long)n);
+  KH_RETURN_LAST_ERROR();
+}
+
+KH_EXPORT int kh_residual_add_bf16(void* dst, const void* const* srcs, int n_srcs, float inv_count, int64_t n,
+                                   void* stream) {
+  if (!dst || n <= 0 || n_srcs <= 0) return KH_ERR_INVALID_ARG;
+  if (n % 8 != 0) return KH_ERR_UNSUPPORTED;
+  if (!kh_aligned16(dst)) return KH_ERR_ALIGNMENT;
+  SrcList s;
+  const int rc = fill_srcs(s, srcs, n_srcs, inv_count);
+  if (rc != KH_OK) return rc;
+  hipLaunchKernelGGL(residual_add_kernel, dim3(ew_grid(n / 8)), dim3(EW_THREADS), 0, (hipStream_t)stream,
+                     (bf16_t*)dst, s, (long)n);
+  KH_RETURN_LAST_ERROR();
+}
+
+KH_EXPORT int kh_concat_residual_bf16(const void* h, const void* skip, const void* const* residuals, int n_residuals,
+                                      float inv_count, void* out, int64_t rows, int64_t C1, int64_t C2, void* stream) {
+  if (!h || !skip || !out || rows <= 0 || C1 <= 0 || C2 <= 0) return KH_ERR_INVALID_ARG;
+  if (C1 % 8 != 0 || C2 % 8 != 0) return KH_ERR_UNSUPPORTED;
+  if (!kh_aligned16(h) || !kh_aligned16(skip) || !kh_aligned16(out)) return KH_ERR_ALIGNMENT;
+  SrcList s;
+  const int rc = fill_srcs(s, residuals, n_residuals, inv_count);
+  if (rc != KH_OK) return rc;
+  hipLaunchKernelGGL(concat_residual_kernel, dim3(ew_grid(rows * ((C1 + C2) / 8))), dim3(EW_THREADS), 0,
+                     (hipStream_t)stream, (const bf16_t*)h, (const bf16_t*)skip, s, (bf16_t*)out, (long)rows, (int)C1,
+                     (int)C2);
+  KH_RETURN_LAST_ERROR();
+}

@@ -1,0 +1,63 @@
+// Shared device/host helpers for the katz_hip kernels (gfx950 / CDNA4 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define KH_OK 0
+#define KH_ERR_INVALID_ARG (-1)
+#define KH_ERR_UNSUPPORTED (-2)
+#define KH_ERR_ALIGNMENT (-3)
+#define KH_ERR_TOO_LARGE (-4)
+
+#define KH_EXPORT extern "C" __attribute__((visibility("default")))
+
+// Launch-error check: kernels are asynchronous, so only launch-time errors are
+// visible here; a positive return value is the hipError_t.
+#define KH_RETURN_LAST_ERROR()                      \
+  do {                                              \
+    hipError_t e__ = hipGetLastError();             \
+    return e__ == hipSuccess ? KH_OK : (int)e__;    \
+  } while (0)
+
+typedef __bf16 bf16_t;
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t lo16) {
+  return __uint_as_float(lo16 << 16);
+}
+// Low / high bf16 of a packed 32-bit word, widened to fp32.
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+
+// Round-to-nearest-even fp32 -> bf16 (the compiler emits v_cvt_pk_bf16_f32 on gfx950).
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+  bf16x2 v;
+  v[0] = (bf16_t)a;
+  v[1] = (bf16_t)b;
+  return __builtin_bit_cast(uint32_t, v);
+}
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float a) {
+  bf16_t v = (bf16_t)a;
+  return __builtin_bit_cast(uint16_t, v);
+}
+
+__device__ __forceinline__ float silu_f(float x) { return x / (1.0f + __expf(-x)); }
+
+static inline bool kh_aligned16(const void* p) { return (((uintptr_t)p) & 15u) == 0; }
+
+// Workgroups are dealt round-robin to the 8 XCDs (each with its own L2). Map a
+// hardware block id to a logical tile id such that every XCD walks one
+// contiguous range of logical tiles, so neighbouring tiles share an L2.
+__device__ __forceinline__ uint32_t xcd_remap(uint32_t bid, uint32_t total) {
+  const uint32_t NX = 8;
+  uint32_t xcd = bid % NX, local = bid / NX;
+  uint32_t per = total / NX, rem = total % NX;
+  return xcd * per + (xcd < rem ? xcd : rem) + local;
+}

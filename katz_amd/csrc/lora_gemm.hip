@@ -1,0 +1,514 @@
+// K1: fused base GEMM + low-rank (LoRA) delta on bf16 MFMA for gfx950.
+//
+//   y[M,N] = x[M,K] . W[N,K]^T + bias[N] + ((x . A_cat[R,K]^T) * col_scale[R]) . B_cat[N,R]^T (+ residual[M,N])
+//
+// A_cat / B_cat are the active adapters concatenated along the rank axis, so a
+// sum over adapters is one rank-R product; col_scale carries s_i * alpha_i / r_i
+// for every rank column of adapter i.  This is the closed form of the
+// reference's LoRA-patched Linear (diffusers-hf/src/diffusers/models/lora.py:222-232
+// for the low-rank branch, :451-457 for base + scale * delta).
+//
+// The rank-R intermediate T = x . A_cat^T is accumulated by extra MFMAs inside
+// the base GEMM's K loop (the x tile is already in LDS), scaled, rounded to
+// bf16 and parked in LDS; the expand product T . B_cat^T is then accumulated
+// into the same fp32 accumulators as the base GEMM before the epilogue.  T
+// never goes to HBM.  One workgroup walks several N tiles of the same M block
+// so that T is computed once per chunk of N tiles rather than once per tile.
+#include "kh_common.h"
+
+namespace {
+
+constexpr int BK = 64;       // K slab per LDS stage (bf16 elements)
+constexpr int LDK = BK + 8;  // padded LDS row: 144 B, so the 16 rows one ds_read_b128 phase touches hit 16 distinct bank groups
+
+struct LoraGemmParams {
+  const bf16_t* x;
+  const bf16_t* w;
+  const bf16_t* bias;      // may be null
+  const bf16_t* a_cat;     // [R,K] (unused when R == 0)
+  const bf16_t* b_cat;     // [N,R]
+  const float* col_scale;  // [R]
+  const bf16_t* res;       // [M,N] residual added in the epilogue, may be null
+  bf16_t* y;
+  int M, N, K, R;
+  int m_tiles, n_tiles, n_chunk, n_chunks;  // n_chunk = N tiles walked by one workgroup
+  int geglu;                                // 1: W rows are (value,gate) interleaved in 32-column groups, y is [M,N/2]
+};
+
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int NRT_>
+struct Cfg {
+  static constexpr int BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, NRT = NRT_;
+  static constexpr int NW = WAVES_M * WAVES_N;
+  static constexpr int NT = NW * 64;
+  static constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
+  static constexpr int TM = WTM / 32, TN = WTN / 32;
+  static constexpr int R = NRT * 32;
+  static constexpr int SM = (NRT > 0) ? TM / WAVES_N : 0;  // shrink m-tiles per wave
+  static constexpr int LDT = R + 8;                        // padded row of the T / B_cat tiles
+  static constexpr int LDC = BN + 8;                       // padded row of the epilogue staging tile
+  static constexpr int XCH = BM * 8 / NT, WCH = BN * 8 / NT, ACH = R * 8 / NT;
+  static constexpr size_t SX = (size_t)BM * LDK * 2, SW = (size_t)BN * LDK * 2, SA = (size_t)R * LDK * 2;
+  static constexpr size_t SB = (size_t)BN * LDT * 2;
+  static constexpr size_t SC = (size_t)WAVES_M * 32 * LDC * 2;
+  static constexpr size_t STAGE = SX + SW + SA;
+  static constexpr size_t STAGE_MAX = STAGE > SB ? (STAGE > SC ? STAGE : SC) : (SB > SC ? SB : SC);
+  static constexpr size_t ST = (NRT > 0) ? (size_t)BM * LDT * 2 : 0;
+  static constexpr size_t LDS_BYTES = STAGE_MAX + ST;
+  static_assert(BM % (32 * WAVES_M) == 0 && BN % (32 * WAVES_N) == 0, "tile/wave mismatch");
+  static_assert(NRT == 0 || (TM % WAVES_N == 0), "shrink tiles must split evenly over the waves of a row");
+  static_assert((BM * 8) % NT == 0 && (BN * 8) % NT == 0 && (R * 8) % NT == 0, "load split");
+};
+
+__device__ __forceinline__ u32x4 ld16(const bf16_t* p) { return *reinterpret_cast<const u32x4*>(p); }
+__device__ __forceinline__ bf16x8 lds_frag(const bf16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
+
+template <class C>
+__global__ __launch_bounds__(C::NT) void lora_gemm_kernel(const LoraGemmParams p) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  constexpr int BM = C::BM, BN = C::BN, TM = C::TM, TN = C::TN, NRT = C::NRT, R = C::R;
+  constexpr int SMT = C::SM > 0 ? C::SM : 1, NRTT = NRT > 0 ? NRT : 1;
+  bf16_t* sX = reinterpret_cast<bf16_t*>(smem);
+  bf16_t* sW = reinterpret_cast<bf16_t*>(smem + C::SX);
+  bf16_t* sA = reinterpret_cast<bf16_t*>(smem + C::SX + C::SW);
+  bf16_t* sB = reinterpret_cast<bf16_t*>(smem);                 // aliases the K-loop stage
+  bf16_t* sC = reinterpret_cast<bf16_t*>(smem);                 // aliases the K-loop stage
+  bf16_t* sT = reinterpret_cast<bf16_t*>(smem + C::STAGE_MAX);  // lives across N tiles
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / C::WAVES_N, wn = wave % C::WAVES_N;
+  const int l32 = lane & 31, lh = lane >> 5;
+
+  const uint32_t total = (uint32_t)p.m_tiles * (uint32_t)p.n_chunks;
+  const uint32_t logical = xcd_remap(blockIdx.x, total);
+  const int m_blk = logical / p.n_chunks, chunk = logical % p.n_chunks;
+  const int m0 = m_blk * BM;
+  const int K = p.K, M = p.M, N = p.N;
+  const int KT = (K + BK - 1) / BK;
+
+  for (int jt = 0; jt < p.n_chunk; ++jt) {
+    const int n_tile = chunk * p.n_chunk + jt;
+    if (n_tile >= p.n_tiles) break;  // uniform over the workgroup
+    const int n0 = n_tile * BN;
+    const bool shrink = (NRT > 0) && (jt == 0);
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+    f32x16 tacc[SMT][NRTT];
+#pragma unroll
+    for (int s = 0; s < SMT; ++s)
+#pragma unroll
+      for (int r = 0; r < NRTT; ++r)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) tacc[s][r][v] = 0.f;
+
+    u32x4 rx[C::XCH], rw[C::WCH], ra[C::ACH > 0 ? C::ACH : 1];
+
+    auto load_tile = [&](int kt) {
+      const int k0 = kt * BK;
+#pragma unroll
+      for (int q = 0; q < C::XCH; ++q) {
+        const int c = tid + q * C::NT, row = c >> 3, ch = c & 7;
+        const int gk = k0 + ch * 8;
+        int gr = m0 + row; gr = gr < M ? gr : M - 1;
+        rx[q] = (gk < K) ? ld16(p.x + (size_t)gr * K + gk) : u32x4{0, 0, 0, 0};
+      }
+#pragma unroll
+      for (int q = 0; q < C::WCH; ++q) {
+        const int c = tid + q * C::NT, row = c >> 3, ch = c & 7;
+        const int gk = k0 + ch * 8;
+        int gr = n0 + row; gr = gr < N ? gr : N - 1;
+        rw[q] = (gk < K) ? ld16(p.w + (size_t)gr * K + gk) : u32x4{0, 0, 0, 0};
+      }
+      if constexpr (NRT > 0) {
+        if (shrink) {
+#pragma unroll
+          for (int q = 0; q < C::ACH; ++q) {
+            const int c = tid + q * C::NT, row = c >> 3, ch = c & 7;
+            const int gk = k0 + ch * 8;
+            ra[q] = (gk < K) ? ld16(p.a_cat + (size_t)row * K + gk) : u32x4{0, 0, 0, 0};
+          }
+        }
+      }
+    };
+    auto store_tile = [&]() {
+#pragma unroll
+      for (int q = 0; q < C::XCH; ++q) {
+        const int c = tid + q * C::NT, row = c >> 3, ch = c & 7;
+        *reinterpret_cast<u32x4*>(sX + row * LDK + ch * 8) = rx[q];
+      }
+#pragma unroll
+      for (int q = 0; q < C::WCH; ++q) {
+        const int c = tid + q * C::NT, row = c >> 3, ch = c & 7;
+        *reinterpret_cast<u32x4*>(sW + row * LDK + ch * 8) = rw[q];
+      }
+      if constexpr (NRT > 0) {
+        if (shrink) {
+#pragma unroll
+          for (int q = 0; q < C::ACH; ++q) {
+            const int c = tid + q * C::NT, row = c >> 3, ch = c & 7;
+            *reinterpret_cast<u32x4*>(sA + row * LDK + ch * 8) = ra[q];
+          }
+        }
+      }
+    };
+
+    load_tile(0);
+    store_tile();
+    __syncthreads();
+    for (int kt = 0; kt < KT; ++kt) {
+      if (kt + 1 < KT) load_tile(kt + 1);  // global loads stay in flight under the MFMAs below
+#pragma unroll
+      for (int ks = 0; ks < BK / 16; ++ks) {
+        bf16x8 a[TM], b[TN];
+        const int ko = ks * 16 + lh * 8;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) a[i] = lds_frag(sX + (wm * C::WTM + i * 32 + l32) * LDK + ko);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) b[j] = lds_frag(sW + (wn * C::WTN + j * 32 + l32) * LDK + ko);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+        if constexpr (NRT > 0) {
+          if (shrink) {
+            // this wave owns shrink m-tiles wn*SM .. wn*SM+SM-1 of its wave row: their x fragments are in a[]
+#pragma unroll
+            for (int r = 0; r < NRT; ++r) {
+              const bf16x8 ar = lds_frag(sA + (r * 32 + l32) * LDK + ko);
+#pragma unroll
+              for (int q = 0; q < C::WAVES_N; ++q) {
+                if (wn == q) {  // wave-uniform: keeps the index into a[] a compile-time constant
+#pragma unroll
+                  for (int s = 0; s < C::SM; ++s)
+                    tacc[s][r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[q * C::SM + s], ar, tacc[s][r], 0, 0, 0);
+                }
+              }
+            }
+          }
+        }
+      }
+      __syncthreads();
+      if (kt + 1 < KT) {
+        store_tile();
+        __syncthreads();
+      }
+    }
+
+    if constexpr (NRT > 0) {
+      if (shrink) {
+        // T = (x . A_cat^T) * col_scale -> bf16 -> LDS.  Accumulator element v of lane (l32, lh)
+        // is row 8*(v/4) + 4*lh + v%4, column l32 of its 32x32 tile.
+#pragma unroll
+        for (int r = 0; r < NRT; ++r) {
+          const int col = r * 32 + l32;
+          const float sc = p.col_scale[col];
+#pragma unroll
+          for (int s = 0; s < C::SM; ++s) {
+            const int rbase = wm * C::WTM + (wn * C::SM + s) * 32 + 4 * lh;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+              const int row = rbase + 8 * (v >> 2) + (v & 3);
+              sT[row * C::LDT + col] = (bf16_t)(tacc[s][r][v] * sc);
+            }
+          }
+        }
+      }
+      // expand: acc += T[BM,R] . B_cat[n0:n0+BN, R]^T
+      for (int c = tid; c < BN * (R / 8); c += C::NT) {
+        const int row = c / (R / 8), ch = c % (R / 8);
+        int gr = n0 + row; gr = gr < N ? gr : N - 1;
+        *reinterpret_cast<u32x4*>(sB + row * C::LDT + ch * 8) = ld16(p.b_cat + (size_t)gr * R + ch * 8);
+      }
+      __syncthreads();
+#pragma unroll
+      for (int ks = 0; ks < R / 16; ++ks) {
+        bf16x8 a[TM], b[TN];
+        const int ko = ks * 16 + lh * 8;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) a[i] = lds_frag(sT + (wm * C::WTM + i * 32 + l32) * C::LDT + ko);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) b[j] = lds_frag(sB + (wn * C::WTN + j * 32 + l32) * C::LDT + ko);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+      }
+      __syncthreads();  // sB is dead before sC overwrites it
+    }
+
+    // Epilogue: bias in fp32, round to bf16, transpose through LDS so that every
+    // global store is a 16-byte piece of a contiguous output row.
+    float bv[TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int col = n0 + wn * C::WTN + j * 32 + l32;
+      bv[j] = (p.bias != nullptr && col < N) ? (float)p.bias[col] : 0.f;
+    }
+    const int out_ld = p.geglu ? (N >> 1) : N;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int col = wn * C::WTN + j * 32 + l32;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int row = wm * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+          sC[row * C::LDC + col] = (bf16_t)(acc[i][j][v] + bv[j]);
+        }
+      }
+      __syncthreads();
+      if (!p.geglu) {
+        constexpr int CPR = BN / 8;  // 16-byte chunks per staged row
+        for (int c = tid; c < C::WAVES_M * 32 * CPR; c += C::NT) {
+          const int srow = c / CPR, ch = c % CPR;
+          const int grow = m0 + (srow >> 5) * C::WTM + i * 32 + (srow & 31);
+          const int gcol = n0 + ch * 8;
+          if (grow < M && gcol < N) {
+            u32x4 o = *reinterpret_cast<const u32x4*>(sC + srow * C::LDC + ch * 8);
+            if (p.res != nullptr) {
+              const u32x4 rr = ld16(p.res + (size_t)grow * N + gcol);
+#pragma unroll
+              for (int e = 0; e < 4; ++e)
+                o[e] = pack_bf16x2(bf16_lo(o[e]) + bf16_lo(rr[e]), bf16_hi(o[e]) + bf16_hi(rr[e]));
+            }
+            *reinterpret_cast<u32x4*>(p.y + (size_t)grow * N + gcol) = o;
+          }
+        }
+      } else {
+        // GEGLU epilogue: staged columns come in groups of 64 = 32 value columns then their 32 gate
+        // columns; out = value * gelu_erf(gate), written to y[M, N/2].
+        constexpr int OPR = BN / 16;  // 8-element output chunks per staged row
+        for (int c = tid; c < C::WAVES_M * 32 * OPR; c += C::NT) {
+          const int srow = c / OPR, oc = c % OPR;          // oc: output chunk, 4 chunks per 64-col group
+          const int grp = oc >> 2, sub = oc & 3;
+          const int grow = m0 + (srow >> 5) * C::WTM + i * 32 + (srow & 31);
+          const int gcol = (n0 >> 1) + grp * 32 + sub * 8;
+          if (grow < M && gcol < out_ld) {
+            const u32x4 hv = *reinterpret_cast<const u32x4*>(sC + srow * C::LDC + grp * 64 + sub * 8);
+            const u32x4 gv = *reinterpret_cast<const u32x4*>(sC + srow * C::LDC + grp * 64 + 32 + sub * 8);
+            u32x4 o;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const float g0 = bf16_lo(gv[e]), g1 = bf16_hi(gv[e]);
+              const float a0 = 0.5f * g0 * (1.f + erff(g0 * 0.70710678118654752f));
+              const float a1 = 0.5f * g1 * (1.f + erff(g1 * 0.70710678118654752f));
+              // the reference rounds gelu(gate) to the activation dtype before the product
+              const float r0 = bf16_lo(pack_bf16x2(a0, 0.f)), r1 = bf16_lo(pack_bf16x2(a1, 0.f));
+              o[e] = pack_bf16x2(bf16_lo(hv[e]) * r0, bf16_hi(hv[e]) * r1);
+            }
+            *reinterpret_cast<u32x4*>(p.y + (size_t)grow * out_ld + gcol) = o;
+          }
+        }
+      }
+      __syncthreads();
+    }
+  }
+}
+
+template <class C>
+int launch_cfg(LoraGemmParams p, hipStream_t stream) {
+  p.m_tiles = (p.M + C::BM - 1) / C::BM;
+  p.n_tiles = (p.N + C::BN - 1) / C::BN;
+  // Walk several N tiles per workgroup (T is reused from LDS) as long as the grid still
+  // covers the 256 CUs at least twice over.
+  int nc = 1;
+  if (C::NRT > 0) {
+    while (nc < p.n_tiles && (long)p.m_tiles * ((p.n_tiles + 2 * nc - 1) / (2 * nc)) >= 512) nc *= 2;
+  }
+  p.n_chunk = nc;
+  p.n_chunks = (p.n_tiles + nc - 1) / nc;
+  static bool attr_done = false;  // per template instantiation
+  if (!attr_done) {
+    hipError_t e = hipFuncSetAttribute((const void*)lora_gemm_kernel<C>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)C::LDS_BYTES);
+    if (e != hipSuccess) return (int)e;
+    attr_done = true;
+  }
+  const unsigned grid = (unsigned)(p.m_tiles * p.n_chunks);
+  hipLaunchKernelGGL(lora_gemm_kernel<C>, dim3(grid), dim3(C::NT), C::LDS_BYTES, stream, p);
+  KH_RETURN_LAST_ERROR();
+}
+
+template <int BM, int BN, int WM, int WN>
+int launch_rank(const LoraGemmParams& p, hipStream_t stream) {
+  switch (p.R / 32) {
+    case 0: return launch_cfg<Cfg<BM, BN, WM, WN, 0>>(p, stream);
+    case 1: return launch_cfg<Cfg<BM, BN, WM, WN, 1>>(p, stream);
+    case 2: return launch_cfg<Cfg<BM, BN, WM, WN, 2>>(p, stream);
+    case 3: return launch_cfg<Cfg<BM, BN, WM, WN, 3>>(p, stream);
+    case 4: return launch_cfg<Cfg<BM, BN, WM, WN, 4>>(p, stream);
+    default: return KH_ERR_UNSUPPORTED;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// fp32 variant (debug / fp32 parity path): plain FMA tiles, same fusion (T kept in LDS).
+// ---------------------------------------------------------------------------------------------
+constexpr int F_BM = 64, F_BN = 64, F_BK = 16, F_RMAX = 128;
+
+__global__ __launch_bounds__(256) void lora_gemm_f32_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                            const float* __restrict__ bias,
+                                                            const float* __restrict__ a_cat,
+                                                            const float* __restrict__ b_cat,
+                                                            const float* __restrict__ col_scale,
+                                                            const float* __restrict__ res, float* __restrict__ y,
+                                                            int M, int N, int K, int R) {
+  __shared__ float sX[F_BK][F_BM + 1];
+  __shared__ float sW[F_BK][F_BN + 1];
+  __shared__ float sT[F_BM][F_RMAX + 1];
+  const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+  const int m0 = blockIdx.y * F_BM, n0 = blockIdx.x * F_BN;
+  float acc[4][4] = {};
+
+  // shrink: T[r_local, 0..R) for the 64 rows of this block; thread (ty,tx): rows ty*4.., ranks tx, tx+16, ...
+  for (int rb = 0; rb < R; rb += F_BN) {
+    float t[4][4] = {};
+    for (int k0 = 0; k0 < K; k0 += F_BK) {
+      for (int c = tid; c < F_BM * F_BK; c += 256) {
+        const int r = c / F_BK, kk = c % F_BK;
+        const int gr = min(m0 + r, M - 1), gk = k0 + kk;
+        sX[kk][r] = gk < K ? x[(size_t)gr * K + gk] : 0.f;
+      }
+      for (int c = tid; c < F_BN * F_BK; c += 256) {
+        const int r = c / F_BK, kk = c % F_BK;
+        const int gr = rb + r, gk = k0 + kk;
+        sW[kk][r] = (gr < R && gk < K) ? a_cat[(size_t)gr * K + gk] : 0.f;
+      }
+      __syncthreads();
+#pragma unroll
+      for (int kk = 0; kk < F_BK; ++kk) {
+        float xv[4], av[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) xv[i] = sX[kk][ty * 4 + i];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) av[j] = sW[kk][tx + 16 * j];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) t[i][j] = fmaf(xv[i], av[j], t[i][j]);
+      }
+      __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int rr = rb + tx + 16 * j;
+        if (rr < R) sT[ty * 4 + i][rr] = t[i][j] * col_scale[rr];
+      }
+  }
+  __syncthreads();
+
+  for (int k0 = 0; k0 < K; k0 += F_BK) {
+    for (int c = tid; c < F_BM * F_BK; c += 256) {
+      const int r = c / F_BK, kk = c % F_BK;
+      const int gr = min(m0 + r, M - 1), gk = k0 + kk;
+      sX[kk][r] = gk < K ? x[(size_t)gr * K + gk] : 0.f;
+    }
+    for (int c = tid; c < F_BN * F_BK; c += 256) {
+      const int r = c / F_BK, kk = c % F_BK;
+      const int gr = min(n0 + r, N - 1), gk = k0 + kk;
+      sW[kk][r] = gk < K ? w[(size_t)gr * K + gk] : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < F_BK; ++kk) {
+      float xv[4], wv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) xv[i] = sX[kk][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) wv[j] = sW[kk][tx + 16 * j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(xv[i], wv[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+  // expand: acc += T . B_cat^T
+  for (int r0 = 0; r0 < R; r0 += F_BK) {
+    for (int c = tid; c < F_BN * F_BK; c += 256) {
+      const int r = c / F_BK, kk = c % F_BK;
+      const int gr = min(n0 + r, N - 1), gk = r0 + kk;
+      sW[kk][r] = gk < R ? b_cat[(size_t)gr * R + gk] : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < F_BK; ++kk) {
+      if (r0 + kk < R) {
+        float tv[4], bv[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) tv[i] = sT[ty * 4 + i][r0 + kk];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) bv[j] = sW[kk][tx + 16 * j];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(tv[i], bv[j], acc[i][j]);
+      }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int gr = m0 + ty * 4 + i;
+    if (gr >= M) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int gc = n0 + tx + 16 * j;
+      if (gc >= N) continue;
+      float v = acc[i][j] + (bias ? bias[gc] : 0.f);
+      if (res) v += res[(size_t)gr * N + gc];
+      y[(size_t)gr * N + gc] = v;
+    }
+  }
+}
+
+}  // namespace
+
+// See include/katz_hip.h for the contract.
+KH_EXPORT int kh_lora_linear_bf16(const void* x, const void* w, const void* bias, const void* a_cat,
+                                  const void* b_cat, const float* col_scale, const void* residual, void* y,
+                                  int64_t M, int64_t N, int64_t K, int64_t R, int flags, void* stream) {
+  if (!x || !w || !y || M <= 0 || N <= 0 || K <= 0 || R < 0) return KH_ERR_INVALID_ARG;
+  if (R > 0 && (!a_cat || !b_cat || !col_scale)) return KH_ERR_INVALID_ARG;
+  if (K % 8 != 0 || N % 8 != 0 || R % 32 != 0) return KH_ERR_UNSUPPORTED;
+  if (R > 128) return KH_ERR_TOO_LARGE;
+  if (M > (1 << 24) || N > (1 << 24) || K > (1 << 24)) return KH_ERR_TOO_LARGE;
+  const bool geglu = (flags & 1) != 0;
+  if (geglu && (N % 64 != 0 || residual != nullptr)) return KH_ERR_UNSUPPORTED;
+  if (!kh_aligned16(x) || !kh_aligned16(w) || !kh_aligned16(y) || (R > 0 && (!kh_aligned16(a_cat) || !kh_aligned16(b_cat))) ||
+      (residual && !kh_aligned16(residual)))
+    return KH_ERR_ALIGNMENT;
+  LoraGemmParams p;
+  p.x = (const bf16_t*)x; p.w = (const bf16_t*)w; p.bias = (const bf16_t*)bias;
+  p.a_cat = (const bf16_t*)a_cat; p.b_cat = (const bf16_t*)b_cat; p.col_scale = col_scale;
+  p.res = (const bf16_t*)residual; p.y = (bf16_t*)y;
+  p.M = (int)M; p.N = (int)N; p.K = (int)K; p.R = (int)R;
+  p.m_tiles = p.n_tiles = p.n_chunk = p.n_chunks = 0;
+  p.geglu = geglu ? 1 : 0;
+  hipStream_t s = (hipStream_t)stream;
+  const int tile_sel = (flags >> 8) & 0xff;  // 0 = automatic
+  if (tile_sel == 2) return R > 96 ? KH_ERR_UNSUPPORTED : launch_rank<256, 128, 2, 2>(p, s);
+  if (tile_sel == 1) return launch_rank<128, 128, 2, 2>(p, s);
+  return launch_rank<128, 128, 2, 2>(p, s);
+}
+
+KH_EXPORT int kh_lora_linear_f32(const float* x, const float* w, const float* bias, const float* a_cat,
+                                 const float* b_cat, const float* col_scale, const float* residual, float* y,
+                                 int64_t M, int64_t N, int64_t K, int64_t R, void* stream) {
+  if (!x || !w || !y || M <= 0 || N <= 0 || K <= 0 || R < 0) return KH_ERR_INVALID_ARG;
+  if (R > 0 && (!a_cat || !b_cat || !col_scale)) return KH_ERR_INVALID_ARG;
+  if (R > F_RMAX) return KH_ERR_TOO_LARGE;
+  dim3 grid((unsigned)((N + F_BN - 1) / F_BN), (unsigned)((M + F_BM - 1) / F_BM));
+  hipLaunchKernelGGL(lora_gemm_f32_kernel, grid, dim3(256), 0, (hipStream_t)stream, x, w, bias, a_cat, b_cat,
+                     col_scale, residual, y, (int)M, (int)N, (int)K, (int)R);
+  KH_RETURN_LAST_ERROR();
+}

@@ -1,0 +1,106 @@
+"""Host side of the LoRA surface: adapter registry per layer and the packed layout the kernels read.
+
+The reference keeps one (lora_A, lora_B, alpha, rank, weight) set per adapter inside peft's Linear
+wrappers and turns them on / off and scales them from the host
+(set_weights_and_activate_adapters, diffusers-hf/src/diffusers/utils/peft_utils.py:238-269;
+scale_lora_layers / unscale_lora_layers :103-147).  Here the ACTIVE adapters of a layer are packed
+once per activation change into
+
+    A_cat [R, in]   rows of all active A_i stacked, zero padded to R % 32 == 0
+    B_cat [out, R]  columns of all active B_i side by side, zero padded
+    col_scale [R]   fp32, weight_i * alpha_i / rank_i * global_scale for the columns of adapter i
+
+so that sum_i s_i B_i A_i x is ONE rank-R product inside the fused kernel, and changing a scale only
+rewrites col_scale.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence
+
+import torch
+
+RANK_PAD = 32
+MAX_PACKED_RANK = 128
+
+
+@dataclass
+class Adapter:
+    """One LoRA on one layer: down = lora_A [r, in], up = lora_B [out, r]
+    (LoRALinearLayer.down/up, diffusers-hf/src/diffusers/models/lora.py:210-211)."""
+
+    down: torch.Tensor
+    up: torch.Tensor
+    alpha: Optional[float] = None  # network_alpha; None means alpha == rank (lora.py:227-228)
+    weight: float = 1.0            # set_adapters weight
+
+    @property
+    def rank(self) -> int:
+        return self.down.shape[0]
+
+    def multiplier(self, global_scale: float = 1.0) -> float:
+        a = self.rank if self.alpha is None else self.alpha
+        return float(self.weight) * float(a) / float(self.rank) * float(global_scale)
+
+
+@dataclass
+class PackedAdapters:
+    a_cat: torch.Tensor
+    b_cat: torch.Tensor
+    col_scale: torch.Tensor
+    spans: List[tuple] = field(default_factory=list)  # (name, first column, rank)
+
+    @property
+    def R(self) -> int:
+        return self.a_cat.shape[0]
+
+
+def interleave_geglu_rows(t: torch.Tensor) -> torch.Tensor:
+    """Reorder the output-feature axis (dim 0) of a GEGLU projection tensor from
+    [value(0..D) | gate(0..D)] (hidden, gate = proj(x).chunk(2, -1),
+    diffusers-hf/src/diffusers/models/activations.py:148) to blocks of 32 value rows followed by
+    their 32 gate rows, the order the fused GEGLU epilogue consumes."""
+    two_d = t.shape[0]
+    D = two_d // 2
+    if two_d % 64 != 0:
+        raise ValueError("GEGLU interleave needs 2*D % 64 == 0")
+    v = t[:D].reshape(D // 32, 1, 32, *t.shape[1:])
+    g = t[D:].reshape(D // 32, 1, 32, *t.shape[1:])
+    return torch.cat([v, g], dim=1).reshape(t.shape).contiguous()
+
+
+def pack_adapters(adapters: Dict[str, Adapter], active: Sequence[str], in_features: int, out_features: int,
+                  dtype, device, global_scale: float = 1.0, geglu_interleave: bool = False) -> Optional[PackedAdapters]:
+    """Build A_cat / B_cat / col_scale for the active adapters (in the given order). Returns None when
+    nothing is active (the layer then runs as a plain Linear, like peft with adapters disabled)."""
+    names = [n for n in active if n in adapters]
+    if not names:
+        return None
+    total = sum(adapters[n].rank for n in names)
+    R = (total + RANK_PAD - 1) // RANK_PAD * RANK_PAD
+    if R > MAX_PACKED_RANK:
+        raise ValueError(f"sum of active ranks {total} exceeds the fused kernel's maximum {MAX_PACKED_RANK}")
+    a_cat = torch.zeros((R, in_features), dtype=dtype, device=device)
+    b_cat = torch.zeros((out_features, R), dtype=dtype, device=device)
+    col_scale = torch.zeros((R,), dtype=torch.float32, device=device)
+    spans, c = [], 0
+    for n in names:
+        ad = adapters[n]
+        r = ad.rank
+        if ad.down.shape != (r, in_features) or ad.up.shape != (out_features, r):
+            raise ValueError(f"adapter {n!r}: down {tuple(ad.down.shape)} / up {tuple(ad.up.shape)} do not fit "
+                             f"a [{out_features},{in_features}] layer")
+        a_cat[c:c + r] = ad.down.to(device=device, dtype=dtype)
+        b_cat[:, c:c + r] = ad.up.to(device=device, dtype=dtype)
+        col_scale[c:c + r] = ad.multiplier(global_scale)
+        spans.append((n, c, r))
+        c += r
+    if geglu_interleave:
+        b_cat = interleave_geglu_rows(b_cat)
+    return PackedAdapters(a_cat, b_cat, col_scale, spans)
+
+
+def rescale_(packed: PackedAdapters, adapters: Dict[str, Adapter], global_scale: float = 1.0) -> None:
+    """Rewrite col_scale only (scale_lora_layers / set_adapters weight change); A_cat/B_cat stay put."""
+    for n, c, r in packed.spans:
+        packed.col_scale[c:c + r] = adapters[n].multiplier(global_scale)

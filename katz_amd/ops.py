@@ -1,0 +1,283 @@
+"""Tensor-level wrappers over the katz_hip C ABI.
+
+Every function validates shapes / dtypes / device, passes raw device pointers and torch's current
+HIP stream to the library, and returns torch tensors.  Work is enqueued on the current stream, so the
+calls compose with other torch ops and with torch.cuda.graph capture.  Nothing here computes on the
+CPU: without a GPU (or without the built library) the functions raise.
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+from typing import Optional, Sequence
+
+import torch
+
+from . import _lib
+
+BF16 = torch.bfloat16
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _req(t: torch.Tensor, dtype, name: str) -> None:
+    if not t.is_cuda:
+        raise _lib.KatzHipError(f"{name} must live on the GPU (got {t.device}); katz_hip has no CPU path")
+    if t.dtype != dtype:
+        raise TypeError(f"{name} must be {dtype}, got {t.dtype}")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+
+
+# --------------------------------------------------------------------------------------- K1
+def lora_linear(
+    x: torch.Tensor,
+    weight: torch.Tensor,
+    bias: Optional[torch.Tensor] = None,
+    a_cat: Optional[torch.Tensor] = None,
+    b_cat: Optional[torch.Tensor] = None,
+    col_scale: Optional[torch.Tensor] = None,
+    residual: Optional[torch.Tensor] = None,
+    geglu: bool = False,
+    tile: int = 0,
+    out: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """y = x W^T + b + ((x A_cat^T) * col_scale) B_cat^T (+ residual); bf16 or fp32 by x.dtype.
+
+    a_cat [R,K], b_cat [N,R], col_scale [R] fp32 describe the active adapters concatenated along the
+    rank axis (R % 32 == 0 for bf16).  With geglu=True the rows of weight / bias / b_cat must be in the
+    interleaved (32 value, 32 gate) order produced by `katz_amd.lora.interleave_geglu_rows`.
+    """
+    lib = _lib.load()
+    K = x.shape[-1]
+    N = weight.shape[0]
+    M = x.numel() // K
+    dt = x.dtype
+    _req(x, dt, "x"); _req(weight, dt, "weight")
+    if weight.shape[1] != K:
+        raise ValueError(f"weight {tuple(weight.shape)} does not match x[..., {K}]")
+    R = 0
+    if a_cat is not None:
+        _req(a_cat, dt, "a_cat"); _req(b_cat, dt, "b_cat"); _req(col_scale, torch.float32, "col_scale")
+        R = a_cat.shape[0]
+        if a_cat.shape != (R, K) or b_cat.shape != (N, R) or col_scale.shape != (R,):
+            raise ValueError("a_cat/b_cat/col_scale shapes must be [R,K], [N,R], [R]")
+    if bias is not None:
+        _req(bias, dt, "bias")
+    n_out = N // 2 if geglu else N
+    out_shape = tuple(x.shape[:-1]) + (n_out,)
+    if residual is not None:
+        _req(residual, dt, "residual")
+        if residual.numel() != M * N:
+            raise ValueError("residual must have the shape of the output")
+    if out is None:
+        out = torch.empty(out_shape, dtype=dt, device=x.device)
+    else:
+        _req(out, dt, "out")
+        if out.numel() != M * n_out:
+            raise ValueError("out has the wrong size")
+    if dt == BF16:
+        flags = (1 if geglu else 0) | ((tile & 0xFF) << 8)
+        rc = lib.kh_lora_linear_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(a_cat), _ptr(b_cat), _ptr(col_scale),
+                                     _ptr(residual), _ptr(out), M, N, K, R, flags, _stream())
+    elif dt == torch.float32:
+        if geglu:
+            raise ValueError("the GEGLU epilogue exists for bf16 only")
+        rc = lib.kh_lora_linear_f32(_ptr(x), _ptr(weight), _ptr(bias), _ptr(a_cat), _ptr(b_cat), _ptr(col_scale),
+                                    _ptr(residual), _ptr(out), M, N, K, R, _stream())
+    else:
+        raise TypeError(f"lora_linear supports bfloat16 and float32, got {dt}")
+    _lib.check(rc, "kh_lora_linear")
+    return out
+
+
+# --------------------------------------------------------------------------------------- K2
+def sgmv_shrink(x, a_all, seg_start, seg_adapter, adapter_rank, max_seg_rows: int, out=None):
+    """t[rows, :r_a] = x[rows] A_a^T per segment. a_all [n_adapters, RP, K]; returns t [rows, RP]."""
+    lib = _lib.load()
+    _req(x, BF16, "x"); _req(a_all, BF16, "a_all")
+    for n, t in (("seg_start", seg_start), ("seg_adapter", seg_adapter), ("adapter_rank", adapter_rank)):
+        _req(t, torch.int32, n)
+    rows, K = x.shape
+    RP = a_all.shape[1]
+    if a_all.shape[2] != K:
+        raise ValueError("a_all must be [n_adapters, RP, K]")
+    if out is None:
+        out = torch.zeros((rows, RP), dtype=BF16, device=x.device)
+    nseg = seg_adapter.numel()
+    rc = lib.kh_sgmv_shrink_bf16(_ptr(x), _ptr(a_all), _ptr(out), _ptr(seg_start), _ptr(seg_adapter),
+                                 _ptr(adapter_rank), nseg, max_seg_rows, K, RP, _stream())
+    _lib.check(rc, "kh_sgmv_shrink_bf16")
+    return out
+
+
+def sgmv_expand_(y, t, b_all, seg_start, seg_adapter, adapter_rank, adapter_scale, max_seg_rows: int):
+    """y[rows] += scale_a * t[rows, :r_a] B_a^T per segment, in place. b_all [n_adapters, N, RP]."""
+    lib = _lib.load()
+    _req(y, BF16, "y"); _req(t, BF16, "t"); _req(b_all, BF16, "b_all"); _req(adapter_scale, torch.float32, "adapter_scale")
+    rows, N = y.shape
+    RP = b_all.shape[2]
+    if b_all.shape[1] != N or t.shape != (rows, RP):
+        raise ValueError("b_all must be [n_adapters, N, RP] and t [rows, RP]")
+    nseg = seg_adapter.numel()
+    rc = lib.kh_sgmv_expand_bf16(_ptr(t), _ptr(b_all), _ptr(y), _ptr(seg_start), _ptr(seg_adapter),
+                                 _ptr(adapter_rank), _ptr(adapter_scale), nseg, max_seg_rows, N, RP, _stream())
+    _lib.check(rc, "kh_sgmv_expand_bf16")
+    return y
+
+
+# --------------------------------------------------------------------------------------- K3
+def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, heads: int, scale: Optional[float] = None,
+              out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """softmax(q k^T * scale) v. q [B,T,H*64], k/v [B,S,H*64] (last-dim-contiguous views allowed)."""
+    lib = _lib.load()
+    B, T, inner = q.shape
+    S = k.shape[1]
+    hd = inner // heads
+    for n, t in (("q", q), ("k", k), ("v", v)):
+        if not t.is_cuda:
+            raise _lib.KatzHipError(f"{n} must live on the GPU; katz_hip has no CPU path")
+        if t.dtype != BF16 or t.stride(-1) != 1:
+            raise TypeError(f"{n} must be bfloat16 with a contiguous last axis")
+    if k.shape != (B, S, inner) or v.shape != (B, S, inner):
+        raise ValueError("k and v must be [B,S,H*head_dim]")
+    if scale is None:
+        scale = 1.0 / math.sqrt(hd)
+    if out is None:
+        out = torch.empty((B, T, inner), dtype=BF16, device=q.device)
+    rc = lib.kh_attention_bf16(_ptr(q), _ptr(k), _ptr(v), _ptr(out), B, heads, T, S, hd,
+                               q.stride(1), k.stride(1), v.stride(1), out.stride(1),
+                               q.stride(0), k.stride(0), v.stride(0), out.stride(0), float(scale), _stream())
+    _lib.check(rc, "kh_attention_bf16")
+    return out
+
+
+# --------------------------------------------------------------------------------------- K4
+_gn_workspace: dict = {}
+
+
+def _workspace(nbytes: int, device) -> torch.Tensor:
+    """One grow-only fp32 scratch buffer per device (allocated outside graph capture on first use)."""
+    key = (device.type, device.index)
+    buf = _gn_workspace.get(key)
+    if buf is None or buf.numel() * 4 < nbytes:
+        buf = torch.empty(max(nbytes // 4, 1 << 16), dtype=torch.float32, device=device)
+        _gn_workspace[key] = buf
+    return buf
+
+
+def group_norm(x: torch.Tensor, num_groups: int, weight: Optional[torch.Tensor], bias: Optional[torch.Tensor],
+               eps: float, activation: str = "none", out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """GroupNorm(+SiLU) of a 4-D [N,C,H,W] tensor, either contiguous (NCHW) or channels_last (NHWC
+    memory); the output has the memory format of the input."""
+    lib = _lib.load()
+    if activation not in ("none", "silu"):
+        raise ValueError(f"unknown activation {activation!r}")  # the reference only printf's here
+    if not x.is_cuda:
+        raise _lib.KatzHipError("x must live on the GPU; katz_hip has no CPU path")
+    if x.dtype != BF16 or x.dim() != 4:
+        raise TypeError("group_norm expects a 4-D bfloat16 tensor")
+    N, C, H, W = x.shape
+    is_cl, is_cf = x.is_contiguous(memory_format=torch.channels_last), x.is_contiguous()
+    if not (is_cl or is_cf):
+        raise ValueError("x must be contiguous in NCHW or channels_last memory format")
+    # both hold only when the two layouts coincide (C == 1 or H*W == 1): take whichever the kernels accept
+    cl = 1 if (is_cl and (not is_cf or C % 8 == 0)) else 0
+    if out is None:
+        out = torch.empty_like(x)  # preserves the memory format
+    elif out.stride() != x.stride() or out.dtype != BF16:
+        raise ValueError("out must match x in dtype and strides")
+    nbytes = lib.kh_group_norm_workspace_bytes(N, C, H * W, num_groups, cl)
+    if nbytes < 0:
+        _lib.check(int(nbytes), "kh_group_norm_workspace_bytes")
+    ws = _workspace(int(nbytes), x.device)
+    rc = lib.kh_group_norm_bf16(_ptr(x), _ptr(out), _ptr(weight), _ptr(bias), _ptr(ws), N, C, H * W, num_groups,
+                                float(eps), 1 if activation == "silu" else 0, cl, _stream())
+    _lib.check(rc, "kh_group_norm_bf16")
+    return out
+
+
+def layer_norm(x: torch.Tensor, weight: Optional[torch.Tensor], bias: Optional[torch.Tensor], eps: float = 1e-5,
+               out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    lib = _lib.load()
+    _req(x, BF16, "x")
+    D = x.shape[-1]
+    M = x.numel() // D
+    if out is None:
+        out = torch.empty_like(x)
+    rc = lib.kh_layer_norm_bf16(_ptr(x), _ptr(out), _ptr(weight), _ptr(bias), M, D, float(eps), _stream())
+    _lib.check(rc, "kh_layer_norm_bf16")
+    return out
+
+
+# --------------------------------------------------------------------------------------- K5
+def geglu(proj: torch.Tensor, approximate: str = "none") -> torch.Tensor:
+    """value * gelu(gate) with [value | gate] = proj.chunk(2, -1)."""
+    lib = _lib.load()
+    _req(proj, BF16, "proj")
+    D = proj.shape[-1] // 2
+    M = proj.numel() // (2 * D)
+    out = torch.empty(tuple(proj.shape[:-1]) + (D,), dtype=BF16, device=proj.device)
+    rc = lib.kh_geglu_bf16(_ptr(proj), _ptr(out), M, D, 1 if approximate == "tanh" else 0, _stream())
+    _lib.check(rc, "kh_geglu_bf16")
+    return out
+
+
+def gelu_mul(x: torch.Tensor, m: torch.Tensor, approximate: str = "tanh") -> torch.Tensor:
+    """gelu(x) * m -- the argument order and tanh default of fast_kernel.fast_gelu_mul_fp16(x, m)."""
+    lib = _lib.load()
+    _req(x, BF16, "x"); _req(m, BF16, "m")
+    if x.shape != m.shape:
+        raise ValueError("x and m must have the same shape")
+    out = torch.empty_like(x)
+    rc = lib.kh_gelu_mul_bf16(_ptr(x), _ptr(m), _ptr(out), x.numel(), 1 if approximate == "tanh" else 0, _stream())
+    _lib.check(rc, "kh_gelu_mul_bf16")
+    return out
+
+
+# --------------------------------------------------------------------------------------- residuals
+def _ptr_array(ts: Sequence[torch.Tensor]):
+    arr = (ctypes.c_void_p * max(len(ts), 1))()
+    for i, t in enumerate(ts):
+        arr[i] = t.data_ptr()
+    return arr
+
+
+def residual_add_(dst: torch.Tensor, residuals: Sequence[torch.Tensor]) -> torch.Tensor:
+    """dst += mean_k(residuals[k]) in place (one residual: a plain add).  All tensors must share dst's
+    memory layout."""
+    lib = _lib.load()
+    if not dst.is_cuda or dst.dtype != BF16:
+        raise _lib.KatzHipError("dst must be a bfloat16 GPU tensor; katz_hip has no CPU path")
+    for r in residuals:
+        if r.shape != dst.shape or r.stride() != dst.stride() or r.dtype != BF16:
+            raise ValueError("every residual must match dst in shape, strides and dtype")
+    rc = lib.kh_residual_add_bf16(_ptr(dst), _ptr_array(residuals), len(residuals), 1.0 / len(residuals),
+                                  dst.numel(), _stream())
+    _lib.check(rc, "kh_residual_add_bf16")
+    return dst
+
+
+def concat_residual(h: torch.Tensor, skip: torch.Tensor, residuals: Sequence[torch.Tensor] = ()) -> torch.Tensor:
+    """cat([h, skip + mean_k residuals[k]], dim=1) for channels_last 4-D tensors."""
+    lib = _lib.load()
+    for n, t in (("h", h), ("skip", skip), *[("residual", r) for r in residuals]):
+        if not t.is_cuda or t.dtype != BF16 or t.dim() != 4 or not t.is_contiguous(memory_format=torch.channels_last):
+            raise ValueError(f"{n} must be a channels_last bfloat16 GPU tensor")
+    N, C1, H, W = h.shape
+    C2 = skip.shape[1]
+    for r in residuals:
+        if r.shape != skip.shape:
+            raise ValueError("residuals must have the shape of skip")
+    out = torch.empty((N, C1 + C2, H, W), dtype=BF16, device=h.device, memory_format=torch.channels_last)
+    inv = 1.0 / len(residuals) if residuals else 1.0
+    rc = lib.kh_concat_residual_bf16(_ptr(h), _ptr(skip), _ptr_array(residuals), len(residuals), inv, _ptr(out),
+                                     N * H * W, C1, C2, _stream())
+    _lib.check(rc, "kh_concat_residual_bf16")
+    return out

@@ -1,0 +1,383 @@
+"""Parity of every katz_hip kernel (through the C ABI) against the CPU oracle on seeded inputs.
+
+Tolerances: bf16 kernels -- elementwise |err| <= 2e-2 * (|ref| + rms(ref)) against the oracle evaluated
+in fp32 on the same bf16-rounded inputs; fp32 path -- 1e-4; pure data movement / single-rounding adds --
+bit exact.
+"""
+import math
+
+import pytest
+import torch
+
+from helpers import assert_close_rel, bf16_round
+from oracle import ops as O
+
+pytestmark = pytest.mark.gpu
+
+BF = torch.bfloat16
+REL_BF16 = 2e-2
+
+
+def dev():
+    return torch.device("cuda:0")
+
+
+def randn(gen, *shape, std=1.0):
+    return bf16_round(torch.randn(*shape, generator=gen) * std)
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+# ------------------------------------------------------------------------------------------- K1
+def _lora_case(M, N, K, ranks, scales, bias=True, residual=False, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    x = randn(g, M, K)
+    w = randn(g, N, K, std=0.02)
+    b = randn(g, N, std=0.02) if bias else None
+    adapters = []
+    for r, s in zip(ranks, scales):
+        adapters.append((randn(g, r, K, std=0.02), randn(g, N, r, std=0.02), s))
+    res = randn(g, M, N) if residual else None
+    return x, w, b, adapters, res
+
+
+def _run_lora(x, w, b, adapters, res, geglu=False, tile=0):
+    from katz_amd import ops
+    from katz_amd.lora import Adapter, pack_adapters
+
+    d = dev()
+    N, K = w.shape
+    ads = {f"a{i}": Adapter(A, B, alpha=None, weight=s) for i, (A, B, s) in enumerate(adapters)}
+    packed = pack_adapters(ads, list(ads), K, N, BF, d, geglu_interleave=geglu) if ads else None
+    wd, bd = w, b
+    if geglu:
+        from katz_amd.lora import interleave_geglu_rows
+        wd = interleave_geglu_rows(w)
+        bd = interleave_geglu_rows(b) if b is not None else None
+    y = ops.lora_linear(
+        x.to(d, BF), wd.to(d, BF), None if bd is None else bd.to(d, BF),
+        None if packed is None else packed.a_cat, None if packed is None else packed.b_cat,
+        None if packed is None else packed.col_scale, None if res is None else res.to(d, BF),
+        geglu=geglu, tile=tile)
+    torch.cuda.synchronize()
+    return y
+
+
+LORA_SHAPES = [
+    # M, N, K, ranks, scales, bias, residual
+    (2048, 1280, 1280, (64,), (1.0,), False, False),      # to_q at 32x32, one rank-64 adapter
+    (8192, 640, 640, (64, 32), (0.8, 0.6), True, True),   # to_out.0 at 64x64, two adapters + residual
+    (154, 1280, 2048, (64, 32), (0.8, 0.6), False, False),  # cross-attention to_k / to_v (77 tokens x 2)
+    (2048, 1280, 5120, (64, 32), (0.8, 0.6), True, True),   # ff.net.2
+    (8192, 640, 640, (), (), True, False),                  # adapter-free
+    (100, 136, 72, (8,), (2.0,), True, True),               # ragged: partial tiles in M, N, K and rank padding
+    (1, 8, 8, (16, 8, 4), (1.0, 0.5, 0.25), True, False),   # minimum sizes
+    (300, 1280, 320, (128,), (1.0,), True, False),          # maximum packed rank
+]
+
+
+@pytest.mark.parametrize("tile", [1, 2])
+@pytest.mark.parametrize("case", LORA_SHAPES, ids=lambda c: f"M{c[0]}N{c[1]}K{c[2]}r{'+'.join(map(str, c[3])) or '0'}")
+def test_lora_linear_bf16(case, tile):
+    M, N, K, ranks, scales, bias, residual = case
+    if tile == 2 and sum(ranks) > 96:
+        pytest.skip("256x128 tile is built for packed rank <= 96")
+    say("lora_linear_bf16", case, "tile", tile)
+    x, w, b, adapters, res = _lora_case(M, N, K, ranks, scales, bias, residual)
+    y = _run_lora(x, w, b, adapters, res, tile=tile)
+    ref = O.lora_linear(x, w, b, adapters, res)
+    assert_close_rel(y, ref, REL_BF16, "lora_linear_bf16")
+    # merge identity: the same result as a plain linear with W + sum s B A
+    ref2 = torch.nn.functional.linear(x, O.lora_merged_weight(w, adapters), b)
+    if res is not None:
+        ref2 = ref2 + res
+    assert_close_rel(y, ref2, REL_BF16, "lora_linear_bf16 vs merged weight")
+
+
+def test_lora_linear_bf16_scale_zero_is_base():
+    say("lora_linear_bf16 scale 0")
+    x, w, b, adapters, _ = _lora_case(512, 640, 640, (64,), (0.0,), True, False, seed=3)
+    y0 = _run_lora(x, w, b, adapters, None)
+    y1 = _run_lora(x, w, b, [], None)
+    assert torch.equal(y0, y1)
+
+
+def test_lora_linear_bf16_geglu_epilogue():
+    say("lora_linear_bf16 geglu")
+    M, K, D = 2048, 1280, 5120
+    x, w, b, adapters, _ = _lora_case(M, 2 * D, K, (64,), (1.0,), True, False, seed=5)
+    y = _run_lora(x, w, b, adapters, None, geglu=True)
+    proj = bf16_round(O.lora_linear(x, w, b, adapters))
+    ref = O.geglu(proj)
+    assert y.shape == (M, D)
+    assert_close_rel(y, ref, REL_BF16, "geglu epilogue")
+
+
+def test_lora_linear_f32_config1():
+    """BASELINE config 1: x [2,4096,640], W [640,640], rank 32, scale 0.8, fp32, <= 1e-4."""
+    from katz_amd import ops
+
+    say("lora_linear_f32 config1")
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(2, 4096, 640, generator=g)
+    w = torch.randn(640, 640, generator=g) * 0.02
+    b = torch.randn(640, generator=g) * 0.02
+    A = torch.randn(32, 640, generator=g) * 0.02
+    Bm = torch.randn(640, 32, generator=g) * 0.02
+    d = dev()
+    cs = torch.full((32,), 0.8, dtype=torch.float32, device=d)
+    y = ops.lora_linear(x.to(d), w.to(d), b.to(d), A.to(d), Bm.to(d).contiguous(), cs)
+    torch.cuda.synchronize()
+    ref = O.lora_linear(x.double(), w.double(), b.double(), [(A.double(), Bm.double(), 0.8)]).float()
+    err = (y.cpu() - ref).abs().max().item()
+    rel = err / ref.abs().max().item()
+    assert y.shape == (2, 4096, 640)
+    assert err <= 1e-4 and rel <= 1e-4, (err, rel)
+
+
+def test_lora_linear_f32_ragged():
+    from katz_amd import ops
+
+    say("lora_linear_f32 ragged")
+    g = torch.Generator().manual_seed(1)
+    M, N, K, r = 70, 50, 37, 5
+    x = torch.randn(M, K, generator=g); w = torch.randn(N, K, generator=g) * 0.1
+    A = torch.randn(r, K, generator=g) * 0.1; Bm = torch.randn(N, r, generator=g) * 0.1
+    res = torch.randn(M, N, generator=g)
+    d = dev()
+    cs = torch.full((r,), 1.5, dtype=torch.float32, device=d)
+    y = ops.lora_linear(x.to(d), w.to(d), None, A.to(d), Bm.to(d), cs, residual=res.to(d))
+    torch.cuda.synchronize()
+    ref = O.lora_linear(x.double(), w.double(), None, [(A.double(), Bm.double(), 1.5)], res.double()).float()
+    assert (y.cpu() - ref).abs().max().item() <= 1e-4
+
+
+# ------------------------------------------------------------------------------------------- K3
+ATTN_SHAPES = [
+    # B, H, T, S
+    (1, 2, 4096, 4096),   # self-attention at 64x64 (two of the ten heads)
+    (2, 20, 1024, 1024),  # self-attention at 32x32, full head count
+    (2, 10, 4096, 77),    # cross-attention at 64x64
+    (2, 20, 1024, 77),    # cross-attention at 32x32
+    (1, 1, 100, 77),      # ragged query block and key tile
+    (2, 3, 130, 200),
+    (1, 1, 1, 1),
+]
+
+
+@pytest.mark.parametrize("shape", ATTN_SHAPES, ids=lambda s: "B%dH%dT%dS%d" % s)
+def test_attention_bf16(shape):
+    from katz_amd import ops
+
+    B, H, T, S = shape
+    say("attention_bf16", shape)
+    g = torch.Generator().manual_seed(7)
+    q = randn(g, B, T, H * 64); k = randn(g, B, S, H * 64); v = randn(g, B, S, H * 64)
+    d = dev()
+    o = ops.attention(q.to(d, BF), k.to(d, BF), v.to(d, BF), H)
+    torch.cuda.synchronize()
+    ref = O.attention(q, k, v, H)
+    assert_close_rel(o, ref, REL_BF16, "attention_bf16")
+
+
+def test_attention_bf16_strided_views():
+    """q/k/v as column slices of one fused [B,T,3*H*64] projection buffer."""
+    from katz_amd import ops
+
+    say("attention_bf16 strided")
+    B, H, T = 2, 5, 333
+    g = torch.Generator().manual_seed(8)
+    qkv = randn(g, B, T, 3 * H * 64)
+    d = dev()
+    qkv_d = qkv.to(d, BF)
+    q, k, v = qkv_d.split(H * 64, dim=-1)
+    o = ops.attention(q, k, v, H)
+    torch.cuda.synchronize()
+    qr, kr, vr = qkv.split(H * 64, dim=-1)
+    ref = O.attention(qr.contiguous(), kr.contiguous(), vr.contiguous(), H)
+    assert_close_rel(o, ref, REL_BF16, "attention strided")
+
+
+# ------------------------------------------------------------------------------------------- K4
+GN_SHAPES = [
+    # N, C, H, W, G
+    (2, 320, 128, 128, 32),
+    (2, 960, 64, 64, 32),
+    (2, 1920, 32, 32, 32),
+    (2, 2560, 32, 32, 32),
+    (1, 32, 8, 8, 32),    # one channel per group
+    (3, 64, 5, 8, 4),
+]
+
+
+@pytest.mark.parametrize("channels_last", [True, False], ids=["nhwc", "nchw"])
+@pytest.mark.parametrize("act", ["silu", "none"])
+@pytest.mark.parametrize("shape", GN_SHAPES, ids=lambda s: "N%dC%dH%dW%dG%d" % s)
+def test_group_norm_bf16(shape, act, channels_last):
+    from katz_amd import ops
+
+    N, C, H, W, G = shape
+    say("group_norm_bf16", shape, act, "nhwc" if channels_last else "nchw")
+    g = torch.Generator().manual_seed(11)
+    x = bf16_round(torch.randn(N, C, H, W, generator=g) * 2.0 + 3.0)  # non-zero mean: exercises the variance
+    gamma = randn(g, C) + 1.0
+    beta = randn(g, C, std=0.5)
+    d = dev()
+    xd = x.to(d, BF)
+    if channels_last:
+        xd = xd.contiguous(memory_format=torch.channels_last)
+    eps = 1e-5 if act == "silu" else 1e-6
+    y = ops.group_norm(xd, G, gamma.to(d, BF), beta.to(d, BF), eps, act)
+    torch.cuda.synchronize()
+    assert y.stride() == xd.stride()
+    ref = O.group_norm(x, G, gamma, beta, eps, act)
+    assert_close_rel(y, ref, REL_BF16, "group_norm_bf16")
+
+
+def test_group_norm_no_affine():
+    from katz_amd import ops
+
+    say("group_norm no affine")
+    g = torch.Generator().manual_seed(12)
+    x = randn(g, 2, 64, 16, 16)
+    d = dev()
+    y = ops.group_norm(x.to(d, BF).contiguous(memory_format=torch.channels_last), 8, None, None, 1e-5, "none")
+    torch.cuda.synchronize()
+    assert_close_rel(y, O.group_norm(x, 8, None, None, 1e-5), REL_BF16, "group_norm no affine")
+
+
+def test_group_norm_unknown_activation_raises():
+    from katz_amd import ops
+
+    x = torch.zeros(1, 32, 8, 8, dtype=BF, device=dev())
+    with pytest.raises(ValueError):
+        ops.group_norm(x, 32, None, None, 1e-5, "relu")
+
+
+@pytest.mark.parametrize("shape", [(8192, 640), (2048, 1280), (154, 2048), (5, 8), (3, 72)], ids=str)
+def test_layer_norm_bf16(shape):
+    from katz_amd import ops
+
+    say("layer_norm_bf16", shape)
+    M, D = shape
+    g = torch.Generator().manual_seed(13)
+    x = bf16_round(torch.randn(M, D, generator=g) * 1.5 + 0.7)
+    gamma = randn(g, D) + 1.0
+    beta = randn(g, D, std=0.3)
+    d = dev()
+    y = ops.layer_norm(x.to(d, BF), gamma.to(d, BF), beta.to(d, BF), 1e-5)
+    torch.cuda.synchronize()
+    assert_close_rel(y, O.layer_norm(x, gamma, beta, 1e-5), REL_BF16, "layer_norm_bf16")
+
+
+# ------------------------------------------------------------------------------------------- K5
+@pytest.mark.parametrize("approx", ["none", "tanh"])
+@pytest.mark.parametrize("shape", [(2048, 5120), (8192, 2560), (7, 8)], ids=str)
+def test_geglu_bf16(shape, approx):
+    from katz_amd import ops
+
+    say("geglu_bf16", shape, approx)
+    M, D = shape
+    g = torch.Generator().manual_seed(17)
+    proj = randn(g, M, 2 * D, std=2.0)
+    y = ops.geglu(proj.to(dev(), BF), approx)
+    torch.cuda.synchronize()
+    assert_close_rel(y, O.geglu(proj, approx), REL_BF16, "geglu_bf16")
+
+
+def test_gelu_mul_bf16_matches_reference_argument_order():
+    from katz_amd import ops
+
+    say("gelu_mul_bf16")
+    g = torch.Generator().manual_seed(18)
+    x = randn(g, 3, 77, 40, std=2.0); m = randn(g, 3, 77, 40)
+    y = ops.gelu_mul(x.to(dev(), BF), m.to(dev(), BF))
+    torch.cuda.synchronize()
+    assert_close_rel(y, O.gelu_mul(x, m, "tanh"), REL_BF16, "gelu_mul")
+
+
+# ------------------------------------------------------------------------------------------- residuals
+@pytest.mark.parametrize("k", [1, 3])
+def test_residual_add_bf16(k):
+    from katz_amd import ops
+
+    say("residual_add_bf16", k)
+    g = torch.Generator().manual_seed(19)
+    d = dev()
+    skip = randn(g, 2, 640, 64, 64)
+    rs = [randn(g, 2, 640, 64, 64, std=0.1) for _ in range(k)]
+    dst = skip.to(d, BF).contiguous(memory_format=torch.channels_last)
+    rd = [r.to(d, BF).contiguous(memory_format=torch.channels_last) for r in rs]
+    ops.residual_add_(dst, rd)
+    torch.cuda.synchronize()
+    ref = O.residual_add(skip, rs)
+    if k == 1:
+        # one ControlNet: a single rounding, identical to the bf16 add of the reference
+        assert torch.equal(dst.cpu(), (skip.to(BF) + rs[0].to(BF)))
+    assert_close_rel(dst, ref, REL_BF16, "residual_add")
+
+
+@pytest.mark.parametrize("k", [0, 1, 2])
+def test_concat_residual_bf16(k):
+    from katz_amd import ops
+
+    say("concat_residual_bf16", k)
+    g = torch.Generator().manual_seed(23)
+    d = dev()
+    h = randn(g, 2, 1280, 32, 32); skip = randn(g, 2, 640, 32, 32)
+    rs = [randn(g, 2, 640, 32, 32, std=0.1) for _ in range(k)]
+    cl = lambda t: t.to(d, BF).contiguous(memory_format=torch.channels_last)
+    out = ops.concat_residual(cl(h), cl(skip), [cl(r) for r in rs])
+    torch.cuda.synchronize()
+    assert out.shape == (2, 1920, 32, 32) and out.is_contiguous(memory_format=torch.channels_last)
+    ref = O.concat_residual(h, skip, rs)
+    if k <= 1:
+        exp = torch.cat([h.to(BF), skip.to(BF) + rs[0].to(BF) if k else skip.to(BF)], dim=1)
+        assert torch.equal(out.cpu(), exp)
+    assert_close_rel(out, ref, REL_BF16, "concat_residual")
+
+
+# ------------------------------------------------------------------------------------------- K2
+@pytest.mark.parametrize("T,dm", [(1024, 1280), (4096, 640), (77, 640)], ids=str)
+def test_sgmv_heterogeneous_batch(T, dm):
+    """BASELINE config 4: 8 requests, each with its own adapter, ranks drawn (seed 2) from {8,16,32,64,128}."""
+    from katz_amd import ops
+
+    say("sgmv", T, dm)
+    g = torch.Generator().manual_seed(2)
+    n_req = 8
+    choices = [8, 16, 32, 64, 128]
+    ranks = [choices[i] for i in torch.randint(0, 5, (n_req,), generator=g).tolist()]
+    seg_adapter = torch.randperm(n_req, generator=g).tolist()
+    seg_adapter[3] = -1  # one request without an adapter
+    K = N = dm
+    x = randn(g, n_req * T, K)
+    w = randn(g, N, K, std=0.02)
+    adapters = [(randn(g, r, K, std=0.02), randn(g, N, r, std=0.02), 0.5 + 0.1 * i) for i, r in enumerate(ranks)]
+    seg_start = [i * T for i in range(n_req + 1)]
+    d = dev()
+    RP = 128
+    a_all = torch.zeros(n_req, RP, K); b_all = torch.zeros(n_req, N, RP)
+    for i, (A, B, _) in enumerate(adapters):
+        a_all[i, : A.shape[0]] = A
+        b_all[i, :, : B.shape[1]] = B
+    rank_pad = torch.tensor([(r + 31) // 32 * 32 for r in ranks], dtype=torch.int32, device=d)
+    scales = torch.tensor([a[2] for a in adapters], dtype=torch.float32, device=d)
+    ss = torch.tensor(seg_start, dtype=torch.int32, device=d)
+    sa = torch.tensor(seg_adapter, dtype=torch.int32, device=d)
+    xd = x.to(d, BF)
+    y = ops.lora_linear(xd, w.to(d, BF))          # base projection, adapter-free
+    y_base = y.clone()
+    t = ops.sgmv_shrink(xd, a_all.to(d, BF), ss, sa, rank_pad, T)
+    ops.sgmv_expand_(y, t, b_all.to(d, BF), ss, sa, rank_pad, scales, T)
+    torch.cuda.synchronize()
+    ref = O.sgmv(x, seg_start, seg_adapter, adapters, torch.nn.functional.linear(x, w))
+    assert_close_rel(y, ref, REL_BF16, "sgmv")
+    # the request without an adapter keeps the base projection bit for bit
+    assert torch.equal(y[3 * T:4 * T], y_base[3 * T:4 * T])
+    # shrink alone: t[:, :r] = x A^T
+    a0 = seg_adapter[0]
+    t_ref = torch.nn.functional.linear(x[:T], adapters[a0][0])
+    assert_close_rel(t[:T, : ranks[a0]], t_ref, REL_BF16, "sgmv shrink")
