@@ -36,6 +36,17 @@ int kh_version(void);
 /* Static string for a KH_ERR_* code or a hipError_t (host pointer, never NULL). */
 const char* kh_error_string(int code);
 
+/* Per-launch timing for benchmarks (no counterpart in the reference, which times whole steps with
+ * torch.cuda.synchronize + time.time, pipeline_controlnet_sd_xl_katz.py:1588-1644).  Between
+ * kh_profile_begin and kh_profile_end every kernel of this library is launched with its own HIP
+ * start/stop event pair on the launch stream.  kh_profile_end waits for them and writes, in launch
+ * order, a kernel tag (1 lora_gemm, 2 lora_gemm_f32, 3 attention, 4 group_norm stats, 5 group_norm apply,
+ * 6 layer_norm, 7 geglu, 8 residual_add, 9 concat_residual, 10 sgmv_shrink, 11 sgmv_expand) and the
+ * duration in ms into HOST arrays; returns the number of launches (or -hipError_t).  Do not use under
+ * graph capture. */
+int kh_profile_begin(void);
+int kh_profile_end(int32_t* tags, float* ms, int capacity);
+
 /* ---- K1: LoRA-patched Linear ------------------------------------------------------------------
  * y[M,N] = x[M,K] W[N,K]^T + bias[N] + ((x A_cat[R,K]^T) * col_scale[R]) B_cat[N,R]^T (+ residual[M,N])
  * Replaces base Linear + per-adapter low-rank branch of the reference:
@@ -88,13 +99,16 @@ int kh_attention_bf16(const void* q, const void* k, const void* v, void* o, int6
  * affine, channels_last) (csrc/group_norm.cu:264-274, called at
  * diffusers-hf/src/diffusers/models/normalization.py:90-91); y is caller-allocated as there.
  * activation: 0 none, 1 silu.  channels_last: 1 = x,y are [N,HW,C] (NHWC), 0 = [N,C,HW] (NCHW).
- * gamma/beta may be NULL (affine=False).  workspace: kh_group_norm_workspace_bytes(...) bytes of
+ * gamma/beta may be NULL (affine=False).  add_nc (may be NULL): bf16 [N,C] added to x per (sample,
+ * channel) before the statistics and the normalisation -- folds the resnet's `hidden_states + temb`
+ * (diffusers-hf/src/diffusers/models/resnet.py:388-390) into the norm that follows it.  workspace: kh_group_norm_workspace_bytes(...) bytes of
  * device memory owned by the caller (the reference allocates its mean/inv_variance tensors per call,
  * group_norm.cu:240-242, which is not graph-capturable).  NHWC needs C % 8 == 0, C <= 4096, G <= 512;
  * NCHW needs HW % 8 == 0. */
 int64_t kh_group_norm_workspace_bytes(int64_t N, int64_t C, int64_t HW, int64_t G, int channels_last);
-int kh_group_norm_bf16(const void* x, void* y, const void* gamma, const void* beta, float* workspace, int64_t N,
-                       int64_t C, int64_t HW, int64_t G, float eps, int activation, int channels_last, void* stream);
+int kh_group_norm_bf16(const void* x, void* y, const void* gamma, const void* beta, const void* add_nc,
+                       float* workspace, int64_t N, int64_t C, int64_t HW, int64_t G, float eps, int activation,
+                       int channels_last, void* stream);
 /* nn.LayerNorm over the last axis (norm1/2/3 of BasicTransformerBlock,
  * diffusers-hf/src/diffusers/models/attention.py:195,225,253); D % 8 == 0, D <= 2048. */
 int kh_layer_norm_bf16(const void* x, void* y, const void* gamma, const void* beta, int64_t M, int64_t D, float eps,

@@ -18,13 +18,15 @@ _I = c_int64
 SIGNATURES = {
     "kh_version": (c_int, []),
     "kh_error_string": (c_char_p, [c_int]),
+    "kh_profile_begin": (c_int, []),
+    "kh_profile_end": (c_int, [_P, _P, c_int]),
     "kh_lora_linear_bf16": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, c_int, _P]),
     "kh_lora_linear_f32": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
     "kh_sgmv_shrink_bf16": (c_int, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
     "kh_sgmv_expand_bf16": (c_int, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
     "kh_attention_bf16": (c_int, [_P, _P, _P, _P] + [_I] * 13 + [c_float, _P]),
     "kh_group_norm_workspace_bytes": (c_int64, [_I, _I, _I, _I, c_int]),
-    "kh_group_norm_bf16": (c_int, [_P, _P, _P, _P, _P, _I, _I, _I, _I, c_float, c_int, c_int, _P]),
+    "kh_group_norm_bf16": (c_int, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, c_float, c_int, c_int, _P]),
     "kh_layer_norm_bf16": (c_int, [_P, _P, _P, _P, _I, _I, c_float, _P]),
     "kh_geglu_bf16": (c_int, [_P, _P, _I, _I, c_int, _P]),
     "kh_gelu_mul_bf16": (c_int, [_P, _P, _P, _I, c_int, _P]),
@@ -49,6 +51,10 @@ def load() -> ctypes.CDLL:
             f"{LIB_PATH} is missing: build the HIP kernels with `python -m katz_amd.build` "
             "(needs hipcc); there is no CPU fallback for these ops"
         )
+    # torch first: its HIP runtime must be the one this process initialises.  If libkatz_hip.so pulls in
+    # a HIP runtime of its own before torch is imported, launches fail with hipErrorNoDevice.
+    import torch  # noqa: F401
+
     lib = ctypes.CDLL(str(LIB_PATH))
     for name, (res, args) in SIGNATURES.items():
         fn = getattr(lib, name)  # AttributeError here means header and library disagree

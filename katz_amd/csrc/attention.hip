@@ -213,6 +213,6 @@ KH_EXPORT int kh_attention_bf16(const void* q, const void* k, const void* v, voi
   p.q_blocks = (int)((T + 127) / 128);
   const long grid = (long)p.q_blocks * H * B;
   if (grid > 0x7fffffffL) return KH_ERR_TOO_LARGE;
-  hipLaunchKernelGGL(attention_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, p);
+  kh_launch(KH_TAG_ATTENTION, attention_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, p);
   KH_RETURN_LAST_ERROR();
 }

@@ -157,10 +157,10 @@ KH_EXPORT int kh_geglu_bf16(const void* proj, void* out, int64_t M, int64_t D, i
   if (!kh_aligned16(proj) || !kh_aligned16(out)) return KH_ERR_ALIGNMENT;
   const unsigned grid = ew_grid(M * (D / 8));
   if (approximate_tanh)
-    hipLaunchKernelGGL(geglu_kernel<true>, dim3(grid), dim3(EW_THREADS), 0, (hipStream_t)stream, (const bf16_t*)proj,
+    kh_launch(KH_TAG_GEGLU, geglu_kernel<true>, dim3(grid), dim3(EW_THREADS), 0, (hipStream_t)stream, (const bf16_t*)proj,
                        (bf16_t*)out, (long)M, (int)D);
   else
-    hipLaunchKernelGGL(geglu_kernel<false>, dim3(grid), dim3(EW_THREADS), 0, (hipStream_t)stream, (const bf16_t*)proj,
+    kh_launch(KH_TAG_GEGLU, geglu_kernel<false>, dim3(grid), dim3(EW_THREADS), 0, (hipStream_t)stream, (const bf16_t*)proj,
                        (bf16_t*)out, (long)M, (int)D);
   KH_RETURN_LAST_ERROR();
 }
@@ -170,10 +170,10 @@ KH_EXPORT int kh_gelu_mul_bf16(const void* x, const void* m, void* out, int64_t 
   if (!kh_aligned16(x) || !kh_aligned16(m) || !kh_aligned16(out)) return KH_ERR_ALIGNMENT;
   const unsigned grid = ew_grid(n / 8 + 1);
   if (approximate_tanh)
-    hipLaunchKernelGGL(gelu_mul_kernel<true>, dim3(grid), dim3(EW_THREADS), 0, (hipStream_t)stream, (const bf16_t*)x,
+    kh_launch(KH_TAG_GEGLU, gelu_mul_kernel<true>, dim3(grid), dim3(EW_THREADS), 0, (hipStream_t)stream, (const bf16_t*)x,
                        (const bf16_t*)m, (bf16_t*)out, (long)n);
   else
-    hipLaunchKernelGGL(gelu_mul_kernel<false>, dim3(grid), dim3(EW_THREADS), 0, (hipStream_t)stream, (const bf16_t*)x,
+    kh_launch(KH_TAG_GEGLU, gelu_mul_kernel<false>, dim3(grid), dim3(EW_THREADS), 0, (hipStream_t)stream, (const bf16_t*)x,
                        (const bf16_t*)m, (bf16_t*)out, (long)n);
   KH_RETURN_LAST_ERROR();
 }
@@ -186,7 +186,7 @@ KH_EXPORT int kh_residual_add_bf16(void* dst, const void* const* srcs, int n_src
   SrcList s;
   const int rc = fill_srcs(s, srcs, n_srcs, inv_count);
   if (rc != KH_OK) return rc;
-  hipLaunchKernelGGL(residual_add_kernel, dim3(ew_grid(n / 8)), dim3(EW_THREADS), 0, (hipStream_t)stream,
+  kh_launch(KH_TAG_RESIDUAL_ADD, residual_add_kernel, dim3(ew_grid(n / 8)), dim3(EW_THREADS), 0, (hipStream_t)stream,
                      (bf16_t*)dst, s, (long)n);
   KH_RETURN_LAST_ERROR();
 }
@@ -199,7 +199,7 @@ KH_EXPORT int kh_concat_residual_bf16(const void* h, const void* skip, const voi
   SrcList s;
   const int rc = fill_srcs(s, residuals, n_residuals, inv_count);
   if (rc != KH_OK) return rc;
-  hipLaunchKernelGGL(concat_residual_kernel, dim3(ew_grid(rows * ((C1 + C2) / 8))), dim3(EW_THREADS), 0,
+  kh_launch(KH_TAG_CONCAT_RESIDUAL, concat_residual_kernel, dim3(ew_grid(rows * ((C1 + C2) / 8))), dim3(EW_THREADS), 0,
                      (hipStream_t)stream, (const bf16_t*)h, (const bf16_t*)skip, s, (bf16_t*)out, (long)rows, (int)C1,
                      (int)C2);
   KH_RETURN_LAST_ERROR();

@@ -1,6 +1,7 @@
 // Shared device/host helpers for the katz_hip kernels (gfx950 / CDNA4 only).
 #pragma once
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stdint.h>
 
 #define KH_OK 0
@@ -18,6 +19,32 @@
     hipError_t e__ = hipGetLastError();             \
     return e__ == hipSuccess ? KH_OK : (int)e__;    \
   } while (0)
+
+// ---- optional per-launch timing (host) -----------------------------------------------------------
+// While profiling is on (kh_profile_begin .. kh_profile_end) every kernel goes out through
+// hipExtLaunchKernelGGL with its own start/stop event pair, which time exactly that dispatch on the
+// stream it was launched on.  Off (the default) launches are plain and graph-capturable.
+enum KhKernelTag {
+  KH_TAG_LORA_GEMM = 1, KH_TAG_LORA_GEMM_F32 = 2, KH_TAG_ATTENTION = 3, KH_TAG_GN_STATS = 4, KH_TAG_GN_APPLY = 5,
+  KH_TAG_LAYER_NORM = 6, KH_TAG_GEGLU = 7, KH_TAG_RESIDUAL_ADD = 8, KH_TAG_CONCAT_RESIDUAL = 9,
+  KH_TAG_SGMV_SHRINK = 10, KH_TAG_SGMV_EXPAND = 11
+};
+bool kh_prof_enabled();
+void kh_prof_events(int tag, hipEvent_t* start, hipEvent_t* stop);
+
+template <typename F, typename... Args>
+inline void kh_launch(int tag, F kernel, dim3 grid, dim3 block, size_t lds, hipStream_t stream, Args... args) {
+  // hipGetLastError is per thread and sticky across libraries: drop whatever an earlier, unrelated
+  // runtime call left behind so that the check after the launch reports this launch only.
+  (void)hipGetLastError();
+  if (kh_prof_enabled()) {
+    hipEvent_t a, b;
+    kh_prof_events(tag, &a, &b);
+    hipExtLaunchKernelGGL(kernel, grid, block, lds, stream, a, b, 0, args...);
+  } else {
+    hipLaunchKernelGGL(kernel, grid, block, lds, stream, args...);
+  }
+}
 
 typedef __bf16 bf16_t;
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));

@@ -332,7 +332,7 @@ int launch_cfg(LoraGemmParams p, hipStream_t stream) {
     attr_done = true;
   }
   const unsigned grid = (unsigned)(p.m_tiles * p.n_chunks);
-  hipLaunchKernelGGL(lora_gemm_kernel<C>, dim3(grid), dim3(C::NT), C::LDS_BYTES, stream, p);
+  kh_launch(KH_TAG_LORA_GEMM, lora_gemm_kernel<C>, dim3(grid), dim3(C::NT), C::LDS_BYTES, stream, p);
   KH_RETURN_LAST_ERROR();
 }
 
@@ -508,7 +508,7 @@ KH_EXPORT int kh_lora_linear_f32(const float* x, const float* w, const float* bi
   if (R > 0 && (!a_cat || !b_cat || !col_scale)) return KH_ERR_INVALID_ARG;
   if (R > F_RMAX) return KH_ERR_TOO_LARGE;
   dim3 grid((unsigned)((N + F_BN - 1) / F_BN), (unsigned)((M + F_BM - 1) / F_BM));
-  hipLaunchKernelGGL(lora_gemm_f32_kernel, grid, dim3(256), 0, (hipStream_t)stream, x, w, bias, a_cat, b_cat,
+  kh_launch(KH_TAG_LORA_GEMM_F32, lora_gemm_f32_kernel, grid, dim3(256), 0, (hipStream_t)stream, x, w, bias, a_cat, b_cat,
                      col_scale, residual, y, (int)M, (int)N, (int)K, (int)R);
   KH_RETURN_LAST_ERROR();
 }

@@ -16,7 +16,7 @@
 namespace {
 
 constexpr int GN_THREADS = 256;
-constexpr int GN_MAX_C = 4096;  // per-channel scale/shift table in LDS (32 KB)
+constexpr int GN_MAX_C = 4096;
 
 __device__ __forceinline__ float block_sum(float v, float* red) {
 #pragma unroll
@@ -32,7 +32,12 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
 
 // ---------------------------------------------------------------- NHWC
 // grid (splits, N); a workgroup owns pixels [p0,p1) of sample n over all channels.
-// Thread (tx,ty): 16-byte channel chunks tx, tx+NTX, ... of pixels ty, ty+PL, ...
+// Thread (tx,ty) owns the 16-byte channel chunks tx, tx+NTX, ... (at most GN_MAX_CPT of them) for
+// the pixels ty, ty+PL, ...: its channels never change, so per-channel constants live in registers
+// and consecutive threads read consecutive 16-byte pieces of a pixel row.
+constexpr int GN_MAX_CPT = 2;
+constexpr int GN_UNROLL = 4;
+
 struct GnGeom {
   int N, C, HW, G, Cg, splits;
   int CP;   // 16-byte chunks per pixel (C/8)
@@ -41,51 +46,68 @@ struct GnGeom {
   int PL;   // pixel lanes
 };
 
-__global__ __launch_bounds__(GN_THREADS) void gn_stats_nhwc(const bf16_t* __restrict__ x, float* __restrict__ ws,
-                                                            const GnGeom g) {
-  __shared__ float bins[2 * 512];  // per group (sum, sumsq); G <= 512
+__device__ __forceinline__ void unpack8(const u32x4 v, float (&f)[8]) {
+#pragma unroll
+  for (int e = 0; e < 4; ++e) { f[2 * e] = bf16_lo(v[e]); f[2 * e + 1] = bf16_hi(v[e]); }
+}
+
+// add_nc (optional): a per-(sample, channel) term added to x before the statistics and the
+// normalisation -- the resnet's time-embedding projection, which the reference adds in a separate
+// pass between conv1 and norm2 (diffusers-hf/src/diffusers/models/resnet.py:388-390).
+__global__ __launch_bounds__(GN_THREADS) void gn_stats_nhwc(const bf16_t* __restrict__ x,
+                                                            const bf16_t* __restrict__ add_nc,
+                                                            float* __restrict__ ws, const GnGeom g) {
+  extern __shared__ float part[];  // [2][PL][C]: per pixel-lane, per channel (sum, sumsq)
   const int n = blockIdx.y, split = blockIdx.x;
   const int tid = threadIdx.x;
-  for (int i = tid; i < 2 * g.G; i += GN_THREADS) bins[i] = 0.f;
-  __syncthreads();
   const int per = (g.HW + g.splits - 1) / g.splits;
   const int p0 = split * per, p1 = min(g.HW, p0 + per);
   const int tx = tid % g.NTX, ty = tid / g.NTX;
+  float* psum = part;
+  float* psq = part + g.PL * g.C;
   if (ty < g.PL) {
     for (int k = 0; k < g.CPT; ++k) {
-      const int cc = tx + k * g.NTX;
+      const int c0 = (tx + k * g.NTX) * 8;
+      float sh[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) sh[e] = 0.f;
+      if (add_nc) unpack8(*reinterpret_cast<const u32x4*>(add_nc + (size_t)n * g.C + c0), sh);
       float s[8], q[8];
 #pragma unroll
       for (int e = 0; e < 8; ++e) s[e] = q[e] = 0.f;
-      const bf16_t* base = x + ((size_t)n * g.HW) * g.C + cc * 8;
-      for (int p = p0 + ty; p < p1; p += g.PL) {
-        const u32x4 v = *reinterpret_cast<const u32x4*>(base + (size_t)p * g.C);
+      const bf16_t* base = x + ((size_t)n * g.HW) * g.C + c0;
+      int p = p0 + ty;
+      for (; p + (GN_UNROLL - 1) * g.PL < p1; p += GN_UNROLL * g.PL) {
+        u32x4 v[GN_UNROLL];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const float a = bf16_lo(v[e]), b = bf16_hi(v[e]);
-          s[2 * e] += a; q[2 * e] = fmaf(a, a, q[2 * e]);
-          s[2 * e + 1] += b; q[2 * e + 1] = fmaf(b, b, q[2 * e + 1]);
+        for (int u = 0; u < GN_UNROLL; ++u)
+          v[u] = *reinterpret_cast<const u32x4*>(base + (size_t)(p + u * g.PL) * g.C);
+#pragma unroll
+        for (int u = 0; u < GN_UNROLL; ++u) {
+          float f[8];
+          unpack8(v[u], f);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) { const float a = f[e] + sh[e]; s[e] += a; q[e] = fmaf(a, a, q[e]); }
         }
       }
-      // fold the 8 channels into their groups (a chunk may straddle group boundaries)
-      int cur = (cc * 8) / g.Cg;
-      float cs = 0.f, cq = 0.f;
+      for (; p < p1; p += g.PL) {
+        float f[8];
+        unpack8(*reinterpret_cast<const u32x4*>(base + (size_t)p * g.C), f);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const int grp = (cc * 8 + e) / g.Cg;
-        if (grp != cur) {
-          atomicAdd(&bins[2 * cur], cs); atomicAdd(&bins[2 * cur + 1], cq);
-          cur = grp; cs = 0.f; cq = 0.f;
-        }
-        cs += s[e]; cq += q[e];
+        for (int e = 0; e < 8; ++e) { const float a = f[e] + sh[e]; s[e] += a; q[e] = fmaf(a, a, q[e]); }
       }
-      atomicAdd(&bins[2 * cur], cs); atomicAdd(&bins[2 * cur + 1], cq);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) { psum[ty * g.C + c0 + e] = s[e]; psq[ty * g.C + c0 + e] = q[e]; }
     }
   }
   __syncthreads();
-  for (int i = tid; i < g.G; i += GN_THREADS) {
-    float* o = ws + (((size_t)n * g.G + i) * g.splits + split) * 2;
-    o[0] = bins[2 * i]; o[1] = bins[2 * i + 1];
+  // fixed-order fold per group: deterministic (no atomics)
+  for (int grp = tid; grp < g.G; grp += GN_THREADS) {
+    float s = 0.f, q = 0.f;
+    for (int l = 0; l < g.PL; ++l)
+      for (int c = grp * g.Cg; c < (grp + 1) * g.Cg; ++c) { s += psum[l * g.C + c]; q += psq[l * g.C + c]; }
+    float* o = ws + (((size_t)n * g.G + grp) * g.splits + split) * 2;
+    o[0] = s; o[1] = q;
   }
 }
 
@@ -93,9 +115,8 @@ template <bool SILU>
 __global__ __launch_bounds__(GN_THREADS) void gn_apply_nhwc(const bf16_t* __restrict__ x, bf16_t* __restrict__ y,
                                                             const bf16_t* __restrict__ gamma,
                                                             const bf16_t* __restrict__ beta,
+                                                            const bf16_t* __restrict__ add_nc,
                                                             const float* __restrict__ ws, const GnGeom g, float eps) {
-  __shared__ float s_scale[GN_MAX_C];
-  __shared__ float s_shift[GN_MAX_C];
   __shared__ float s_mean[512], s_rstd[512];
   const int n = blockIdx.y, split = blockIdx.x;
   const int tid = threadIdx.x;
@@ -111,38 +132,55 @@ __global__ __launch_bounds__(GN_THREADS) void gn_apply_nhwc(const bf16_t* __rest
     s_rstd[i] = (float)(1.0 / sqrt(var + (double)eps));
   }
   __syncthreads();
-  for (int c = tid; c < g.C; c += GN_THREADS) {
-    const int grp = c / g.Cg;
-    const float ga = gamma ? (float)gamma[c] : 1.f, be = beta ? (float)beta[c] : 0.f;
-    const float sc = ga * s_rstd[grp];
-    s_scale[c] = sc;
-    s_shift[c] = be - s_mean[grp] * sc;
-  }
-  __syncthreads();
   const int per = (g.HW + g.splits - 1) / g.splits;
   const int p0 = split * per, p1 = min(g.HW, p0 + per);
-  const long chunks = (long)(p1 - p0) * g.CP;
-  const bf16_t* xb = x + ((size_t)n * g.HW + p0) * g.C;
-  bf16_t* yb = y + ((size_t)n * g.HW + p0) * g.C;
-  for (long i = tid; i < chunks; i += GN_THREADS) {
-    const int c0 = (int)(i % g.CP) * 8;
-    const u32x4 v = *reinterpret_cast<const u32x4*>(xb + i * 8);
-    u32x4 o;
+  const int tx = tid % g.NTX, ty = tid / g.NTX;
+  if (ty >= g.PL) return;
+  for (int k = 0; k < g.CPT; ++k) {
+    const int c0 = (tx + k * g.NTX) * 8;
+    float sc[8], sh[8];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      float a = fmaf(bf16_lo(v[e]), s_scale[c0 + 2 * e], s_shift[c0 + 2 * e]);
-      float b = fmaf(bf16_hi(v[e]), s_scale[c0 + 2 * e + 1], s_shift[c0 + 2 * e + 1]);
-      if (SILU) { a = silu_f(a); b = silu_f(b); }
-      o[e] = pack_bf16x2(a, b);
+    for (int e = 0; e < 8; ++e) {
+      const int c = c0 + e, grp = c / g.Cg;
+      const float ga = gamma ? (float)gamma[c] : 1.f, be = beta ? (float)beta[c] : 0.f;
+      const float ad = add_nc ? (float)add_nc[(size_t)n * g.C + c] : 0.f;
+      sc[e] = ga * s_rstd[grp];
+      sh[e] = be + (ad - s_mean[grp]) * sc[e];
     }
-    *reinterpret_cast<u32x4*>(yb + i * 8) = o;
+    const size_t off = ((size_t)n * g.HW) * g.C + c0;
+    const bf16_t* xb = x + off;
+    bf16_t* yb = y + off;
+    auto emit = [&](const u32x4 v, int p) {
+      float f[8];
+      unpack8(v, f);
+      u32x4 o;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float a = fmaf(f[2 * e], sc[2 * e], sh[2 * e]);
+        float b = fmaf(f[2 * e + 1], sc[2 * e + 1], sh[2 * e + 1]);
+        if (SILU) { a = silu_f(a); b = silu_f(b); }
+        o[e] = pack_bf16x2(a, b);
+      }
+      *reinterpret_cast<u32x4*>(yb + (size_t)p * g.C) = o;
+    };
+    int p = p0 + ty;
+    for (; p + (GN_UNROLL - 1) * g.PL < p1; p += GN_UNROLL * g.PL) {
+      u32x4 v[GN_UNROLL];
+#pragma unroll
+      for (int u = 0; u < GN_UNROLL; ++u) v[u] = *reinterpret_cast<const u32x4*>(xb + (size_t)(p + u * g.PL) * g.C);
+#pragma unroll
+      for (int u = 0; u < GN_UNROLL; ++u) emit(v[u], p + u * g.PL);
+    }
+    for (; p < p1; p += g.PL) emit(*reinterpret_cast<const u32x4*>(xb + (size_t)p * g.C), p);
   }
 }
 
 // ---------------------------------------------------------------- NCHW
 // grid (splits, N*G); row (n,g) is Cg*HW contiguous elements.
-__global__ __launch_bounds__(GN_THREADS) void gn_stats_nchw(const bf16_t* __restrict__ x, float* __restrict__ ws,
-                                                            long row_len, int splits) {
+__global__ __launch_bounds__(GN_THREADS) void gn_stats_nchw(const bf16_t* __restrict__ x,
+                                                            const bf16_t* __restrict__ add_nc,
+                                                            float* __restrict__ ws, long row_len, int splits, int G,
+                                                            int Cg, int HW) {
   __shared__ float red[GN_THREADS / 64];
   const long row = blockIdx.y;
   const int split = blockIdx.x;
@@ -150,12 +188,14 @@ __global__ __launch_bounds__(GN_THREADS) void gn_stats_nchw(const bf16_t* __rest
   const long per = (chunks + splits - 1) / splits;
   const long c0 = split * per, c1 = min(chunks, c0 + per);
   const bf16_t* xb = x + row * row_len;
+  const long cbase = (row / G) * (long)G * Cg + (row % G) * Cg;  // n*C + g*Cg
   float s = 0.f, q = 0.f;
   for (long i = c0 + threadIdx.x; i < c1; i += GN_THREADS) {
     const u32x4 v = *reinterpret_cast<const u32x4*>(xb + i * 8);
+    const float ad = add_nc ? (float)add_nc[cbase + (i * 8) / HW] : 0.f;  // HW % 8 == 0: one channel per chunk
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const float a = bf16_lo(v[e]), b = bf16_hi(v[e]);
+      const float a = bf16_lo(v[e]) + ad, b = bf16_hi(v[e]) + ad;
       s += a + b;
       q = fmaf(a, a, q); q = fmaf(b, b, q);
     }
@@ -172,6 +212,7 @@ template <bool SILU>
 __global__ __launch_bounds__(GN_THREADS) void gn_apply_nchw(const bf16_t* __restrict__ x, bf16_t* __restrict__ y,
                                                             const bf16_t* __restrict__ gamma,
                                                             const bf16_t* __restrict__ beta,
+                                                            const bf16_t* __restrict__ add_nc,
                                                             const float* __restrict__ ws, long row_len, int splits,
                                                             int G, int Cg, int HW, float eps) {
   __shared__ float s_mr[2];
@@ -200,7 +241,8 @@ __global__ __launch_bounds__(GN_THREADS) void gn_apply_nchw(const bf16_t* __rest
     // HW % 8 == 0 (host-checked): the 8 elements share one channel
     const int c = grp * Cg + (int)((i * 8) / HW);
     const float ga = gamma ? (float)gamma[c] : 1.f, be = beta ? (float)beta[c] : 0.f;
-    const float sc = ga * rstd, sh = be - mean * sc;
+    const float ad = add_nc ? (float)add_nc[(row / G) * (long)G * Cg + c] : 0.f;
+    const float sc = ga * rstd, sh = be + (ad - mean) * sc;
     u32x4 o;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
@@ -301,8 +343,8 @@ KH_EXPORT int64_t kh_group_norm_workspace_bytes(int64_t N, int64_t C, int64_t HW
   return (int64_t)N * G * splits * 2 * (int64_t)sizeof(float);
 }
 
-KH_EXPORT int kh_group_norm_bf16(const void* x, void* y, const void* gamma, const void* beta, float* workspace,
-                                 int64_t N, int64_t C, int64_t HW, int64_t G, float eps, int activation,
+KH_EXPORT int kh_group_norm_bf16(const void* x, void* y, const void* gamma, const void* beta, const void* add_nc,
+                                 float* workspace, int64_t N, int64_t C, int64_t HW, int64_t G, float eps, int activation,
                                  int channels_last, void* stream) {
   if (!x || !y || !workspace || N <= 0 || C <= 0 || HW <= 0 || G <= 0 || C % G != 0) return KH_ERR_INVALID_ARG;
   if (activation != 0 && activation != 1) return KH_ERR_INVALID_ARG;  // 0 = none, 1 = silu
@@ -312,6 +354,8 @@ KH_EXPORT int kh_group_norm_bf16(const void* x, void* y, const void* gamma, cons
   hipStream_t s = (hipStream_t)stream;
   const bf16_t* xp = (const bf16_t*)x; bf16_t* yp = (bf16_t*)y;
   const bf16_t* gp = (const bf16_t*)gamma; const bf16_t* bp = (const bf16_t*)beta;
+  const bf16_t* ap = (const bf16_t*)add_nc;
+  if (ap && !kh_aligned16(ap)) return KH_ERR_ALIGNMENT;
   if (channels_last) {
     if (C % 8 != 0 || C > GN_MAX_C || G > 512) return KH_ERR_UNSUPPORTED;
     GnGeom g;
@@ -322,24 +366,27 @@ KH_EXPORT int kh_group_norm_bf16(const void* x, void* y, const void* gamma, cons
     int ntx = g.CP < GN_THREADS ? g.CP : GN_THREADS;
     while (g.CP % ntx != 0) --ntx;
     g.NTX = ntx; g.CPT = g.CP / ntx; g.PL = GN_THREADS / ntx;
+    if (g.CPT > GN_MAX_CPT) return KH_ERR_UNSUPPORTED;
     dim3 grid((unsigned)g.splits, (unsigned)N);
-    hipLaunchKernelGGL(gn_stats_nhwc, grid, dim3(GN_THREADS), 0, s, xp, workspace, g);
+    const size_t lds = (size_t)2 * g.PL * g.C * sizeof(float);
+    kh_launch(KH_TAG_GN_STATS, gn_stats_nhwc, grid, dim3(GN_THREADS), lds, s, xp, ap, workspace, g);
     if (activation == 1)
-      hipLaunchKernelGGL(gn_apply_nhwc<true>, grid, dim3(GN_THREADS), 0, s, xp, yp, gp, bp, workspace, g, eps);
+      kh_launch(KH_TAG_GN_APPLY, gn_apply_nhwc<true>, grid, dim3(GN_THREADS), 0, s, xp, yp, gp, bp, ap, workspace, g, eps);
     else
-      hipLaunchKernelGGL(gn_apply_nhwc<false>, grid, dim3(GN_THREADS), 0, s, xp, yp, gp, bp, workspace, g, eps);
+      kh_launch(KH_TAG_GN_APPLY, gn_apply_nhwc<false>, grid, dim3(GN_THREADS), 0, s, xp, yp, gp, bp, ap, workspace, g, eps);
   } else {
     const long Cg = C / G, row_len = Cg * HW, rows = N * G;
     if (HW % 8 != 0) return KH_ERR_UNSUPPORTED;
     if (rows > 65535) return KH_ERR_TOO_LARGE;
     const int splits = gn_splits_nchw(rows, row_len);
     dim3 grid((unsigned)splits, (unsigned)rows);
-    hipLaunchKernelGGL(gn_stats_nchw, grid, dim3(GN_THREADS), 0, s, xp, workspace, row_len, splits);
+    kh_launch(KH_TAG_GN_STATS, gn_stats_nchw, grid, dim3(GN_THREADS), 0, s, xp, ap, workspace, row_len, splits, (int)G,
+                       (int)Cg, (int)HW);
     if (activation == 1)
-      hipLaunchKernelGGL(gn_apply_nchw<true>, grid, dim3(GN_THREADS), 0, s, xp, yp, gp, bp, workspace, row_len, splits,
-                         (int)G, (int)Cg, (int)HW, eps);
+      kh_launch(KH_TAG_GN_APPLY, gn_apply_nchw<true>, grid, dim3(GN_THREADS), 0, s, xp, yp, gp, bp, ap, workspace, row_len,
+                         splits, (int)G, (int)Cg, (int)HW, eps);
     else
-      hipLaunchKernelGGL(gn_apply_nchw<false>, grid, dim3(GN_THREADS), 0, s, xp, yp, gp, bp, workspace, row_len,
+      kh_launch(KH_TAG_GN_APPLY, gn_apply_nchw<false>, grid, dim3(GN_THREADS), 0, s, xp, yp, gp, bp, ap, workspace, row_len,
                          splits, (int)G, (int)Cg, (int)HW, eps);
   }
   KH_RETURN_LAST_ERROR();
@@ -353,7 +400,7 @@ KH_EXPORT int kh_layer_norm_bf16(const void* x, void* y, const void* gamma, cons
     return KH_ERR_ALIGNMENT;
   const long blocks = (M + 3) / 4;
   if (blocks > 0x7fffffffL) return KH_ERR_TOO_LARGE;
-  hipLaunchKernelGGL(layer_norm_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)x,
+  kh_launch(KH_TAG_LAYER_NORM, layer_norm_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const bf16_t*)x,
                      (bf16_t*)y, (const bf16_t*)gamma, (const bf16_t*)beta, (long)M, (int)D, eps);
   KH_RETURN_LAST_ERROR();
 }

@@ -174,7 +174,7 @@ KH_EXPORT int kh_sgmv_shrink_bf16(const void* x, const void* a_all, void* t, con
   p.seg_start = seg_start; p.seg_adapter = seg_adapter; p.adapter_rank = adapter_rank;
   p.K = (int)K; p.RP = (int)RP;
   dim3 grid((unsigned)((max_seg_rows + 127) / 128), (unsigned)n_segments);
-  hipLaunchKernelGGL(sgmv_shrink_kernel, grid, dim3(256), 0, (hipStream_t)stream, p);
+  kh_launch(KH_TAG_SGMV_SHRINK, sgmv_shrink_kernel, grid, dim3(256), 0, (hipStream_t)stream, p);
   KH_RETURN_LAST_ERROR();
 }
 
@@ -194,6 +194,6 @@ KH_EXPORT int kh_sgmv_expand_bf16(const void* t, const void* b_all, void* y, con
   const long gx = ((max_seg_rows + 127) / 128) * p.n_tiles;
   if (gx > 0x7fffffffL) return KH_ERR_TOO_LARGE;
   dim3 grid((unsigned)gx, (unsigned)n_segments);
-  hipLaunchKernelGGL(sgmv_expand_kernel, grid, dim3(256), 0, (hipStream_t)stream, p);
+  kh_launch(KH_TAG_SGMV_EXPAND, sgmv_expand_kernel, grid, dim3(256), 0, (hipStream_t)stream, p);
   KH_RETURN_LAST_ERROR();
 }

@@ -1,0 +1,383 @@
+"""Host-side layers of the adapter-augmented SDXL UNet, running on the katz_hip kernels.
+
+Module, attribute and state-dict names are the reference's (Katz fork of diffusers 0.28):
+`norm_silu1.0`, `to_q/to_k/to_v/to_out.0`, `ff.net.0.proj`, `ff.net.2`, `proj_in/proj_out`, ... so
+checkpoints and LoRA key maps written for the reference address these modules unchanged.
+
+Activations are bf16.  4-D feature maps are torch tensors of shape [N,C,H,W] in channels_last memory
+(NHWC): the convolutions (MIOpen) take and return that format, GroupNorm reads it directly, and the
+token view [N, H*W, C] the transformer blocks need is the same memory -- the NCHW<->token permute +
+.contiguous() copies of the reference (transformer_2d.py:488-490, :516-518) do not exist here.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Sequence
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from . import ops
+from .lora import Adapter, PackedAdapters, interleave_geglu_rows, pack_adapters, rescale_
+
+CL = torch.channels_last
+
+
+# When True, LoRALinear leaves its weights uninitialised (for models whose state dict is loaded next).
+SKIP_INIT = False
+
+
+class LoRALinear(nn.Module):
+    """nn.Linear whose forward is the fused base-GEMM + low-rank-delta kernel.
+
+    Equivalent of the peft `Linear` wrapper the reference injects
+    (diffusers-hf/src/diffusers/loaders/lora.py:409,475-476) and of LoRACompatibleLinear
+    (diffusers-hf/src/diffusers/models/lora.py:386-457): named adapters, an active list, per-adapter
+    weights, a global scale, fuse / unfuse.  geglu=True fuses GEGLU.forward's chunk + gelu + mul
+    (diffusers-hf/src/diffusers/models/activations.py:148-149) into the epilogue.
+    """
+
+    def __init__(self, in_features: int, out_features: int, bias: bool = True, geglu: bool = False,
+                 device=None, dtype=None):
+        super().__init__()
+        self.in_features, self.out_features, self.geglu = in_features, out_features, geglu
+        self.weight = nn.Parameter(torch.empty((out_features, in_features), device=device, dtype=dtype), requires_grad=False)
+        self.bias = nn.Parameter(torch.empty(out_features, device=device, dtype=dtype), requires_grad=False) if bias else None
+        self.adapters: Dict[str, Adapter] = {}
+        self.active: List[str] = []
+        self.global_scale = 1.0
+        self.adapters_enabled = True
+        self._packed: Optional[PackedAdapters] = None
+        self._packed_key = None
+        self._rt = None          # (weight version, weight ptr, runtime weight, runtime bias)
+        self._fused: Dict[str, float] = {}   # adapter name -> multiplier merged into weight
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        if self.weight.device.type != "meta" and not SKIP_INIT:
+            lin = nn.Linear(self.in_features, self.out_features, bias=self.bias is not None)
+            with torch.no_grad():
+                self.weight.copy_(lin.weight)
+                if self.bias is not None:
+                    self.bias.copy_(lin.bias)
+
+    # ---- adapter state (host) ---------------------------------------------------------------
+    def add_adapter(self, name: str, down: torch.Tensor, up: torch.Tensor, alpha: Optional[float] = None,
+                    weight: float = 1.0) -> None:
+        if down.shape[1] != self.in_features or up.shape[0] != self.out_features or down.shape[0] != up.shape[1]:
+            raise ValueError(f"adapter {name!r} does not fit a [{self.out_features},{self.in_features}] layer: "
+                             f"down {tuple(down.shape)}, up {tuple(up.shape)}")
+        self.adapters[name] = Adapter(down.detach(), up.detach(), alpha, weight)
+        self._packed_key = None
+
+    def delete_adapter(self, name: str) -> None:
+        self.adapters.pop(name, None)
+        self.active = [n for n in self.active if n != name]
+        self._packed_key = None
+
+    def set_active(self, names: Sequence[str], weights: Optional[Sequence[float]] = None) -> None:
+        self.active = [n for n in names if n in self.adapters]
+        if weights is not None:
+            for n, w in zip(names, weights):
+                if n in self.adapters:
+                    self.adapters[n].weight = float(w)
+        self.refresh_adapters()
+
+    def set_global_scale(self, scale: float) -> None:
+        """cross_attention_kwargs["scale"]: scale_lora_layers, diffusers-hf/src/diffusers/utils/peft_utils.py:103-123."""
+        if scale != self.global_scale:
+            self.global_scale = float(scale)
+            self.refresh_adapters()
+
+    def refresh_adapters(self) -> None:
+        """(Re)build the packed buffers; a pure scale change only rewrites col_scale in place, so a
+        captured HIP graph that reads the buffers stays valid."""
+        names = [n for n in self.active if n not in self._fused] if self.adapters_enabled else []
+        key = tuple((n, id(self.adapters[n].down)) for n in names)
+        if not names:
+            self._packed, self._packed_key = None, key
+            return
+        if key == self._packed_key and self._packed is not None:
+            rescale_(self._packed, self.adapters, self.global_scale)
+            return
+        self._packed = pack_adapters(self.adapters, names, self.in_features, self.out_features, self.weight.dtype,
+                                     self.weight.device, self.global_scale, geglu_interleave=self.geglu)
+        self._packed_key = key
+
+    def fuse(self, lora_scale: float = 1.0, names: Optional[Sequence[str]] = None) -> None:
+        """W += sum_i (lora_scale * m_i) B_i A_i in fp32, cast back -- _fuse_lora,
+        diffusers-hf/src/diffusers/models/lora.py:403-433 (Katz: pipeline_controlnet_sd_xl_katz.py:1737-1747)."""
+        names = list(self.active if names is None else names)
+        with torch.no_grad():
+            w = self.weight.float()
+            for n in names:
+                if n in self._fused or n not in self.adapters:
+                    continue
+                ad = self.adapters[n]
+                m = lora_scale * ad.multiplier(1.0)
+                dev = self.weight.device
+                w = w + m * (ad.up.to(dev).float() @ ad.down.to(dev).float())
+                self._fused[n] = m
+            if not torch.isfinite(w).all():
+                raise ValueError("fusing produced non-finite weights; LoRA left unfused")
+            self.weight.copy_(w.to(self.weight.dtype))
+        self.refresh_adapters()
+
+    def unfuse(self) -> None:
+        with torch.no_grad():
+            w = self.weight.float()
+            dev = self.weight.device
+            for n, m in self._fused.items():
+                ad = self.adapters[n]
+                w = w - m * (ad.up.to(dev).float() @ ad.down.to(dev).float())
+            self.weight.copy_(w.to(self.weight.dtype))
+        self._fused.clear()
+        self.refresh_adapters()
+
+    # ---- runtime -----------------------------------------------------------------------------------
+    def prepare(self) -> None:
+        """Build the kernel-side weight buffers (the GEGLU row interleave) for the current weights."""
+        ver = (self.weight._version, self.weight.data_ptr(), None if self.bias is None else self.bias._version)
+        if self._rt is not None and self._rt[0] == ver:
+            return
+        if self.geglu:
+            w = interleave_geglu_rows(self.weight.detach())
+            b = interleave_geglu_rows(self.bias.detach()) if self.bias is not None else None
+        else:
+            w = self.weight.detach()
+            b = self.bias.detach() if self.bias is not None else None
+        self._rt = (ver, w, b)
+        self._packed_key = None  # weights moved or changed: repack on their device / dtype
+        self.refresh_adapters()
+
+    def forward(self, x: torch.Tensor, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+        self.prepare()
+        _, w, b = self._rt
+        p = self._packed
+        if p is None:
+            return ops.lora_linear(x, w, b, residual=residual, geglu=self.geglu)
+        return ops.lora_linear(x, w, b, p.a_cat, p.b_cat, p.col_scale, residual=residual, geglu=self.geglu)
+
+    def extra_repr(self) -> str:
+        return f"in_features={self.in_features}, out_features={self.out_features}, bias={self.bias is not None}, geglu={self.geglu}"
+
+
+class GroupNorm(nn.Module):
+    """GroupNorm with the activation fused, replacing the reference's
+    diffusers-hf/src/diffusers/models/normalization.py:40-103 (fast_kernel group_norm_fp16)."""
+
+    def __init__(self, num_groups: int, num_channels: int, eps: float = 1e-5, affine: bool = True,
+                 activation: str = "none", device=None, dtype=None):
+        super().__init__()
+        self.num_groups, self.num_channels, self.eps, self.activation = num_groups, num_channels, eps, activation
+        if affine:
+            self.weight = nn.Parameter(torch.ones(num_channels, device=device, dtype=dtype), requires_grad=False)
+            self.bias = nn.Parameter(torch.zeros(num_channels, device=device, dtype=dtype), requires_grad=False)
+        else:
+            self.weight = self.bias = None
+
+    def forward(self, x: torch.Tensor, add_nc: Optional[torch.Tensor] = None) -> torch.Tensor:
+        return ops.group_norm(x, self.num_groups, self.weight, self.bias, self.eps, self.activation, add_nc=add_nc)
+
+
+def fused_norm_silu(num_channels: int, norm_num_groups: int, eps: float, affine: bool = True):
+    """One fused module where the reference returns [GroupNorm(activation fused)] under
+    ENABLE_FUSED_NORM_SILU=1 (normalization.py:30-35): keeps the `<name>.0.weight` state-dict keys."""
+    return [GroupNorm(norm_num_groups, num_channels, eps=eps, affine=affine, activation="silu")]
+
+
+class LayerNorm(nn.Module):
+    def __init__(self, dim: int, eps: float = 1e-5, device=None, dtype=None):
+        super().__init__()
+        self.eps = eps
+        self.weight = nn.Parameter(torch.ones(dim, device=device, dtype=dtype), requires_grad=False)
+        self.bias = nn.Parameter(torch.zeros(dim, device=device, dtype=dtype), requires_grad=False)
+
+    def forward(self, x):
+        return ops.layer_norm(x, self.weight, self.bias, self.eps)
+
+
+class TimestepEmbedding(nn.Module):
+    """linear_1 -> SiLU -> linear_2 on [B, C] (two rows: not worth a custom kernel)."""
+
+    def __init__(self, in_channels: int, time_embed_dim: int):
+        super().__init__()
+        self.linear_1 = nn.Linear(in_channels, time_embed_dim)
+        self.linear_2 = nn.Linear(time_embed_dim, time_embed_dim)
+
+    def forward(self, sample):
+        return self.linear_2(F.silu(self.linear_1(sample)))
+
+
+class Downsample2D(nn.Module):
+    def __init__(self, channels, use_conv=True, out_channels=None, padding=1, name="op"):
+        super().__init__()
+        self.padding = padding
+        self.conv = nn.Conv2d(channels, out_channels or channels, 3, stride=2, padding=padding)
+
+    def forward(self, x):
+        if self.padding == 0:
+            x = F.pad(x, (0, 1, 0, 1))
+        return self.conv(x)
+
+
+class Upsample2D(nn.Module):
+    def __init__(self, channels, use_conv=True, out_channels=None):
+        super().__init__()
+        self.conv = nn.Conv2d(channels, out_channels or channels, 3, padding=1)
+
+    def forward(self, x, output_size=None):
+        if output_size is None:
+            x = F.interpolate(x, scale_factor=2.0, mode="nearest")
+        else:
+            x = F.interpolate(x, size=output_size, mode="nearest")
+        return self.conv(x)
+
+
+class ResnetBlock2D(nn.Module):
+    """diffusers-hf/src/diffusers/models/resnet.py:352-415 with both GroupNorm+SiLU pairs on the fused kernel."""
+
+    def __init__(self, *, in_channels, out_channels=None, temb_channels=512, groups=32, eps=1e-6,
+                 output_scale_factor=1.0):
+        super().__init__()
+        out_channels = in_channels if out_channels is None else out_channels
+        self.output_scale_factor = output_scale_factor
+        self.norm_silu1 = nn.Sequential(*fused_norm_silu(in_channels, groups, eps))
+        self.conv1 = nn.Conv2d(in_channels, out_channels, 3, padding=1)
+        self.time_emb_proj = nn.Linear(temb_channels, out_channels)
+        self.norm_silu2 = nn.Sequential(*fused_norm_silu(out_channels, groups, eps))
+        self.conv2 = nn.Conv2d(out_channels, out_channels, 3, padding=1)
+        self.conv_shortcut = nn.Conv2d(in_channels, out_channels, 1) if in_channels != out_channels else None
+
+    def forward(self, input_tensor, temb_act):
+        """temb_act = silu(temb), computed once per step by the caller."""
+        h = self.norm_silu1(input_tensor)
+        h = self.conv1(h)
+        # hidden_states + temb[:, :, None, None] rides inside the second norm (no separate pass)
+        h = self.norm_silu2[0](h, add_nc=self.time_emb_proj(temb_act))
+        h = self.conv2(h)
+        if self.conv_shortcut is not None:
+            input_tensor = self.conv_shortcut(input_tensor)
+        out = input_tensor + h
+        if self.output_scale_factor != 1.0:
+            out = out / self.output_scale_factor
+        return out
+
+
+class KatzAttnProcessor:
+    """Attention processor on the katz_hip flash kernel; plugs into the reference's processor API
+    (Attention.set_processor, attention_processor.py:374-392; call signature :1219-1228).
+    q/k/v stay in the projection layout [B, tokens, heads*64]; `residual` (optional) is added inside
+    the to_out projection's epilogue."""
+
+    def __call__(self, attn, hidden_states, encoder_hidden_states=None, attention_mask=None, temb=None,
+                 residual=None, **kwargs):
+        if attention_mask is not None:
+            raise NotImplementedError("attention masks are not used on the SDXL path and not implemented")
+        ctx = hidden_states if encoder_hidden_states is None else encoder_hidden_states
+        q = attn.to_q(hidden_states)
+        k = attn.to_k(ctx)
+        v = attn.to_v(ctx)
+        o = ops.attention(q, k, v, attn.heads, attn.scale)
+        o = attn.to_out[0](o, residual=residual)
+        return attn.to_out[1](o)
+
+
+class Attention(nn.Module):
+    """diffusers-hf/src/diffusers/models/attention_processor.py:91-210, :484-525."""
+
+    def __init__(self, query_dim, cross_attention_dim=None, heads=8, dim_head=64, bias=False, out_bias=True,
+                 processor=None):
+        super().__init__()
+        inner = heads * dim_head
+        self.heads, self.scale = heads, dim_head ** -0.5
+        kv_dim = cross_attention_dim if cross_attention_dim is not None else query_dim
+        self.to_q = LoRALinear(query_dim, inner, bias=bias)
+        self.to_k = LoRALinear(kv_dim, inner, bias=bias)
+        self.to_v = LoRALinear(kv_dim, inner, bias=bias)
+        self.to_out = nn.ModuleList([LoRALinear(inner, query_dim, bias=out_bias), nn.Dropout(0.0)])
+        self.processor = processor or KatzAttnProcessor()
+
+    def set_processor(self, processor) -> None:
+        self.processor = processor
+
+    def get_processor(self):
+        return self.processor
+
+    def forward(self, hidden_states, encoder_hidden_states=None, attention_mask=None, **cross_attention_kwargs):
+        return self.processor(self, hidden_states, encoder_hidden_states=encoder_hidden_states,
+                              attention_mask=attention_mask, **cross_attention_kwargs)
+
+
+class GEGLU(nn.Module):
+    """`proj` holds the reference's [2*inner, dim] weight (value rows then gate rows); the kernel reads a
+    row-interleaved copy and applies value * gelu(gate) in the GEMM epilogue."""
+
+    def __init__(self, dim_in, dim_out):
+        super().__init__()
+        self.proj = LoRALinear(dim_in, dim_out * 2, geglu=True)
+
+    def forward(self, x):
+        return self.proj(x)
+
+
+class FeedForward(nn.Module):
+    def __init__(self, dim, mult=4):
+        super().__init__()
+        inner = dim * mult
+        self.net = nn.ModuleList([GEGLU(dim, inner), nn.Dropout(0.0), LoRALinear(inner, dim)])
+
+    def forward(self, x, residual=None):
+        return self.net[2](self.net[0](x), residual=residual)
+
+
+class BasicTransformerBlock(nn.Module):
+    """diffusers-hf/src/diffusers/models/attention.py:283-403 (layer_norm variant); the three residual
+    adds run in the epilogues of to_out.0 (x2) and ff.net.2."""
+
+    def __init__(self, dim, num_attention_heads, attention_head_dim, cross_attention_dim=None):
+        super().__init__()
+        self.norm1 = LayerNorm(dim, 1e-5)
+        self.attn1 = Attention(dim, None, num_attention_heads, attention_head_dim)
+        if cross_attention_dim is not None:
+            self.norm2 = LayerNorm(dim, 1e-5)
+            self.attn2 = Attention(dim, cross_attention_dim, num_attention_heads, attention_head_dim)
+        else:
+            self.norm2 = self.attn2 = None
+        self.norm3 = LayerNorm(dim, 1e-5)
+        self.ff = FeedForward(dim)
+
+    def forward(self, h, encoder_hidden_states=None):
+        h = self.attn1(self.norm1(h), residual=h)
+        if self.attn2 is not None:
+            h = self.attn2(self.norm2(h), encoder_hidden_states=encoder_hidden_states, residual=h)
+        return self.ff(self.norm3(h), residual=h)
+
+
+class Transformer2DModel(nn.Module):
+    """diffusers-hf/src/diffusers/models/transformers/transformer_2d.py:327-527, linear-projection variant
+    (the only one SDXL uses).  Input / output: channels_last [N,C,H,W]."""
+
+    def __init__(self, num_attention_heads, attention_head_dim, in_channels, num_layers=1, cross_attention_dim=None,
+                 norm_num_groups=32, use_linear_projection=True):
+        super().__init__()
+        if not use_linear_projection:
+            raise NotImplementedError("only use_linear_projection=True (SDXL) is implemented")
+        inner = num_attention_heads * attention_head_dim
+        self.norm = GroupNorm(norm_num_groups, in_channels, eps=1e-6, affine=True, activation="none")
+        self.proj_in = LoRALinear(in_channels, inner)
+        self.transformer_blocks = nn.ModuleList(
+            [BasicTransformerBlock(inner, num_attention_heads, attention_head_dim, cross_attention_dim)
+             for _ in range(num_layers)])
+        self.proj_out = LoRALinear(inner, in_channels)
+
+    def forward(self, hidden_states, encoder_hidden_states=None):
+        N, C, H, W = hidden_states.shape
+        tokens = lambda t: t.permute(0, 2, 3, 1).reshape(N, H * W, C)  # a view of channels_last memory
+        residual = tokens(hidden_states)
+        h = tokens(self.norm(hidden_states))
+        h = self.proj_in(h)
+        for blk in self.transformer_blocks:
+            h = blk(h, encoder_hidden_states)
+        h = self.proj_out(h, residual=residual)
+        return h.view(N, H, W, C).permute(0, 3, 1, 2)

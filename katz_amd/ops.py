@@ -17,6 +17,9 @@ from . import _lib
 
 BF16 = torch.bfloat16
 
+# When set to a list, lora_linear / attention append their problem sizes to it (benchmark accounting).
+CALL_LOG = None
+
 
 def _stream() -> int:
     return torch.cuda.current_stream().cuda_stream
@@ -82,6 +85,8 @@ def lora_linear(
         _req(out, dt, "out")
         if out.numel() != M * n_out:
             raise ValueError("out has the wrong size")
+    if CALL_LOG is not None:
+        CALL_LOG.append(("lora_linear", M, N, K, R, bool(geglu), residual is not None))
     if dt == BF16:
         flags = (1 if geglu else 0) | ((tile & 0xFF) << 8)
         rc = lib.kh_lora_linear_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(a_cat), _ptr(b_cat), _ptr(col_scale),
@@ -151,6 +156,8 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, heads: int, sca
         scale = 1.0 / math.sqrt(hd)
     if out is None:
         out = torch.empty((B, T, inner), dtype=BF16, device=q.device)
+    if CALL_LOG is not None:
+        CALL_LOG.append(("attention", B, heads, T, S, hd))
     rc = lib.kh_attention_bf16(_ptr(q), _ptr(k), _ptr(v), _ptr(out), B, heads, T, S, hd,
                                q.stride(1), k.stride(1), v.stride(1), out.stride(1),
                                q.stride(0), k.stride(0), v.stride(0), out.stride(0), float(scale), _stream())
@@ -173,9 +180,11 @@ def _workspace(nbytes: int, device) -> torch.Tensor:
 
 
 def group_norm(x: torch.Tensor, num_groups: int, weight: Optional[torch.Tensor], bias: Optional[torch.Tensor],
-               eps: float, activation: str = "none", out: Optional[torch.Tensor] = None) -> torch.Tensor:
+               eps: float, activation: str = "none", out: Optional[torch.Tensor] = None,
+               add_nc: Optional[torch.Tensor] = None) -> torch.Tensor:
     """GroupNorm(+SiLU) of a 4-D [N,C,H,W] tensor, either contiguous (NCHW) or channels_last (NHWC
-    memory); the output has the memory format of the input."""
+    memory); the output has the memory format of the input.  add_nc [N,C] (optional) is added to x
+    per (sample, channel) before the statistics: norm(x + add_nc[:, :, None, None])."""
     lib = _lib.load()
     if activation not in ("none", "silu"):
         raise ValueError(f"unknown activation {activation!r}")  # the reference only printf's here
@@ -197,7 +206,11 @@ def group_norm(x: torch.Tensor, num_groups: int, weight: Optional[torch.Tensor],
     if nbytes < 0:
         _lib.check(int(nbytes), "kh_group_norm_workspace_bytes")
     ws = _workspace(int(nbytes), x.device)
-    rc = lib.kh_group_norm_bf16(_ptr(x), _ptr(out), _ptr(weight), _ptr(bias), _ptr(ws), N, C, H * W, num_groups,
+    if add_nc is not None:
+        _req(add_nc, BF16, "add_nc")
+        if add_nc.shape != (N, C):
+            raise ValueError(f"add_nc must be [N,C] = [{N},{C}], got {tuple(add_nc.shape)}")
+    rc = lib.kh_group_norm_bf16(_ptr(x), _ptr(out), _ptr(weight), _ptr(bias), _ptr(add_nc), _ptr(ws), N, C, H * W, num_groups,
                                 float(eps), 1 if activation == "silu" else 0, cl, _stream())
     _lib.check(rc, "kh_group_norm_bf16")
     return out
@@ -281,3 +294,25 @@ def concat_residual(h: torch.Tensor, skip: torch.Tensor, residuals: Sequence[tor
                                      N * H * W, C1, C2, _stream())
     _lib.check(rc, "kh_concat_residual_bf16")
     return out
+
+
+# --------------------------------------------------------------------------------------- per-launch timing
+KERNEL_TAGS = {1: "lora_gemm", 2: "lora_gemm_f32", 3: "attention", 4: "group_norm_stats", 5: "group_norm_apply",
+               6: "layer_norm", 7: "geglu", 8: "residual_add", 9: "concat_residual", 10: "sgmv_shrink",
+               11: "sgmv_expand"}
+
+
+def profile_begin() -> None:
+    """From now on every katz_hip launch carries its own HIP start/stop events (not graph-capturable)."""
+    _lib.check(_lib.load().kh_profile_begin(), "kh_profile_begin")
+
+
+def profile_end(capacity: int = 1 << 16):
+    """Stop per-launch timing; returns [(kernel name, milliseconds)] in launch order (synchronises)."""
+    tags = (ctypes.c_int32 * capacity)()
+    ms = (ctypes.c_float * capacity)()
+    n = _lib.load().kh_profile_end(tags, ms, capacity)
+    if n < 0:
+        _lib.check(-n, "kh_profile_end")
+    n = min(n, capacity)
+    return [(KERNEL_TAGS.get(tags[i], str(tags[i])), float(ms[i])) for i in range(n)]

@@ -1,0 +1,390 @@
+"""UNet2DConditionModel (SDXL configuration) on the katz_hip kernels.
+
+Drop-in for the reference's model at the call boundary
+(diffusers-hf/src/diffusers/models/unets/unet_2d_condition.py:1955-1974): same forward keyword
+arguments -- including ControlNet's `down_block_additional_residuals` / `mid_block_additional_residual`
+and the Katz extras `controlnet_skt, serve_mode, time_stats, controlnet_num` -- same module / state-dict
+names, and the LoRA surface (`load_lora_into_unet`, `set_adapters`, `fuse_lora`, `unfuse_lora`,
+`unload_lora`, `disable_lora` / `enable_lora`, `cross_attention_kwargs={"scale": s}`) of
+diffusers-hf/src/diffusers/loaders/unet.py:514-618 and diffusers-hf/src/diffusers/loaders/lora.py:382-496,
+implemented without peft: every LoRA-able Linear is a `LoRALinear` that runs the fused kernel.
+
+Semantics follow the reference's CUDA-graph path (_down_forward :1127-1252, _up_forward :1254-1341),
+which adds all nine skip residuals and the mid residual; the eager variant's `is not None` guard that
+drops the skip adds (:1886-1898) is not reproduced.
+"""
+from __future__ import annotations
+
+import math
+import re
+from dataclasses import dataclass
+from typing import Any, Dict, List, Optional, Sequence, Tuple, Union
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from . import ops
+from .layers import LoRALinear, TimestepEmbedding, fused_norm_silu
+from .unet_blocks import (CrossAttnDownBlock2D, CrossAttnUpBlock2D, DownBlock2D, UNetMidBlock2DCrossAttn, UpBlock2D)
+
+
+@dataclass
+class UNetConfig:
+    in_channels: int = 4
+    out_channels: int = 4
+    block_out_channels: Tuple[int, ...] = (320, 640, 1280)
+    down_block_types: Tuple[str, ...] = ("DownBlock2D", "CrossAttnDownBlock2D", "CrossAttnDownBlock2D")
+    up_block_types: Tuple[str, ...] = ("CrossAttnUpBlock2D", "CrossAttnUpBlock2D", "UpBlock2D")
+    layers_per_block: int = 2
+    transformer_layers_per_block: Tuple[int, ...] = (1, 2, 10)
+    num_attention_heads: Tuple[int, ...] = (5, 10, 20)  # stored as `attention_head_dim` in SDXL's config.json
+    cross_attention_dim: int = 2048
+    norm_num_groups: int = 32
+    norm_eps: float = 1e-5
+    addition_time_embed_dim: int = 256
+    projection_class_embeddings_input_dim: int = 2816
+    use_linear_projection: bool = True
+
+    @staticmethod
+    def sdxl() -> "UNetConfig":
+        return UNetConfig()
+
+    @staticmethod
+    def tiny() -> "UNetConfig":
+        return UNetConfig(block_out_channels=(64, 128, 256), transformer_layers_per_block=(1, 1, 2),
+                          num_attention_heads=(1, 2, 4), cross_attention_dim=128, addition_time_embed_dim=32,
+                          projection_class_embeddings_input_dim=64 + 6 * 32)
+
+
+@dataclass
+class UNet2DConditionOutput:
+    sample: torch.Tensor
+
+
+def get_timestep_embedding(timesteps, embedding_dim, flip_sin_to_cos=False, downscale_freq_shift=1.0, scale=1.0,
+                           max_period=10000):
+    """diffusers-hf/src/diffusers/models/embeddings.py:26-66, evaluated on the device of `timesteps`."""
+    half = embedding_dim // 2
+    exponent = -math.log(max_period) * torch.arange(0, half, dtype=torch.float32, device=timesteps.device)
+    exponent = exponent / (half - downscale_freq_shift)
+    emb = scale * timesteps[:, None].float() * torch.exp(exponent)[None, :]
+    emb = torch.cat([torch.sin(emb), torch.cos(emb)], dim=-1)
+    if flip_sin_to_cos:
+        emb = torch.cat([emb[:, half:], emb[:, :half]], dim=-1)
+    if embedding_dim % 2 == 1:
+        emb = F.pad(emb, (0, 1, 0, 0))
+    return emb
+
+
+# LoRA key spellings accepted by load_lora_into_unet -> (module path, "down" | "up")
+_LORA_PATTERNS = [
+    (re.compile(r"^(.*)\.processor\.(to_q|to_k|to_v|to_out)_lora\.(down|up)\.weight$"), "processor"),
+    (re.compile(r"^(.*)\.(to_q|to_k|to_v)_lora\.(down|up)\.weight$"), "attn_old"),
+    (re.compile(r"^(.*)\.lora\.(down|up)\.weight$"), "plain"),
+    (re.compile(r"^(.*)\.lora_(A|B)(?:\.[^.]+)?\.weight$"), "peft"),
+]
+
+
+def parse_lora_key(key: str) -> Optional[Tuple[str, str]]:
+    """Map one LoRA state-dict key to (UNet module path, 'down'|'up').
+
+    Spellings: the kohya->diffusers converted keys the reference stores in shared memory
+    (`<attn>.processor.to_q_lora.down.weight`, `<module>.lora.up.weight`; lora_info_shm/*_key_match_unet.json,
+    built by gen_lora_diffuser_key_match.py:131-175) and the peft spelling they are converted to
+    (`<module>.lora_A.weight`, diffusers-hf/src/diffusers/utils/state_dict_utils.py:38-50)."""
+    if key.startswith("unet."):
+        key = key[len("unet."):]
+    for pat, kind in _LORA_PATTERNS:
+        m = pat.match(key)
+        if not m:
+            continue
+        if kind == "processor" or kind == "attn_old":
+            proj = m.group(2)
+            mod = f"{m.group(1)}.{'to_out.0' if proj == 'to_out' else proj}"
+            return mod, m.group(3)
+        if kind == "plain":
+            return m.group(1), m.group(2)
+        return m.group(1), "down" if m.group(2) == "A" else "up"
+    return None
+
+
+class UNet2DConditionModel(nn.Module):
+    def __init__(self, cfg: Optional[UNetConfig] = None):
+        super().__init__()
+        cfg = cfg or UNetConfig.sdxl()
+        self.cfg = cfg
+        boc = cfg.block_out_channels
+        ted = boc[0] * 4
+        self.conv_in = nn.Conv2d(cfg.in_channels, boc[0], 3, padding=1)
+        self.time_embedding = TimestepEmbedding(boc[0], ted)
+        self.add_embedding = TimestepEmbedding(cfg.projection_class_embeddings_input_dim, ted)
+        n = len(boc)
+        self.down_blocks = nn.ModuleList()
+        out_ch = boc[0]
+        for i, typ in enumerate(cfg.down_block_types):
+            in_ch, out_ch = out_ch, boc[i]
+            common = dict(in_channels=in_ch, out_channels=out_ch, temb_channels=ted, num_layers=cfg.layers_per_block,
+                          resnet_eps=cfg.norm_eps, resnet_groups=cfg.norm_num_groups, add_downsample=i != n - 1)
+            if typ == "DownBlock2D":
+                self.down_blocks.append(DownBlock2D(**common))
+            elif typ == "CrossAttnDownBlock2D":
+                self.down_blocks.append(CrossAttnDownBlock2D(
+                    **common, transformer_layers_per_block=cfg.transformer_layers_per_block[i],
+                    num_attention_heads=cfg.num_attention_heads[i], cross_attention_dim=cfg.cross_attention_dim,
+                    use_linear_projection=cfg.use_linear_projection))
+            else:
+                raise ValueError(f"unsupported down block {typ}")
+        self.mid_block = UNetMidBlock2DCrossAttn(
+            in_channels=boc[-1], temb_channels=ted, transformer_layers_per_block=cfg.transformer_layers_per_block[-1],
+            resnet_eps=cfg.norm_eps, resnet_groups=cfg.norm_num_groups, num_attention_heads=cfg.num_attention_heads[-1],
+            cross_attention_dim=cfg.cross_attention_dim, use_linear_projection=cfg.use_linear_projection)
+        self.up_blocks = nn.ModuleList()
+        rev, rev_heads = list(reversed(boc)), list(reversed(cfg.num_attention_heads))
+        rev_tl = list(reversed(cfg.transformer_layers_per_block))
+        out_ch = rev[0]
+        for i, typ in enumerate(cfg.up_block_types):
+            prev, out_ch = out_ch, rev[i]
+            in_ch = rev[min(i + 1, n - 1)]
+            common = dict(in_channels=in_ch, out_channels=out_ch, prev_output_channel=prev, temb_channels=ted,
+                          num_layers=cfg.layers_per_block + 1, resnet_eps=cfg.norm_eps,
+                          resnet_groups=cfg.norm_num_groups, add_upsample=i != n - 1)
+            if typ == "UpBlock2D":
+                self.up_blocks.append(UpBlock2D(**common))
+            elif typ == "CrossAttnUpBlock2D":
+                self.up_blocks.append(CrossAttnUpBlock2D(
+                    **common, transformer_layers_per_block=rev_tl[i], num_attention_heads=rev_heads[i],
+                    cross_attention_dim=cfg.cross_attention_dim, use_linear_projection=cfg.use_linear_projection))
+            else:
+                raise ValueError(f"unsupported up block {typ}")
+        self.conv_norm_silu = nn.Sequential(*fused_norm_silu(boc[0], cfg.norm_num_groups, cfg.norm_eps))
+        self.conv_out = nn.Conv2d(boc[0], cfg.out_channels, 3, padding=1)
+        self.num_upsamplers = n - 1
+        self._register_load_state_dict_pre_hook(self._remap_upstream_keys)
+
+    # ---- checkpoints ---------------------------------------------------------------------------
+    @staticmethod
+    def _remap_upstream_keys(state_dict, prefix, *args):
+        """Accept upstream-diffusers key names, as the reference's load hooks do:
+        conv_norm_out.* -> conv_norm_silu.0.* (unet_2d_condition.py:521-529),
+        resnet norm1/norm2 -> norm_silu1.0/norm_silu2.0 (diffusers-hf/src/diffusers/models/resnet.py:336-350),
+        and the fused-GEGLU split proj_1 / proj_2 -> proj (activations.py:151-170, inverted)."""
+        for k in list(state_dict.keys()):
+            nk = k
+            if k.startswith(prefix + "conv_norm_out."):
+                nk = k.replace("conv_norm_out.", "conv_norm_silu.0.", 1)
+            elif re.search(r"\.resnets\.\d+\.norm[12]\.(weight|bias)$", k):
+                nk = re.sub(r"\.norm([12])\.(weight|bias)$", r".norm_silu\1.0.\2", k)
+            if nk != k:
+                state_dict[nk] = state_dict.pop(k)
+        for k in [k for k in state_dict if ".ff.net.0.proj_1." in k]:
+            k2 = k.replace(".proj_1.", ".proj_2.")
+            if k2 in state_dict:  # proj_1 = value half, proj_2 = gate half of `proj` (chunk(2, dim=0))
+                state_dict[k.replace(".proj_1.", ".proj.")] = torch.cat([state_dict.pop(k), state_dict.pop(k2)], dim=0)
+
+    def to_runtime(self, device="cuda", dtype=torch.bfloat16) -> "UNet2DConditionModel":
+        """Move to the GPU in the kernel formats: bf16, conv weights channels_last, packed GEGLU rows."""
+        self.to(device=device, dtype=dtype)
+        self.to(memory_format=torch.channels_last)
+        self.prepare()
+        return self.eval()
+
+    def prepare(self) -> None:
+        for m in self.lora_linears().values():
+            m.prepare()
+
+    # ---- LoRA surface ----------------------------------------------------------------------------
+    def lora_linears(self) -> Dict[str, LoRALinear]:
+        return {n: m for n, m in self.named_modules() if isinstance(m, LoRALinear)}
+
+    def load_lora_into_unet(self, state_dict: Dict[str, torch.Tensor], network_alphas: Optional[Dict[str, float]] = None,
+                            adapter_name: Optional[str] = None) -> str:
+        """Register one adapter from a LoRA state dict (load_lora_into_unet,
+        diffusers-hf/src/diffusers/loaders/lora.py:382-496).  Keys in any spelling parse_lora_key accepts;
+        keys of other components (text encoders) are ignored; network_alphas maps
+        "<module or down key>.alpha" to alpha (:261-270), default alpha = rank."""
+        lin = self.lora_linears()
+        pairs: Dict[str, Dict[str, torch.Tensor]] = {}
+        for k, v in state_dict.items():
+            if k.startswith("text_encoder"):
+                continue
+            parsed = parse_lora_key(k)
+            if parsed is None:
+                continue
+            mod, which = parsed
+            pairs.setdefault(mod, {})[which] = v
+            pairs[mod][which + "_key"] = k
+        if not pairs:
+            raise ValueError("no UNet LoRA keys found in the state dict")
+        adapter_name = adapter_name or f"default_{len(self.adapter_names())}"
+        if adapter_name in self.adapter_names():
+            raise ValueError(f"adapter name {adapter_name!r} is already in use in the UNet")
+        for mod, pr in pairs.items():
+            if mod not in lin:
+                raise ValueError(f"LoRA targets {mod!r}, which is not a LoRA-able linear of this UNet")
+            if "down" not in pr or "up" not in pr:
+                raise ValueError(f"LoRA for {mod!r} lacks its {'down' if 'down' not in pr else 'up'} matrix")
+            alpha = None
+            if network_alphas:
+                for cand in (pr["down_key"] + ".alpha", "unet." + mod + ".alpha", mod + ".alpha",
+                             pr["down_key"].removeprefix("unet.") + ".alpha"):
+                    if cand in network_alphas:
+                        alpha = float(network_alphas[cand])
+                        break
+            lin[mod].add_adapter(adapter_name, pr["down"], pr["up"], alpha)
+        self.set_adapters(self.adapter_names())  # a freshly loaded adapter is active, like peft's
+        return adapter_name
+
+    def adapter_names(self) -> List[str]:
+        names: List[str] = []
+        for m in self.lora_linears().values():
+            for n in m.adapters:
+                if n not in names:
+                    names.append(n)
+        return names
+
+    def set_adapters(self, adapter_names: Union[str, Sequence[str]],
+                     weights: Optional[Union[float, Sequence[float]]] = None) -> None:
+        """UNet2DConditionLoadersMixin.set_adapters, diffusers-hf/src/diffusers/loaders/unet.py:565-618."""
+        names = [adapter_names] if isinstance(adapter_names, str) else list(adapter_names)
+        if weights is None:
+            weights = [1.0] * len(names)
+        elif isinstance(weights, (int, float)):
+            weights = [float(weights)] * len(names)
+        if len(weights) != len(names):
+            raise ValueError(f"Length of adapter names {len(names)} is not equal to the length of their weights {len(weights)}.")
+        for m in self.lora_linears().values():
+            m.set_active(names, weights)
+
+    def disable_lora(self) -> None:
+        for m in self.lora_linears().values():
+            m.adapters_enabled = False
+            m.refresh_adapters()
+
+    def enable_lora(self) -> None:
+        for m in self.lora_linears().values():
+            m.adapters_enabled = True
+            m.refresh_adapters()
+
+    def fuse_lora(self, lora_scale: float = 1.0, adapter_names: Optional[Sequence[str]] = None) -> None:
+        for m in self.lora_linears().values():
+            m.fuse(lora_scale, adapter_names)
+
+    def unfuse_lora(self) -> None:
+        for m in self.lora_linears().values():
+            m.unfuse()
+
+    def unload_lora(self) -> None:
+        for m in self.lora_linears().values():
+            if m._fused:
+                m.unfuse()
+            for n in list(m.adapters):
+                m.delete_adapter(n)
+            m.refresh_adapters()
+
+    def delete_adapters(self, adapter_names: Union[str, Sequence[str]]) -> None:
+        names = [adapter_names] if isinstance(adapter_names, str) else list(adapter_names)
+        for m in self.lora_linears().values():
+            for n in names:
+                m.delete_adapter(n)
+            m.refresh_adapters()
+
+    def scale_lora_layers(self, scale: float) -> None:
+        for m in self.lora_linears().values():
+            m.set_global_scale(scale)
+
+    def set_attn_processor(self, processor) -> None:
+        """unet_2d_condition.py:800-832: one processor for all, or a dict keyed '<module>.processor'."""
+        from .layers import Attention
+        for name, m in self.named_modules():
+            if isinstance(m, Attention):
+                m.set_processor(processor[f"{name}.processor"] if isinstance(processor, dict) else processor)
+
+    @property
+    def attn_processors(self) -> Dict[str, Any]:
+        from .layers import Attention
+        return {f"{n}.processor": m.get_processor() for n, m in self.named_modules() if isinstance(m, Attention)}
+
+    # ---- forward -------------------------------------------------------------------------------------
+    def _embed(self, sample, timestep, added_cond_kwargs):
+        cfg = self.cfg
+        B = sample.shape[0]
+        if not torch.is_tensor(timestep):
+            timestep = torch.tensor([timestep], dtype=torch.float32, device=sample.device)
+        t = timestep.reshape(-1).to(sample.device)
+        if t.numel() == 1:
+            t = t.expand(B)
+        t_emb = get_timestep_embedding(t, cfg.block_out_channels[0], flip_sin_to_cos=True, downscale_freq_shift=0)
+        emb = self.time_embedding(t_emb.to(sample.dtype))
+        if added_cond_kwargs is None or "text_embeds" not in added_cond_kwargs or "time_ids" not in added_cond_kwargs:
+            raise ValueError("addition_embed_type 'text_time' requires `text_embeds` and `time_ids` in `added_cond_kwargs`")
+        text_embeds, time_ids = added_cond_kwargs["text_embeds"], added_cond_kwargs["time_ids"]
+        tid = get_timestep_embedding(time_ids.flatten(), cfg.addition_time_embed_dim, flip_sin_to_cos=True,
+                                     downscale_freq_shift=0).reshape(B, -1)
+        add = torch.cat([text_embeds.to(sample.dtype), tid.to(sample.dtype)], dim=-1)
+        return emb + self.add_embedding(add)
+
+    @staticmethod
+    def _residual_sets(res, n_expected):
+        """Normalise ControlNet residuals to a list (per skip) of lists (per ControlNet) of channels_last tensors."""
+        if res is None:
+            return [[] for _ in range(n_expected)]
+        res = list(res)
+        if len(res) and isinstance(res[0], (list, tuple)):   # several ControlNets: list of residual sets
+            sets = [list(s) for s in res]
+            if any(len(s) != n_expected for s in sets):
+                raise ValueError(f"every ControlNet residual set must hold {n_expected} tensors")
+            per_skip = [[s[j] for s in sets] for j in range(n_expected)]
+        else:
+            if len(res) != n_expected:
+                raise ValueError(f"expected {n_expected} down-block residuals, got {len(res)}")
+            per_skip = [[r] for r in res]
+        return [[r.to(torch.bfloat16).contiguous(memory_format=torch.channels_last) for r in rs] for rs in per_skip]
+
+    def forward(self, sample, timestep, encoder_hidden_states, class_labels=None, timestep_cond=None,
+                attention_mask=None, cross_attention_kwargs=None, added_cond_kwargs=None,
+                down_block_additional_residuals=None, mid_block_additional_residual=None,
+                down_intrablock_additional_residuals=None, encoder_attention_mask=None, return_dict: bool = True,
+                controlnet_skt=None, serve_mode=None, time_stats=None, controlnet_num=None):
+        for name, val in (("class_labels", class_labels), ("timestep_cond", timestep_cond),
+                          ("attention_mask", attention_mask), ("encoder_attention_mask", encoder_attention_mask),
+                          ("down_intrablock_additional_residuals", down_intrablock_additional_residuals),
+                          ("controlnet_skt", controlnet_skt)):
+            if val is not None:
+                raise NotImplementedError(f"`{name}` is not used on the SDXL + ControlNet + LoRA path and is not implemented")
+        if cross_attention_kwargs is not None:
+            self.scale_lora_layers(float(cross_attention_kwargs.get("scale", 1.0)))
+        if sample.dtype != torch.bfloat16 or not sample.is_contiguous(memory_format=torch.channels_last):
+            sample = sample.to(torch.bfloat16).contiguous(memory_format=torch.channels_last)
+        ctx = encoder_hidden_states.to(torch.bfloat16).contiguous()
+
+        emb = self._embed(sample, timestep, added_cond_kwargs)
+        temb_act = F.silu(emb)
+        sample = self.conv_in(sample)
+        skips = (sample,)
+        for blk in self.down_blocks:
+            sample, res = blk(sample, temb_act, ctx)
+            skips += res
+        sample = self.mid_block(sample, temb_act, ctx)
+
+        extra = self._residual_sets(down_block_additional_residuals, len(skips))
+        if mid_block_additional_residual is not None:
+            mids = mid_block_additional_residual
+            mids = list(mids) if isinstance(mids, (list, tuple)) else [mids]
+            mids = [m.to(torch.bfloat16).contiguous(memory_format=torch.channels_last) for m in mids]
+            if not sample.is_contiguous(memory_format=torch.channels_last):
+                sample = sample.contiguous(memory_format=torch.channels_last)
+            sample = ops.residual_add_(sample, mids)
+
+        for blk in self.up_blocks:
+            n = len(blk.resnets)
+            res, skips = skips[-n:], skips[:-n]
+            ex, extra = extra[-n:], extra[:-n]
+            sample = blk(sample, res, ex, temb_act, ctx)
+        sample = self.conv_norm_silu(sample)
+        sample = self.conv_out(sample)
+        if cross_attention_kwargs is not None:
+            self.scale_lora_layers(1.0)  # unscale_lora_layers, unet_2d_condition.py:1334-1336
+        if not return_dict:
+            return (sample,)
+        return UNet2DConditionOutput(sample=sample)

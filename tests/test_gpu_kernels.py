@@ -104,6 +104,35 @@ def test_lora_linear_bf16_scale_zero_is_base():
     assert torch.equal(y0, y1)
 
 
+def test_kernels_are_bit_reproducible():
+    """Same inputs, same bits, call after call: GEMM with LoRA + residual, GEGLU epilogue, attention."""
+    from katz_amd import ops
+    from katz_amd.layers import LoRALinear
+
+    say("reproducibility")
+    d = dev()
+    g = torch.Generator().manual_seed(31)
+    x = randn(g, 2048, 640).to(d, BF)
+    lin = LoRALinear(640, 640).to(d, BF)
+    lin.add_adapter("a", randn(g, 16, 640, std=0.05), randn(g, 640, 16, std=0.05))
+    base = lin(x).clone()
+    lin.set_active(["a"], [0.0])
+    assert torch.equal(lin(x), base)           # scale 0 == no adapter, bit for bit
+    lin.set_active(["a"], [1.0])
+    y = lin(x, residual=base).clone()
+    assert not torch.equal(lin(x), base)
+    for _ in range(3):
+        assert torch.equal(lin(x, residual=base), y)
+    geg = LoRALinear(640, 5120, geglu=True).to(d, BF)
+    geg.add_adapter("a", randn(g, 16, 640, std=0.05), randn(g, 5120, 16, std=0.05))
+    geg.set_active(["a"], [0.7])
+    y = geg(x).clone()
+    assert torch.equal(geg(x), y)
+    q = randn(g, 2, 1024, 640).to(d, BF)
+    o = ops.attention(q, q, q, 10).clone()
+    assert torch.equal(ops.attention(q, q, q, 10), o)
+
+
 def test_lora_linear_bf16_geglu_epilogue():
     say("lora_linear_bf16 geglu")
     M, K, D = 2048, 1280, 5120
@@ -246,6 +275,37 @@ def test_group_norm_no_affine():
     y = ops.group_norm(x.to(d, BF).contiguous(memory_format=torch.channels_last), 8, None, None, 1e-5, "none")
     torch.cuda.synchronize()
     assert_close_rel(y, O.group_norm(x, 8, None, None, 1e-5), REL_BF16, "group_norm no affine")
+
+
+def test_group_norm_fused_channel_add():
+    """norm(x + t[:, :, None, None]): the resnet's time-embedding add folded into the norm."""
+    from katz_amd import ops
+
+    say("group_norm add_nc")
+    g = torch.Generator().manual_seed(14)
+    d = dev()
+    for (N, C, H, W, G), cl in [((2, 320, 32, 32, 32), True), ((2, 320, 32, 32, 32), False), ((2, 2560, 16, 16, 32), True)]:
+        x = randn(g, N, C, H, W, std=2.0)
+        t = randn(g, N, C)
+        gamma = randn(g, C) + 1.0; beta = randn(g, C, std=0.5)
+        xd = x.to(d, BF)
+        if cl:
+            xd = xd.contiguous(memory_format=torch.channels_last)
+        y = ops.group_norm(xd, G, gamma.to(d, BF), beta.to(d, BF), 1e-5, "silu", add_nc=t.to(d, BF))
+        torch.cuda.synchronize()
+        ref = O.group_norm(x + t[:, :, None, None], G, gamma, beta, 1e-5, "silu")
+        assert_close_rel(y, ref, REL_BF16, "group_norm add_nc")
+
+
+def test_group_norm_is_deterministic():
+    from katz_amd import ops
+
+    x = torch.randn(2, 640, 64, 64, generator=torch.Generator().manual_seed(15)).to(dev(), BF)
+    x = x.contiguous(memory_format=torch.channels_last)
+    w = torch.ones(640, device=dev(), dtype=BF); b = torch.zeros(640, device=dev(), dtype=BF)
+    y0 = ops.group_norm(x, 32, w, b, 1e-5, "silu").clone()
+    for _ in range(3):
+        assert torch.equal(ops.group_norm(x, 32, w, b, 1e-5, "silu"), y0)
 
 
 def test_group_norm_unknown_activation_raises():
