@@ -1,0 +1,20 @@
+// Parameters shared by the LoRA GEMM kernels (host fills, kernels read by value).
+#pragma once
+#include "kh_common.h"
+
+struct LoraGemmParams {
+  const bf16_t* x;
+  const bf16_t* w;
+  const bf16_t* bias;      // may be null
+  const bf16_t* a_cat;     // [R,K] (unused when R == 0)
+  const bf16_t* b_cat;     // [N,R]
+  const float* col_scale;  // [R]
+  const bf16_t* res;       // [M,N] residual added in the epilogue, may be null
+  bf16_t* y;
+  int M, N, K, R;
+  int m_tiles, n_tiles, n_chunk, n_chunks;  // n_chunk = N tiles walked by one workgroup
+  int geglu;                                // 1: W rows are (value,gate) interleaved in 32-column groups, y is [M,N/2]
+};
+
+// Software-pipelined kernel (lora_gemm_pipe.hip); needs K % 32 == 0.  tile_sel: 0 automatic, >= 16 forces a tile.
+int lora_gemm_pipe_launch(const LoraGemmParams& p, int tile_sel, hipStream_t stream);

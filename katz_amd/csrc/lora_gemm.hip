@@ -15,25 +15,13 @@
 // never goes to HBM.  One workgroup walks several N tiles of the same M block
 // so that T is computed once per chunk of N tiles rather than once per tile.
 #include "kh_common.h"
+#include "lora_gemm.h"
 
 namespace {
 
 constexpr int BK = 64;       // K slab per LDS stage (bf16 elements)
 constexpr int LDK = BK + 8;  // padded LDS row: 144 B, so the 16 rows one ds_read_b128 phase touches hit 16 distinct bank groups
 
-struct LoraGemmParams {
-  const bf16_t* x;
-  const bf16_t* w;
-  const bf16_t* bias;      // may be null
-  const bf16_t* a_cat;     // [R,K] (unused when R == 0)
-  const bf16_t* b_cat;     // [N,R]
-  const float* col_scale;  // [R]
-  const bf16_t* res;       // [M,N] residual added in the epilogue, may be null
-  bf16_t* y;
-  int M, N, K, R;
-  int m_tiles, n_tiles, n_chunk, n_chunks;  // n_chunk = N tiles walked by one workgroup
-  int geglu;                                // 1: W rows are (value,gate) interleaved in 32-column groups, y is [M,N/2]
-};
 
 template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int NRT_>
 struct Cfg {
@@ -496,6 +484,8 @@ KH_EXPORT int kh_lora_linear_bf16(const void* x, const void* w, const void* bias
   p.geglu = geglu ? 1 : 0;
   hipStream_t s = (hipStream_t)stream;
   const int tile_sel = (flags >> 8) & 0xff;  // 0 = automatic
+  // K % 32 == 0 (every SDXL layer): the software-pipelined kernel; tile_sel 1/2 force the simple kernel
+  if (K % 32 == 0 && (tile_sel == 0 || tile_sel >= 16)) return lora_gemm_pipe_launch(p, tile_sel, s);
   if (tile_sel == 2) return R > 96 ? KH_ERR_UNSUPPORTED : launch_rank<256, 128, 2, 2>(p, s);
   if (tile_sel == 1) return launch_rank<128, 128, 2, 2>(p, s);
   return launch_rank<128, 128, 2, 2>(p, s);

@@ -1,0 +1,419 @@
+// K1, software-pipelined variant: fused base GEMM + LoRA delta on bf16 MFMA (gfx950), K % 32 == 0.
+//
+// Same arithmetic as lora_gemm.hip (see there for the formula and the reference citations); what
+// differs is how operands reach the MFMAs:
+//   * x / W / A_cat tiles go global -> LDS directly (global_load_lds_dwordx4, no VGPR staging) into
+//     a ring of NST stages of 32 K-columns each; loads run NST-1 tiles ahead of the MFMAs, each
+//     wave waits only for its own oldest loads (s_waitcnt vmcnt(n)) and one barrier per K tile
+//     publishes them;
+//   * LDS rows are 64 bytes, unpadded; the four 16-byte pieces of a row are XOR-swizzled with
+//     (row/4)%4 so that the 16 rows one ds_read_b128 phase touches fall into 16 distinct bank
+//     groups (the DMA writes lane i to slot i, so the swizzle is applied to the global address a
+//     lane fetches, not to where it lands).
+#include "kh_common.h"
+#include "lora_gemm.h"
+#include <type_traits>
+
+namespace {
+
+constexpr int BKP = 32;    // K columns per stage
+constexpr int ROWB = 64;   // bytes per LDS row
+
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int NRT_, int NST_>
+struct PCfg {
+  static constexpr int BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, NRT = NRT_, NST = NST_;
+  static constexpr int NW = WAVES_M * WAVES_N, NT = NW * 64;
+  static constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
+  static constexpr int TM = WTM / 32, TN = WTN / 32;
+  static constexpr int R = NRT * 32;
+  static constexpr int SM = (NRT > 0) ? TM / WAVES_N : 0;
+  static constexpr int UX = BM / 16, UW = BN / 16, UA = R / 16;        // 16-row DMA units per stage
+  static constexpr int MU = (UX + UW + UA + NW - 1) / NW;              // most units one wave issues per stage
+  static constexpr int SW_OFF = BM * ROWB, SA_OFF = (BM + BN) * ROWB;
+  static constexpr int STAGE = (BM + BN + R) * ROWB;
+  static constexpr int LDT = R + 8, LDC = BN + 8;
+  static constexpr size_t RING = (size_t)NST * STAGE;
+  static constexpr size_t SB = (size_t)BN * LDT * 2;
+  static constexpr size_t SC = (size_t)WAVES_M * 32 * LDC * 2;
+  static constexpr size_t RING_MAX = RING > SB ? (RING > SC ? RING : SC) : (SB > SC ? SB : SC);
+  static constexpr size_t ST = (NRT > 0) ? (size_t)BM * LDT * 2 : 0;
+  static constexpr size_t LDS_BYTES = RING_MAX + ST;
+  static_assert(BM % (32 * WAVES_M) == 0 && BN % (32 * WAVES_N) == 0, "tile/wave mismatch");
+  static_assert(NRT == 0 || (TM % WAVES_N == 0), "shrink tiles must split evenly over the waves of a row");
+  static_assert(NST >= 2 && NST <= 5, "ring depth");
+  static_assert(UX % NW == 0 && UW % NW == 0 && (R / 8) % NW == 0, "DMA work must split evenly over the waves");
+  static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
+};
+
+// s_waitcnt with vmcnt = VM and lgkmcnt = LGKM (15 = unconstrained), expcnt unconstrained
+// (gfx9 encoding: vmcnt = [15:14|3:0], expcnt = [6:4], lgkmcnt = [11:8]).
+template <int VM, int LGKM>
+__device__ __forceinline__ void wait_cnt() {
+  __builtin_amdgcn_s_waitcnt((VM & 15) | (7 << 4) | ((LGKM & 15) << 8) | ((VM >> 4) << 14));
+}
+
+typedef const __attribute__((address_space(1))) void* gptr_t;
+typedef __attribute__((address_space(3))) void* lptr_t;
+
+__device__ __forceinline__ u32x4 ld16(const bf16_t* p) { return *reinterpret_cast<const u32x4*>(p); }
+__device__ __forceinline__ bf16x8 lds_frag(const char* p) { return *reinterpret_cast<const bf16x8*>(p); }
+__device__ __forceinline__ bf16x8 lds_fragb(const bf16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
+
+// Fragments of one K tile (32 columns = two 16-wide MFMA steps) held in registers.
+template <class C, bool SHRINK>
+struct Frags {
+  bf16x8 a[2][C::TM];
+  bf16x8 b[2][C::TN];
+  bf16x8 r[2][SHRINK ? C::NRT : 1];
+};
+
+// DMA work of one wave for one K tile: the same number of global_load_lds instructions for every
+// wave (so the vmcnt that isolates "my loads of tile t" is a compile-time constant): XI x-units and
+// WI W-units of 16 rows, and R/NW rows of A_cat as AI instructions (the last one half-masked when
+// R/NW is 8 mod 16).
+template <class C, bool SHRINK>
+struct Dma {
+  static constexpr int XI = C::UX / C::NW, WI = C::UW / C::NW;
+  static constexpr int RA = SHRINK ? C::R / C::NW : 0;       // A_cat rows per wave
+  static constexpr int AI = (RA + 15) / 16;
+  static constexpr int LPS = XI + WI + AI;                    // loads per stage per wave
+  static constexpr int N = LPS > 0 ? LPS : 1;
+  const bf16_t* src[N];
+  int dst[N];
+};
+
+// The K loop.  Three things overlap: DMA loads run NST-1 tiles ahead (global -> LDS ring); the LDS ->
+// register fragment reads of tile kt+1 are issued right after the barrier that publishes it; the
+// MFMAs of tile kt execute from the other register buffer -- half of them before that barrier, so the
+// matrix pipe has work queued while the wave waits for its neighbours, half after it, under the reads.
+// SHRINK also accumulates T = x . A_cat^T for the shrink m-tiles of this wave (m-tile wn*SM + s of
+// its wave row, selected branch-free from the x fragments it holds).
+template <class C, bool SHRINK>
+__device__ __forceinline__ void k_loop(char* smem, const Dma<C, SHRINK>& dma, int KT, int lane, int wm, int wn,
+                                       int l32, int lh, int sw, f32x16 (&acc)[C::TM][C::TN],
+                                       f32x16 (&tacc)[C::SM > 0 ? C::SM : 1][C::NRT > 0 ? C::NRT : 1]) {
+  constexpr int TM = C::TM, TN = C::TN, NRT = C::NRT, NST = C::NST;
+  constexpr int PD = NST - 1;  // prefetch distance in K tiles
+  using D = Dma<C, SHRINK>;
+  auto issue = [&](int t) {
+    char* stage = smem + (t % NST) * C::STAGE;
+#pragma unroll
+    for (int q = 0; q < D::LPS; ++q) {
+      const bool partial = SHRINK && (q == D::LPS - 1) && (D::RA % 16 != 0);
+      if (!partial || lane < 32)
+        __builtin_amdgcn_global_load_lds((gptr_t)(dma.src[q] + t * BKP), (lptr_t)(stage + dma.dst[q]), 16, 0, 0);
+    }
+  };
+  auto read_frags = [&](int t, Frags<C, SHRINK>& f) {
+    const char* st = smem + (t % NST) * C::STAGE;
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      const int po = ((2 * ks + lh) ^ sw) * 16;
+#pragma unroll
+      for (int i = 0; i < TM; ++i) f.a[ks][i] = lds_frag(st + (wm * C::WTM + i * 32 + l32) * ROWB + po);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) f.b[ks][j] = lds_frag(st + C::SW_OFF + (wn * C::WTN + j * 32 + l32) * ROWB + po);
+      if constexpr (SHRINK) {
+#pragma unroll
+        for (int r = 0; r < NRT; ++r) f.r[ks][r] = lds_frag(st + C::SA_OFF + (r * 32 + l32) * ROWB + po);
+      }
+    }
+  };
+  auto mma = [&](const Frags<C, SHRINK>& f, int ks) {
+    if constexpr (SHRINK) {
+#pragma unroll
+      for (int s = 0; s < C::SM; ++s) {
+        bf16x8 as = f.a[ks][s];  // wn == 0
+#pragma unroll
+        for (int q = 1; q < C::WAVES_N; ++q) as = (wn == q) ? f.a[ks][q * C::SM + s] : as;
+#pragma unroll
+        for (int r = 0; r < NRT; ++r)
+          tacc[s][r] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as, f.r[ks][r], tacc[s][r], 0, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a[ks][i], f.b[ks][j], acc[i][j], 0, 0, 0);
+  };
+  // Steady-state step: tile kt is in `cur`; tile kt+1 becomes visible, tile kt+1+PD is requested.
+  // Bare s_barrier (no workgroup fence: a fence is s_waitcnt vmcnt(0) and would drain the prefetches).
+  // Before it: this wave's DMA loads of tile kt+1 are complete (only the PD-1 later tiles may be
+  // outstanding) and so are its LDS reads of tile kt (lgkmcnt 0), whose stage the DMA after the
+  // barrier refills.
+  auto step_steady = [&](int kt, const Frags<C, SHRINK>& cur, Frags<C, SHRINK>& nxt) {
+    mma(cur, 0);
+    wait_cnt<D::LPS*(PD - 1), 0>();
+    __builtin_amdgcn_s_barrier();
+    issue(kt + 1 + PD);
+    read_frags(kt + 1, nxt);
+    mma(cur, 1);
+  };
+  auto step_tail = [&](int kt, const Frags<C, SHRINK>& cur, Frags<C, SHRINK>& nxt) {
+    mma(cur, 0);
+    if (kt + 1 < KT) {
+      wait_cnt<0, 0>();
+      __builtin_amdgcn_s_barrier();
+      read_frags(kt + 1, nxt);
+    }
+    mma(cur, 1);
+  };
+
+  wait_cnt<0, 15>();  // stores of the previous tile's epilogue are out of the way of the counting below
+#pragma unroll
+  for (int t = 0; t < PD; ++t)
+    if (t < KT) issue(t);
+  Frags<C, SHRINK> f0, f1;
+  wait_cnt<0, 15>();
+  __builtin_amdgcn_s_barrier();
+  if (PD < KT) issue(PD);
+  read_frags(0, f0);
+  int kt = 0;
+  for (; kt + 2 + PD < KT; kt += 2) {
+    step_steady(kt, f0, f1);
+    step_steady(kt + 1, f1, f0);
+  }
+  for (; kt < KT; kt += 2) {
+    step_tail(kt, f0, f1);
+    if (kt + 1 < KT) step_tail(kt + 1, f1, f0);
+  }
+}
+
+template <class C>
+__global__ __launch_bounds__(C::NT) void lora_gemm_pipe_kernel(const LoraGemmParams p) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  constexpr int BM = C::BM, BN = C::BN, TM = C::TM, TN = C::TN, NRT = C::NRT, R = C::R, NST = C::NST;
+  constexpr int SMT = C::SM > 0 ? C::SM : 1, NRTT = NRT > 0 ? NRT : 1;
+  bf16_t* sB = reinterpret_cast<bf16_t*>(smem);                // aliases the ring (after the K loop)
+  bf16_t* sC = reinterpret_cast<bf16_t*>(smem);                // aliases the ring (after the expand)
+  bf16_t* sT = reinterpret_cast<bf16_t*>(smem + C::RING_MAX);  // lives across N tiles
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / C::WAVES_N, wn = wave % C::WAVES_N;
+  const int l32 = lane & 31, lh = lane >> 5;
+
+  const uint32_t total = (uint32_t)p.m_tiles * (uint32_t)p.n_chunks;
+  const uint32_t logical = xcd_remap(blockIdx.x, total);
+  const int m_blk = logical / p.n_chunks, chunk = logical % p.n_chunks;
+  const int m0 = m_blk * BM;
+  const int K = p.K, M = p.M, N = p.N;
+  const int KT = K / BKP;
+
+  // DMA geometry of this lane inside a 16-row unit: LDS slot = lane (16 bytes each); it holds row
+  // lane/4, physical piece lane%4, which stores logical piece (lane%4) ^ ((row/4)%4).
+  const int u_row = lane >> 2;
+  // fragment read: logical piece (2*ks + lh) of row (.. + l32) sits at physical piece ^ ((l32/4)%4)
+  const int sw = (l32 >> 2) & 3;
+
+  for (int jt = 0; jt < p.n_chunk; ++jt) {
+    const int n_tile = chunk * p.n_chunk + jt;
+    if (n_tile >= p.n_tiles) break;  // uniform over the workgroup
+    const int n0 = n_tile * BN;
+    const bool shrink = (NRT > 0) && (jt == 0);
+
+    // this wave's DMA sources / LDS destinations for one stage (K offset 0; the loop adds t*32 columns)
+    auto dma_setup = [&](auto& d) {
+      using D = typename std::remove_reference<decltype(d)>::type;
+      int q = 0;
+#pragma unroll
+      for (int i = 0; i < D::XI; ++i, ++q) {
+        const int r = (wave * D::XI + i) * 16 + u_row;  // row inside the x tile
+        int row = m0 + r; row = row < M ? row : M - 1;
+        d.src[q] = p.x + (size_t)row * K + (((lane & 3) ^ ((r >> 2) & 3)) * 8);
+        d.dst[q] = (wave * D::XI + i) * 1024;
+      }
+#pragma unroll
+      for (int i = 0; i < D::WI; ++i, ++q) {
+        const int r = (wave * D::WI + i) * 16 + u_row;
+        int row = n0 + r; row = row < N ? row : N - 1;
+        d.src[q] = p.w + (size_t)row * K + (((lane & 3) ^ ((r >> 2) & 3)) * 8);
+        d.dst[q] = C::SW_OFF + (wave * D::WI + i) * 1024;
+      }
+#pragma unroll
+      for (int i = 0; i < D::AI; ++i, ++q) {
+        int r = wave * D::RA + i * 16 + u_row;          // rank row; lanes >= 32 of a half instruction are masked off
+        r = r < C::R ? r : C::R - 1;
+        d.src[q] = p.a_cat + (size_t)r * K + (((lane & 3) ^ ((r >> 2) & 3)) * 8);
+        d.dst[q] = C::SA_OFF + (wave * D::RA + i * 16) * ROWB;
+      }
+    };
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+    f32x16 tacc[SMT][NRTT];
+#pragma unroll
+    for (int s = 0; s < SMT; ++s)
+#pragma unroll
+      for (int r = 0; r < NRTT; ++r)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) tacc[s][r][v] = 0.f;
+
+    if (shrink) {
+      if constexpr (NRT > 0) {
+        Dma<C, true> d;
+        dma_setup(d);
+        k_loop<C, true>(smem, d, KT, lane, wm, wn, l32, lh, sw, acc, tacc);
+      }
+    } else {
+      Dma<C, false> d;
+      dma_setup(d);
+      k_loop<C, false>(smem, d, KT, lane, wm, wn, l32, lh, sw, acc, tacc);
+    }
+    __syncthreads();  // every wave is done reading the ring before sB / sC reuse it
+
+    if constexpr (NRT > 0) {
+      if (shrink) {
+#pragma unroll
+        for (int r = 0; r < NRT; ++r) {
+          const int col = r * 32 + l32;
+          const float sc = p.col_scale[col];
+#pragma unroll
+          for (int s = 0; s < C::SM; ++s) {
+            const int rbase = wm * C::WTM + (wn * C::SM + s) * 32 + 4 * lh;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+              const int row = rbase + 8 * (v >> 2) + (v & 3);
+              sT[row * C::LDT + col] = (bf16_t)(tacc[s][r][v] * sc);
+            }
+          }
+        }
+      }
+      for (int c = tid; c < BN * (R / 8); c += C::NT) {
+        const int row = c / (R / 8), ch = c % (R / 8);
+        int gr = n0 + row; gr = gr < N ? gr : N - 1;
+        *reinterpret_cast<u32x4*>(sB + row * C::LDT + ch * 8) = ld16(p.b_cat + (size_t)gr * R + ch * 8);
+      }
+      __syncthreads();
+#pragma unroll
+      for (int ks = 0; ks < R / 16; ++ks) {
+        bf16x8 a[TM], b[TN];
+        const int ko = ks * 16 + lh * 8;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) a[i] = lds_fragb(sT + (wm * C::WTM + i * 32 + l32) * C::LDT + ko);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) b[j] = lds_fragb(sB + (wn * C::WTN + j * 32 + l32) * C::LDT + ko);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+      }
+      __syncthreads();  // sB is dead before sC overwrites it
+    }
+
+    // Epilogue: bias in fp32, round to bf16, transpose through LDS so that every global store is a
+    // 16-byte piece of a contiguous output row.
+    float bv[TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int col = n0 + wn * C::WTN + j * 32 + l32;
+      bv[j] = (p.bias != nullptr && col < N) ? (float)p.bias[col] : 0.f;
+    }
+    const int out_ld = p.geglu ? (N >> 1) : N;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int col = wn * C::WTN + j * 32 + l32;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int row = wm * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+          sC[row * C::LDC + col] = (bf16_t)(acc[i][j][v] + bv[j]);
+        }
+      }
+      __syncthreads();
+      if (!p.geglu) {
+        constexpr int CPR = BN / 8;
+        for (int c = tid; c < C::WAVES_M * 32 * CPR; c += C::NT) {
+          const int srow = c / CPR, ch = c % CPR;
+          const int grow = m0 + (srow >> 5) * C::WTM + i * 32 + (srow & 31);
+          const int gcol = n0 + ch * 8;
+          if (grow < M && gcol < N) {
+            u32x4 o = *reinterpret_cast<const u32x4*>(sC + srow * C::LDC + ch * 8);
+            if (p.res != nullptr) {
+              const u32x4 rr = ld16(p.res + (size_t)grow * N + gcol);
+#pragma unroll
+              for (int e = 0; e < 4; ++e)
+                o[e] = pack_bf16x2(bf16_lo(o[e]) + bf16_lo(rr[e]), bf16_hi(o[e]) + bf16_hi(rr[e]));
+            }
+            *reinterpret_cast<u32x4*>(p.y + (size_t)grow * N + gcol) = o;
+          }
+        }
+      } else {
+        constexpr int OPR = BN / 16;
+        for (int c = tid; c < C::WAVES_M * 32 * OPR; c += C::NT) {
+          const int srow = c / OPR, oc = c % OPR;
+          const int grp = oc >> 2, sub = oc & 3;
+          const int grow = m0 + (srow >> 5) * C::WTM + i * 32 + (srow & 31);
+          const int gcol = (n0 >> 1) + grp * 32 + sub * 8;
+          if (grow < M && gcol < out_ld) {
+            const u32x4 hv = *reinterpret_cast<const u32x4*>(sC + srow * C::LDC + grp * 64 + sub * 8);
+            const u32x4 gv = *reinterpret_cast<const u32x4*>(sC + srow * C::LDC + grp * 64 + 32 + sub * 8);
+            u32x4 o;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const float g0 = bf16_lo(gv[e]), g1 = bf16_hi(gv[e]);
+              const float a0 = 0.5f * g0 * (1.f + erff(g0 * 0.70710678118654752f));
+              const float a1 = 0.5f * g1 * (1.f + erff(g1 * 0.70710678118654752f));
+              const uint32_t ar = pack_bf16x2(a0, a1);  // gelu(gate) rounded to bf16 before the product
+              o[e] = pack_bf16x2(bf16_lo(hv[e]) * bf16_lo(ar), bf16_hi(hv[e]) * bf16_hi(ar));
+            }
+            *reinterpret_cast<u32x4*>(p.y + (size_t)grow * out_ld + gcol) = o;
+          }
+        }
+      }
+      __syncthreads();
+    }
+  }
+}
+
+template <class C>
+int launch_pcfg(LoraGemmParams p, hipStream_t stream) {
+  p.m_tiles = (p.M + C::BM - 1) / C::BM;
+  p.n_tiles = (p.N + C::BN - 1) / C::BN;
+  int nc = 1;
+  if (C::NRT > 0) {
+    // walk several N tiles per workgroup (T reused from LDS) while the grid still covers the chip
+    while (nc < p.n_tiles && (long)p.m_tiles * ((p.n_tiles + 2 * nc - 1) / (2 * nc)) >= 256) nc *= 2;
+  }
+  p.n_chunk = nc;
+  p.n_chunks = (p.n_tiles + nc - 1) / nc;
+  static bool attr_done = false;  // per template instantiation
+  if (!attr_done) {
+    hipError_t e = hipFuncSetAttribute((const void*)lora_gemm_pipe_kernel<C>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)C::LDS_BYTES);
+    if (e != hipSuccess) return (int)e;
+    attr_done = true;
+  }
+  const unsigned grid = (unsigned)(p.m_tiles * p.n_chunks);
+  kh_launch(KH_TAG_LORA_GEMM, lora_gemm_pipe_kernel<C>, dim3(grid), dim3(C::NT), C::LDS_BYTES, stream, p);
+  KH_RETURN_LAST_ERROR();
+}
+
+template <int BM, int BN, int WM, int WN, int NST>
+int launch_prank(const LoraGemmParams& p, hipStream_t stream) {
+  switch (p.R / 32) {
+    case 0: return launch_pcfg<PCfg<BM, BN, WM, WN, 0, NST>>(p, stream);
+    case 1: return launch_pcfg<PCfg<BM, BN, WM, WN, 1, NST>>(p, stream);
+    case 2: return launch_pcfg<PCfg<BM, BN, WM, WN, 2, NST>>(p, stream);
+    case 3: return launch_pcfg<PCfg<BM, BN, WM, WN, 3, NST>>(p, stream);
+    case 4: return launch_pcfg<PCfg<BM, BN, WM, WN, 4, NST>>(p, stream);
+    default: return KH_ERR_UNSUPPORTED;
+  }
+}
+
+}  // namespace
+
+int lora_gemm_pipe_launch(const LoraGemmParams& p, int tile_sel, hipStream_t stream) {
+  switch (tile_sel) {
+    case 17: return launch_prank<128, 128, 2, 2, 3>(p, stream);
+    case 18: return launch_prank<128, 128, 2, 2, 2>(p, stream);
+    default: return launch_prank<128, 128, 2, 2, 4>(p, stream);
+  }
+}
