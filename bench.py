@@ -203,8 +203,11 @@ def main():
     gemm_calls = [c for c in log if c[0] == "lora_linear"]
     gemm_ms = [d for n, d in launches if n == "lora_gemm"]
     assert len(gemm_calls) == len(gemm_ms), (len(gemm_calls), len(gemm_ms))
+    # two-launch layers: the shrink launch belongs to the layer whose GEMM follows it
+    shrink_calls = [c for c in log if c[0] == "lora_shrink"]
+    shrink_ms = sum(d for n, d in launches if n == "lora_shrink")
     gemm_flops = sum(lora_linear_flops(c[1], c[2], c[3], c[4]) for c in gemm_calls)
-    gemm_total_ms = sum(gemm_ms)
+    gemm_total_ms = sum(gemm_ms) + shrink_ms
     attn_flops = sum(4.0 * c[1] * c[2] * c[3] * c[4] * c[5] for c in log if c[0] == "attention")
     step_flops = gemm_flops + attn_flops + conv_flops
     achieved_tf = gemm_flops / (gemm_total_ms * 1e-3) / 1e12
@@ -244,7 +247,8 @@ def main():
         "roofline": {"kernel": "lora_gemm_kernel (fused base GEMM + LoRA delta, all launches of one step)",
                      "bound": "mfma", "achieved": round(achieved_tf, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved_tf / PEAK_BF16_TFLOPS, 4), "traffic": None,
-                     "launches_per_step": len(gemm_ms), "avg_launch_us": round(gemm_total_ms / len(gemm_ms) * 1e3, 2),
+                     "launches_per_step": len(gemm_ms), "shrink_launches_per_step": len(shrink_calls),
+                     "shrink_ms_per_step": round(shrink_ms, 3), "avg_launch_us": round(gemm_total_ms / len(gemm_ms) * 1e3, 2),
                      "algorithmic_gflop_per_step": round(gemm_flops / 1e9, 1), "by_shape": shape_rows[:8]},
         "kernel_ms_per_step": {k: {"launches": v[0], "ms": round(v[1], 3)} for k, v in sorted(by_kernel.items())},
     }

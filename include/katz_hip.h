@@ -41,7 +41,7 @@ const char* kh_error_string(int code);
  * kh_profile_begin and kh_profile_end every kernel of this library is launched with its own HIP
  * start/stop event pair on the launch stream.  kh_profile_end waits for them and writes, in launch
  * order, a kernel tag (1 lora_gemm, 2 lora_gemm_f32, 3 attention, 4 group_norm stats, 5 group_norm apply,
- * 6 layer_norm, 7 geglu, 8 residual_add, 9 concat_residual, 10 sgmv_shrink, 11 sgmv_expand) and the
+ * 6 layer_norm, 7 geglu, 8 residual_add, 9 concat_residual, 10 sgmv_shrink, 11 sgmv_expand, 12 lora_shrink) and the
  * duration in ms into HOST arrays; returns the number of launches (or -hipError_t).  Do not use under
  * graph capture. */
 int kh_profile_begin(void);
@@ -65,6 +65,18 @@ int kh_profile_end(int32_t* tags, float* ms, int capacity);
 int kh_lora_linear_bf16(const void* x, const void* w, const void* bias, const void* a_cat, const void* b_cat,
                         const float* col_scale, const void* residual, void* y, int64_t M, int64_t N, int64_t K,
                         int64_t R, int flags, void* stream);
+/* The same layer in two launches, for inputs whose rank-R product is better computed once than once per
+ * output tile (and for several layers sharing one input, e.g. to_q/to_k/to_v: stack their A matrices):
+ *   kh_lora_shrink_bf16:      t[M,R] = bf16((x[M,K] A_cat[R,K]^T) * col_scale[R])      K % 64 == 0, R % 32 == 0, R <= 1024
+ *   kh_lora_linear_pre_bf16:  y = x W^T + bias + t[:, 0:R] B_cat[N,R]^T (+ residual | GEGLU)
+ * t is [M, ldt] with ldt >= R (a column slice of a wider shrink result is addressed by offsetting the
+ * pointer); it is ~1 MB and stays in L2 between the two launches.  Same reference formula as above
+ * (lora.py:222-232: up(down(x)) * scale).  K % 32 == 0, R <= 128, flags as for kh_lora_linear_bf16. */
+int kh_lora_shrink_bf16(const void* x, const void* a_cat, const float* col_scale, void* t, int64_t M, int64_t K,
+                        int64_t R, void* stream);
+int kh_lora_linear_pre_bf16(const void* x, const void* w, const void* bias, const void* t, int64_t ldt,
+                            const void* b_cat, const void* residual, void* y, int64_t M, int64_t N, int64_t K,
+                            int64_t R, int flags, void* stream);
 /* fp32 variant of the same formula (fp32 parity path); R <= 128, any M/N/K. */
 int kh_lora_linear_f32(const float* x, const float* w, const float* bias, const float* a_cat, const float* b_cat,
                        const float* col_scale, const float* residual, float* y, int64_t M, int64_t N, int64_t K,

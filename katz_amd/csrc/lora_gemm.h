@@ -9,6 +9,8 @@ struct LoraGemmParams {
   const bf16_t* a_cat;     // [R,K] (unused when R == 0)
   const bf16_t* b_cat;     // [N,R]
   const float* col_scale;  // [R]
+  const bf16_t* t_ext;     // [M, ldt] precomputed, already scaled shrink result (null: compute it in the kernel)
+  int ldt;
   const bf16_t* res;       // [M,N] residual added in the epilogue, may be null
   bf16_t* y;
   int M, N, K, R;

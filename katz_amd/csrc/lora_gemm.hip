@@ -479,6 +479,7 @@ KH_EXPORT int kh_lora_linear_bf16(const void* x, const void* w, const void* bias
   p.x = (const bf16_t*)x; p.w = (const bf16_t*)w; p.bias = (const bf16_t*)bias;
   p.a_cat = (const bf16_t*)a_cat; p.b_cat = (const bf16_t*)b_cat; p.col_scale = col_scale;
   p.res = (const bf16_t*)residual; p.y = (bf16_t*)y;
+  p.t_ext = nullptr; p.ldt = 0;
   p.M = (int)M; p.N = (int)N; p.K = (int)K; p.R = (int)R;
   p.m_tiles = p.n_tiles = p.n_chunk = p.n_chunks = 0;
   p.geglu = geglu ? 1 : 0;
@@ -489,6 +490,30 @@ KH_EXPORT int kh_lora_linear_bf16(const void* x, const void* w, const void* bias
   if (tile_sel == 2) return R > 96 ? KH_ERR_UNSUPPORTED : launch_rank<256, 128, 2, 2>(p, s);
   if (tile_sel == 1) return launch_rank<128, 128, 2, 2>(p, s);
   return launch_rank<128, 128, 2, 2>(p, s);
+}
+
+// Base GEMM + expand with a precomputed shrink result t (kh_lora_shrink_bf16); see include/katz_hip.h.
+KH_EXPORT int kh_lora_linear_pre_bf16(const void* x, const void* w, const void* bias, const void* t, int64_t ldt,
+                                      const void* b_cat, const void* residual, void* y, int64_t M, int64_t N,
+                                      int64_t K, int64_t R, int flags, void* stream) {
+  if (!x || !w || !y || !t || !b_cat || M <= 0 || N <= 0 || K <= 0 || R <= 0 || ldt < R) return KH_ERR_INVALID_ARG;
+  if (K % 32 != 0 || N % 8 != 0 || R % 32 != 0 || ldt % 8 != 0) return KH_ERR_UNSUPPORTED;
+  if (R > 128) return KH_ERR_TOO_LARGE;
+  if (M > (1 << 24) || N > (1 << 24) || K > (1 << 24)) return KH_ERR_TOO_LARGE;
+  const bool geglu = (flags & 1) != 0;
+  if (geglu && (N % 64 != 0 || residual != nullptr)) return KH_ERR_UNSUPPORTED;
+  if (!kh_aligned16(x) || !kh_aligned16(w) || !kh_aligned16(y) || !kh_aligned16(t) || !kh_aligned16(b_cat) ||
+      (residual && !kh_aligned16(residual)))
+    return KH_ERR_ALIGNMENT;
+  LoraGemmParams p;
+  p.x = (const bf16_t*)x; p.w = (const bf16_t*)w; p.bias = (const bf16_t*)bias;
+  p.a_cat = nullptr; p.b_cat = (const bf16_t*)b_cat; p.col_scale = nullptr;
+  p.t_ext = (const bf16_t*)t; p.ldt = (int)ldt;
+  p.res = (const bf16_t*)residual; p.y = (bf16_t*)y;
+  p.M = (int)M; p.N = (int)N; p.K = (int)K; p.R = (int)R;
+  p.m_tiles = p.n_tiles = p.n_chunk = p.n_chunks = 0;
+  p.geglu = geglu ? 1 : 0;
+  return lora_gemm_pipe_launch(p, (flags >> 8) & 0xff, (hipStream_t)stream);
 }
 
 KH_EXPORT int kh_lora_linear_f32(const float* x, const float* w, const float* bias, const float* a_cat,

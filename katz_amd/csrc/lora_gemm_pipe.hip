@@ -27,21 +27,23 @@ struct PCfg {
   static constexpr int TM = WTM / 32, TN = WTN / 32;
   static constexpr int R = NRT * 32;
   static constexpr int SM = (NRT > 0) ? TM / WAVES_N : 0;
-  static constexpr int UX = BM / 16, UW = BN / 16, UA = R / 16;        // 16-row DMA units per stage
+  static constexpr int RS = R;                                         // A_cat rows staged per K tile
+  static constexpr int UX = BM / 16, UW = BN / 16, UA = RS / 16;       // 16-row DMA units per stage
   static constexpr int MU = (UX + UW + UA + NW - 1) / NW;              // most units one wave issues per stage
   static constexpr int SW_OFF = BM * ROWB, SA_OFF = (BM + BN) * ROWB;
-  static constexpr int STAGE = (BM + BN + R) * ROWB;
+  static constexpr int STAGE = (BM + BN + RS) * ROWB;
   static constexpr int LDT = R + 8, LDC = BN + 8;
   static constexpr size_t RING = (size_t)NST * STAGE;
   static constexpr size_t SB = (size_t)BN * LDT * 2;
   static constexpr size_t SC = (size_t)WAVES_M * 32 * LDC * 2;
   static constexpr size_t RING_MAX = RING > SB ? (RING > SC ? RING : SC) : (SB > SC ? SB : SC);
   static constexpr size_t ST = (NRT > 0) ? (size_t)BM * LDT * 2 : 0;
+  static constexpr size_t ST_OFF = RING_MAX;
   static constexpr size_t LDS_BYTES = RING_MAX + ST;
   static_assert(BM % (32 * WAVES_M) == 0 && BN % (32 * WAVES_N) == 0, "tile/wave mismatch");
   static_assert(NRT == 0 || (TM % WAVES_N == 0), "shrink tiles must split evenly over the waves of a row");
-  static_assert(NST >= 2 && NST <= 5, "ring depth");
-  static_assert(UX % NW == 0 && UW % NW == 0 && (R / 8) % NW == 0, "DMA work must split evenly over the waves");
+  static_assert(NST >= 2 && NST <= 4, "ring depth");
+  static_assert(UX % NW == 0 && UW % NW == 0 && (RS / 8) % NW == 0, "DMA work must split evenly over the waves");
   static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
 };
 
@@ -78,7 +80,11 @@ struct Dma {
   static constexpr int AI = (RA + 15) / 16;
   static constexpr int LPS = XI + WI + AI;                    // loads per stage per wave
   static constexpr int N = LPS > 0 ? LPS : 1;
-  const bf16_t* src[N];
+  // per instruction: element offset of the lane's source row in its matrix (row * K + swizzled piece),
+  // the same for the K-extension operand (row * ld2 + piece; T for the x rows, B_cat for the W rows),
+  // which matrix it is, and the LDS byte offset inside a stage
+  long off[N];
+  int off2[N];
   int dst[N];
 };
 
@@ -88,10 +94,13 @@ struct Dma {
 // matrix pipe has work queued while the wave waits for its neighbours, half after it, under the reads.
 // SHRINK also accumulates T = x . A_cat^T for the shrink m-tiles of this wave (m-tile wn*SM + s of
 // its wave row, selected branch-free from the x fragments it holds).
-template <class C, bool SHRINK>
-__device__ __forceinline__ void k_loop(char* smem, const Dma<C, SHRINK>& dma, int KT, int lane, int wm, int wn,
+template <class C, bool SHRINK, int NX, class TailLoads>
+__device__ __forceinline__ void k_loop(char* smem, const Dma<C, SHRINK>& dma, const bf16_t* px, const bf16_t* pw,
+                                       const bf16_t* pa, const bf16_t* px2, const bf16_t* pw2, int KT, int KT1,
+                                       int lane, int wm, int wn,
                                        int l32, int lh, int sw, f32x16 (&acc)[C::TM][C::TN],
-                                       f32x16 (&tacc)[C::SM > 0 ? C::SM : 1][C::NRT > 0 ? C::NRT : 1]) {
+                                       f32x16 (&tacc)[C::SM > 0 ? C::SM : 1][C::NRT > 0 ? C::NRT : 1],
+                                       TailLoads tail_loads) {
   constexpr int TM = C::TM, TN = C::TN, NRT = C::NRT, NST = C::NST;
   constexpr int PD = NST - 1;  // prefetch distance in K tiles
   using D = Dma<C, SHRINK>;
@@ -100,8 +109,12 @@ __device__ __forceinline__ void k_loop(char* smem, const Dma<C, SHRINK>& dma, in
 #pragma unroll
     for (int q = 0; q < D::LPS; ++q) {
       const bool partial = SHRINK && (q == D::LPS - 1) && (D::RA % 16 != 0);
+      // K tiles >= KT1 come from the extension operands: y = [x | T] . [W | B_cat]^T
+      const bf16_t* base = q < D::XI ? px : (q < D::XI + D::WI ? pw : pa);
+      const bf16_t* base2 = q < D::XI ? px2 : pw2;
+      const bf16_t* g = (SHRINK || t < KT1) ? base + dma.off[q] + t * BKP : base2 + dma.off2[q] + (t - KT1) * BKP;
       if (!partial || lane < 32)
-        __builtin_amdgcn_global_load_lds((gptr_t)(dma.src[q] + t * BKP), (lptr_t)(stage + dma.dst[q]), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((gptr_t)g, (lptr_t)(stage + dma.dst[q]), 16, 0, 0);
     }
   };
   auto read_frags = [&](int t, Frags<C, SHRINK>& f) {
@@ -137,11 +150,11 @@ __device__ __forceinline__ void k_loop(char* smem, const Dma<C, SHRINK>& dma, in
       for (int j = 0; j < TN; ++j)
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a[ks][i], f.b[ks][j], acc[i][j], 0, 0, 0);
   };
-  // Steady-state step: tile kt is in `cur`; tile kt+1 becomes visible, tile kt+1+PD is requested.
-  // Bare s_barrier (no workgroup fence: a fence is s_waitcnt vmcnt(0) and would drain the prefetches).
-  // Before it: this wave's DMA loads of tile kt+1 are complete (only the PD-1 later tiles may be
-  // outstanding) and so are its LDS reads of tile kt (lgkmcnt 0), whose stage the DMA after the
-  // barrier refills.
+  // Publish tile t and fetch its fragments.  Bare s_barrier (no workgroup fence: a fence is
+  // s_waitcnt vmcnt(0) and would drain the prefetches).  Before it: this wave's DMA loads of tile t
+  // are complete (VM = number of younger loads that may stay outstanding) and so are its LDS reads
+  // of tile t-1 (lgkmcnt 0), whose stage the DMA issued after the barrier refills.
+  // Steady state: tile kt is in `cur`; tile kt+1 becomes visible, tile kt+1+PD is requested.
   auto step_steady = [&](int kt, const Frags<C, SHRINK>& cur, Frags<C, SHRINK>& nxt) {
     mma(cur, 0);
     wait_cnt<D::LPS*(PD - 1), 0>();
@@ -150,44 +163,70 @@ __device__ __forceinline__ void k_loop(char* smem, const Dma<C, SHRINK>& dma, in
     read_frags(kt + 1, nxt);
     mma(cur, 1);
   };
-  auto step_tail = [&](int kt, const Frags<C, SHRINK>& cur, Frags<C, SHRINK>& nxt) {
-    mma(cur, 0);
-    if (kt + 1 < KT) {
-      wait_cnt<0, 0>();
-      __builtin_amdgcn_s_barrier();
-      read_frags(kt + 1, nxt);
-    }
-    mma(cur, 1);
-  };
 
   wait_cnt<0, 15>();  // stores of the previous tile's epilogue are out of the way of the counting below
-#pragma unroll
-  for (int t = 0; t < PD; ++t)
-    if (t < KT) issue(t);
   Frags<C, SHRINK> f0, f1;
-  wait_cnt<0, 15>();
-  __builtin_amdgcn_s_barrier();
-  if (PD < KT) issue(PD);
-  read_frags(0, f0);
-  int kt = 0;
-  for (; kt + 2 + PD < KT; kt += 2) {
-    step_steady(kt, f0, f1);
-    step_steady(kt + 1, f1, f0);
-  }
-  for (; kt < KT; kt += 2) {
-    step_tail(kt, f0, f1);
-    if (kt + 1 < KT) step_tail(kt + 1, f1, f0);
+  if (KT > PD) {
+#pragma unroll
+    for (int t = 0; t < PD; ++t) issue(t);
+    wait_cnt<D::LPS*(PD - 1), 15>();
+    __builtin_amdgcn_s_barrier();
+    issue(PD);
+    read_frags(0, f0);
+    int kt = 0;
+    for (; kt + 2 + PD < KT; kt += 2) {
+      step_steady(kt, f0, f1);
+      step_steady(kt + 1, f1, f0);
+    }
+    if (kt + 1 + PD < KT) {  // odd number of steady steps: one more, then rename f1 -> f0
+      step_steady(kt, f0, f1);
+      f0 = f1;
+      ++kt;
+    }
+    // Tail: kt == KT-PD-1, tile kt in f0, tiles kt+1 .. KT-1 in flight, nothing left to request.
+    // `tail_loads` may start NX extra global loads per wave (operands of the expand phase): they are
+    // younger than every DMA load, so the waits below leave them outstanding.
+    tail_loads();
+#pragma unroll
+    for (int j = 0; j < PD; ++j) {
+      Frags<C, SHRINK>& cur = (j & 1) ? f1 : f0;
+      Frags<C, SHRINK>& nxt = (j & 1) ? f0 : f1;
+      mma(cur, 0);
+      switch (j) {  // compile-time after unrolling: PD-1-j DMA tiles younger than tile kt+1+j
+        case 0: wait_cnt<D::LPS*(PD - 1) + NX, 0>(); break;
+        case 1: wait_cnt<D::LPS*(PD > 2 ? PD - 2 : 0) + NX, 0>(); break;
+        case 2: wait_cnt<D::LPS*(PD > 3 ? PD - 3 : 0) + NX, 0>(); break;
+        default: wait_cnt<NX, 0>(); break;
+      }
+      __builtin_amdgcn_s_barrier();
+      read_frags(kt + 1 + j, nxt);
+      mma(cur, 1);
+    }
+    const Frags<C, SHRINK>& last = (PD & 1) ? f1 : f0;
+    mma(last, 0);
+    mma(last, 1);
+  } else {
+    // fewer K tiles than ring stages (tiny K): request everything, wait for everything
+    for (int t = 0; t < KT; ++t) issue(t);
+    tail_loads();
+    wait_cnt<NX, 15>();
+    __builtin_amdgcn_s_barrier();
+    for (int t = 0; t < KT; ++t) {
+      read_frags(t, f0);
+      mma(f0, 0);
+      mma(f0, 1);
+    }
   }
 }
 
 template <class C>
-__global__ __launch_bounds__(C::NT) void lora_gemm_pipe_kernel(const LoraGemmParams p) {
+__global__ __launch_bounds__(C::NT, C::NRT == 0 ? 2 : 1) void lora_gemm_pipe_kernel(const LoraGemmParams p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   constexpr int BM = C::BM, BN = C::BN, TM = C::TM, TN = C::TN, NRT = C::NRT, R = C::R, NST = C::NST;
   constexpr int SMT = C::SM > 0 ? C::SM : 1, NRTT = NRT > 0 ? NRT : 1;
   bf16_t* sB = reinterpret_cast<bf16_t*>(smem);                // aliases the ring (after the K loop)
   bf16_t* sC = reinterpret_cast<bf16_t*>(smem);                // aliases the ring (after the expand)
-  bf16_t* sT = reinterpret_cast<bf16_t*>(smem + C::RING_MAX);  // lives across N tiles
+  bf16_t* sT = reinterpret_cast<bf16_t*>(smem + C::ST_OFF);    // fused mode: lives across N tiles
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -199,7 +238,8 @@ __global__ __launch_bounds__(C::NT) void lora_gemm_pipe_kernel(const LoraGemmPar
   const int m_blk = logical / p.n_chunks, chunk = logical % p.n_chunks;
   const int m0 = m_blk * BM;
   const int K = p.K, M = p.M, N = p.N;
-  const int KT = K / BKP;
+  const int KT1 = K / BKP;                                             // K tiles of x / W
+  const int KT = KT1 + (p.t_ext != nullptr ? p.R / BKP : 0);           // + rank tiles of T / B_cat (two-launch form)
 
   // DMA geometry of this lane inside a 16-row unit: LDS slot = lane (16 bytes each); it holds row
   // lane/4, physical piece lane%4, which stores logical piece (lane%4) ^ ((row/4)%4).
@@ -221,21 +261,24 @@ __global__ __launch_bounds__(C::NT) void lora_gemm_pipe_kernel(const LoraGemmPar
       for (int i = 0; i < D::XI; ++i, ++q) {
         const int r = (wave * D::XI + i) * 16 + u_row;  // row inside the x tile
         int row = m0 + r; row = row < M ? row : M - 1;
-        d.src[q] = p.x + (size_t)row * K + (((lane & 3) ^ ((r >> 2) & 3)) * 8);
+        d.off[q] = (long)row * K + (((lane & 3) ^ ((r >> 2) & 3)) * 8);
+        d.off2[q] = row * p.ldt + (((lane & 3) ^ ((r >> 2) & 3)) * 8);
         d.dst[q] = (wave * D::XI + i) * 1024;
       }
 #pragma unroll
       for (int i = 0; i < D::WI; ++i, ++q) {
         const int r = (wave * D::WI + i) * 16 + u_row;
         int row = n0 + r; row = row < N ? row : N - 1;
-        d.src[q] = p.w + (size_t)row * K + (((lane & 3) ^ ((r >> 2) & 3)) * 8);
+        d.off[q] = (long)row * K + (((lane & 3) ^ ((r >> 2) & 3)) * 8);
+        d.off2[q] = row * p.R + (((lane & 3) ^ ((r >> 2) & 3)) * 8);
         d.dst[q] = C::SW_OFF + (wave * D::WI + i) * 1024;
       }
 #pragma unroll
       for (int i = 0; i < D::AI; ++i, ++q) {
         int r = wave * D::RA + i * 16 + u_row;          // rank row; lanes >= 32 of a half instruction are masked off
         r = r < C::R ? r : C::R - 1;
-        d.src[q] = p.a_cat + (size_t)r * K + (((lane & 3) ^ ((r >> 2) & 3)) * 8);
+        d.off[q] = (long)r * K + (((lane & 3) ^ ((r >> 2) & 3)) * 8);
+        d.off2[q] = 0;
         d.dst[q] = C::SA_OFF + (wave * D::RA + i * 16) * ROWB;
       }
     };
@@ -254,16 +297,40 @@ __global__ __launch_bounds__(C::NT) void lora_gemm_pipe_kernel(const LoraGemmPar
 #pragma unroll
         for (int v = 0; v < 16; ++v) tacc[s][r][v] = 0.f;
 
+    // operands of the phases after the K loop, requested early: bias / col_scale before the loop, the
+    // B_cat tile when the loop enters its tail
+    float bv[TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int col = n0 + wn * C::WTN + j * 32 + l32;
+      bv[j] = (p.bias != nullptr && col < N) ? (float)p.bias[col] : 0.f;
+    }
+    float csv[NRTT];
+#pragma unroll
+    for (int r = 0; r < NRTT; ++r) csv[r] = (shrink && NRT > 0) ? p.col_scale[r * 32 + l32] : 0.f;
+    constexpr int RCH = R > 0 ? R / 8 : 1;                       // 16-byte pieces per T / B_cat row
+    constexpr int BCH = NRT > 0 ? BN * RCH / C::NT : 0;          // pieces of the B_cat tile per thread
+    static_assert(NRT == 0 || (BN * RCH) % C::NT == 0, "expand tile split");
+    u32x4 breg[BCH > 0 ? BCH : 1];
+    auto tail_loads = [&]() {
+#pragma unroll
+      for (int q = 0; q < BCH; ++q) {
+        const int c = tid + q * C::NT, row = c / RCH, ch = c % RCH;
+        int gr = n0 + row; gr = gr < N ? gr : N - 1;
+        breg[q] = ld16(p.b_cat + (size_t)gr * R + ch * 8);
+      }
+    };
+
     if (shrink) {
       if constexpr (NRT > 0) {
         Dma<C, true> d;
         dma_setup(d);
-        k_loop<C, true>(smem, d, KT, lane, wm, wn, l32, lh, sw, acc, tacc);
+        k_loop<C, true, BCH>(smem, d, p.x, p.w, p.a_cat, p.t_ext, p.b_cat, KT, KT1, lane, wm, wn, l32, lh, sw, acc, tacc, tail_loads);
       }
     } else {
       Dma<C, false> d;
       dma_setup(d);
-      k_loop<C, false>(smem, d, KT, lane, wm, wn, l32, lh, sw, acc, tacc);
+      k_loop<C, false, BCH>(smem, d, p.x, p.w, p.a_cat, p.t_ext, p.b_cat, KT, KT1, lane, wm, wn, l32, lh, sw, acc, tacc, tail_loads);
     }
     __syncthreads();  // every wave is done reading the ring before sB / sC reuse it
 
@@ -272,22 +339,21 @@ __global__ __launch_bounds__(C::NT) void lora_gemm_pipe_kernel(const LoraGemmPar
 #pragma unroll
         for (int r = 0; r < NRT; ++r) {
           const int col = r * 32 + l32;
-          const float sc = p.col_scale[col];
 #pragma unroll
           for (int s = 0; s < C::SM; ++s) {
             const int rbase = wm * C::WTM + (wn * C::SM + s) * 32 + 4 * lh;
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
               const int row = rbase + 8 * (v >> 2) + (v & 3);
-              sT[row * C::LDT + col] = (bf16_t)(tacc[s][r][v] * sc);
+              sT[row * C::LDT + col] = (bf16_t)(tacc[s][r][v] * csv[r]);
             }
           }
         }
       }
-      for (int c = tid; c < BN * (R / 8); c += C::NT) {
-        const int row = c / (R / 8), ch = c % (R / 8);
-        int gr = n0 + row; gr = gr < N ? gr : N - 1;
-        *reinterpret_cast<u32x4*>(sB + row * C::LDT + ch * 8) = ld16(p.b_cat + (size_t)gr * R + ch * 8);
+#pragma unroll
+      for (int q = 0; q < BCH; ++q) {
+        const int c = tid + q * C::NT, row = c / RCH, ch = c % RCH;
+        *reinterpret_cast<u32x4*>(sB + row * C::LDT + ch * 8) = breg[q];
       }
       __syncthreads();
 #pragma unroll
@@ -308,16 +374,25 @@ __global__ __launch_bounds__(C::NT) void lora_gemm_pipe_kernel(const LoraGemmPar
     }
 
     // Epilogue: bias in fp32, round to bf16, transpose through LDS so that every global store is a
-    // 16-byte piece of a contiguous output row.
-    float bv[TN];
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int col = n0 + wn * C::WTN + j * 32 + l32;
-      bv[j] = (p.bias != nullptr && col < N) ? (float)p.bias[col] : 0.f;
-    }
+    // 16-byte piece of a contiguous output row.  Residual pieces are requested before the staging
+    // writes so their latency hides behind the transpose.
     const int out_ld = p.geglu ? (N >> 1) : N;
+    constexpr int CPR = BN / 8;                                   // 16-byte pieces per staged row
+    constexpr int ECH = C::WAVES_M * 32 * CPR / C::NT;            // pieces per thread per pass
+    constexpr int OPR = BN / 16;                                  // GEGLU: output pieces per staged row
+    constexpr int GCH = C::WAVES_M * 32 * OPR / C::NT;
+    static_assert((C::WAVES_M * 32 * CPR) % C::NT == 0 && (C::WAVES_M * 32 * OPR) % C::NT == 0, "epilogue split");
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
+      u32x4 rr[ECH];
+      if (p.res != nullptr) {
+#pragma unroll
+        for (int q = 0; q < ECH; ++q) {
+          const int c = tid + q * C::NT, srow = c / CPR, ch = c % CPR;
+          const int grow = m0 + (srow >> 5) * C::WTM + i * 32 + (srow & 31), gcol = n0 + ch * 8;
+          rr[q] = (grow < M && gcol < N) ? ld16(p.res + (size_t)grow * N + gcol) : u32x4{0, 0, 0, 0};
+        }
+      }
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
         const int col = wn * C::WTN + j * 32 + l32;
@@ -329,26 +404,25 @@ __global__ __launch_bounds__(C::NT) void lora_gemm_pipe_kernel(const LoraGemmPar
       }
       __syncthreads();
       if (!p.geglu) {
-        constexpr int CPR = BN / 8;
-        for (int c = tid; c < C::WAVES_M * 32 * CPR; c += C::NT) {
-          const int srow = c / CPR, ch = c % CPR;
-          const int grow = m0 + (srow >> 5) * C::WTM + i * 32 + (srow & 31);
-          const int gcol = n0 + ch * 8;
+#pragma unroll
+        for (int q = 0; q < ECH; ++q) {
+          const int c = tid + q * C::NT, srow = c / CPR, ch = c % CPR;
+          const int grow = m0 + (srow >> 5) * C::WTM + i * 32 + (srow & 31), gcol = n0 + ch * 8;
           if (grow < M && gcol < N) {
             u32x4 o = *reinterpret_cast<const u32x4*>(sC + srow * C::LDC + ch * 8);
             if (p.res != nullptr) {
-              const u32x4 rr = ld16(p.res + (size_t)grow * N + gcol);
 #pragma unroll
               for (int e = 0; e < 4; ++e)
-                o[e] = pack_bf16x2(bf16_lo(o[e]) + bf16_lo(rr[e]), bf16_hi(o[e]) + bf16_hi(rr[e]));
+                o[e] = pack_bf16x2(bf16_lo(o[e]) + bf16_lo(rr[q][e]), bf16_hi(o[e]) + bf16_hi(rr[q][e]));
             }
             *reinterpret_cast<u32x4*>(p.y + (size_t)grow * N + gcol) = o;
           }
         }
       } else {
-        constexpr int OPR = BN / 16;
-        for (int c = tid; c < C::WAVES_M * 32 * OPR; c += C::NT) {
-          const int srow = c / OPR, oc = c % OPR;
+        // staged columns come in groups of 64 = 32 value columns then their 32 gate columns
+#pragma unroll
+        for (int q = 0; q < GCH; ++q) {
+          const int c = tid + q * C::NT, srow = c / OPR, oc = c % OPR;
           const int grp = oc >> 2, sub = oc & 3;
           const int grow = m0 + (srow >> 5) * C::WTM + i * 32 + (srow & 31);
           const int gcol = (n0 >> 1) + grp * 32 + sub * 8;
@@ -398,6 +472,8 @@ int launch_pcfg(LoraGemmParams p, hipStream_t stream) {
 
 template <int BM, int BN, int WM, int WN, int NST>
 int launch_prank(const LoraGemmParams& p, hipStream_t stream) {
+  // two-launch form: T is an input, the rank columns ride along as extra K tiles of the plain GEMM
+  if (p.t_ext != nullptr) return launch_pcfg<PCfg<BM, BN, WM, WN, 0, NST>>(p, stream);
   switch (p.R / 32) {
     case 0: return launch_pcfg<PCfg<BM, BN, WM, WN, 0, NST>>(p, stream);
     case 1: return launch_pcfg<PCfg<BM, BN, WM, WN, 1, NST>>(p, stream);

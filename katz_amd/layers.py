@@ -11,6 +11,7 @@ token view [N, H*W, C] the transformer blocks need is the same memory -- the NCH
 """
 from __future__ import annotations
 
+import os
 from typing import Dict, List, Optional, Sequence
 
 import torch
@@ -25,6 +26,11 @@ CL = torch.channels_last
 
 # When True, LoRALinear leaves its weights uninitialised (for models whose state dict is loaded next).
 SKIP_INIT = False
+
+# How a LoRALinear with active adapters runs:
+#   "fused": one launch, the rank-R product is computed per output tile and kept in LDS;
+#   "split": kh_lora_shrink_bf16 once per layer input, then the base GEMM + expand reading it from L2.
+LORA_MODE = os.getenv("KATZ_LORA_MODE", "split")
 
 
 class LoRALinear(nn.Module):
@@ -156,6 +162,9 @@ class LoRALinear(nn.Module):
         p = self._packed
         if p is None:
             return ops.lora_linear(x, w, b, residual=residual, geglu=self.geglu)
+        if LORA_MODE == "split" and x.dtype == torch.bfloat16 and self.in_features % 64 == 0:
+            t = ops.lora_shrink(x, p.a_cat, p.col_scale)
+            return ops.lora_linear_pre(x, w, b, t, p.b_cat, residual=residual, geglu=self.geglu)
         return ops.lora_linear(x, w, b, p.a_cat, p.b_cat, p.col_scale, residual=residual, geglu=self.geglu)
 
     def extra_repr(self) -> str:

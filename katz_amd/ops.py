@@ -102,6 +102,56 @@ def lora_linear(
     return out
 
 
+def lora_shrink(x: torch.Tensor, a_cat: torch.Tensor, col_scale: torch.Tensor, out: Optional[torch.Tensor] = None):
+    """t = bf16((x A_cat^T) * col_scale), [M, R]; A_cat may stack the adapters of several layers that read x."""
+    lib = _lib.load()
+    _req(x, BF16, "x"); _req(a_cat, BF16, "a_cat"); _req(col_scale, torch.float32, "col_scale")
+    K = x.shape[-1]
+    M = x.numel() // K
+    R = a_cat.shape[0]
+    if a_cat.shape != (R, K) or col_scale.shape != (R,):
+        raise ValueError("a_cat / col_scale must be [R,K] / [R]")
+    if out is None:
+        out = torch.empty((M, R), dtype=BF16, device=x.device)
+    if CALL_LOG is not None:
+        CALL_LOG.append(("lora_shrink", M, K, R))
+    rc = lib.kh_lora_shrink_bf16(_ptr(x), _ptr(a_cat), _ptr(col_scale), _ptr(out), M, K, R, _stream())
+    _lib.check(rc, "kh_lora_shrink_bf16")
+    return out
+
+
+def lora_linear_pre(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], t: torch.Tensor,
+                    b_cat: torch.Tensor, residual: Optional[torch.Tensor] = None, geglu: bool = False,
+                    tile: int = 0) -> torch.Tensor:
+    """y = x W^T + b + t B_cat^T (+ residual | GEGLU) with t = lora_shrink(x, ...)[:, cols] (a column
+    slice of a wider shrink result is fine: only its last axis must be contiguous)."""
+    lib = _lib.load()
+    _req(x, BF16, "x"); _req(weight, BF16, "weight"); _req(b_cat, BF16, "b_cat")
+    K = x.shape[-1]
+    N = weight.shape[0]
+    M = x.numel() // K
+    R = b_cat.shape[1]
+    if t.dtype != BF16 or not t.is_cuda or t.dim() != 2 or t.stride(1) != 1 or t.shape != (M, R):
+        raise ValueError(f"t must be a bfloat16 [M,R] = [{M},{R}] GPU matrix with a contiguous last axis")
+    if weight.shape[1] != K or b_cat.shape[0] != N:
+        raise ValueError("weight / b_cat do not match x")
+    if bias is not None:
+        _req(bias, BF16, "bias")
+    if residual is not None:
+        _req(residual, BF16, "residual")
+        if residual.numel() != M * N:
+            raise ValueError("residual must have the shape of the output")
+    n_out = N // 2 if geglu else N
+    out = torch.empty(tuple(x.shape[:-1]) + (n_out,), dtype=BF16, device=x.device)
+    if CALL_LOG is not None:
+        CALL_LOG.append(("lora_linear", M, N, K, R, bool(geglu), residual is not None))
+    flags = (1 if geglu else 0) | ((tile & 0xFF) << 8)
+    rc = lib.kh_lora_linear_pre_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(t), t.stride(0), _ptr(b_cat),
+                                     _ptr(residual), _ptr(out), M, N, K, R, flags, _stream())
+    _lib.check(rc, "kh_lora_linear_pre_bf16")
+    return out
+
+
 # --------------------------------------------------------------------------------------- K2
 def sgmv_shrink(x, a_all, seg_start, seg_adapter, adapter_rank, max_seg_rows: int, out=None):
     """t[rows, :r_a] = x[rows] A_a^T per segment. a_all [n_adapters, RP, K]; returns t [rows, RP]."""
@@ -299,7 +349,7 @@ def concat_residual(h: torch.Tensor, skip: torch.Tensor, residuals: Sequence[tor
 # --------------------------------------------------------------------------------------- per-launch timing
 KERNEL_TAGS = {1: "lora_gemm", 2: "lora_gemm_f32", 3: "attention", 4: "group_norm_stats", 5: "group_norm_apply",
                6: "layer_norm", 7: "geglu", 8: "residual_add", 9: "concat_residual", 10: "sgmv_shrink",
-               11: "sgmv_expand"}
+               11: "sgmv_expand", 12: "lora_shrink"}
 
 
 def profile_begin() -> None:

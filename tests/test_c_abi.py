@@ -1,0 +1,55 @@
+"""The C-ABI library loads without a GPU and exports exactly what include/katz_hip.h declares."""
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+
+ROOT = Path(__file__).resolve().parent.parent
+HEADER = ROOT / "include" / "katz_hip.h"
+
+
+def declared_symbols():
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    return sorted(set(re.findall(r"\b(kh_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    syms = declared_symbols()
+    for must in ("kh_lora_linear_bf16", "kh_lora_linear_f32", "kh_lora_shrink_bf16", "kh_lora_linear_pre_bf16",
+                 "kh_sgmv_shrink_bf16", "kh_sgmv_expand_bf16", "kh_attention_bf16", "kh_group_norm_bf16",
+                 "kh_layer_norm_bf16", "kh_geglu_bf16", "kh_gelu_mul_bf16", "kh_residual_add_bf16",
+                 "kh_concat_residual_bf16", "kh_version", "kh_error_string"):
+        assert must in syms
+
+
+def test_library_exports_every_declared_symbol():
+    from katz_amd import _lib
+
+    if not _lib.LIB_PATH.exists():
+        pytest.skip("libkatz_hip.so not built (run python -m katz_amd.build)")
+    lib = ctypes.CDLL(str(_lib.LIB_PATH))
+    for name in declared_symbols():
+        assert hasattr(lib, name), f"{name} is declared in katz_hip.h but not exported"
+    # the ctypes prototype table covers the header one to one
+    assert sorted(_lib.SIGNATURES) == declared_symbols()
+
+
+def test_argument_validation_needs_no_gpu():
+    """Entry points reject bad arguments before touching the device."""
+    from katz_amd import _lib
+
+    if not _lib.LIB_PATH.exists():
+        pytest.skip("libkatz_hip.so not built")
+    lib = _lib.load()
+    assert lib.kh_version() >= 1
+    assert b"aligned" in lib.kh_error_string(-3)
+    assert lib.kh_lora_linear_bf16(None, None, None, None, None, None, None, None, 1, 8, 8, 0, 0, None) == -1
+    assert lib.kh_lora_linear_bf16(16, 16, None, None, None, None, None, 16, 4, 8, 12, 0, 0, None) == -2   # K % 8
+    assert lib.kh_lora_linear_bf16(16, 16, None, 16, 16, 16, None, 16, 4, 8, 8, 160, 0, None) == -4        # R > 128
+    assert lib.kh_lora_linear_bf16(8, 16, None, None, None, None, None, 16, 4, 8, 8, 0, 0, None) == -3     # alignment
+    assert lib.kh_attention_bf16(16, 16, 16, 16, 1, 1, 4, 4, 32, 64, 64, 64, 64, 256, 256, 256, 256, 0.1, None) == -2
+    assert lib.kh_group_norm_workspace_bytes(2, 320, 16384, 32, 1) > 0
+    assert lib.kh_group_norm_workspace_bytes(2, 30, 64, 4, 1) == -1   # C % G != 0
+    assert lib.kh_layer_norm_bf16(16, 16, None, None, 4, 4096, 1e-5, None) == -2  # D > 2048
+    assert lib.kh_lora_shrink_bf16(16, 16, 16, 16, 4, 72, 32, None) == -2        # K % 64

@@ -96,6 +96,36 @@ def test_lora_linear_bf16(case, tile):
     assert_close_rel(y, ref2, REL_BF16, "lora_linear_bf16 vs merged weight")
 
 
+@pytest.mark.parametrize("case", [c for c in LORA_SHAPES if c[3] and c[2] % 64 == 0],
+                         ids=lambda c: f"M{c[0]}N{c[1]}K{c[2]}r{'+'.join(map(str, c[3]))}")
+def test_lora_shrink_then_pre_gemm(case):
+    """Two-launch form: t = shrink(x), y = x W^T + b + t B^T; same oracle, same tolerance."""
+    from katz_amd import ops
+    from katz_amd.lora import Adapter, pack_adapters
+
+    M, N, K, ranks, scales, bias, residual = case
+    say("lora shrink + pre gemm", case)
+    x, w, b, adapters, res = _lora_case(M, N, K, ranks, scales, bias, residual)
+    d = dev()
+    ads = {f"a{i}": Adapter(A, B, alpha=None, weight=s) for i, (A, B, s) in enumerate(adapters)}
+    pk = pack_adapters(ads, list(ads), K, N, BF, d)
+    xd = x.to(d, BF)
+    t = ops.lora_shrink(xd, pk.a_cat, pk.col_scale)
+    torch.cuda.synchronize()
+    t_ref = torch.cat([s * torch.nn.functional.linear(x, A) for A, _, s in adapters], dim=1)
+    assert_close_rel(t[:, : t_ref.shape[1]], t_ref, REL_BF16, "lora_shrink")
+    y = ops.lora_linear_pre(xd, w.to(d, BF), None if b is None else b.to(d, BF), t, pk.b_cat,
+                            None if res is None else res.to(d, BF))
+    torch.cuda.synchronize()
+    assert_close_rel(y, O.lora_linear(x, w, b, adapters, res), REL_BF16, "lora_linear_pre")
+    # a column slice of a wider shrink result (layers sharing one input)
+    wide = torch.zeros(M, pk.R + 64, dtype=BF, device=d)
+    wide[:, 32:32 + pk.R] = t
+    y2 = ops.lora_linear_pre(xd, w.to(d, BF), None if b is None else b.to(d, BF), wide[:, 32:32 + pk.R], pk.b_cat,
+                             None if res is None else res.to(d, BF))
+    assert torch.equal(y, y2)
+
+
 def test_lora_linear_bf16_scale_zero_is_base():
     say("lora_linear_bf16 scale 0")
     x, w, b, adapters, _ = _lora_case(512, 640, 640, (64,), (0.0,), True, False, seed=3)
