@@ -200,13 +200,14 @@ def main():
         e = by_kernel.setdefault(name, [0, 0.0])
         e[0] += 1
         e[1] += dur
-    gemm_calls = [c for c in log if c[0] == "lora_linear"]
+    gemm_calls = [c for c in log if c[0] in ("lora_linear", "lora_linear_grouped")]
     gemm_ms = [d for n, d in launches if n == "lora_gemm"]
     assert len(gemm_calls) == len(gemm_ms), (len(gemm_calls), len(gemm_ms))
     # two-launch layers: the shrink launch belongs to the layer whose GEMM follows it
     shrink_calls = [c for c in log if c[0] == "lora_shrink"]
     shrink_ms = sum(d for n, d in launches if n == "lora_shrink")
-    gemm_flops = sum(lora_linear_flops(c[1], c[2], c[3], c[4]) for c in gemm_calls)
+    n_layers = lambda c: c[5] if c[0] == "lora_linear_grouped" else 1
+    gemm_flops = sum(n_layers(c) * lora_linear_flops(c[1], c[2], c[3], c[4]) for c in gemm_calls)
     gemm_total_ms = sum(gemm_ms) + shrink_ms
     attn_flops = sum(4.0 * c[1] * c[2] * c[3] * c[4] * c[5] for c in log if c[0] == "attention")
     step_flops = gemm_flops + attn_flops + conv_flops
@@ -214,13 +215,13 @@ def main():
     # the largest fused-LoRA GEMM shape class, for the headline "fused LoRA-GEMM TFLOP/s"
     by_shape = {}
     for c, d in zip(gemm_calls, gemm_ms):
-        e = by_shape.setdefault(c[1:5], [0, 0.0])
+        e = by_shape.setdefault(tuple(c[1:5]) + (n_layers(c),), [0, 0.0])
         e[0] += 1
         e[1] += d
     shape_rows = []
-    for (M, N, K, R), (cnt, tot) in sorted(by_shape.items(), key=lambda kv: -kv[1][1]):
-        fl = lora_linear_flops(M, N, K, R)
-        shape_rows.append({"M": M, "N": N, "K": K, "R": R, "launches": cnt, "avg_us": round(tot / cnt * 1e3, 2),
+    for (M, N, K, R, G), (cnt, tot) in sorted(by_shape.items(), key=lambda kv: -kv[1][1]):
+        fl = G * lora_linear_flops(M, N, K, R)
+        shape_rows.append({"M": M, "N": N, "K": K, "R": R, "layers_per_launch": G, "launches": cnt, "avg_us": round(tot / cnt * 1e3, 2),
                            "tflops": round(fl / (tot / cnt * 1e-3) / 1e12, 1)})
 
     result = {

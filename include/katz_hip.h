@@ -67,7 +67,7 @@ int kh_lora_linear_bf16(const void* x, const void* w, const void* bias, const vo
                         int64_t R, int flags, void* stream);
 /* The same layer in two launches, for inputs whose rank-R product is better computed once than once per
  * output tile (and for several layers sharing one input, e.g. to_q/to_k/to_v: stack their A matrices):
- *   kh_lora_shrink_bf16:      t[M,R] = bf16((x[M,K] A_cat[R,K]^T) * col_scale[R])      K % 64 == 0, R % 32 == 0, R <= 1024
+ *   kh_lora_shrink_bf16:      t[M,R] = bf16((x[M,K] A_cat[R,K]^T) * col_scale[R])      K % 64 == 0, R % 32 == 0
  *   kh_lora_linear_pre_bf16:  y = x W^T + bias + t[:, 0:R] B_cat[N,R]^T (+ residual | GEGLU)
  * t is [M, ldt] with ldt >= R (a column slice of a wider shrink result is addressed by offsetting the
  * pointer); it is ~1 MB and stays in L2 between the two launches.  Same reference formula as above
@@ -77,6 +77,15 @@ int kh_lora_shrink_bf16(const void* x, const void* a_cat, const float* col_scale
 int kh_lora_linear_pre_bf16(const void* x, const void* w, const void* bias, const void* t, int64_t ldt,
                             const void* b_cat, const void* residual, void* y, int64_t M, int64_t N, int64_t K,
                             int64_t R, int flags, void* stream);
+/* n_groups layers that read the SAME x in one launch (the context K/V projections of every cross-attention
+ * of the UNet: 140 GEMMs of 154 rows each, which individually cannot fill the chip):
+ *   y_g = x W_g^T + bias_g + t_g B_cat_g^T        g = 0 .. n_groups-1, all with the same M, N, K, R
+ * table: DEVICE array of n_groups rows of five 64-bit device addresses {W_g, bias_g or 0, B_cat_g or 0,
+ * t_g or 0, y_g}; t_g addresses a [M, ldt] matrix (typically a column slice of one wide shrink result).
+ * R == 0: plain linears.  No counterpart in the reference (it issues the layers one by one,
+ * attention_processor.py:1260-1262).  K % 32 == 0, R <= 128, no GEGLU / residual. */
+int kh_lora_linear_grouped_bf16(const void* x, const uint64_t* table, int64_t n_groups, int64_t ldt, int64_t M,
+                                int64_t N, int64_t K, int64_t R, int flags, void* stream);
 /* fp32 variant of the same formula (fp32 parity path); R <= 128, any M/N/K. */
 int kh_lora_linear_f32(const float* x, const float* w, const float* bias, const float* a_cat, const float* b_cat,
                        const float* col_scale, const float* residual, float* y, int64_t M, int64_t N, int64_t K,

@@ -11,6 +11,8 @@ struct LoraGemmParams {
   const float* col_scale;  // [R]
   const bf16_t* t_ext;     // [M, ldt] precomputed, already scaled shrink result (null: compute it in the kernel)
   int ldt;
+  // grouped launch: blockIdx.y selects a row {w, bias, b_cat, t_ext, y} of this device table (null: single layer)
+  const uint64_t* grp;
   const bf16_t* res;       // [M,N] residual added in the epilogue, may be null
   bf16_t* y;
   int M, N, K, R;
@@ -20,3 +22,5 @@ struct LoraGemmParams {
 
 // Software-pipelined kernel (lora_gemm_pipe.hip); needs K % 32 == 0.  tile_sel: 0 automatic, >= 16 forces a tile.
 int lora_gemm_pipe_launch(const LoraGemmParams& p, int tile_sel, hipStream_t stream);
+// Grouped form: grid.y = n_groups, per-group pointers from p.grp; rank columns (p.R > 0) as extra K tiles.
+int lora_gemm_pipe_launch_grouped(const LoraGemmParams& p, int n_groups, hipStream_t stream);

@@ -479,7 +479,7 @@ KH_EXPORT int kh_lora_linear_bf16(const void* x, const void* w, const void* bias
   p.x = (const bf16_t*)x; p.w = (const bf16_t*)w; p.bias = (const bf16_t*)bias;
   p.a_cat = (const bf16_t*)a_cat; p.b_cat = (const bf16_t*)b_cat; p.col_scale = col_scale;
   p.res = (const bf16_t*)residual; p.y = (bf16_t*)y;
-  p.t_ext = nullptr; p.ldt = 0;
+  p.t_ext = nullptr; p.ldt = 0; p.grp = nullptr;
   p.M = (int)M; p.N = (int)N; p.K = (int)K; p.R = (int)R;
   p.m_tiles = p.n_tiles = p.n_chunk = p.n_chunks = 0;
   p.geglu = geglu ? 1 : 0;
@@ -508,12 +508,31 @@ KH_EXPORT int kh_lora_linear_pre_bf16(const void* x, const void* w, const void* 
   LoraGemmParams p;
   p.x = (const bf16_t*)x; p.w = (const bf16_t*)w; p.bias = (const bf16_t*)bias;
   p.a_cat = nullptr; p.b_cat = (const bf16_t*)b_cat; p.col_scale = nullptr;
-  p.t_ext = (const bf16_t*)t; p.ldt = (int)ldt;
+  p.t_ext = (const bf16_t*)t; p.ldt = (int)ldt; p.grp = nullptr;
   p.res = (const bf16_t*)residual; p.y = (bf16_t*)y;
   p.M = (int)M; p.N = (int)N; p.K = (int)K; p.R = (int)R;
   p.m_tiles = p.n_tiles = p.n_chunk = p.n_chunks = 0;
   p.geglu = geglu ? 1 : 0;
   return lora_gemm_pipe_launch(p, (flags >> 8) & 0xff, (hipStream_t)stream);
+}
+
+// Many layers that share one input in one launch; see include/katz_hip.h.
+KH_EXPORT int kh_lora_linear_grouped_bf16(const void* x, const uint64_t* table, int64_t n_groups, int64_t ldt,
+                                          int64_t M, int64_t N, int64_t K, int64_t R, int flags, void* stream) {
+  if (!x || !table || n_groups <= 0 || M <= 0 || N <= 0 || K <= 0 || R < 0) return KH_ERR_INVALID_ARG;
+  if (K % 32 != 0 || N % 8 != 0 || R % 32 != 0 || ldt % 8 != 0 || (R > 0 && ldt < R)) return KH_ERR_UNSUPPORTED;
+  if (R > 128 || n_groups > 65535) return KH_ERR_TOO_LARGE;
+  if (M > (1 << 24) || N > (1 << 24) || K > (1 << 24)) return KH_ERR_TOO_LARGE;
+  if ((flags & 1) != 0) return KH_ERR_UNSUPPORTED;  // no GEGLU epilogue in grouped launches
+  if (!kh_aligned16(x) || !kh_aligned16(table)) return KH_ERR_ALIGNMENT;
+  LoraGemmParams p;
+  p.x = (const bf16_t*)x; p.w = nullptr; p.bias = nullptr; p.a_cat = nullptr; p.b_cat = nullptr; p.col_scale = nullptr;
+  p.t_ext = nullptr; p.ldt = (int)ldt; p.grp = table;
+  p.res = nullptr; p.y = nullptr;
+  p.M = (int)M; p.N = (int)N; p.K = (int)K; p.R = (int)R;
+  p.m_tiles = p.n_tiles = p.n_chunk = p.n_chunks = 0;
+  p.geglu = 0;
+  return lora_gemm_pipe_launch_grouped(p, (int)n_groups, (hipStream_t)stream);
 }
 
 KH_EXPORT int kh_lora_linear_f32(const float* x, const float* w, const float* bias, const float* a_cat,

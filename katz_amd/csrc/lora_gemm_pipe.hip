@@ -220,8 +220,17 @@ __device__ __forceinline__ void k_loop(char* smem, const Dma<C, SHRINK>& dma, co
 }
 
 template <class C>
-__global__ __launch_bounds__(C::NT, C::NRT == 0 ? 2 : 1) void lora_gemm_pipe_kernel(const LoraGemmParams p) {
+__global__ __launch_bounds__(C::NT, C::NRT == 0 ? 2 : 1) void lora_gemm_pipe_kernel(const LoraGemmParams pin) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
+  LoraGemmParams p = pin;
+  if (pin.grp != nullptr) {  // grouped launch: this workgroup's layer
+    const uint64_t* g = pin.grp + (size_t)blockIdx.y * 5;
+    p.w = reinterpret_cast<const bf16_t*>(g[0]);
+    p.bias = reinterpret_cast<const bf16_t*>(g[1]);
+    p.b_cat = reinterpret_cast<const bf16_t*>(g[2]);
+    p.t_ext = reinterpret_cast<const bf16_t*>(g[3]);
+    p.y = reinterpret_cast<bf16_t*>(g[4]);
+  }
   constexpr int BM = C::BM, BN = C::BN, TM = C::TM, TN = C::TN, NRT = C::NRT, R = C::R, NST = C::NST;
   constexpr int SMT = C::SM > 0 ? C::SM : 1, NRTT = NRT > 0 ? NRT : 1;
   bf16_t* sB = reinterpret_cast<bf16_t*>(smem);                // aliases the ring (after the K loop)
@@ -448,7 +457,7 @@ __global__ __launch_bounds__(C::NT, C::NRT == 0 ? 2 : 1) void lora_gemm_pipe_ker
 }
 
 template <class C>
-int launch_pcfg(LoraGemmParams p, hipStream_t stream) {
+int launch_pcfg(LoraGemmParams p, hipStream_t stream, int n_groups = 1) {
   p.m_tiles = (p.M + C::BM - 1) / C::BM;
   p.n_tiles = (p.N + C::BN - 1) / C::BN;
   int nc = 1;
@@ -466,7 +475,7 @@ int launch_pcfg(LoraGemmParams p, hipStream_t stream) {
     attr_done = true;
   }
   const unsigned grid = (unsigned)(p.m_tiles * p.n_chunks);
-  kh_launch(KH_TAG_LORA_GEMM, lora_gemm_pipe_kernel<C>, dim3(grid), dim3(C::NT), C::LDS_BYTES, stream, p);
+  kh_launch(KH_TAG_LORA_GEMM, lora_gemm_pipe_kernel<C>, dim3(grid, (unsigned)n_groups), dim3(C::NT), C::LDS_BYTES, stream, p);
   KH_RETURN_LAST_ERROR();
 }
 
@@ -485,6 +494,10 @@ int launch_prank(const LoraGemmParams& p, hipStream_t stream) {
 }
 
 }  // namespace
+
+int lora_gemm_pipe_launch_grouped(const LoraGemmParams& p, int n_groups, hipStream_t stream) {
+  return launch_pcfg<PCfg<128, 128, 2, 2, 0, 4>>(p, stream, n_groups);
+}
 
 int lora_gemm_pipe_launch(const LoraGemmParams& p, int tile_sel, hipStream_t stream) {
   switch (tile_sel) {

@@ -10,6 +10,9 @@
 // Bound: HBM/L2 (x is streamed from L2; 2*M*K*R FLOPs are ~1 GFLOP).  Grid (M/32, R/32): a workgroup owns
 // 32 rows x 32 rank columns; its 4 waves split K four ways (direct global -> register fragments,
 // 64 contiguous bytes per row per step), partial sums meet in LDS in a fixed order (deterministic).
+// Tried and dropped: splitting K across workgroups with a last-arriver reduction (the device-scope
+// release is an L2 write-back on a multi-XCD part: 40 us) and 8-wave workgroups over 96 rank columns
+// (too few workgroups: 18 us).
 #include "kh_common.h"
 
 namespace {
@@ -88,7 +91,7 @@ KH_EXPORT int kh_lora_shrink_bf16(const void* x, const void* a_cat, const float*
                                   int64_t K, int64_t R, void* stream) {
   if (!x || !a_cat || !col_scale || !t || M <= 0 || K <= 0 || R <= 0) return KH_ERR_INVALID_ARG;
   if (K % 64 != 0 || R % 32 != 0) return KH_ERR_UNSUPPORTED;
-  if (R > 1024 || M > (1 << 24)) return KH_ERR_TOO_LARGE;
+  if (R > 65535 * SR_COLS || M > (1 << 24)) return KH_ERR_TOO_LARGE;
   if (!kh_aligned16(x) || !kh_aligned16(a_cat) || !kh_aligned16(t)) return KH_ERR_ALIGNMENT;
   ShrinkParams p;
   p.x = (const bf16_t*)x; p.a_cat = (const bf16_t*)a_cat; p.col_scale = col_scale; p.t = (bf16_t*)t;

@@ -32,6 +32,10 @@ SKIP_INIT = False
 #   "split": kh_lora_shrink_bf16 once per layer input, then the base GEMM + expand reading it from L2.
 LORA_MODE = os.getenv("KATZ_LORA_MODE", "split")
 
+# bumped whenever any layer rebuilds its packed adapter buffers (not on pure scale changes): consumers
+# that cache pointers into those buffers (grouped launches) rebuild when it moves
+_pack_epoch = 0
+
 
 class LoRALinear(nn.Module):
     """nn.Linear whose forward is the fused base-GEMM + low-rank-delta kernel.
@@ -98,9 +102,12 @@ class LoRALinear(nn.Module):
     def refresh_adapters(self) -> None:
         """(Re)build the packed buffers; a pure scale change only rewrites col_scale in place, so a
         captured HIP graph that reads the buffers stays valid."""
+        global _pack_epoch
         names = [n for n in self.active if n not in self._fused] if self.adapters_enabled else []
         key = tuple((n, id(self.adapters[n].down)) for n in names)
         if not names:
+            if self._packed is not None:
+                _pack_epoch += 1
             self._packed, self._packed_key = None, key
             return
         if key == self._packed_key and self._packed is not None:
@@ -109,6 +116,7 @@ class LoRALinear(nn.Module):
         self._packed = pack_adapters(self.adapters, names, self.in_features, self.out_features, self.weight.dtype,
                                      self.weight.device, self.global_scale, geglu_interleave=self.geglu)
         self._packed_key = key
+        _pack_epoch += 1
 
     def fuse(self, lora_scale: float = 1.0, names: Optional[Sequence[str]] = None) -> None:
         """W += sum_i (lora_scale * m_i) B_i A_i in fp32, cast back -- _fuse_lora,
@@ -285,8 +293,11 @@ class KatzAttnProcessor:
             raise NotImplementedError("attention masks are not used on the SDXL path and not implemented")
         ctx = hidden_states if encoder_hidden_states is None else encoder_hidden_states
         q = attn.to_q(hidden_states)
-        k = attn.to_k(ctx)
-        v = attn.to_v(ctx)
+        if encoder_hidden_states is not None and attn.ctx_kv is not None and attn.ctx_kv[0] is encoder_hidden_states:
+            _, k, v = attn.ctx_kv  # projected for every cross-attention at once at the start of the step
+        else:
+            k = attn.to_k(ctx)
+            v = attn.to_v(ctx)
         o = ops.attention(q, k, v, attn.heads, attn.scale)
         o = attn.to_out[0](o, residual=residual)
         return attn.to_out[1](o)
@@ -306,6 +317,8 @@ class Attention(nn.Module):
         self.to_v = LoRALinear(kv_dim, inner, bias=bias)
         self.to_out = nn.ModuleList([LoRALinear(inner, query_dim, bias=out_bias), nn.Dropout(0.0)])
         self.processor = processor or KatzAttnProcessor()
+        self.is_cross = cross_attention_dim is not None
+        self.ctx_kv = None  # (context tensor, k, v) filled by ContextKVProjector for the current step
 
     def set_processor(self, processor) -> None:
         self.processor = processor
@@ -390,3 +403,81 @@ class Transformer2DModel(nn.Module):
             h = blk(h, encoder_hidden_states)
         h = self.proj_out(h, residual=residual)
         return h.view(N, H, W, C).permute(0, 3, 1, 2)
+
+
+class ContextKVProjector:
+    """to_k / to_v of EVERY cross-attention of the model in one grouped launch per width.
+
+    The text context is the same tensor for all 70 cross-attentions of a step, and each of their
+    K/V projections is a 154-row GEMM that cannot fill 256 CUs on its own (the reference issues
+    them one by one, attention_processor.py:1260-1262).  Here the 2 x 70 projections run as one launch
+    per output width (grid.y = layer), and with adapters active one shrink launch computes
+    context . A^T for all of them (their A matrices stacked).  The step's arithmetic is unchanged --
+    nothing is cached across steps.
+    """
+
+    def __init__(self, attentions: Sequence["Attention"]):
+        self.groups: Dict[int, List[Attention]] = {}
+        for a in attentions:
+            if a.is_cross:
+                self.groups.setdefault(a.to_k.out_features, []).append(a)
+        self._built = {}  # width -> dict(state)
+
+    def _layers(self, width):
+        out = []
+        for a in self.groups[width]:
+            out += [a.to_k, a.to_v]
+        return out
+
+    def _build(self, width: int, M: int, ctx: torch.Tensor):
+        layers = self._layers(width)
+        for l in layers:
+            l.prepare()
+        K = layers[0].in_features
+        packs = [l._packed for l in layers]
+        uniform = all(p is None for p in packs) or (all(p is not None for p in packs) and len({p.R for p in packs}) == 1)
+        ok = uniform and LORA_MODE == "split" and all(l.weight.dtype == torch.bfloat16 and not l.geglu for l in layers)
+        st = dict(epoch=_pack_epoch, M=M, ok=ok, wptr=[l.weight.data_ptr() for l in layers])
+        if ok:
+            dev = ctx.device
+            G = len(layers)
+            R = 0 if packs[0] is None else packs[0].R
+            y = torch.empty((G, M, width), dtype=torch.bfloat16, device=dev)
+            t = a_all = s_all = None
+            if R > 0:
+                a_all = torch.cat([p.a_cat for p in packs], dim=0).contiguous()
+                s_all = torch.cat([p.col_scale for p in packs], dim=0).contiguous()
+                for g, p in enumerate(packs):  # the layers now read (and rescale) the stacked storage
+                    p.a_cat = a_all[g * R:(g + 1) * R]
+                    p.col_scale = s_all[g * R:(g + 1) * R]
+                t = torch.empty((M, G * R), dtype=torch.bfloat16, device=dev)
+            rows = []
+            for g, l in enumerate(layers):
+                _, w, b = l._rt
+                rows.append([w.data_ptr(), 0 if b is None else b.data_ptr(), 0 if R == 0 else packs[g].b_cat.data_ptr(),
+                             0 if R == 0 else t.data_ptr() + g * R * 2, y[g].data_ptr()])
+            st.update(G=G, R=R, K=K, y=y, t=t, a_all=a_all, s_all=s_all,
+                      table=torch.tensor(rows, dtype=torch.int64, device=dev))
+        self._built[width] = st
+        return st
+
+    def run(self, ctx: torch.Tensor) -> None:
+        """Project `ctx` [B,S,K] for every cross-attention; results are handed to the Attention modules."""
+        B, S, K = ctx.shape
+        M = B * S
+        for width, attns in self.groups.items():
+            st = self._built.get(width)
+            layers = self._layers(width)
+            if (st is None or st["epoch"] != _pack_epoch or st["M"] != M
+                    or st["wptr"] != [l.weight.data_ptr() for l in layers]):
+                st = self._build(width, M, ctx)
+            if not st["ok"]:
+                for a in attns:
+                    a.ctx_kv = None
+                continue
+            x2 = ctx.reshape(M, K)
+            if st["R"] > 0:
+                ops.lora_shrink(x2, st["a_all"], st["s_all"], out=st["t"])
+            ops.lora_linear_grouped(x2, st["table"], M, width, K, st["R"], st["G"] * st["R"] if st["R"] else 8)
+            for i, a in enumerate(attns):
+                a.ctx_kv = (ctx, st["y"][2 * i].view(B, S, width), st["y"][2 * i + 1].view(B, S, width))

@@ -152,6 +152,21 @@ def lora_linear_pre(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.
     return out
 
 
+def lora_linear_grouped(x: torch.Tensor, table: torch.Tensor, M: int, N: int, K: int, R: int, ldt: int) -> None:
+    """y_g = x W_g^T + b_g + t_g B_cat_g^T for every row {W, bias, B_cat, t, y} of the int64 device
+    `table` [n_groups, 5] in one launch; the caller owns every buffer the table points to."""
+    lib = _lib.load()
+    _req(x, BF16, "x"); _req(table, torch.int64, "table")
+    if table.dim() != 2 or table.shape[1] != 5:
+        raise ValueError("table must be [n_groups, 5] int64")
+    if x.numel() != M * K:
+        raise ValueError("x does not match M x K")
+    if CALL_LOG is not None:
+        CALL_LOG.append(("lora_linear_grouped", M, N, K, R, int(table.shape[0])))
+    rc = lib.kh_lora_linear_grouped_bf16(_ptr(x), _ptr(table), table.shape[0], ldt, M, N, K, R, 0, _stream())
+    _lib.check(rc, "kh_lora_linear_grouped_bf16")
+
+
 # --------------------------------------------------------------------------------------- K2
 def sgmv_shrink(x, a_all, seg_start, seg_adapter, adapter_rank, max_seg_rows: int, out=None):
     """t[rows, :r_a] = x[rows] A_a^T per segment. a_all [n_adapters, RP, K]; returns t [rows, RP]."""

@@ -160,6 +160,7 @@ class UNet2DConditionModel(nn.Module):
         self.conv_norm_silu = nn.Sequential(*fused_norm_silu(boc[0], cfg.norm_num_groups, cfg.norm_eps))
         self.conv_out = nn.Conv2d(boc[0], cfg.out_channels, 3, padding=1)
         self.num_upsamplers = n - 1
+        self._ctx_kv = None
         self._register_load_state_dict_pre_hook(self._remap_upstream_keys)
 
     # ---- checkpoints ---------------------------------------------------------------------------
@@ -192,6 +193,9 @@ class UNet2DConditionModel(nn.Module):
     def prepare(self) -> None:
         for m in self.lora_linears().values():
             m.prepare()
+        if self._ctx_kv is None:
+            from .layers import Attention, ContextKVProjector
+            self._ctx_kv = ContextKVProjector([m for m in self.modules() if isinstance(m, Attention)])
 
     # ---- LoRA surface ----------------------------------------------------------------------------
     def lora_linears(self) -> Dict[str, LoRALinear]:
@@ -358,6 +362,9 @@ class UNet2DConditionModel(nn.Module):
             sample = sample.to(torch.bfloat16).contiguous(memory_format=torch.channels_last)
         ctx = encoder_hidden_states.to(torch.bfloat16).contiguous()
 
+        if self._ctx_kv is None:
+            self.prepare()
+        self._ctx_kv.run(ctx)  # K/V projections of all cross-attentions, grouped
         emb = self._embed(sample, timestep, added_cond_kwargs)
         temb_act = F.silu(emb)
         sample = self.conv_in(sample)

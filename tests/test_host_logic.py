@@ -1,0 +1,114 @@
+"""Host-side logic that needs no GPU: imports, LoRA key parsing, adapter packing, state-dict hooks."""
+import torch
+
+from helpers import katz_lora_state_dict
+
+
+def test_package_imports_without_gpu():
+    import katz_amd.graph  # noqa: F401
+    import katz_amd.layers  # noqa: F401
+    import katz_amd.lora  # noqa: F401
+    import katz_amd.ops  # noqa: F401
+    import katz_amd.unet_2d_condition  # noqa: F401
+    import katz_amd.unet_blocks  # noqa: F401
+
+
+def test_ops_fail_loudly_without_gpu():
+    """No CPU fallback: a CPU tensor is rejected with an explicit error."""
+    import pytest
+    from katz_amd import _lib, ops
+
+    if not _lib.LIB_PATH.exists():
+        pytest.skip("libkatz_hip.so not built")
+    x = torch.zeros(4, 8, dtype=torch.bfloat16)
+    with pytest.raises(_lib.KatzHipError):
+        ops.lora_linear(x, torch.zeros(8, 8, dtype=torch.bfloat16))
+    with pytest.raises(_lib.KatzHipError):
+        ops.group_norm(torch.zeros(1, 8, 2, 2, dtype=torch.bfloat16), 2, None, None, 1e-5)
+
+
+def test_parse_lora_key_spellings():
+    from katz_amd.unet_2d_condition import parse_lora_key
+
+    base = "down_blocks.1.attentions.0.transformer_blocks.0"
+    assert parse_lora_key(f"unet.{base}.attn1.processor.to_q_lora.down.weight") == (f"{base}.attn1.to_q", "down")
+    assert parse_lora_key(f"unet.{base}.attn2.processor.to_out_lora.up.weight") == (f"{base}.attn2.to_out.0", "up")
+    assert parse_lora_key(f"unet.{base}.ff.net.0.proj.lora.down.weight") == (f"{base}.ff.net.0.proj", "down")
+    assert parse_lora_key(f"{base}.ff.net.2.lora_A.weight") == (f"{base}.ff.net.2", "down")
+    assert parse_lora_key(f"{base}.attn1.to_v.lora_B.default_0.weight") == (f"{base}.attn1.to_v", "up")
+    assert parse_lora_key("text_encoder.something.weight") is None
+
+
+def test_every_reference_lora_key_resolves_to_a_module():
+    """All 1444 down/up keys of the reference's adapter metadata parse to one of the 722 LoRA linears."""
+    import json
+    from pathlib import Path
+
+    import katz_amd.layers as L
+    from katz_amd.unet_2d_condition import UNet2DConditionModel, UNetConfig, parse_lora_key
+
+    keys = json.loads((Path(__file__).parent / "golden" / "sdxl_lora_keys.json").read_text())
+    L.SKIP_INIT = True
+    try:
+        with torch.device("meta"):
+            unet = UNet2DConditionModel(UNetConfig.sdxl())
+    finally:
+        L.SKIP_INIT = False
+    lin = unet.lora_linears()
+    assert len(lin) == 722
+    for unet_key, meta in keys.items():
+        mod = unet_key[: -len(".weight")]
+        assert parse_lora_key(meta["down_key"]) == (mod, "down")
+        assert parse_lora_key(meta["up_key"]) == (mod, "up")
+        assert (lin[mod].in_features, lin[mod].out_features) == (meta["down"][1], meta["up"][0])
+
+
+def test_pack_adapters_layout_and_rescale():
+    from katz_amd.lora import Adapter, interleave_geglu_rows, pack_adapters, rescale_
+
+    g = torch.Generator().manual_seed(0)
+    ads = {"a": Adapter(torch.randn(8, 16, generator=g), torch.randn(64, 8, generator=g), alpha=16.0, weight=0.5),
+           "b": Adapter(torch.randn(4, 16, generator=g), torch.randn(64, 4, generator=g), alpha=None, weight=2.0)}
+    pk = pack_adapters(ads, ["b", "a"], 16, 64, torch.float32, "cpu", global_scale=0.5)
+    assert pk.R == 32 and pk.a_cat.shape == (32, 16) and pk.b_cat.shape == (64, 32)
+    assert torch.equal(pk.a_cat[:4], ads["b"].down) and torch.equal(pk.a_cat[4:12], ads["a"].down)
+    assert torch.all(pk.a_cat[12:] == 0) and torch.all(pk.b_cat[:, 12:] == 0)
+    assert torch.allclose(pk.col_scale[:4], torch.tensor(2.0 * 1.0 * 0.5))          # alpha = rank
+    assert torch.allclose(pk.col_scale[4:12], torch.tensor(0.5 * 16.0 / 8 * 0.5))   # weight * alpha / rank * scale
+    # the packed product equals the sum over adapters
+    x = torch.randn(5, 16, generator=g)
+    got = ((x @ pk.a_cat.T) * pk.col_scale) @ pk.b_cat.T
+    ref = sum(ad.multiplier(0.5) * (x @ ad.down.T) @ ad.up.T for ad in ads.values())
+    assert torch.allclose(got, ref, atol=1e-5)
+    ads["a"].weight = 0.0
+    rescale_(pk, ads, 1.0)
+    assert torch.all(pk.col_scale[4:12] == 0) and torch.allclose(pk.col_scale[:4], torch.tensor(2.0))
+    # GEGLU interleave: blocks of 32 value rows then their 32 gate rows
+    t = torch.arange(128).float()[:, None].repeat(1, 2)
+    it = interleave_geglu_rows(t)
+    assert it[:32, 0].tolist() == list(range(32)) and it[32:64, 0].tolist() == list(range(64, 96))
+    assert it[64:96, 0].tolist() == list(range(32, 64)) and it[96:, 0].tolist() == list(range(96, 128))
+
+
+def test_upstream_state_dict_names_are_remapped():
+    import katz_amd.layers as L
+    from katz_amd.unet_2d_condition import UNet2DConditionModel, UNetConfig
+
+    L.SKIP_INIT = True
+    try:
+        unet = UNet2DConditionModel(UNetConfig.tiny())
+    finally:
+        L.SKIP_INIT = False
+    sd = {k: torch.randn_like(v) for k, v in unet.state_dict().items()}
+    up = {}
+    for k, v in sd.items():
+        k2 = k.replace("conv_norm_silu.0.", "conv_norm_out.").replace(".norm_silu1.0.", ".norm1.").replace(".norm_silu2.0.", ".norm2.")
+        if ".ff.net.0.proj." in k2:  # the fork's fused-GEGLU split
+            h = v.shape[0] // 2
+            up[k2.replace(".proj.", ".proj_1.")] = v[:h].clone()
+            up[k2.replace(".proj.", ".proj_2.")] = v[h:].clone()
+        else:
+            up[k2] = v
+    unet.load_state_dict(up, strict=True)
+    for k, v in unet.state_dict().items():
+        assert torch.equal(v, sd[k]), k
