@@ -71,12 +71,15 @@ int kh_lora_linear_bf16(const void* x, const void* w, const void* bias, const vo
  *   kh_lora_linear_pre_bf16:  y = x W^T + bias + t[:, 0:R] B_cat[N,R]^T (+ residual | GEGLU)
  * t is [M, ldt] with ldt >= R (a column slice of a wider shrink result is addressed by offsetting the
  * pointer); it is ~1 MB and stays in L2 between the two launches.  Same reference formula as above
- * (lora.py:222-232: up(down(x)) * scale).  K % 32 == 0, R <= 128, flags as for kh_lora_linear_bf16. */
+ * (lora.py:222-232: up(down(x)) * scale).  K % 32 == 0, R <= 128, flags as for kh_lora_linear_bf16.
+ * n_split > 0 fuses several layers with one input into one GEMM (to_q/to_k/to_v): W, bias, B_cat are the
+ * layers stacked along N in blocks of n_split rows (n_split % 128 == 0) and block j takes T columns
+ * [j*R, (j+1)*R) of the shared shrink result; 0 = a single layer. */
 int kh_lora_shrink_bf16(const void* x, const void* a_cat, const float* col_scale, void* t, int64_t M, int64_t K,
                         int64_t R, void* stream);
 int kh_lora_linear_pre_bf16(const void* x, const void* w, const void* bias, const void* t, int64_t ldt,
-                            const void* b_cat, const void* residual, void* y, int64_t M, int64_t N, int64_t K,
-                            int64_t R, int flags, void* stream);
+                            int64_t n_split, const void* b_cat, const void* residual, void* y, int64_t M, int64_t N,
+                            int64_t K, int64_t R, int flags, void* stream);
 /* n_groups layers that read the SAME x in one launch (the context K/V projections of every cross-attention
  * of the UNet: 140 GEMMs of 154 rows each, which individually cannot fill the chip):
  *   y_g = x W_g^T + bias_g + t_g B_cat_g^T        g = 0 .. n_groups-1, all with the same M, N, K, R

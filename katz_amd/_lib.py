@@ -22,7 +22,7 @@ SIGNATURES = {
     "kh_profile_end": (c_int, [_P, _P, c_int]),
     "kh_lora_linear_bf16": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, c_int, _P]),
     "kh_lora_shrink_bf16": (c_int, [_P, _P, _P, _P, _I, _I, _I, _P]),
-    "kh_lora_linear_pre_bf16": (c_int, [_P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, c_int, _P]),
+    "kh_lora_linear_pre_bf16": (c_int, [_P, _P, _P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, c_int, _P]),
     "kh_lora_linear_grouped_bf16": (c_int, [_P, _P, _I, _I, _I, _I, _I, _I, c_int, _P]),
     "kh_lora_linear_f32": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
     "kh_sgmv_shrink_bf16": (c_int, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),

@@ -11,8 +11,10 @@ struct LoraGemmParams {
   const float* col_scale;  // [R]
   const bf16_t* t_ext;     // [M, ldt] precomputed, already scaled shrink result (null: compute it in the kernel)
   int ldt;
+  int t_nsplit;            // > 0: W rows come in blocks of t_nsplit rows; block j uses T columns [j*R, (j+1)*R)
   // grouped launch: blockIdx.y selects a row {w, bias, b_cat, t_ext, y} of this device table (null: single layer)
   const uint64_t* grp;
+  int dbg;  // tuning experiments only (flags bits 16..23); 0 in production
   const bf16_t* res;       // [M,N] residual added in the epilogue, may be null
   bf16_t* y;
   int M, N, K, R;

@@ -479,10 +479,11 @@ KH_EXPORT int kh_lora_linear_bf16(const void* x, const void* w, const void* bias
   p.x = (const bf16_t*)x; p.w = (const bf16_t*)w; p.bias = (const bf16_t*)bias;
   p.a_cat = (const bf16_t*)a_cat; p.b_cat = (const bf16_t*)b_cat; p.col_scale = col_scale;
   p.res = (const bf16_t*)residual; p.y = (bf16_t*)y;
-  p.t_ext = nullptr; p.ldt = 0; p.grp = nullptr;
+  p.t_ext = nullptr; p.ldt = 0; p.grp = nullptr; p.dbg = 0; p.t_nsplit = 0;
   p.M = (int)M; p.N = (int)N; p.K = (int)K; p.R = (int)R;
   p.m_tiles = p.n_tiles = p.n_chunk = p.n_chunks = 0;
   p.geglu = geglu ? 1 : 0;
+  p.dbg = (flags >> 16) & 0xff;
   hipStream_t s = (hipStream_t)stream;
   const int tile_sel = (flags >> 8) & 0xff;  // 0 = automatic
   // K % 32 == 0 (every SDXL layer): the software-pipelined kernel; tile_sel 1/2 force the simple kernel
@@ -494,9 +495,11 @@ KH_EXPORT int kh_lora_linear_bf16(const void* x, const void* w, const void* bias
 
 // Base GEMM + expand with a precomputed shrink result t (kh_lora_shrink_bf16); see include/katz_hip.h.
 KH_EXPORT int kh_lora_linear_pre_bf16(const void* x, const void* w, const void* bias, const void* t, int64_t ldt,
-                                      const void* b_cat, const void* residual, void* y, int64_t M, int64_t N,
-                                      int64_t K, int64_t R, int flags, void* stream) {
+                                      int64_t n_split, const void* b_cat, const void* residual, void* y, int64_t M,
+                                      int64_t N, int64_t K, int64_t R, int flags, void* stream) {
   if (!x || !w || !y || !t || !b_cat || M <= 0 || N <= 0 || K <= 0 || R <= 0 || ldt < R) return KH_ERR_INVALID_ARG;
+  if (n_split < 0 || (n_split > 0 && (n_split % 128 != 0 || N % n_split != 0 || ldt < (N / n_split) * R)))
+    return KH_ERR_INVALID_ARG;
   if (K % 32 != 0 || N % 8 != 0 || R % 32 != 0 || ldt % 8 != 0) return KH_ERR_UNSUPPORTED;
   if (R > 128) return KH_ERR_TOO_LARGE;
   if (M > (1 << 24) || N > (1 << 24) || K > (1 << 24)) return KH_ERR_TOO_LARGE;
@@ -508,7 +511,7 @@ KH_EXPORT int kh_lora_linear_pre_bf16(const void* x, const void* w, const void* 
   LoraGemmParams p;
   p.x = (const bf16_t*)x; p.w = (const bf16_t*)w; p.bias = (const bf16_t*)bias;
   p.a_cat = nullptr; p.b_cat = (const bf16_t*)b_cat; p.col_scale = nullptr;
-  p.t_ext = (const bf16_t*)t; p.ldt = (int)ldt; p.grp = nullptr;
+  p.t_ext = (const bf16_t*)t; p.ldt = (int)ldt; p.grp = nullptr; p.dbg = 0; p.t_nsplit = (int)n_split;
   p.res = (const bf16_t*)residual; p.y = (bf16_t*)y;
   p.M = (int)M; p.N = (int)N; p.K = (int)K; p.R = (int)R;
   p.m_tiles = p.n_tiles = p.n_chunk = p.n_chunks = 0;
@@ -527,7 +530,7 @@ KH_EXPORT int kh_lora_linear_grouped_bf16(const void* x, const uint64_t* table, 
   if (!kh_aligned16(x) || !kh_aligned16(table)) return KH_ERR_ALIGNMENT;
   LoraGemmParams p;
   p.x = (const bf16_t*)x; p.w = nullptr; p.bias = nullptr; p.a_cat = nullptr; p.b_cat = nullptr; p.col_scale = nullptr;
-  p.t_ext = nullptr; p.ldt = (int)ldt; p.grp = table;
+  p.t_ext = nullptr; p.ldt = (int)ldt; p.grp = table; p.dbg = 0; p.t_nsplit = 0;
   p.res = nullptr; p.y = nullptr;
   p.M = (int)M; p.N = (int)N; p.K = (int)K; p.R = (int)R;
   p.m_tiles = p.n_tiles = p.n_chunk = p.n_chunks = 0;

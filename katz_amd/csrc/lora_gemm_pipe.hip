@@ -16,19 +16,25 @@
 
 namespace {
 
-constexpr int BKP = 32;    // K columns per stage
-constexpr int ROWB = 64;   // bytes per LDS row
+// K columns per stage (BKP) are a template parameter: 32 (64-byte LDS rows) or 64 (128-byte rows).
 
-template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int NRT_, int NST_>
+template <int BM_, int BN_, int WAVES_M_, int WAVES_N_, int NRT_, int NST_, int BKP_ = 32>
 struct PCfg {
   static constexpr int BM = BM_, BN = BN_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, NRT = NRT_, NST = NST_;
+  static constexpr int BKP = BKP_;              // K columns per stage
+  static constexpr int ROWB = BKP * 2;          // bytes per LDS row
+  static constexpr int PPR = BKP / 8;           // 16-byte pieces per row
+  static constexpr int UROWS = 64 / PPR;        // rows one DMA instruction (64 lanes x 16 B) covers
+  static constexpr int SWR = 256 / ROWB;        // rows per 256 bytes: piece p of row r is stored at p ^ ((r / SWR) % PPR)
+  static constexpr int KS = BKP / 16;           // MFMA k-steps per stage
+  static_assert(BKP == 32 || BKP == 64, "stage depth");
   static constexpr int NW = WAVES_M * WAVES_N, NT = NW * 64;
   static constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
   static constexpr int TM = WTM / 32, TN = WTN / 32;
   static constexpr int R = NRT * 32;
   static constexpr int SM = (NRT > 0) ? TM / WAVES_N : 0;
   static constexpr int RS = R;                                         // A_cat rows staged per K tile
-  static constexpr int UX = BM / 16, UW = BN / 16, UA = RS / 16;       // 16-row DMA units per stage
+  static constexpr int UX = BM / UROWS, UW = BN / UROWS, UA = RS / UROWS;  // DMA units per stage
   static constexpr int MU = (UX + UW + UA + NW - 1) / NW;              // most units one wave issues per stage
   static constexpr int SW_OFF = BM * ROWB, SA_OFF = (BM + BN) * ROWB;
   static constexpr int STAGE = (BM + BN + RS) * ROWB;
@@ -40,10 +46,11 @@ struct PCfg {
   static constexpr size_t ST = (NRT > 0) ? (size_t)BM * LDT * 2 : 0;
   static constexpr size_t ST_OFF = RING_MAX;
   static constexpr size_t LDS_BYTES = RING_MAX + ST;
+  static constexpr int OCC = (LDS_BYTES <= 80 * 1024 && TM * TN <= 4) ? 2 : 1;  // workgroups per CU that LDS and registers allow
   static_assert(BM % (32 * WAVES_M) == 0 && BN % (32 * WAVES_N) == 0, "tile/wave mismatch");
   static_assert(NRT == 0 || (TM % WAVES_N == 0), "shrink tiles must split evenly over the waves of a row");
   static_assert(NST >= 2 && NST <= 4, "ring depth");
-  static_assert(UX % NW == 0 && UW % NW == 0 && (RS / 8) % NW == 0, "DMA work must split evenly over the waves");
+  static_assert(UX % NW == 0 && UW % NW == 0 && (RS / 8) % NW == 0 && (NRT == 0 || BKP == 32), "DMA work must split evenly over the waves");
   static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
 };
 
@@ -61,12 +68,12 @@ __device__ __forceinline__ u32x4 ld16(const bf16_t* p) { return *reinterpret_cas
 __device__ __forceinline__ bf16x8 lds_frag(const char* p) { return *reinterpret_cast<const bf16x8*>(p); }
 __device__ __forceinline__ bf16x8 lds_fragb(const bf16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
 
-// Fragments of one K tile (32 columns = two 16-wide MFMA steps) held in registers.
+// Fragments of one K tile (BKP columns = KS 16-wide MFMA steps) held in registers.
 template <class C, bool SHRINK>
 struct Frags {
-  bf16x8 a[2][C::TM];
-  bf16x8 b[2][C::TN];
-  bf16x8 r[2][SHRINK ? C::NRT : 1];
+  bf16x8 a[C::KS][C::TM];
+  bf16x8 b[C::KS][C::TN];
+  bf16x8 r[C::KS][SHRINK ? C::NRT : 1];
 };
 
 // DMA work of one wave for one K tile: the same number of global_load_lds instructions for every
@@ -102,6 +109,7 @@ __device__ __forceinline__ void k_loop(char* smem, const Dma<C, SHRINK>& dma, co
                                        f32x16 (&tacc)[C::SM > 0 ? C::SM : 1][C::NRT > 0 ? C::NRT : 1],
                                        TailLoads tail_loads) {
   constexpr int TM = C::TM, TN = C::TN, NRT = C::NRT, NST = C::NST;
+  constexpr int BKP = C::BKP, ROWB = C::ROWB, KS = C::KS;
   constexpr int PD = NST - 1;  // prefetch distance in K tiles
   using D = Dma<C, SHRINK>;
   auto issue = [&](int t) {
@@ -120,7 +128,7 @@ __device__ __forceinline__ void k_loop(char* smem, const Dma<C, SHRINK>& dma, co
   auto read_frags = [&](int t, Frags<C, SHRINK>& f) {
     const char* st = smem + (t % NST) * C::STAGE;
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
+    for (int ks = 0; ks < KS; ++ks) {
       const int po = ((2 * ks + lh) ^ sw) * 16;
 #pragma unroll
       for (int i = 0; i < TM; ++i) f.a[ks][i] = lds_frag(st + (wm * C::WTM + i * 32 + l32) * ROWB + po);
@@ -132,7 +140,7 @@ __device__ __forceinline__ void k_loop(char* smem, const Dma<C, SHRINK>& dma, co
       }
     }
   };
-  auto mma = [&](const Frags<C, SHRINK>& f, int ks) {
+  auto mma1 = [&](const Frags<C, SHRINK>& f, int ks) {
     if constexpr (SHRINK) {
 #pragma unroll
       for (int s = 0; s < C::SM; ++s) {
@@ -149,6 +157,10 @@ __device__ __forceinline__ void k_loop(char* smem, const Dma<C, SHRINK>& dma, co
 #pragma unroll
       for (int j = 0; j < TN; ++j)
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a[ks][i], f.b[ks][j], acc[i][j], 0, 0, 0);
+  };
+  auto mma = [&](const Frags<C, SHRINK>& f, int half) {  // half 0 / 1 of the tile's k-steps
+#pragma unroll
+    for (int ks = 0; ks < KS / 2; ++ks) mma1(f, half * (KS / 2) + ks);
   };
   // Publish tile t and fetch its fragments.  Bare s_barrier (no workgroup fence: a fence is
   // s_waitcnt vmcnt(0) and would drain the prefetches).  Before it: this wave's DMA loads of tile t
@@ -220,7 +232,7 @@ __device__ __forceinline__ void k_loop(char* smem, const Dma<C, SHRINK>& dma, co
 }
 
 template <class C>
-__global__ __launch_bounds__(C::NT, C::NRT == 0 ? 2 : 1) void lora_gemm_pipe_kernel(const LoraGemmParams pin) {
+__global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const LoraGemmParams pin) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   LoraGemmParams p = pin;
   if (pin.grp != nullptr) {  // grouped launch: this workgroup's layer
@@ -247,15 +259,21 @@ __global__ __launch_bounds__(C::NT, C::NRT == 0 ? 2 : 1) void lora_gemm_pipe_ker
   const int m_blk = logical / p.n_chunks, chunk = logical % p.n_chunks;
   const int m0 = m_blk * BM;
   const int K = p.K, M = p.M, N = p.N;
+  constexpr int BKP = C::BKP, ROWB = C::ROWB;
   const int KT1 = K / BKP;                                             // K tiles of x / W
   const int KT = KT1 + (p.t_ext != nullptr ? p.R / BKP : 0);           // + rank tiles of T / B_cat (two-launch form)
 
   // DMA geometry of this lane inside a 16-row unit: LDS slot = lane (16 bytes each); it holds row
   // lane/4, physical piece lane%4, which stores logical piece (lane%4) ^ ((row/4)%4).
-  const int u_row = lane >> 2;
-  // fragment read: logical piece (2*ks + lh) of row (.. + l32) sits at physical piece ^ ((l32/4)%4)
-  const int sw = (l32 >> 2) & 3;
+  const int u_row = lane / C::PPR;
+  // fragment read: logical piece (2*ks + lh) of row (.. + l32) sits at physical piece ^ ((l32/SWR) % PPR)
+  const int sw = (l32 / C::SWR) % C::PPR;
 
+  // tuning only: dbg & 16 turns `res` into a timestamp buffer (8 x int64 per workgroup), no residual
+  long long* ts = (p.dbg & 16) ? reinterpret_cast<long long*>(const_cast<bf16_t*>(p.res)) + (size_t)blockIdx.x * 8 : nullptr;
+  if (p.dbg & 16) p.res = nullptr;
+  auto stamp = [&](int i) { if (ts != nullptr && tid == 0) ts[i] = (long long)__builtin_readcyclecounter(); };
+  stamp(0);
   for (int jt = 0; jt < p.n_chunk; ++jt) {
     const int n_tile = chunk * p.n_chunk + jt;
     if (n_tile >= p.n_tiles) break;  // uniform over the workgroup
@@ -268,18 +286,20 @@ __global__ __launch_bounds__(C::NT, C::NRT == 0 ? 2 : 1) void lora_gemm_pipe_ker
       int q = 0;
 #pragma unroll
       for (int i = 0; i < D::XI; ++i, ++q) {
-        const int r = (wave * D::XI + i) * 16 + u_row;  // row inside the x tile
+        const int r = (wave * D::XI + i) * C::UROWS + u_row;  // row inside the x tile
+        const int pc = ((lane % C::PPR) ^ ((r / C::SWR) % C::PPR)) * 8;
         int row = m0 + r; row = row < M ? row : M - 1;
-        d.off[q] = (long)row * K + (((lane & 3) ^ ((r >> 2) & 3)) * 8);
-        d.off2[q] = row * p.ldt + (((lane & 3) ^ ((r >> 2) & 3)) * 8);
+        d.off[q] = (long)row * K + pc;
+        d.off2[q] = row * p.ldt + pc + (p.t_nsplit > 0 ? (n0 / p.t_nsplit) * p.R : 0);
         d.dst[q] = (wave * D::XI + i) * 1024;
       }
 #pragma unroll
       for (int i = 0; i < D::WI; ++i, ++q) {
-        const int r = (wave * D::WI + i) * 16 + u_row;
+        const int r = (wave * D::WI + i) * C::UROWS + u_row;
+        const int pc = ((lane % C::PPR) ^ ((r / C::SWR) % C::PPR)) * 8;
         int row = n0 + r; row = row < N ? row : N - 1;
-        d.off[q] = (long)row * K + (((lane & 3) ^ ((r >> 2) & 3)) * 8);
-        d.off2[q] = row * p.R + (((lane & 3) ^ ((r >> 2) & 3)) * 8);
+        d.off[q] = (long)row * K + pc;
+        d.off2[q] = row * p.R + pc;
         d.dst[q] = C::SW_OFF + (wave * D::WI + i) * 1024;
       }
 #pragma unroll
@@ -330,6 +350,7 @@ __global__ __launch_bounds__(C::NT, C::NRT == 0 ? 2 : 1) void lora_gemm_pipe_ker
       }
     };
 
+    stamp(1);
     if (shrink) {
       if constexpr (NRT > 0) {
         Dma<C, true> d;
@@ -341,7 +362,9 @@ __global__ __launch_bounds__(C::NT, C::NRT == 0 ? 2 : 1) void lora_gemm_pipe_ker
       dma_setup(d);
       k_loop<C, false, BCH>(smem, d, p.x, p.w, p.a_cat, p.t_ext, p.b_cat, KT, KT1, lane, wm, wn, l32, lh, sw, acc, tacc, tail_loads);
     }
+    stamp(2);
     __syncthreads();  // every wave is done reading the ring before sB / sC reuse it
+    stamp(3);
 
     if constexpr (NRT > 0) {
       if (shrink) {
@@ -385,6 +408,7 @@ __global__ __launch_bounds__(C::NT, C::NRT == 0 ? 2 : 1) void lora_gemm_pipe_ker
     // Epilogue: bias in fp32, round to bf16, transpose through LDS so that every global store is a
     // 16-byte piece of a contiguous output row.  Residual pieces are requested before the staging
     // writes so their latency hides behind the transpose.
+    stamp(4);
     const int out_ld = p.geglu ? (N >> 1) : N;
     constexpr int CPR = BN / 8;                                   // 16-byte pieces per staged row
     constexpr int ECH = C::WAVES_M * 32 * CPR / C::NT;            // pieces per thread per pass
@@ -453,6 +477,7 @@ __global__ __launch_bounds__(C::NT, C::NRT == 0 ? 2 : 1) void lora_gemm_pipe_ker
       }
       __syncthreads();
     }
+    stamp(5);
   }
 }
 
@@ -493,6 +518,14 @@ int launch_prank(const LoraGemmParams& p, hipStream_t stream) {
   }
 }
 
+// plain GEMM (optionally K-extended by the rank columns) with 64 K columns per stage
+bool deep_stage_ok(const LoraGemmParams& p) {
+  const bool plain = p.R == 0 || p.t_ext != nullptr;
+  return plain && p.K % 64 == 0 && (p.t_ext == nullptr || p.R % 64 == 0);
+}
+
+bool plain_ok(const LoraGemmParams& p) { return p.R == 0 || p.t_ext != nullptr; }
+
 }  // namespace
 
 int lora_gemm_pipe_launch_grouped(const LoraGemmParams& p, int n_groups, hipStream_t stream) {
@@ -501,8 +534,15 @@ int lora_gemm_pipe_launch_grouped(const LoraGemmParams& p, int n_groups, hipStre
 
 int lora_gemm_pipe_launch(const LoraGemmParams& p, int tile_sel, hipStream_t stream) {
   switch (tile_sel) {
+    case 16: return launch_prank<128, 128, 2, 2, 4>(p, stream);
     case 17: return launch_prank<128, 128, 2, 2, 3>(p, stream);
     case 18: return launch_prank<128, 128, 2, 2, 2>(p, stream);
-    default: return launch_prank<128, 128, 2, 2, 4>(p, stream);
+    case 20: return deep_stage_ok(p) ? launch_pcfg<PCfg<128, 128, 2, 2, 0, 3, 64>>(p, stream) : KH_ERR_UNSUPPORTED;
+    case 21: return deep_stage_ok(p) ? launch_pcfg<PCfg<128, 128, 2, 2, 0, 2, 64>>(p, stream) : KH_ERR_UNSUPPORTED;
+    case 24: return plain_ok(p) ? launch_pcfg<PCfg<128, 256, 2, 2, 0, 3>>(p, stream) : KH_ERR_UNSUPPORTED;
+    case 25: return plain_ok(p) ? launch_pcfg<PCfg<128, 256, 2, 2, 0, 4>>(p, stream) : KH_ERR_UNSUPPORTED;
+    case 26: return plain_ok(p) ? launch_pcfg<PCfg<256, 128, 2, 2, 0, 3>>(p, stream) : KH_ERR_UNSUPPORTED;
+    default: break;
   }
+  return launch_prank<128, 128, 2, 2, 4>(p, stream);
 }

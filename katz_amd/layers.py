@@ -292,8 +292,14 @@ class KatzAttnProcessor:
         if attention_mask is not None:
             raise NotImplementedError("attention masks are not used on the SDXL path and not implemented")
         ctx = hidden_states if encoder_hidden_states is None else encoder_hidden_states
-        q = attn.to_q(hidden_states)
-        if encoder_hidden_states is not None and attn.ctx_kv is not None and attn.ctx_kv[0] is encoder_hidden_states:
+        qkv = attn.fused_qkv(hidden_states) if encoder_hidden_states is None else None
+        if qkv is not None:
+            q, k, v = qkv  # self-attention: one shrink + one GEMM for the three projections
+        else:
+            q = attn.to_q(hidden_states)
+        if qkv is not None:
+            pass
+        elif encoder_hidden_states is not None and attn.ctx_kv is not None and attn.ctx_kv[0] is encoder_hidden_states:
             _, k, v = attn.ctx_kv  # projected for every cross-attention at once at the start of the step
         else:
             k = attn.to_k(ctx)
@@ -319,6 +325,45 @@ class Attention(nn.Module):
         self.processor = processor or KatzAttnProcessor()
         self.is_cross = cross_attention_dim is not None
         self.ctx_kv = None  # (context tensor, k, v) filled by ContextKVProjector for the current step
+        self._qkv = None    # fused to_q/to_k/to_v state (self-attention only)
+
+    def fused_qkv(self, x: torch.Tensor):
+        """to_q / to_k / to_v of a self-attention as ONE GEMM over the stacked weights ([3N,K]: three
+        times the workgroups of a single projection, which alone covers 160 of 256 CUs) and, with
+        adapters, ONE shrink over the stacked A matrices.  Returns (q, k, v) as column views of the
+        [.., 3N] result, or None when the layers cannot be fused (then they run one by one)."""
+        layers = (self.to_q, self.to_k, self.to_v)
+        N, K = self.to_q.out_features, self.to_q.in_features
+        if self.is_cross or x.dtype != torch.bfloat16 or N % 128 != 0 or K % 64 != 0:
+            return None
+        for l in layers:
+            l.prepare()
+        sig = (_pack_epoch, tuple((l.weight.data_ptr(), l.weight._version) for l in layers), LORA_MODE)
+        st = self._qkv
+        if st is None or st["sig"] != sig:
+            packs = [l._packed for l in layers]
+            same = all(p is None for p in packs) or (all(p is not None for p in packs) and len({p.R for p in packs}) == 1)
+            ok = same and (packs[0] is None or LORA_MODE == "split") and all(l.bias is None for l in layers)
+            st = dict(sig=sig, ok=ok)
+            if ok:
+                st["w"] = torch.cat([l.weight.detach() for l in layers], dim=0).contiguous()
+                st["R"] = 0 if packs[0] is None else packs[0].R
+                if st["R"]:
+                    R = st["R"]
+                    st["a"] = torch.cat([p.a_cat for p in packs], dim=0).contiguous()
+                    st["s"] = torch.cat([p.col_scale for p in packs], dim=0).contiguous()
+                    st["b"] = torch.cat([p.b_cat for p in packs], dim=0).contiguous()
+                    for g, p in enumerate(packs):  # the layers now read (and rescale) the stacked storage
+                        p.a_cat, p.col_scale = st["a"][g * R:(g + 1) * R], st["s"][g * R:(g + 1) * R]
+            self._qkv = st
+        if not st["ok"]:
+            return None
+        if st["R"]:
+            t = ops.lora_shrink(x, st["a"], st["s"])
+            y = ops.lora_linear_pre(x, st["w"], None, t, st["b"], n_split=N)
+        else:
+            y = ops.lora_linear(x, st["w"], None)
+        return y.split(N, dim=-1)
 
     def set_processor(self, processor) -> None:
         self.processor = processor

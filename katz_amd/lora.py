@@ -20,7 +20,7 @@ from typing import Dict, List, Optional, Sequence
 
 import torch
 
-RANK_PAD = 32
+RANK_PAD = 64   # packed rank is padded to the K-stage depth of the GEMM that consumes it
 MAX_PACKED_RANK = 128
 
 

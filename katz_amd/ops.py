@@ -50,6 +50,7 @@ def lora_linear(
     geglu: bool = False,
     tile: int = 0,
     out: Optional[torch.Tensor] = None,
+    dbg: int = 0,
 ) -> torch.Tensor:
     """y = x W^T + b + ((x A_cat^T) * col_scale) B_cat^T (+ residual); bf16 or fp32 by x.dtype.
 
@@ -88,7 +89,7 @@ def lora_linear(
     if CALL_LOG is not None:
         CALL_LOG.append(("lora_linear", M, N, K, R, bool(geglu), residual is not None))
     if dt == BF16:
-        flags = (1 if geglu else 0) | ((tile & 0xFF) << 8)
+        flags = (1 if geglu else 0) | ((tile & 0xFF) << 8) | ((dbg & 0xFF) << 16)
         rc = lib.kh_lora_linear_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(a_cat), _ptr(b_cat), _ptr(col_scale),
                                      _ptr(residual), _ptr(out), M, N, K, R, flags, _stream())
     elif dt == torch.float32:
@@ -122,17 +123,19 @@ def lora_shrink(x: torch.Tensor, a_cat: torch.Tensor, col_scale: torch.Tensor, o
 
 def lora_linear_pre(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], t: torch.Tensor,
                     b_cat: torch.Tensor, residual: Optional[torch.Tensor] = None, geglu: bool = False,
-                    tile: int = 0) -> torch.Tensor:
+                    tile: int = 0, n_split: int = 0) -> torch.Tensor:
     """y = x W^T + b + t B_cat^T (+ residual | GEGLU) with t = lora_shrink(x, ...)[:, cols] (a column
-    slice of a wider shrink result is fine: only its last axis must be contiguous)."""
+    slice of a wider shrink result is fine: only its last axis must be contiguous).  n_split > 0: weight /
+    bias / b_cat stack several layers of n_split rows each and t holds their shrink results side by side."""
     lib = _lib.load()
     _req(x, BF16, "x"); _req(weight, BF16, "weight"); _req(b_cat, BF16, "b_cat")
     K = x.shape[-1]
     N = weight.shape[0]
     M = x.numel() // K
     R = b_cat.shape[1]
-    if t.dtype != BF16 or not t.is_cuda or t.dim() != 2 or t.stride(1) != 1 or t.shape != (M, R):
-        raise ValueError(f"t must be a bfloat16 [M,R] = [{M},{R}] GPU matrix with a contiguous last axis")
+    t_cols = R * (N // n_split) if n_split else R
+    if t.dtype != BF16 or not t.is_cuda or t.dim() != 2 or t.stride(1) != 1 or t.shape != (M, t_cols):
+        raise ValueError(f"t must be a bfloat16 [M,{t_cols}] GPU matrix with a contiguous last axis")
     if weight.shape[1] != K or b_cat.shape[0] != N:
         raise ValueError("weight / b_cat do not match x")
     if bias is not None:
@@ -146,7 +149,7 @@ def lora_linear_pre(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.
     if CALL_LOG is not None:
         CALL_LOG.append(("lora_linear", M, N, K, R, bool(geglu), residual is not None))
     flags = (1 if geglu else 0) | ((tile & 0xFF) << 8)
-    rc = lib.kh_lora_linear_pre_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(t), t.stride(0), _ptr(b_cat),
+    rc = lib.kh_lora_linear_pre_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(t), t.stride(0), n_split, _ptr(b_cat),
                                      _ptr(residual), _ptr(out), M, N, K, R, flags, _stream())
     _lib.check(rc, "kh_lora_linear_pre_bf16")
     return out

@@ -70,7 +70,7 @@ def test_pack_adapters_layout_and_rescale():
     ads = {"a": Adapter(torch.randn(8, 16, generator=g), torch.randn(64, 8, generator=g), alpha=16.0, weight=0.5),
            "b": Adapter(torch.randn(4, 16, generator=g), torch.randn(64, 4, generator=g), alpha=None, weight=2.0)}
     pk = pack_adapters(ads, ["b", "a"], 16, 64, torch.float32, "cpu", global_scale=0.5)
-    assert pk.R == 32 and pk.a_cat.shape == (32, 16) and pk.b_cat.shape == (64, 32)
+    assert pk.R == 64 and pk.a_cat.shape == (64, 16) and pk.b_cat.shape == (64, 64)
     assert torch.equal(pk.a_cat[:4], ads["b"].down) and torch.equal(pk.a_cat[4:12], ads["a"].down)
     assert torch.all(pk.a_cat[12:] == 0) and torch.all(pk.b_cat[:, 12:] == 0)
     assert torch.allclose(pk.col_scale[:4], torch.tensor(2.0 * 1.0 * 0.5))          # alpha = rank
