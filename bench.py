@@ -206,6 +206,15 @@ def main():
     # two-launch layers: the shrink launch belongs to the layer whose GEMM follows it
     shrink_calls = [c for c in log if c[0] == "lora_shrink"]
     shrink_ms = sum(d for n, d in launches if n == "lora_shrink")
+    shrink_us = [d * 1e3 for n, d in launches if n == "lora_shrink"]
+    assert len(shrink_calls) == len(shrink_us)
+    shrink_shapes = {}
+    for c, d in zip(shrink_calls, shrink_us):
+        e = shrink_shapes.setdefault(tuple(c[1:4]), [0, 0.0])
+        e[0] += 1
+        e[1] += d
+    shrink_rows = [{"M": M, "K": K, "R": R, "launches": cnt, "avg_us": round(tot / cnt, 2)}
+                   for (M, K, R), (cnt, tot) in sorted(shrink_shapes.items(), key=lambda kv: -kv[1][1])]
     n_layers = lambda c: c[5] if c[0] == "lora_linear_grouped" else 1
     gemm_flops = sum(n_layers(c) * lora_linear_flops(c[1], c[2], c[3], c[4]) for c in gemm_calls)
     gemm_total_ms = sum(gemm_ms) + shrink_ms
@@ -250,7 +259,8 @@ def main():
                      "frac": round(achieved_tf / PEAK_BF16_TFLOPS, 4), "traffic": None,
                      "launches_per_step": len(gemm_ms), "shrink_launches_per_step": len(shrink_calls),
                      "shrink_ms_per_step": round(shrink_ms, 3), "avg_launch_us": round(gemm_total_ms / len(gemm_ms) * 1e3, 2),
-                     "algorithmic_gflop_per_step": round(gemm_flops / 1e9, 1), "by_shape": shape_rows[:8]},
+                     "algorithmic_gflop_per_step": round(gemm_flops / 1e9, 1), "by_shape": shape_rows[:8],
+                     "shrink_by_shape": shrink_rows[:6]},
         "kernel_ms_per_step": {k: {"launches": v[0], "ms": round(v[1], 3)} for k, v in sorted(by_kernel.items())},
     }
     if not args.no_cpu_baseline:

@@ -107,12 +107,13 @@ __device__ __forceinline__ void k_loop(char* smem, const Dma<C, SHRINK>& dma, co
                                        int lane, int wm, int wn,
                                        int l32, int lh, int sw, f32x16 (&acc)[C::TM][C::TN],
                                        f32x16 (&tacc)[C::SM > 0 ? C::SM : 1][C::NRT > 0 ? C::NRT : 1],
-                                       TailLoads tail_loads) {
+                                       TailLoads tail_loads, bool nodma = false, bool fixk = false) {
   constexpr int TM = C::TM, TN = C::TN, NRT = C::NRT, NST = C::NST;
   constexpr int BKP = C::BKP, ROWB = C::ROWB, KS = C::KS;
   constexpr int PD = NST - 1;  // prefetch distance in K tiles
   using D = Dma<C, SHRINK>;
   auto issue = [&](int t) {
+    if (nodma) return;  // tuning only
     char* stage = smem + (t % NST) * C::STAGE;
 #pragma unroll
     for (int q = 0; q < D::LPS; ++q) {
@@ -120,7 +121,7 @@ __device__ __forceinline__ void k_loop(char* smem, const Dma<C, SHRINK>& dma, co
       // K tiles >= KT1 come from the extension operands: y = [x | T] . [W | B_cat]^T
       const bf16_t* base = q < D::XI ? px : (q < D::XI + D::WI ? pw : pa);
       const bf16_t* base2 = q < D::XI ? px2 : pw2;
-      const bf16_t* g = (SHRINK || t < KT1) ? base + dma.off[q] + t * BKP : base2 + dma.off2[q] + (t - KT1) * BKP;
+      const bf16_t* g = (SHRINK || t < KT1) ? base + dma.off[q] + (fixk ? 0 : t * BKP) : base2 + dma.off2[q] + (t - KT1) * BKP;
       if (!partial || lane < 32)
         __builtin_amdgcn_global_load_lds((gptr_t)g, (lptr_t)(stage + dma.dst[q]), 16, 0, 0);
     }
@@ -288,7 +289,7 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
       for (int i = 0; i < D::XI; ++i, ++q) {
         const int r = (wave * D::XI + i) * C::UROWS + u_row;  // row inside the x tile
         const int pc = ((lane % C::PPR) ^ ((r / C::SWR) % C::PPR)) * 8;
-        int row = m0 + r; row = row < M ? row : M - 1;
+        int row = ((p.dbg & 32) ? 0 : m0) + r; row = row < M ? row : M - 1;
         d.off[q] = (long)row * K + pc;
         d.off2[q] = row * p.ldt + pc + (p.t_nsplit > 0 ? (n0 / p.t_nsplit) * p.R : 0);
         d.dst[q] = (wave * D::XI + i) * 1024;
@@ -297,7 +298,7 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
       for (int i = 0; i < D::WI; ++i, ++q) {
         const int r = (wave * D::WI + i) * C::UROWS + u_row;
         const int pc = ((lane % C::PPR) ^ ((r / C::SWR) % C::PPR)) * 8;
-        int row = n0 + r; row = row < N ? row : N - 1;
+        int row = ((p.dbg & 32) ? 0 : n0) + r; row = row < N ? row : N - 1;
         d.off[q] = (long)row * K + pc;
         d.off2[q] = row * p.R + pc;
         d.dst[q] = C::SW_OFF + (wave * D::WI + i) * 1024;
@@ -360,7 +361,7 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
     } else {
       Dma<C, false> d;
       dma_setup(d);
-      k_loop<C, false, BCH>(smem, d, p.x, p.w, p.a_cat, p.t_ext, p.b_cat, KT, KT1, lane, wm, wn, l32, lh, sw, acc, tacc, tail_loads);
+      k_loop<C, false, BCH>(smem, d, p.x, p.w, p.a_cat, p.t_ext, p.b_cat, KT, KT1, lane, wm, wn, l32, lh, sw, acc, tacc, tail_loads, (p.dbg & 64) != 0, (p.dbg & 128) != 0);
     }
     stamp(2);
     __syncthreads();  // every wave is done reading the ring before sB / sC reuse it
@@ -542,7 +543,23 @@ int lora_gemm_pipe_launch(const LoraGemmParams& p, int tile_sel, hipStream_t str
     case 24: return plain_ok(p) ? launch_pcfg<PCfg<128, 256, 2, 2, 0, 3>>(p, stream) : KH_ERR_UNSUPPORTED;
     case 25: return plain_ok(p) ? launch_pcfg<PCfg<128, 256, 2, 2, 0, 4>>(p, stream) : KH_ERR_UNSUPPORTED;
     case 26: return plain_ok(p) ? launch_pcfg<PCfg<256, 128, 2, 2, 0, 3>>(p, stream) : KH_ERR_UNSUPPORTED;
+    case 27: return plain_ok(p) ? launch_pcfg<PCfg<256, 128, 4, 2, 0, 4>>(p, stream) : KH_ERR_UNSUPPORTED;
+    case 28: return plain_ok(p) ? launch_pcfg<PCfg<128, 256, 2, 4, 0, 4>>(p, stream) : KH_ERR_UNSUPPORTED;
+    case 29: return deep_stage_ok(p) ? launch_pcfg<PCfg<256, 128, 4, 2, 0, 3, 64>>(p, stream) : KH_ERR_UNSUPPORTED;
+    case 30: return plain_ok(p) ? launch_pcfg<PCfg<256, 256, 4, 2, 0, 3>>(p, stream) : KH_ERR_UNSUPPORTED;
+    case 31: return plain_ok(p) ? launch_pcfg<PCfg<256, 256, 4, 2, 0, 4>>(p, stream) : KH_ERR_UNSUPPORTED;
+    case 32: return deep_stage_ok(p) ? launch_pcfg<PCfg<128, 128, 2, 4, 0, 3, 64>>(p, stream) : KH_ERR_UNSUPPORTED;
     default: break;
+  }
+  // Default choice.  The limiter is the vector L1 path (every operand byte enters LDS through it), so
+  // FLOPs per loaded byte decide: 256x128 tiles (8 waves) when there are enough tiles to keep the chip
+  // busy with them; when the 128x128 tiles do not even fill one round of 256 CUs, one 8-wave workgroup
+  // per CU with 64-column stages (full 128-byte lines) beats two 4-wave ones; 128x128 / 4 waves /
+  // two workgroups per CU otherwise.
+  if (plain_ok(p)) {
+    const long tiles = (long)((p.M + 127) / 128) * ((p.N + 127) / 128);
+    if (tiles >= 480 && p.K >= 1024 && !p.geglu) return launch_pcfg<PCfg<256, 128, 4, 2, 0, 4>>(p, stream);
+    if (tiles <= 256 && p.M >= 1024 && deep_stage_ok(p)) return launch_pcfg<PCfg<128, 128, 2, 4, 0, 3, 64>>(p, stream);
   }
   return launch_prank<128, 128, 2, 2, 4>(p, stream);
 }
