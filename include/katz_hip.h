@@ -160,6 +160,18 @@ int kh_residual_add_bf16(void* dst, const void* const* srcs, int n_srcs, float i
 int kh_concat_residual_bf16(const void* h, const void* skip, const void* const* residuals, int n_residuals,
                             float inv_count, void* out, int64_t rows, int64_t C1, int64_t C2, void* stream);
 
+/* ---- 3x3 convolution of the residual blocks ------------------------------------------------------------
+ * y[n,ho,wo,co] = bias[co] + sum_{kh,kw,ci} x[n, ho*stride+kh-1, wo*stride+kw-1, ci] * w[co,kh,kw,ci]
+ *                 (+ residual[n,ho,wo,co]); zero padding 1, stride 1 or 2, Ho = (H-1)/stride + 1.
+ * conv1 / conv2 of ResnetBlock2D (diffusers-hf/src/diffusers/models/resnet.py:275, :295, applied at :351, :369),
+ * the stride-2 conv of Downsample2D and the conv of Upsample2D (diffusers-hf/src/diffusers/models/downsampling.py,
+ * upsampling.py), with the block's `input_tensor + hidden_states` (resnet.py:374) as the optional residual.
+ * Layout: x NHWC [Nb,H,W,Cin], w [Cout,3,3,Cin] (the nn.Conv2d weight permuted to O,KH,KW,I), y and residual
+ * NHWC [Nb,Ho,Wo,Cout], all bf16; bias bf16 [Cout] or NULL.  Runs as an implicit GEMM (M = Nb*Ho*Wo,
+ * K = 9*Cin) on the MFMA pipeline of kh_lora_linear_bf16.  Cin % 32 == 0, Cout % 8 == 0. */
+int kh_conv3x3_nhwc_bf16(const void* x, const void* w, const void* bias, const void* residual, void* y, int64_t Nb,
+                         int64_t H, int64_t W, int64_t Cin, int64_t Cout, int64_t stride, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -20,9 +20,14 @@ struct LoraGemmParams {
   int M, N, K, R;
   int m_tiles, n_tiles, n_chunk, n_chunks;  // n_chunk = N tiles walked by one workgroup
   int geglu;                                // 1: W rows are (value,gate) interleaved in 32-column groups, y is [M,N/2]
+  // 3x3 convolution as an implicit GEMM (conv_cin > 0): x is an NHWC image [Nb, conv_h, conv_w, conv_cin], row m
+  // of the GEMM is output pixel m of [Nb, conv_ho, conv_wo], K = 9 * conv_cin ordered (kh, kw, ci), padding 1
+  int conv_cin, conv_h, conv_w, conv_ho, conv_wo, conv_stride;
 };
 
 // Software-pipelined kernel (lora_gemm_pipe.hip); needs K % 32 == 0.  tile_sel: 0 automatic, >= 16 forces a tile.
 int lora_gemm_pipe_launch(const LoraGemmParams& p, int tile_sel, hipStream_t stream);
+// 3x3 convolution (conv_* fields set, R == 0, K == 9 * conv_cin, conv_cin % 32 == 0).
+int lora_gemm_pipe_launch_conv(const LoraGemmParams& p, hipStream_t stream);
 // Grouped form: grid.y = n_groups, per-group pointers from p.grp; rank columns (p.R > 0) as extra K tiles.
 int lora_gemm_pipe_launch_grouped(const LoraGemmParams& p, int n_groups, hipStream_t stream);

@@ -483,6 +483,7 @@ KH_EXPORT int kh_lora_linear_bf16(const void* x, const void* w, const void* bias
   p.M = (int)M; p.N = (int)N; p.K = (int)K; p.R = (int)R;
   p.m_tiles = p.n_tiles = p.n_chunk = p.n_chunks = 0;
   p.geglu = geglu ? 1 : 0;
+  p.conv_cin = p.conv_h = p.conv_w = p.conv_ho = p.conv_wo = p.conv_stride = 0;
   p.dbg = (flags >> 16) & 0xff;
   hipStream_t s = (hipStream_t)stream;
   const int tile_sel = (flags >> 8) & 0xff;  // 0 = automatic
@@ -516,7 +517,33 @@ KH_EXPORT int kh_lora_linear_pre_bf16(const void* x, const void* w, const void* 
   p.M = (int)M; p.N = (int)N; p.K = (int)K; p.R = (int)R;
   p.m_tiles = p.n_tiles = p.n_chunk = p.n_chunks = 0;
   p.geglu = geglu ? 1 : 0;
+  p.conv_cin = p.conv_h = p.conv_w = p.conv_ho = p.conv_wo = p.conv_stride = 0;
   return lora_gemm_pipe_launch(p, (flags >> 8) & 0xff, (hipStream_t)stream);
+}
+
+// 3x3 convolution, padding 1, NHWC, as an implicit GEMM on the pipelined kernel; see include/katz_hip.h.
+KH_EXPORT int kh_conv3x3_nhwc_bf16(const void* x, const void* w, const void* bias, const void* residual, void* y,
+                                   int64_t Nb, int64_t H, int64_t W, int64_t Cin, int64_t Cout, int64_t stride,
+                                   void* stream) {
+  if (!x || !w || !y || Nb <= 0 || H <= 0 || W <= 0 || Cin <= 0 || Cout <= 0) return KH_ERR_INVALID_ARG;
+  if (stride != 1 && stride != 2) return KH_ERR_UNSUPPORTED;
+  if (Cin % 32 != 0 || Cout % 8 != 0) return KH_ERR_UNSUPPORTED;
+  const int64_t Ho = (H + 2 - 3) / stride + 1, Wo = (W + 2 - 3) / stride + 1;
+  const int64_t M = Nb * Ho * Wo;
+  if (M > (1 << 24) || Cout > (1 << 24) || 9 * Cin > (1 << 24) || Nb * H * W * Cin >= ((int64_t)1 << 40)) return KH_ERR_TOO_LARGE;
+  if (!kh_aligned16(x) || !kh_aligned16(w) || !kh_aligned16(y) || (residual && !kh_aligned16(residual)))
+    return KH_ERR_ALIGNMENT;
+  LoraGemmParams p;
+  p.x = (const bf16_t*)x; p.w = (const bf16_t*)w; p.bias = (const bf16_t*)bias;
+  p.a_cat = nullptr; p.b_cat = nullptr; p.col_scale = nullptr;
+  p.t_ext = nullptr; p.ldt = 0; p.grp = nullptr; p.dbg = 0; p.t_nsplit = 0;
+  p.res = (const bf16_t*)residual; p.y = (bf16_t*)y;
+  p.M = (int)M; p.N = (int)Cout; p.K = (int)(9 * Cin); p.R = 0;
+  p.m_tiles = p.n_tiles = p.n_chunk = p.n_chunks = 0;
+  p.geglu = 0;
+  p.conv_cin = (int)Cin; p.conv_h = (int)H; p.conv_w = (int)W; p.conv_ho = (int)Ho; p.conv_wo = (int)Wo;
+  p.conv_stride = (int)stride;
+  return lora_gemm_pipe_launch_conv(p, (hipStream_t)stream);
 }
 
 // Many layers that share one input in one launch; see include/katz_hip.h.
@@ -535,6 +562,7 @@ KH_EXPORT int kh_lora_linear_grouped_bf16(const void* x, const uint64_t* table, 
   p.M = (int)M; p.N = (int)N; p.K = (int)K; p.R = (int)R;
   p.m_tiles = p.n_tiles = p.n_chunk = p.n_chunks = 0;
   p.geglu = 0;
+  p.conv_cin = p.conv_h = p.conv_w = p.conv_ho = p.conv_wo = p.conv_stride = 0;
   return lora_gemm_pipe_launch_grouped(p, (int)n_groups, (hipStream_t)stream);
 }
 

@@ -101,20 +101,46 @@ struct Dma {
 // matrix pipe has work queued while the wave waits for its neighbours, half after it, under the reads.
 // SHRINK also accumulates T = x . A_cat^T for the shrink m-tiles of this wave (m-tile wn*SM + s of
 // its wave row, selected branch-free from the x fragments it holds).
-template <class C, bool SHRINK, int NX, class TailLoads>
+// 16 bytes of zeros (and more): what a 3x3 convolution's DMA reads for taps that fall into the padding
+__device__ __attribute__((aligned(256))) const uint32_t kh_zero_page[64] = {0};
+
+struct ConvGeom { int w, cin; };  // input width and channels (elements)
+
+template <class C, bool SHRINK, int NX, bool CONV, class TailLoads>
 __device__ __forceinline__ void k_loop(char* smem, const Dma<C, SHRINK>& dma, const bf16_t* px, const bf16_t* pw,
                                        const bf16_t* pa, const bf16_t* px2, const bf16_t* pw2, int KT, int KT1,
                                        int lane, int wm, int wn,
                                        int l32, int lh, int sw, f32x16 (&acc)[C::TM][C::TN],
                                        f32x16 (&tacc)[C::SM > 0 ? C::SM : 1][C::NRT > 0 ? C::NRT : 1],
-                                       TailLoads tail_loads, bool nodma = false, bool fixk = false) {
+                                       TailLoads tail_loads, ConvGeom cg, bool nodma = false, bool fixk = false) {
   constexpr int TM = C::TM, TN = C::TN, NRT = C::NRT, NST = C::NST;
   constexpr int BKP = C::BKP, ROWB = C::ROWB, KS = C::KS;
   constexpr int PD = NST - 1;  // prefetch distance in K tiles
   using D = Dma<C, SHRINK>;
+  // convolution: K tiles are requested in order, so the tap (kh, kw) and channel offset of the next
+  // request are running scalars; x rows of tap (kh, kw) sit (kh*W + kw)*Cin elements after the row's
+  // base (the pixel above-left), rows whose tap falls outside the image read zeros instead
+  int cv_tap = 0, cv_kw = 0, cv_c0 = 0, cv_shift = 0, cv_row = 0;
   auto issue = [&](int t) {
     if (nodma) return;  // tuning only
     char* stage = smem + (t % NST) * C::STAGE;
+    if constexpr (CONV) {
+#pragma unroll
+      for (int q = 0; q < D::XI; ++q) {
+        const bool valid = (dma.off2[q] >> cv_tap) & 1;
+        const bf16_t* g = valid ? px + dma.off[q] + (cv_shift + cv_c0) : reinterpret_cast<const bf16_t*>(kh_zero_page);
+        __builtin_amdgcn_global_load_lds((gptr_t)g, (lptr_t)(stage + dma.dst[q]), 16, 0, 0);
+      }
+#pragma unroll
+      for (int q = D::XI; q < D::LPS; ++q)
+        __builtin_amdgcn_global_load_lds((gptr_t)(pw + dma.off[q] + t * BKP), (lptr_t)(stage + dma.dst[q]), 16, 0, 0);
+      cv_c0 += BKP;
+      if (cv_c0 == cg.cin) {
+        cv_c0 = 0; ++cv_tap; ++cv_kw; cv_shift += cg.cin;
+        if (cv_kw == 3) { cv_kw = 0; cv_row += cg.w * cg.cin; cv_shift = cv_row; }
+      }
+      return;
+    }
 #pragma unroll
     for (int q = 0; q < D::LPS; ++q) {
       const bool partial = SHRINK && (q == D::LPS - 1) && (D::RA % 16 != 0);
@@ -232,7 +258,7 @@ __device__ __forceinline__ void k_loop(char* smem, const Dma<C, SHRINK>& dma, co
   }
 }
 
-template <class C>
+template <class C, bool CONV = false>
 __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const LoraGemmParams pin) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   LoraGemmParams p = pin;
@@ -290,8 +316,22 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
         const int r = (wave * D::XI + i) * C::UROWS + u_row;  // row inside the x tile
         const int pc = ((lane % C::PPR) ^ ((r / C::SWR) % C::PPR)) * 8;
         int row = ((p.dbg & 32) ? 0 : m0) + r; row = row < M ? row : M - 1;
-        d.off[q] = (long)row * K + pc;
-        d.off2[q] = row * p.ldt + pc + (p.t_nsplit > 0 ? (n0 / p.t_nsplit) * p.R : 0);
+        if constexpr (CONV) {
+          // output pixel -> the input pixel above-left of its 3x3 window, and which taps are inside the image
+          const int wo = row % p.conv_wo, t2 = row / p.conv_wo, ho = t2 % p.conv_ho, nb = t2 / p.conv_ho;
+          const int hi0 = ho * p.conv_stride - 1, wi0 = wo * p.conv_stride - 1;
+          int mask = 0;
+#pragma unroll
+          for (int tap = 0; tap < 9; ++tap) {
+            const int hi = hi0 + tap / 3, wi = wi0 + tap % 3;
+            mask |= (hi >= 0 && hi < p.conv_h && wi >= 0 && wi < p.conv_w) ? (1 << tap) : 0;
+          }
+          d.off[q] = ((long)(nb * p.conv_h + hi0) * p.conv_w + wi0) * p.conv_cin + pc;
+          d.off2[q] = mask;
+        } else {
+          d.off[q] = (long)row * K + pc;
+          d.off2[q] = row * p.ldt + pc + (p.t_nsplit > 0 ? (n0 / p.t_nsplit) * p.R : 0);
+        }
         d.dst[q] = (wave * D::XI + i) * 1024;
       }
 #pragma unroll
@@ -356,12 +396,12 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
       if constexpr (NRT > 0) {
         Dma<C, true> d;
         dma_setup(d);
-        k_loop<C, true, BCH>(smem, d, p.x, p.w, p.a_cat, p.t_ext, p.b_cat, KT, KT1, lane, wm, wn, l32, lh, sw, acc, tacc, tail_loads);
+        k_loop<C, true, BCH, false>(smem, d, p.x, p.w, p.a_cat, p.t_ext, p.b_cat, KT, KT1, lane, wm, wn, l32, lh, sw, acc, tacc, tail_loads, ConvGeom{0, 0});
       }
     } else {
       Dma<C, false> d;
       dma_setup(d);
-      k_loop<C, false, BCH>(smem, d, p.x, p.w, p.a_cat, p.t_ext, p.b_cat, KT, KT1, lane, wm, wn, l32, lh, sw, acc, tacc, tail_loads, (p.dbg & 64) != 0, (p.dbg & 128) != 0);
+      k_loop<C, false, BCH, CONV>(smem, d, p.x, p.w, p.a_cat, p.t_ext, p.b_cat, KT, KT1, lane, wm, wn, l32, lh, sw, acc, tacc, tail_loads, ConvGeom{p.conv_w, p.conv_cin}, (p.dbg & 64) != 0, (p.dbg & 128) != 0);
     }
     stamp(2);
     __syncthreads();  // every wave is done reading the ring before sB / sC reuse it
@@ -482,7 +522,7 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
   }
 }
 
-template <class C>
+template <class C, bool CONV = false>
 int launch_pcfg(LoraGemmParams p, hipStream_t stream, int n_groups = 1) {
   p.m_tiles = (p.M + C::BM - 1) / C::BM;
   p.n_tiles = (p.N + C::BN - 1) / C::BN;
@@ -495,13 +535,13 @@ int launch_pcfg(LoraGemmParams p, hipStream_t stream, int n_groups = 1) {
   p.n_chunks = (p.n_tiles + nc - 1) / nc;
   static bool attr_done = false;  // per template instantiation
   if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void*)lora_gemm_pipe_kernel<C>,
+    hipError_t e = hipFuncSetAttribute((const void*)lora_gemm_pipe_kernel<C, CONV>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)C::LDS_BYTES);
     if (e != hipSuccess) return (int)e;
     attr_done = true;
   }
   const unsigned grid = (unsigned)(p.m_tiles * p.n_chunks);
-  kh_launch(KH_TAG_LORA_GEMM, lora_gemm_pipe_kernel<C>, dim3(grid, (unsigned)n_groups), dim3(C::NT), C::LDS_BYTES, stream, p);
+  kh_launch(CONV ? KH_TAG_CONV : KH_TAG_LORA_GEMM, lora_gemm_pipe_kernel<C, CONV>, dim3(grid, (unsigned)n_groups), dim3(C::NT), C::LDS_BYTES, stream, p);
   KH_RETURN_LAST_ERROR();
 }
 
@@ -528,6 +568,12 @@ bool deep_stage_ok(const LoraGemmParams& p) {
 bool plain_ok(const LoraGemmParams& p) { return p.R == 0 || p.t_ext != nullptr; }
 
 }  // namespace
+
+int lora_gemm_pipe_launch_conv(const LoraGemmParams& p, hipStream_t stream) {
+  const long tiles = (long)((p.M + 127) / 128) * ((p.N + 127) / 128);
+  if (tiles <= 256 && p.conv_cin % 64 == 0) return launch_pcfg<PCfg<128, 128, 2, 4, 0, 3, 64>, true>(p, stream);
+  return launch_pcfg<PCfg<128, 128, 2, 2, 0, 4>, true>(p, stream);
+}
 
 int lora_gemm_pipe_launch_grouped(const LoraGemmParams& p, int n_groups, hipStream_t stream) {
   return launch_pcfg<PCfg<128, 128, 2, 2, 0, 4>>(p, stream, n_groups);

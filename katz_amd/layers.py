@@ -226,11 +226,39 @@ class TimestepEmbedding(nn.Module):
         return self.linear_2(F.silu(self.linear_1(sample)))
 
 
+class Conv3x3(nn.Conv2d):
+    """nn.Conv2d(kernel 3, padding 1, stride 1 or 2) whose forward runs the katz_hip implicit-GEMM kernel on
+    channels_last bf16 GPU tensors; parameters and state-dict keys are nn.Conv2d's.  forward(x, residual)
+    also folds the residual add that follows the convolution (resnet.py:374) into the kernel's epilogue.
+    Shapes the kernel does not take (Cin % 32 != 0, Cout % 8 != 0, other dtypes / layouts) run torch's conv2d."""
+
+    def __init__(self, in_channels, out_channels, stride=1, padding=1):
+        super().__init__(in_channels, out_channels, 3, stride=stride, padding=padding)
+        self._packed = None  # (weight data_ptr, weight version, [Cout,3,3,Cin] copy)
+
+    def packed_weight(self) -> torch.Tensor:
+        w = self.weight
+        if self._packed is None or self._packed[0] != w.data_ptr() or self._packed[1] != w._version:
+            self._packed = (w.data_ptr(), w._version, ops.pack_conv3x3_weight(w))
+        return self._packed[2]
+
+    def forward(self, x, residual=None):
+        native = (x.is_cuda and x.dtype == torch.bfloat16 and self.weight.dtype == torch.bfloat16
+                  and self.padding == (1, 1) and self.in_channels % 32 == 0 and self.out_channels % 8 == 0)
+        if not native:
+            y = super().forward(x)
+            return y if residual is None else residual + y
+        x = x.contiguous(memory_format=torch.channels_last)   # no copy when the producer already wrote NHWC
+        if residual is not None:
+            residual = residual.contiguous(memory_format=torch.channels_last)
+        return ops.conv3x3(x, self.packed_weight(), self.bias, stride=self.stride[0], residual=residual)
+
+
 class Downsample2D(nn.Module):
     def __init__(self, channels, use_conv=True, out_channels=None, padding=1, name="op"):
         super().__init__()
         self.padding = padding
-        self.conv = nn.Conv2d(channels, out_channels or channels, 3, stride=2, padding=padding)
+        self.conv = Conv3x3(channels, out_channels or channels, stride=2, padding=padding)
 
     def forward(self, x):
         if self.padding == 0:
@@ -241,7 +269,7 @@ class Downsample2D(nn.Module):
 class Upsample2D(nn.Module):
     def __init__(self, channels, use_conv=True, out_channels=None):
         super().__init__()
-        self.conv = nn.Conv2d(channels, out_channels or channels, 3, padding=1)
+        self.conv = Conv3x3(channels, out_channels or channels)
 
     def forward(self, x, output_size=None):
         if output_size is None:
@@ -260,11 +288,21 @@ class ResnetBlock2D(nn.Module):
         out_channels = in_channels if out_channels is None else out_channels
         self.output_scale_factor = output_scale_factor
         self.norm_silu1 = nn.Sequential(*fused_norm_silu(in_channels, groups, eps))
-        self.conv1 = nn.Conv2d(in_channels, out_channels, 3, padding=1)
+        self.conv1 = Conv3x3(in_channels, out_channels)
         self.time_emb_proj = nn.Linear(temb_channels, out_channels)
         self.norm_silu2 = nn.Sequential(*fused_norm_silu(out_channels, groups, eps))
-        self.conv2 = nn.Conv2d(out_channels, out_channels, 3, padding=1)
+        self.conv2 = Conv3x3(out_channels, out_channels)
         self.conv_shortcut = nn.Conv2d(in_channels, out_channels, 1) if in_channels != out_channels else None
+
+    def _shortcut(self, x):
+        """1x1 convolution = a linear layer over the channels of every pixel (NHWC rows)."""
+        sc = self.conv_shortcut
+        if not (x.is_cuda and x.dtype == torch.bfloat16 and x.is_contiguous(memory_format=torch.channels_last)
+                and sc.in_channels % 32 == 0 and sc.out_channels % 8 == 0):
+            return sc(x)
+        nb, c, hh, ww = x.shape
+        y = ops.lora_linear(x.permute(0, 2, 3, 1).reshape(nb * hh * ww, c), sc.weight.reshape(sc.out_channels, c), sc.bias)
+        return y.view(nb, hh, ww, sc.out_channels).permute(0, 3, 1, 2)
 
     def forward(self, input_tensor, temb_act):
         """temb_act = silu(temb), computed once per step by the caller."""
@@ -272,10 +310,9 @@ class ResnetBlock2D(nn.Module):
         h = self.conv1(h)
         # hidden_states + temb[:, :, None, None] rides inside the second norm (no separate pass)
         h = self.norm_silu2[0](h, add_nc=self.time_emb_proj(temb_act))
-        h = self.conv2(h)
         if self.conv_shortcut is not None:
-            input_tensor = self.conv_shortcut(input_tensor)
-        out = input_tensor + h
+            input_tensor = self._shortcut(input_tensor)
+        out = self.conv2(h, residual=input_tensor)   # input_tensor + conv2(h), the add in the conv's epilogue
         if self.output_scale_factor != 1.0:
             out = out / self.output_scale_factor
         return out

@@ -364,10 +364,43 @@ def concat_residual(h: torch.Tensor, skip: torch.Tensor, residuals: Sequence[tor
     return out
 
 
+def pack_conv3x3_weight(weight: torch.Tensor) -> torch.Tensor:
+    """nn.Conv2d weight [Cout,Cin,3,3] -> the [Cout,3,3,Cin] layout kh_conv3x3_nhwc_bf16 reads (a copy)."""
+    if weight.dim() != 4 or weight.shape[2:] != (3, 3):
+        raise ValueError("expected a [Cout,Cin,3,3] weight")
+    return weight.detach().permute(0, 2, 3, 1).contiguous()
+
+
+def conv3x3(x: torch.Tensor, w_packed: torch.Tensor, bias: Optional[torch.Tensor] = None, stride: int = 1,
+            residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """3x3 convolution, padding 1, of a channels_last [N,Cin,H,W] tensor; returns channels_last [N,Cout,Ho,Wo]
+    (+ residual of that shape).  w_packed: pack_conv3x3_weight(weight)."""
+    lib = _lib.load()
+    if not x.is_cuda or x.dtype != BF16 or x.dim() != 4 or not x.is_contiguous(memory_format=torch.channels_last):
+        raise ValueError("x must be a channels_last bfloat16 GPU tensor")
+    Nb, Cin, H, W = x.shape
+    Cout = w_packed.shape[0]
+    if w_packed.shape != (Cout, 3, 3, Cin) or not w_packed.is_contiguous() or w_packed.dtype != BF16:
+        raise ValueError("w_packed must be a contiguous bfloat16 [Cout,3,3,Cin] tensor")
+    if bias is not None and (bias.shape != (Cout,) or bias.dtype != BF16 or not bias.is_contiguous()):
+        raise ValueError("bias must be a contiguous bfloat16 [Cout] tensor")
+    Ho, Wo = (H - 1) // stride + 1, (W - 1) // stride + 1
+    out = torch.empty((Nb, Cout, Ho, Wo), dtype=BF16, device=x.device, memory_format=torch.channels_last)
+    if residual is not None and (residual.shape != out.shape or residual.dtype != BF16
+                                 or not residual.is_contiguous(memory_format=torch.channels_last)):
+        raise ValueError("residual must be a channels_last bfloat16 tensor of the output's shape")
+    if CALL_LOG is not None:
+        CALL_LOG.append(("conv3x3", Nb * Ho * Wo, Cout, 9 * Cin, stride))
+    rc = lib.kh_conv3x3_nhwc_bf16(_ptr(x), _ptr(w_packed), _ptr(bias), _ptr(residual), _ptr(out), Nb, H, W, Cin, Cout,
+                                  stride, _stream())
+    _lib.check(rc, "kh_conv3x3_nhwc_bf16")
+    return out
+
+
 # --------------------------------------------------------------------------------------- per-launch timing
 KERNEL_TAGS = {1: "lora_gemm", 2: "lora_gemm_f32", 3: "attention", 4: "group_norm_stats", 5: "group_norm_apply",
                6: "layer_norm", 7: "geglu", 8: "residual_add", 9: "concat_residual", 10: "sgmv_shrink",
-               11: "sgmv_expand", 12: "lora_shrink"}
+               11: "sgmv_expand", 12: "lora_shrink", 13: "conv3x3"}
 
 
 def profile_begin() -> None:

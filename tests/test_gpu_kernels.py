@@ -498,3 +498,35 @@ def test_fused_qkv_matches_separate_projections():
     for j in range(3):
         ref = O.lora_linear(x, ws[j], None, ads[j])
         assert_close_rel(y[:, j * N:(j + 1) * N], ref, REL_BF16, f"fused qkv part {j}")
+
+
+@pytest.mark.parametrize("shape", [
+    # (Nb, Cin, H, W, Cout, stride, bias, residual)
+    (2, 64, 16, 16, 64, 1, True, False),
+    (2, 320, 32, 32, 320, 1, True, True),      # 128-row tiles cross image rows
+    (1, 96, 13, 9, 40, 1, True, False),        # ragged: M and Cout not multiples of the tile, Cin = 3 x 32
+    (2, 128, 16, 16, 128, 2, True, False),     # Downsample2D
+    (1, 64, 15, 11, 72, 2, False, True),       # odd sizes, stride 2
+    (2, 1280, 32, 32, 1280, 1, True, True),    # the deepest SDXL resnet conv (8-wave tile path)
+])
+def test_conv3x3_nhwc_bf16(shape):
+    """Implicit-GEMM 3x3 convolution against torch's fp32 conv2d on the same bf16-rounded operands."""
+    from katz_amd import ops
+
+    Nb, Cin, H, W, Cout, stride, has_bias, has_res = shape
+    say("conv3x3", shape)
+    d = dev()
+    g = torch.Generator().manual_seed(7 + Cin + Cout)
+    x = randn(g, Nb, Cin, H, W).to(BF)
+    w = randn(g, Cout, Cin, 3, 3, std=(9 * Cin) ** -0.5).to(BF)
+    b = randn(g, Cout).to(BF) if has_bias else None
+    ref = torch.nn.functional.conv2d(x.float(), w.float(), None if b is None else b.float(), stride=stride, padding=1)
+    res = randn(g, *ref.shape).to(BF) if has_res else None
+    if res is not None:
+        ref = ref.to(BF).float() + res.float()   # the kernel rounds the conv to bf16 before the residual add
+    xd = x.to(d).contiguous(memory_format=torch.channels_last)
+    y = ops.conv3x3(xd, ops.pack_conv3x3_weight(w.to(d)), None if b is None else b.to(d), stride=stride,
+                    residual=None if res is None else res.to(d).contiguous(memory_format=torch.channels_last))
+    torch.cuda.synchronize()
+    assert y.shape == ref.shape and y.is_contiguous(memory_format=torch.channels_last)
+    assert_close_rel(y, ref, REL_BF16, f"conv3x3 {shape}")
