@@ -41,7 +41,7 @@ const char* kh_error_string(int code);
  * kh_profile_begin and kh_profile_end every kernel of this library is launched with its own HIP
  * start/stop event pair on the launch stream.  kh_profile_end waits for them and writes, in launch
  * order, a kernel tag (1 lora_gemm, 2 lora_gemm_f32, 3 attention, 4 group_norm stats, 5 group_norm apply,
- * 6 layer_norm, 7 geglu, 8 residual_add, 9 concat_residual, 10 sgmv_shrink, 11 sgmv_expand, 12 lora_shrink, 13 conv3x3) and the
+ * 6 layer_norm, 7 geglu, 8 residual_add, 9 concat_residual, 10 sgmv_shrink, 11 sgmv_expand, 12 lora_shrink, 13 conv3x3, 14 cfg_euler) and the
  * duration in ms into HOST arrays; returns the number of launches (or -hipError_t).  Do not use under
  * graph capture. */
 int kh_profile_begin(void);
@@ -171,6 +171,19 @@ int kh_concat_residual_bf16(const void* h, const void* skip, const void* const* 
  * K = 9*Cin) on the MFMA pipeline of kh_lora_linear_bf16.  Cin % 32 == 0, Cout % 8 == 0. */
 int kh_conv3x3_nhwc_bf16(const void* x, const void* w, const void* bias, const void* residual, void* y, int64_t Nb,
                          int64_t H, int64_t W, int64_t Cin, int64_t Cout, int64_t stride, void* stream);
+
+/* ---- Classifier-free guidance + Euler step --------------------------------------------------------------
+ * eps = u + g*(t - u) with noise_pred = [u; t] (uncond rows first)      pipeline_controlnet_sd_xl_katz.py:1649-1650
+ * x0 = x - sigma*eps; d = (x - x0)/sigma; x' = x + d*(sigma_next - sigma) scheduling_euler_discrete.py:505-527
+ *                                                                        (epsilon prediction, s_churn = 0)
+ * model_input_next = [x'; x'] / next_scale                               pipeline :1565-1570 + scale_model_input,
+ *                                                                        scheduling_euler_discrete.py:274-298
+ * in one pass over the latents, fp32 arithmetic in that order.  noise_pred [2,n] bf16; latents / latents_out [n]
+ * bf16 (the reference casts prev_sample to the model dtype, :530) or fp32 when latents_f32 != 0; model_input_next
+ * [2,n] bf16 or NULL.  coef: DEVICE pointer to {sigma, sigma_next, next_scale = sqrt(sigma_next^2 + 1)} so that a
+ * captured graph can be replayed for every step with the three floats rewritten between replays.  n % 8 == 0. */
+int kh_cfg_euler_step_bf16(const void* noise_pred, const void* latents, void* latents_out, void* model_input_next,
+                           int64_t n, float guidance_scale, const float* coef, int latents_f32, void* stream);
 
 #ifdef __cplusplus
 }

@@ -11,6 +11,9 @@
 // * kh_concat_residual_bf16: out[..., :C1] = h, out[..., C1:] = skip + (sum_k r_k) * inv_k over
 //   channels-last rows: the up-block torch.cat([hidden, skip], dim=1) is a copy anyway, so the
 //   residual add rides on it for free.
+// * kh_cfg_euler_step_bf16: classifier-free guidance + one Euler step + the next step's input scaling in one
+//   pass (diffusers-hf/src/diffusers/pipelines/controlnet/pipeline_controlnet_sd_xl_katz.py:1565-1570,
+//   :1647-1658; diffusers-hf/src/diffusers/schedulers/scheduling_euler_discrete.py:274-298, :435-545).
 #include "kh_common.h"
 
 namespace {
@@ -150,6 +153,81 @@ int fill_srcs(SrcList& s, const void* const* srcs, int n_srcs, float inv) {
 }
 
 }  // namespace
+
+namespace {
+
+// One thread: 8 latent elements.  Arithmetic in fp32 in the reference's order (epsilon prediction, no churn):
+//   eps = u + g*(t - u); x0 = x - sigma*eps; d = (x - x0)/sigma; x' = x + d*(sigma_next - sigma).
+template <bool LAT_F32>
+__global__ __launch_bounds__(EW_THREADS) void cfg_euler_kernel(const bf16_t* __restrict__ noise, const void* __restrict__ lat_in,
+                                                               void* __restrict__ lat_out, bf16_t* __restrict__ next_in,
+                                                               long n, float g, const float* __restrict__ coef) {
+  const float sigma = coef[0], dt = coef[1] - coef[0], den = coef[2];
+  const long chunks = n / 8;
+  for (long i = (long)blockIdx.x * EW_THREADS + threadIdx.x; i < chunks; i += (long)gridDim.x * EW_THREADS) {
+    const u32x4 uv = *reinterpret_cast<const u32x4*>(noise + i * 8);
+    const u32x4 tv = *reinterpret_cast<const u32x4*>(noise + n + i * 8);
+    float x[8];
+    if (LAT_F32) {
+      const float* p = reinterpret_cast<const float*>(lat_in) + i * 8;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) x[e] = p[e];
+    } else {
+      const u32x4 xv = *reinterpret_cast<const u32x4*>(reinterpret_cast<const bf16_t*>(lat_in) + i * 8);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { x[2 * e] = bf16_lo(xv[e]); x[2 * e + 1] = bf16_hi(xv[e]); }
+    }
+    float y[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float u = (e & 1) ? bf16_hi(uv[e >> 1]) : bf16_lo(uv[e >> 1]);
+      const float t = (e & 1) ? bf16_hi(tv[e >> 1]) : bf16_lo(tv[e >> 1]);
+      const float eps = __fadd_rn(u, __fmul_rn(g, __fsub_rn(t, u)));
+      const float x0 = __fsub_rn(x[e], __fmul_rn(sigma, eps));
+      const float d = __fdiv_rn(__fsub_rn(x[e], x0), sigma);
+      y[e] = __fadd_rn(x[e], __fmul_rn(d, dt));
+    }
+    u32x4 yo;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) yo[e] = pack_bf16x2(y[2 * e], y[2 * e + 1]);
+    if (LAT_F32) {
+      float* p = reinterpret_cast<float*>(lat_out) + i * 8;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) p[e] = y[e];
+    } else {
+      *reinterpret_cast<u32x4*>(reinterpret_cast<bf16_t*>(lat_out) + i * 8) = yo;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { y[2 * e] = bf16_lo(yo[e]); y[2 * e + 1] = bf16_hi(yo[e]); }  // the stored, rounded latents
+    }
+    if (next_in != nullptr) {
+      u32x4 o;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = pack_bf16x2(__fdiv_rn(y[2 * e], den), __fdiv_rn(y[2 * e + 1], den));
+      *reinterpret_cast<u32x4*>(next_in + i * 8) = o;
+      *reinterpret_cast<u32x4*>(next_in + n + i * 8) = o;
+    }
+  }
+}
+
+}  // namespace
+
+KH_EXPORT int kh_cfg_euler_step_bf16(const void* noise_pred, const void* latents, void* latents_out, void* model_input_next,
+                                     int64_t n, float guidance_scale, const float* coef, int latents_f32, void* stream) {
+  if (!noise_pred || !latents || !latents_out || !coef || n <= 0) return KH_ERR_INVALID_ARG;
+  if (n % 8 != 0) return KH_ERR_UNSUPPORTED;
+  if (!kh_aligned16(noise_pred) || !kh_aligned16(latents) || !kh_aligned16(latents_out) ||
+      (model_input_next && !kh_aligned16(model_input_next)) || (n * 2) % 16 != 0)
+    return KH_ERR_ALIGNMENT;
+  const long chunks = n / 8;
+  const unsigned grid = (unsigned)((chunks + EW_THREADS - 1) / EW_THREADS < 4096 ? (chunks + EW_THREADS - 1) / EW_THREADS : 4096);
+  if (latents_f32)
+    kh_launch(KH_TAG_CFG_EULER, cfg_euler_kernel<true>, dim3(grid), dim3(EW_THREADS), 0, (hipStream_t)stream,
+              (const bf16_t*)noise_pred, latents, latents_out, (bf16_t*)model_input_next, (long)n, guidance_scale, coef);
+  else
+    kh_launch(KH_TAG_CFG_EULER, cfg_euler_kernel<false>, dim3(grid), dim3(EW_THREADS), 0, (hipStream_t)stream,
+              (const bf16_t*)noise_pred, latents, latents_out, (bf16_t*)model_input_next, (long)n, guidance_scale, coef);
+  KH_RETURN_LAST_ERROR();
+}
 
 KH_EXPORT int kh_geglu_bf16(const void* proj, void* out, int64_t M, int64_t D, int approximate_tanh, void* stream) {
   if (!proj || !out || M <= 0 || D <= 0) return KH_ERR_INVALID_ARG;

@@ -397,10 +397,37 @@ def conv3x3(x: torch.Tensor, w_packed: torch.Tensor, bias: Optional[torch.Tensor
     return out
 
 
+def cfg_euler_step(noise_pred: torch.Tensor, latents: torch.Tensor, coef: torch.Tensor, guidance_scale: float,
+                   latents_out: Optional[torch.Tensor] = None, model_input_next: Optional[torch.Tensor] = None):
+    """Guidance + Euler step (+ the next step's scaled, duplicated model input) in one kernel.
+    noise_pred [2B,...] bf16 (uncond rows first), latents [B,...] bf16 or fp32, coef: fp32 GPU tensor
+    {sigma, sigma_next, sqrt(sigma_next^2+1)}.  Returns latents_out (allocated unless given)."""
+    lib = _lib.load()
+    _req(noise_pred, BF16, "noise_pred")
+    if latents.dtype not in (BF16, torch.float32) or not latents.is_cuda or not latents.is_contiguous():
+        raise ValueError("latents must be a contiguous bfloat16 or float32 GPU tensor")
+    if not noise_pred.is_contiguous() or noise_pred.numel() != 2 * latents.numel():
+        raise ValueError("noise_pred must be contiguous with twice the elements of latents")
+    if coef.dtype != torch.float32 or not coef.is_cuda or coef.numel() < 3:
+        raise ValueError("coef must be a float32 GPU tensor of at least 3 elements")
+    if latents_out is None:
+        latents_out = torch.empty_like(latents)
+    if latents_out.dtype != latents.dtype or latents_out.shape != latents.shape or not latents_out.is_contiguous():
+        raise ValueError("latents_out must match latents")
+    if model_input_next is not None and (model_input_next.dtype != BF16 or not model_input_next.is_contiguous()
+                                         or model_input_next.numel() != noise_pred.numel()):
+        raise ValueError("model_input_next must be a contiguous bfloat16 tensor of noise_pred's size")
+    rc = lib.kh_cfg_euler_step_bf16(_ptr(noise_pred), _ptr(latents), _ptr(latents_out), _ptr(model_input_next),
+                                    latents.numel(), float(guidance_scale), _ptr(coef),
+                                    1 if latents.dtype == torch.float32 else 0, _stream())
+    _lib.check(rc, "kh_cfg_euler_step_bf16")
+    return latents_out
+
+
 # --------------------------------------------------------------------------------------- per-launch timing
 KERNEL_TAGS = {1: "lora_gemm", 2: "lora_gemm_f32", 3: "attention", 4: "group_norm_stats", 5: "group_norm_apply",
                6: "layer_norm", 7: "geglu", 8: "residual_add", 9: "concat_residual", 10: "sgmv_shrink",
-               11: "sgmv_expand", 12: "lora_shrink", 13: "conv3x3"}
+               11: "sgmv_expand", 12: "lora_shrink", 13: "conv3x3", 14: "cfg_euler"}
 
 
 def profile_begin() -> None:

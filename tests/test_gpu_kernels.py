@@ -530,3 +530,82 @@ def test_conv3x3_nhwc_bf16(shape):
     torch.cuda.synchronize()
     assert y.shape == ref.shape and y.is_contiguous(memory_format=torch.channels_last)
     assert_close_rel(y, ref, REL_BF16, f"conv3x3 {shape}")
+
+
+@pytest.mark.parametrize("lat_f32", [False, True])
+def test_cfg_euler_step_kernel(lat_f32):
+    """Fused guidance + Euler step against (a) the same formula in fp32 on the bf16-rounded inputs (tight) and
+    (b) the oracle's torch-semantics step on bf16 tensors (bf16 tolerance)."""
+    from katz_amd import ops
+    from oracle.euler import EulerDiscreteScheduler as OSched, classifier_free_guidance
+
+    say("cfg_euler", lat_f32)
+    d = dev()
+    g = torch.Generator().manual_seed(3)
+    sch = OSched(beta_start=0.00085, beta_end=0.012, beta_schedule="scaled_linear", timestep_spacing="leading", steps_offset=1)
+    sch.set_timesteps(50)
+    i = 7
+    sigma, sigma_next = sch.sigmas[i], sch.sigmas[i + 1]
+    noise = randn(g, 2, 4, 32, 32).to(BF)
+    lat = (randn(g, 1, 4, 32, 32) * sigma).to(torch.float32 if lat_f32 else BF)
+    gs = 7.5
+    # (a) fp32 restatement
+    u, t = noise[:1].float(), noise[1:].float()
+    eps = u + gs * (t - u)
+    x = lat.float()
+    x0 = x - sigma * eps
+    prev = x + ((x - x0) / sigma) * (sigma_next - sigma)
+    den = (sigma_next ** 2 + 1) ** 0.5
+    coef = torch.tensor([sigma.item(), sigma_next.item(), den.item()], dtype=torch.float32, device=d)
+    nxt = torch.empty(2, 4, 32, 32, dtype=BF, device=d)
+    out = ops.cfg_euler_step(noise.to(d), lat.to(d), coef, gs, model_input_next=nxt)
+    torch.cuda.synchronize()
+    assert out.dtype == lat.dtype
+    ref = prev if lat_f32 else prev.to(BF)
+    err = (out.float().cpu() - ref.float()).abs().max().item()
+    # fp32 latents: rounding-order noise only; bf16 latents: at most one bf16 ulp where that noise crosses a tie
+    assert err <= (1e-5 if lat_f32 else 2.0 ** -8) * max(1.0, prev.abs().max().item()), err
+    if not lat_f32:
+        assert (out.cpu() != ref).float().mean().item() < 1e-2
+    ref_next = (ref.float() / den).to(BF)
+    assert torch.equal(nxt[0].cpu(), ref_next[0]) or (nxt[0].float().cpu() - ref_next[0].float()).abs().max() <= 2 ** -7 * ref_next.abs().max()
+    assert torch.equal(nxt[0], nxt[1])
+    # (b) the reference's op sequence on bf16 tensors (rounds eps and sigma*eps to bf16 on the way)
+    sch.step_index = i
+    o2 = sch.step(classifier_free_guidance(noise, gs), sch.timesteps[i], lat.to(BF))
+    assert_close_rel(out, o2.reshape(out.shape), REL_BF16, "cfg+euler vs oracle op sequence")
+
+
+@pytest.mark.parametrize("lat_f32", [True, False])
+def test_denoise_loop_matches_oracle_loop(lat_f32):
+    """50 guided Euler steps around a cheap elementwise 'model' with bf16 input / output (what the UNet is to the
+    loop): the product loop (fused kernel) against the oracle's loop.  With fp32 latents the two differ by
+    rounding order only; with the reference's model-dtype (bf16) latents every step re-rounds the state, so 50
+    steps of independent bf16 roundings bound the agreement (cosine, and 10 % of |ref| + rms elementwise)."""
+    from katz_amd.scheduler import EulerDiscreteScheduler, denoise_loop
+    from oracle.euler import EulerDiscreteScheduler as OSched, denoise_loop as oracle_loop
+
+    say("denoise loop", lat_f32)
+    d = dev()
+    cfg = dict(beta_start=0.00085, beta_end=0.012, beta_schedule="scaled_linear", timestep_spacing="leading", steps_offset=1)
+    ps, os_ = EulerDiscreteScheduler(**cfg), OSched(**cfg)
+    ps.set_timesteps(50, device=d)
+    os_.set_timesteps(50)
+    assert torch.equal(ps.timesteps.cpu(), os_.timesteps) and torch.equal(ps.sigmas, os_.sigmas)
+    assert ps.init_noise_sigma.item() == os_.init_noise_sigma.item()
+    g = torch.Generator().manual_seed(5)
+    lat0 = (randn(g, 1, 4, 16, 16) * os_.init_noise_sigma).to(BF)
+
+    def model(x, t):  # rows: uncond, text; a smooth, contracting elementwise map of the bf16-rounded input
+        x = x.to(BF).float()
+        scale = torch.tensor([[[[0.8]]], [[[1.1]]]], dtype=torch.float32, device=x.device)
+        y = x / (1.0 + x.abs()) * scale * (1.0 - t.float() / 2000.0)
+        return y.to(BF)
+
+    got = denoise_loop(model, ps, lat0.to(d), 7.5, latents_fp32=lat_f32)
+    ref = oracle_loop(lambda x, t: model(x, t).to(x.dtype), os_, lat0.float() if lat_f32 else lat0, 7.5)
+    torch.cuda.synchronize()
+    assert got.dtype == (torch.float32 if lat_f32 else BF)
+    cos = torch.nn.functional.cosine_similarity(got.float().cpu().flatten(), ref.float().flatten(), dim=0).item()
+    assert cos >= 0.999, cos
+    assert_close_rel(got, ref, 1e-2 if lat_f32 else 1e-1, "50-step loop")

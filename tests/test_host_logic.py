@@ -112,3 +112,29 @@ def test_upstream_state_dict_names_are_remapped():
     unet.load_state_dict(up, strict=True)
     for k, v in unet.state_dict().items():
         assert torch.equal(v, sd[k]), k
+
+
+def test_euler_schedule_matches_oracle():
+    """The product's host-side schedule (numpy) equals the oracle's (torch, KAT-pinned) bit for bit."""
+    import torch
+    from katz_amd.scheduler import EulerDiscreteScheduler
+    from oracle.euler import EulerDiscreteScheduler as OSched
+
+    for cfg, steps in ((dict(beta_start=0.00085, beta_end=0.012, beta_schedule="scaled_linear", timestep_spacing="leading", steps_offset=1), 50),
+                       (dict(num_train_timesteps=1100, beta_start=0.0001, beta_end=0.02, beta_schedule="linear"), 10),
+                       (dict(beta_schedule="scaled_linear", timestep_spacing="trailing"), 30)):
+        p, o = EulerDiscreteScheduler(**cfg), OSched(**cfg)
+        assert torch.equal(p.sigmas, o.sigmas)
+        assert p.init_noise_sigma.item() == o.init_noise_sigma.item()
+        p.set_timesteps(steps)
+        o.set_timesteps(steps)
+        assert torch.equal(p.timesteps, o.timesteps)
+        assert torch.allclose(p.sigmas, o.sigmas, rtol=1e-6, atol=0)
+        t = p.coef_table("cpu")
+        assert t.shape == (steps, 4) and torch.equal(t[:, 0], p.sigmas[:-1]) and torch.equal(t[:, 1], p.sigmas[1:])
+        # unfused step == oracle step on fp32 tensors
+        g = torch.Generator().manual_seed(0)
+        x, eps = torch.randn(1, 4, 8, 8, generator=g), torch.randn(1, 4, 8, 8, generator=g)
+        tt = p.timesteps[0]
+        assert torch.equal(p.scale_model_input(x, tt), o.scale_model_input(x, tt))
+        assert torch.allclose(p.step(eps, tt, x)[0], o.step(eps, tt, x), rtol=1e-6, atol=1e-6)
