@@ -104,3 +104,61 @@ def rescale_(packed: PackedAdapters, adapters: Dict[str, Adapter], global_scale:
     """Rewrite col_scale only (scale_lora_layers / set_adapters weight change); A_cat/B_cat stay put."""
     for n, c, r in packed.spans:
         packed.col_scale[c:c + r] = adapters[n].multiplier(global_scale)
+
+
+# ---- per-block adapter scales -------------------------------------------------------------------------------------
+def _translate_into_actual_layer_name(name: str) -> str:
+    """'mid' -> 'mid_block.attentions.0'; 'down.block_1.0' -> 'down_blocks.1.attentions.0'
+    (diffusers-hf/src/diffusers/loaders/unet_loader_utils.py:28-38)."""
+    if name == "mid":
+        return "mid_block.attentions.0"
+    updown, block, attn = name.split(".")
+    updown = updown.replace("down", "down_blocks").replace("up", "up_blocks")
+    return ".".join((updown, block.replace("block_", ""), "attentions." + attn))
+
+
+def expand_lora_scales_for_one_adapter(scales, blocks_with_transformer: Dict[str, List[int]],
+                                       transformer_per_block: Dict[str, int], module_names: Optional[Sequence[str]] = None):
+    """A float stays a float; a dict like {"down": 2, "mid": 3, "up": {"block_0": 4, "block_1": [5, 6, 7]}} becomes
+    {actual layer name: scale} for every transformer of the UNet, missing parts defaulting to 1
+    (_maybe_expand_lora_scales_for_one_adapter, unet_loader_utils.py:61-141).  module_names: when given, every
+    expanded layer must be a substring of at least one of them (the reference checks the state-dict keys)."""
+    import copy
+    if sorted(blocks_with_transformer.keys()) != ["down", "up"]:
+        raise ValueError("blocks_with_transformer needs to be a dict with keys `'down' and `'up'`")
+    if sorted(transformer_per_block.keys()) != ["down", "up"]:
+        raise ValueError("transformer_per_block needs to be a dict with keys `'down' and `'up'`")
+    if not isinstance(scales, dict):
+        return scales
+    scales = copy.deepcopy(scales)
+    scales.setdefault("mid", 1)
+    for updown in ("up", "down"):
+        scales.setdefault(updown, 1)
+        if not isinstance(scales[updown], dict):
+            scales[updown] = {f"block_{i}": scales[updown] for i in blocks_with_transformer[updown]}
+        for i in blocks_with_transformer[updown]:
+            block = f"block_{i}"
+            if not isinstance(scales[updown][block], list):
+                scales[updown][block] = [scales[updown][block]] * transformer_per_block[updown]
+        for i in blocks_with_transformer[updown]:
+            block = f"block_{i}"
+            for tf_idx, value in enumerate(scales[updown][block]):
+                scales[f"{updown}.{block}.{tf_idx}"] = value
+        del scales[updown]
+    out = {_translate_into_actual_layer_name(k): v for k, v in scales.items()}
+    if module_names is not None:
+        for user, layer in zip(scales.keys(), out.keys()):
+            if not any(layer in m for m in module_names):
+                raise ValueError(f"Can't set lora scale for layer {user}. It either doesn't exist in this unet or it has no attentions.")
+    return out
+
+
+def module_weight(weight_for_adapter, module_name: str) -> float:
+    """The scale of one module: the float itself, or the first expanded layer name contained in the module's name
+    (get_module_weight, diffusers-hf/src/diffusers/utils/peft_utils.py:241-249)."""
+    if not isinstance(weight_for_adapter, dict):
+        return float(weight_for_adapter)
+    for layer_name, w in weight_for_adapter.items():
+        if layer_name in module_name:
+            return float(w)
+    raise RuntimeError(f"No LoRA weight found for module {module_name}.")

@@ -26,6 +26,7 @@ import torch.nn.functional as F
 
 from . import ops
 from .layers import LoRALinear, TimestepEmbedding, fused_norm_silu
+from .lora import expand_lora_scales_for_one_adapter, module_weight
 from .unet_blocks import (CrossAttnDownBlock2D, CrossAttnUpBlock2D, DownBlock2D, UNetMidBlock2DCrossAttn, UpBlock2D)
 
 
@@ -253,12 +254,21 @@ class UNet2DConditionModel(nn.Module):
         names = [adapter_names] if isinstance(adapter_names, str) else list(adapter_names)
         if weights is None:
             weights = [1.0] * len(names)
-        elif isinstance(weights, (int, float)):
-            weights = [float(weights)] * len(names)
+        elif isinstance(weights, (int, float, dict)):
+            weights = [weights] * len(names)
         if len(weights) != len(names):
             raise ValueError(f"Length of adapter names {len(names)} is not equal to the length of their weights {len(weights)}.")
-        for m in self.lora_linears().values():
-            m.set_active(names, weights)
+        weights = [1.0 if w is None else w for w in weights]
+        lin = self.lora_linears()
+        if any(isinstance(w, dict) for w in weights):
+            # per-block scales, e.g. {"down": 0.9, "mid": 1.0, "up": {"block_0": 0.6, "block_1": [0.4, 0.8, 1.0]}}
+            # (_maybe_expand_lora_scales, diffusers-hf/src/diffusers/loaders/unet_loader_utils.py:41-58)
+            bwt = {"down": [i for i, b in enumerate(self.down_blocks) if hasattr(b, "attentions")],
+                   "up": [i for i, b in enumerate(self.up_blocks) if hasattr(b, "attentions")]}
+            tpb = {"down": self.cfg.layers_per_block, "up": self.cfg.layers_per_block + 1}
+            weights = [expand_lora_scales_for_one_adapter(w, bwt, tpb, list(lin.keys())) for w in weights]
+        for mod_name, m in lin.items():
+            m.set_active(names, [module_weight(w, mod_name) for w in weights])
 
     def disable_lora(self) -> None:
         for m in self.lora_linears().values():

@@ -138,3 +138,40 @@ def test_euler_schedule_matches_oracle():
         tt = p.timesteps[0]
         assert torch.equal(p.scale_model_input(x, tt), o.scale_model_input(x, tt))
         assert torch.allclose(p.step(eps, tt, x)[0], o.step(eps, tt, x), rtol=1e-6, atol=1e-6)
+
+
+def test_expand_lora_scales_docstring_example_and_set_adapters():
+    """The worked example in the reference's docstring (unet_loader_utils.py:77-100) is the golden vector."""
+    import pytest
+    from katz_amd.lora import expand_lora_scales_for_one_adapter as expand, module_weight
+    import katz_amd.layers as L
+    from katz_amd.unet_2d_condition import UNet2DConditionModel, UNetConfig
+
+    got = expand({"down": 2, "mid": 3, "up": {"block_0": 4, "block_1": [5, 6, 7]}},
+                 {"down": [1, 2], "up": [0, 1]}, {"down": 2, "up": 3})
+    want = {"down.block_1.0": 2, "down.block_1.1": 2, "down.block_2.0": 2, "down.block_2.1": 2, "mid": 3,
+            "up.block_0.0": 4, "up.block_0.1": 4, "up.block_0.2": 4, "up.block_1.0": 5, "up.block_1.1": 6, "up.block_1.2": 7}
+    tr = lambda n: "mid_block.attentions.0" if n == "mid" else "{}_blocks.{}.attentions.{}".format(*[p.replace("block_", "") for p in n.split(".")])
+    assert got == {tr(k): v for k, v in want.items()}
+    assert expand(0.7, {"down": [1], "up": [0]}, {"down": 2, "up": 3}) == 0.7
+    assert module_weight(got, "up_blocks.1.attentions.2.transformer_blocks.0.attn1.to_q") == 7.0
+    with pytest.raises(RuntimeError):
+        module_weight(got, "down_blocks.0.resnets.0.conv1")
+    with pytest.raises(ValueError):
+        expand({"down": 1.0}, {"down": [1, 2], "up": [0, 1]}, {"down": 2, "up": 3}, ["down_blocks.1.attentions.0.x"])
+
+    L.SKIP_INIT = True
+    try:
+        unet = UNet2DConditionModel(UNetConfig.tiny())
+    finally:
+        L.SKIP_INIT = False
+    import torch
+    for name, m in unet.lora_linears().items():
+        m.add_adapter("a", torch.zeros(4, m.in_features), torch.zeros(m.out_features, 4), None)
+    unet.set_adapters(["a"], [{"down": 0.5, "mid": 0.25, "up": {"block_0": [0.1, 0.2, 0.3], "block_1": 1.0}}])
+    lin = unet.lora_linears()
+    w = lambda n: lin[n].adapters["a"].weight
+    assert w("down_blocks.1.attentions.1.transformer_blocks.0.attn1.to_q") == 0.5
+    assert w("mid_block.attentions.0.proj_in") == 0.25
+    assert w("up_blocks.0.attentions.2.transformer_blocks.0.ff.net.2") == 0.3
+    assert w("up_blocks.1.attentions.0.transformer_blocks.0.attn2.to_k") == 1.0
