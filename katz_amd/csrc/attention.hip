@@ -6,7 +6,7 @@
 // row / batch strides, so the [B,h,T,64] transposes of the reference (:1269-1272, :1280) are never
 // materialised.
 //
-// One workgroup = 4 waves = 128 queries of one (batch, head); each wave owns 32 queries.
+// One workgroup = 4 (or 2) waves = 128 (64) queries of one (batch, head); each wave owns 32 queries.
 // Per 64-key tile (K and V^T staged in LDS, double buffered):
 //   S^T = K . Q^T      (A = K fragment from LDS, B = Q fragment held in registers)
 //   so every lane holds 32 scores of ONE query (query = lane%32): the row max / row sum are
@@ -14,6 +14,7 @@
 //   O^T += V^T . P^T   (A = V^T fragment from LDS, B = P straight from the score registers:
 //   the MFMA K index is a free permutation as long as both operands agree on it.)
 #include "kh_common.h"
+#include <type_traits>
 
 namespace {
 
@@ -22,6 +23,7 @@ constexpr int KV = 64;        // keys per tile
 constexpr int LDH = HD + 8;   // padded LDS rows (144 B)
 constexpr int LDV = KV + 8;
 constexpr float NEG_BIG = -1.0e30f;
+constexpr float RESCALE_LOG2 = 8.0f;   // the running maximum moves only for jumps above 2^8
 
 struct AttnParams {
   const bf16_t* q; const bf16_t* k; const bf16_t* v; bf16_t* o;
@@ -32,7 +34,11 @@ struct AttnParams {
   int q_blocks;
 };
 
-__global__ __launch_bounds__(256) void attention_kernel(const AttnParams p) {
+template <int NW>   // waves per workgroup: NW*32 queries
+// Two waves per SIMD at least: that caps a wave at 256 registers, which makes the compiler keep MFMA results in
+// VGPRs (the softmax reads them every tile; from AGPRs every score and every rescaled output costs extra moves).
+__global__ __launch_bounds__(NW * 64, 8 / NW) void attention_kernel(const AttnParams p) {
+  constexpr int NT = NW * 64, KCH = 512 / NT, VCH = 256 / NT;
   __shared__ __attribute__((aligned(16))) bf16_t sK[2][KV * LDH];
   __shared__ __attribute__((aligned(16))) bf16_t sVt[2][HD * LDV];
 
@@ -50,7 +56,7 @@ __global__ __launch_bounds__(256) void attention_kernel(const AttnParams p) {
   bf16_t* op = p.o + (size_t)b * p.bso + (size_t)h * HD;
 
   // Q fragments: query = q0 + l32, d = ks*16 + lh*8 .. +7
-  const int qrow = qb * 128 + wave * 32 + l32;
+  const int qrow = qb * (NW * 32) + wave * 32 + l32;
   const int qrow_c = qrow < p.T ? qrow : p.T - 1;
   bf16x8 qf[4];
 #pragma unroll
@@ -67,37 +73,44 @@ __global__ __launch_bounds__(256) void attention_kernel(const AttnParams p) {
   const int n_tiles = (p.S + KV - 1) / KV;
 
   // staging registers: K tile = 64 keys x 8 chunks (2 per thread); V tile = 32 key pairs x 8 chunks (1 pair per thread)
-  u32x4 rk[2], rv[2];
-  const int v_kp = tid & 31, v_dch = tid >> 5;
+  u32x4 rk[KCH], rv[VCH][2];
   auto load_tile = [&](int t) {
     const int s0 = t * KV;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int c = tid + i * 256, row = c >> 3, ch = c & 7;
+    for (int i = 0; i < KCH; ++i) {
+      const int c = tid + i * NT, row = c >> 3, ch = c & 7;
       int gr = s0 + row; gr = gr < p.S ? gr : p.S - 1;
       rk[i] = *reinterpret_cast<const u32x4*>(kp + (size_t)gr * p.ldk + ch * 8);
     }
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      int gr = s0 + 2 * v_kp + i; gr = gr < p.S ? gr : p.S - 1;
-      rv[i] = *reinterpret_cast<const u32x4*>(vp + (size_t)gr * p.ldv + v_dch * 8);
+    for (int j = 0; j < VCH; ++j) {
+      const int c = tid + j * NT, v_kp = c & 31, v_dch = c >> 5;
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        int gr = s0 + 2 * v_kp + i; gr = gr < p.S ? gr : p.S - 1;
+        rv[j][i] = *reinterpret_cast<const u32x4*>(vp + (size_t)gr * p.ldv + v_dch * 8);
+      }
     }
   };
   auto store_tile = [&](int buf) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int c = tid + i * 256, row = c >> 3, ch = c & 7;
+    for (int i = 0; i < KCH; ++i) {
+      const int c = tid + i * NT, row = c >> 3, ch = c & 7;
       *reinterpret_cast<u32x4*>(&sK[buf][row * LDH + ch * 8]) = rk[i];
     }
     // transpose: element e of the pair (key 2kp, key 2kp+1) -> sVt[d = dch*8+e][2kp .. 2kp+1] as one dword
     uint32_t* dst = reinterpret_cast<uint32_t*>(&sVt[buf][0]);
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
-      const uint32_t a = rv[0][w], c2 = rv[1][w];
-      const uint32_t lo = (a & 0xffffu) | (c2 << 16);          // d = dch*8 + 2w
-      const uint32_t hi = (a >> 16) | (c2 & 0xffff0000u);      // d = dch*8 + 2w + 1
-      dst[((v_dch * 8 + 2 * w) * LDV) / 2 + v_kp] = lo;
-      dst[((v_dch * 8 + 2 * w + 1) * LDV) / 2 + v_kp] = hi;
+    for (int j = 0; j < VCH; ++j) {
+      const int c = tid + j * NT, v_kp = c & 31, v_dch = c >> 5;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const uint32_t a = rv[j][0][w], c2 = rv[j][1][w];
+        const uint32_t lo = (a & 0xffffu) | (c2 << 16);          // d = dch*8 + 2w
+        const uint32_t hi = (a >> 16) | (c2 & 0xffff0000u);      // d = dch*8 + 2w + 1
+        dst[((v_dch * 8 + 2 * w) * LDV) / 2 + v_kp] = lo;
+        dst[((v_dch * 8 + 2 * w + 1) * LDV) / 2 + v_kp] = hi;
+      }
     }
   };
 
@@ -105,25 +118,25 @@ __global__ __launch_bounds__(256) void attention_kernel(const AttnParams p) {
   store_tile(0);
   __syncthreads();
 
-  for (int t = 0; t < n_tiles; ++t) {
+  // One 64-key tile.  MASK: the tile may reach beyond S (only the last one can).
+  auto tile_step = [&](int t, auto mask_tag) {
+    constexpr bool MASK = decltype(mask_tag)::value;
     const int buf = t & 1;
     if (t + 1 < n_tiles) load_tile(t + 1);
 
     // S^T tiles: st[kt][v] : key = t*64 + kt*32 + 8*(v/4) + 4*lh + v%4, query = l32
     f32x16 st[2];
+    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) st[kt][v] = 0.f;
-#pragma unroll
       for (int ks = 0; ks < 4; ++ks) {
         const bf16x8 kf = *reinterpret_cast<const bf16x8*>(&sK[buf][(kt * 32 + l32) * LDH + ks * 16 + lh * 8]);
-        st[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], st[kt], 0, 0, 0);
+        st[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], ks == 0 ? zero : st[kt], 0, 0, 0);
       }
     }
-    // mask keys beyond S (last tile only)
-    const int s0 = t * KV;
-    if (s0 + KV > p.S) {
+    if constexpr (MASK) {
+      const int s0 = t * KV;
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
@@ -138,26 +151,35 @@ __global__ __launch_bounds__(256) void attention_kernel(const AttnParams p) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) mx = fmaxf(mx, st[kt][v]);
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float m_new = fmaxf(m_run, mx);
-    const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * p.scale_log2e);
-    m_run = m_new;
-    const float mb = m_new * p.scale_log2e;
+    // Lazy running maximum: the reference point of the exponentials only moves when the row maximum has grown by
+    // more than 2^RESCALE_LOG2 in the exponent domain; until then p = exp2(s - m) may exceed 1 (by at most that
+    // factor, harmless in fp32 / bf16) and numerator and denominator stay consistent.  Moving it rescales
+    // the 32 output accumulators, which is then rare -- and skipped for the whole wave when no lane moves.
+    const bool move = (mx - m_run) * p.scale_log2e > RESCALE_LOG2;
+    if (__builtin_amdgcn_ballot_w64(move) != 0) {
+      const float m_new = move ? mx : m_run;
+      const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * p.scale_log2e);
+      m_run = m_new;
+      l_run *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) oacc[dt][v] *= alpha;
+    }
+    const float mb = m_run * p.scale_log2e;
     float rs = 0.f;
     bf16x8 pf[2][2];
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const float e = __builtin_amdgcn_exp2f(st[kt][v] * p.scale_log2e - mb);
-        const bf16_t eb = (bf16_t)e;
-        rs += (float)eb;  // the denominator sums the rounded probabilities the numerator uses
-        pf[kt][v >> 3][v & 7] = eb;
+      for (int v = 0; v < 16; v += 2) {
+        const float e0 = __builtin_amdgcn_exp2f(st[kt][v] * p.scale_log2e - mb);
+        const float e1 = __builtin_amdgcn_exp2f(st[kt][v + 1] * p.scale_log2e - mb);
+        rs += e0 + e1;
+        pf[kt][v >> 3][v & 7] = (bf16_t)e0;
+        pf[kt][v >> 3][(v & 7) + 1] = (bf16_t)e1;
       }
-    l_run = l_run * alpha + rs;
-#pragma unroll
-    for (int dt = 0; dt < 2; ++dt)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) oacc[dt][v] *= alpha;
+    l_run += rs;
 
     // O^T += V^T . P^T : A fragment row d = dt*32 + l32, element e <-> key kt*32 + 8*(2s + e/4) + 4*lh + e%4
 #pragma unroll
@@ -177,7 +199,10 @@ __global__ __launch_bounds__(256) void attention_kernel(const AttnParams p) {
 
     if (t + 1 < n_tiles) store_tile(buf ^ 1);
     __syncthreads();
-  }
+  };
+  const int full_tiles = p.S / KV;
+  for (int t = 0; t < full_tiles; ++t) tile_step(t, std::false_type{});
+  if (full_tiles < n_tiles) tile_step(full_tiles, std::true_type{});
 
   const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
   const float inv = 1.0f / l_tot;
@@ -210,9 +235,15 @@ KH_EXPORT int kh_attention_bf16(const void* q, const void* k, const void* v, voi
   p.ldq = ldq; p.ldk = ldk; p.ldv = ldv; p.ldo = ldo;
   p.bsq = bsq; p.bsk = bsk; p.bsv = bsv; p.bso = bso;
   p.scale_log2e = scale * 1.4426950408889634f;
-  p.q_blocks = (int)((T + 127) / 128);
+  // 128 queries per workgroup; 64 for short key sequences on small grids (cross-attention), for a finer spread
+  const bool small = ((T + 127) / 128) * H * B < 512 && S <= 256;
+  const int qpw = small ? 64 : 128;
+  p.q_blocks = (int)((T + qpw - 1) / qpw);
   const long grid = (long)p.q_blocks * H * B;
   if (grid > 0x7fffffffL) return KH_ERR_TOO_LARGE;
-  kh_launch(KH_TAG_ATTENTION, attention_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, p);
+  if (small)
+    kh_launch(KH_TAG_ATTENTION, attention_kernel<2>, dim3((unsigned)grid), dim3(128), 0, (hipStream_t)stream, p);
+  else
+    kh_launch(KH_TAG_ATTENTION, attention_kernel<4>, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, p);
   KH_RETURN_LAST_ERROR();
 }
