@@ -37,7 +37,7 @@ struct AttnParams {
 template <int NW>   // waves per workgroup: NW*32 queries
 // Two waves per SIMD at least: that caps a wave at 256 registers, which makes the compiler keep MFMA results in
 // VGPRs (the softmax reads them every tile; from AGPRs every score and every rescaled output costs extra moves).
-__global__ __launch_bounds__(NW * 64, 8 / NW) void attention_kernel(const AttnParams p) {
+__global__ __launch_bounds__(NW * 64, 2) void attention_kernel(const AttnParams p) {
   constexpr int NT = NW * 64, KCH = 512 / NT, VCH = 256 / NT;
   __shared__ __attribute__((aligned(16))) bf16_t sK[2][KV * LDH];
   __shared__ __attribute__((aligned(16))) bf16_t sVt[2][HD * LDV];
@@ -74,8 +74,34 @@ __global__ __launch_bounds__(NW * 64, 8 / NW) void attention_kernel(const AttnPa
 
   // staging registers: K tile = 64 keys x 8 chunks (2 per thread); V tile = 32 key pairs x 8 chunks (1 pair per thread)
   u32x4 rk[KCH], rv[VCH][2];
+  // A full tile is read at (uniform tile base) + (per-thread byte offset fixed for the whole kernel): no per-tile
+  // address arithmetic in the vector ALU, which is the unit this kernel is bound by.  Only a last, partial
+  // tile clamps its rows.
+  uint32_t koff[KCH], voff[VCH][2];
+#pragma unroll
+  for (int i = 0; i < KCH; ++i) {
+    const int c = tid + i * NT, row = c >> 3, ch = c & 7;
+    koff[i] = (uint32_t)((row * p.ldk + ch * 8) * 2);
+  }
+#pragma unroll
+  for (int j = 0; j < VCH; ++j) {
+    const int c = tid + j * NT, v_kp = c & 31, v_dch = c >> 5;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) voff[j][i] = (uint32_t)(((2 * v_kp + i) * p.ldv + v_dch * 8) * 2);
+  }
   auto load_tile = [&](int t) {
     const int s0 = t * KV;
+    if (s0 + KV <= p.S) {
+      const char* kb = reinterpret_cast<const char*>(kp + (size_t)s0 * p.ldk);
+      const char* vb = reinterpret_cast<const char*>(vp + (size_t)s0 * p.ldv);
+#pragma unroll
+      for (int i = 0; i < KCH; ++i) rk[i] = *reinterpret_cast<const u32x4*>(kb + koff[i]);
+#pragma unroll
+      for (int j = 0; j < VCH; ++j)
+#pragma unroll
+        for (int i = 0; i < 2; ++i) rv[j][i] = *reinterpret_cast<const u32x4*>(vb + voff[j][i]);
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < KCH; ++i) {
       const int c = tid + i * NT, row = c >> 3, ch = c & 7;
