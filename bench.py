@@ -156,12 +156,49 @@ def cpu_baseline(cores):
     return ts[1], flops
 
 
+# HBM-side bytes of the largest LoRA GEMM launch, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on
+# `bench.py --traffic-probe` and calibrated against a copy of known size (summary under profiles/)
+GEMM_TRAFFIC_BYTES = 164.7e6
+
+
+def traffic_probe():
+    """Counter calibration run: a device copy of known size (64 MiB read + 64 MiB written), then the largest
+    LoRA linear of the step (GEGLU projection, M 2048, K 1280, N 10240, packed rank 128) as shrink + GEMM,
+    three times.  Under `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` the copy gives the factor between
+    the counter and bytes; the GEMM rows give its HBM traffic per launch."""
+    import torch
+    from katz_amd import ops
+
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(0)
+    src = torch.randn(16 << 20, device=dev, generator=g)            # 64 MiB fp32
+    dst = torch.empty_like(src)
+    M, K, N, R = 2048, 1280, 10240, 128
+    x = torch.randn(M, K, device=dev, generator=g).to(torch.bfloat16)
+    w = (torch.randn(N, K, device=dev, generator=g) * 0.02).to(torch.bfloat16)
+    b = torch.randn(N, device=dev, generator=g).to(torch.bfloat16)
+    a_cat = (torch.randn(R, K, device=dev, generator=g) * 0.02).to(torch.bfloat16)
+    b_cat = (torch.randn(N, R, device=dev, generator=g) * 0.02).to(torch.bfloat16)
+    scale = torch.full((R,), 0.8, device=dev)
+    torch.cuda.synchronize()
+    for _ in range(3):
+        dst.copy_(src)
+        t = ops.lora_shrink(x, a_cat, scale)
+        ops.lora_linear_pre(x, w, b, t, b_cat, geglu=True)
+    torch.cuda.synchronize()
+    print(json.dumps({"traffic_probe": {"copy_bytes_read": src.numel() * 4, "copy_bytes_written": src.numel() * 4,
+                                        "gemm": {"M": M, "N": N, "K": K, "R": R, "geglu": True},
+                                        "algorithmic_bytes": 2 * (M * K + K * N + M * N // 2 + R * (K + N))}}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="run only a 64 MiB copy and the dominant LoRA GEMM shape a few times (for rocprofv3 --pmc)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU only (no collectives, no sharding); --gpus must be 1",
@@ -170,6 +207,10 @@ def main():
 
     import torch
     from katz_amd.graph import GraphedUNetStep
+
+    if args.traffic_probe:
+        traffic_probe()
+        return
 
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; the katz_hip kernels have no CPU path", file=sys.stderr)
@@ -256,7 +297,9 @@ def main():
         "output_finite": finite,
         "roofline": {"kernel": "lora_gemm_kernel (fused base GEMM + LoRA delta, all launches of one step)",
                      "bound": "mfma", "achieved": round(achieved_tf, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved_tf / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                     "frac": round(achieved_tf / PEAK_BF16_TFLOPS, 4), "traffic": GEMM_TRAFFIC_BYTES,
+                     "traffic_note": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of `bench.py --traffic-probe`, largest launch "
+                                     "(M 2048, K 1280, N 10240, R 128): 143.7 MB read + 21.0 MB written; algorithmic 55.4 MB",
                      "launches_per_step": len(gemm_ms), "shrink_launches_per_step": len(shrink_calls),
                      "shrink_ms_per_step": round(shrink_ms, 3), "avg_launch_us": round(gemm_total_ms / len(gemm_ms) * 1e3, 2),
                      "algorithmic_gflop_per_step": round(gemm_flops / 1e9, 1), "by_shape": shape_rows[:8],

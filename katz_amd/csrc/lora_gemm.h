@@ -19,6 +19,9 @@ struct LoraGemmParams {
   bf16_t* y;
   int M, N, K, R;
   int m_tiles, n_tiles, n_chunk, n_chunks;  // n_chunk = N tiles walked by one workgroup
+  // tile -> XCD map (xg_n > 0): the 8 XCDs form an xg_m x xg_n grid over the tile matrix, each owning a block of
+  // xr_m x xr_n tiles (see launch_pcfg); 0: contiguous ranges of the (m block, n chunk) list per XCD
+  int xg_n, xr_m, xr_n;
   int geglu;                                // 1: W rows are (value,gate) interleaved in 32-column groups, y is [M,N/2]
   // 3x3 convolution as an implicit GEMM (conv_cin > 0): x is an NHWC image [Nb, conv_h, conv_w, conv_cin], row m
   // of the GEMM is output pixel m of [Nb, conv_ho, conv_wo], K = 9 * conv_cin ordered (kh, kw, ci), padding 1

@@ -483,6 +483,7 @@ KH_EXPORT int kh_lora_linear_bf16(const void* x, const void* w, const void* bias
   p.M = (int)M; p.N = (int)N; p.K = (int)K; p.R = (int)R;
   p.m_tiles = p.n_tiles = p.n_chunk = p.n_chunks = 0;
   p.geglu = geglu ? 1 : 0;
+  p.xg_n = p.xr_m = p.xr_n = 0;
   p.conv_cin = p.conv_h = p.conv_w = p.conv_ho = p.conv_wo = p.conv_stride = 0;
   p.dbg = (flags >> 16) & 0xff;
   hipStream_t s = (hipStream_t)stream;
@@ -517,6 +518,7 @@ KH_EXPORT int kh_lora_linear_pre_bf16(const void* x, const void* w, const void* 
   p.M = (int)M; p.N = (int)N; p.K = (int)K; p.R = (int)R;
   p.m_tiles = p.n_tiles = p.n_chunk = p.n_chunks = 0;
   p.geglu = geglu ? 1 : 0;
+  p.xg_n = p.xr_m = p.xr_n = 0;
   p.conv_cin = p.conv_h = p.conv_w = p.conv_ho = p.conv_wo = p.conv_stride = 0;
   return lora_gemm_pipe_launch(p, (flags >> 8) & 0xff, (hipStream_t)stream);
 }
@@ -541,6 +543,7 @@ KH_EXPORT int kh_conv3x3_nhwc_bf16(const void* x, const void* w, const void* bia
   p.M = (int)M; p.N = (int)Cout; p.K = (int)(9 * Cin); p.R = 0;
   p.m_tiles = p.n_tiles = p.n_chunk = p.n_chunks = 0;
   p.geglu = 0;
+  p.xg_n = p.xr_m = p.xr_n = 0;
   p.conv_cin = (int)Cin; p.conv_h = (int)H; p.conv_w = (int)W; p.conv_ho = (int)Ho; p.conv_wo = (int)Wo;
   p.conv_stride = (int)stride;
   return lora_gemm_pipe_launch_conv(p, (hipStream_t)stream);
@@ -562,6 +565,7 @@ KH_EXPORT int kh_lora_linear_grouped_bf16(const void* x, const uint64_t* table, 
   p.M = (int)M; p.N = (int)N; p.K = (int)K; p.R = (int)R;
   p.m_tiles = p.n_tiles = p.n_chunk = p.n_chunks = 0;
   p.geglu = 0;
+  p.xg_n = p.xr_m = p.xr_n = 0;
   p.conv_cin = p.conv_h = p.conv_w = p.conv_ho = p.conv_wo = p.conv_stride = 0;
   return lora_gemm_pipe_launch_grouped(p, (int)n_groups, (hipStream_t)stream);
 }

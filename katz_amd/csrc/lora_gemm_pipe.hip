@@ -281,9 +281,21 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
   const int wm = wave / C::WAVES_N, wn = wave % C::WAVES_N;
   const int l32 = lane & 31, lh = lane >> 5;
 
-  const uint32_t total = (uint32_t)p.m_tiles * (uint32_t)p.n_chunks;
-  const uint32_t logical = xcd_remap(blockIdx.x, total);
-  const int m_blk = logical / p.n_chunks, chunk = logical % p.n_chunks;
+  int m_blk, chunk;
+  if (p.xg_n > 0) {
+    // Workgroups go round-robin to the 8 XCDs, each with a 4 MB L2 of its own.  XCD (xm, xn) of the
+    // xg_m x xg_n grid owns the block of xr_m x xr_n tiles at (xm*xr_m, xn*xr_n) and walks it row by row, so
+    // the W rows of its xr_n tile columns stay in its L2 while the x rows stream through once.  (With contiguous
+    // ranges of a row-major tile list every XCD reads all of W, twice over: 8.6x the algorithmic bytes.)
+    const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+    m_blk = (xcd / p.xg_n) * p.xr_m + local / p.xr_n;
+    chunk = (xcd % p.xg_n) * p.xr_n + local % p.xr_n;
+    if (local / p.xr_n >= p.xr_m || m_blk >= p.m_tiles || chunk >= p.n_chunks) return;  // padding of the grid
+  } else {
+    const uint32_t total = (uint32_t)p.m_tiles * (uint32_t)p.n_chunks;
+    const uint32_t logical = xcd_remap(blockIdx.x, total);
+    m_blk = logical / p.n_chunks; chunk = logical % p.n_chunks;
+  }
   const int m0 = m_blk * BM;
   const int K = p.K, M = p.M, N = p.N;
   constexpr int BKP = C::BKP, ROWB = C::ROWB;
@@ -540,7 +552,19 @@ int launch_pcfg(LoraGemmParams p, hipStream_t stream, int n_groups = 1) {
     if (e != hipSuccess) return (int)e;
     attr_done = true;
   }
-  const unsigned grid = (unsigned)(p.m_tiles * p.n_chunks);
+  unsigned grid = (unsigned)(p.m_tiles * p.n_chunks);
+  p.xg_n = p.xr_m = p.xr_n = 0;
+  if (C::NRT == 0 && (p.dbg & 8) == 0) {
+    // choose the XCD grid whose per-XCD block touches the fewest operand rows, padding counted as cost
+    double best = 0;
+    for (int gm = 1; gm <= 8; gm *= 2) {
+      const int gn = 8 / gm;
+      const int rm = (p.m_tiles + gm - 1) / gm, rn = (p.n_tiles + gn - 1) / gn;
+      const double cost = ((double)rm * C::BM + (double)rn * C::BN) * (8.0 * rm * rn) / ((double)p.m_tiles * p.n_tiles);
+      if (p.xg_n == 0 || cost < best) { best = cost; p.xg_n = gn; p.xr_m = rm; p.xr_n = rn; }
+    }
+    grid = 8u * (unsigned)p.xr_m * (unsigned)p.xr_n;
+  }
   kh_launch(CONV ? KH_TAG_CONV : KH_TAG_LORA_GEMM, lora_gemm_pipe_kernel<C, CONV>, dim3(grid, (unsigned)n_groups), dim3(C::NT), C::LDS_BYTES, stream, p);
   KH_RETURN_LAST_ERROR();
 }
