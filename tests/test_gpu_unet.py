@@ -243,3 +243,48 @@ def test_sdxl_unet_step_config3():
     say("sdxl unet config3 cosine", c)
     assert got.shape == (2, 4, 128, 128)
     assert c >= 0.999, c
+
+
+def test_patch_on_lora_merge_matches_unmerged_adapter():
+    """Katz's merge path (W += up @ down * alpha/rank as GEMMs on the GPU, keys through the key-match sidecar)
+    gives the weights of the oracle's closed form and the same step output as running the adapter unmerged."""
+    import katz_amd.layers as L
+    from katz_amd.shm_adapters import patch_on_lora
+    from katz_amd.unet_2d_condition import UNet2DConditionModel, UNetConfig
+    from oracle import ops as O
+
+    say("patch_on_lora")
+    torch.manual_seed(0)
+    cfg = OracleCfg.tiny()
+    oracle = round_module_to_bf16_(OracleUNet(cfg).eval())
+    merged = _product_from_oracle(oracle, "tiny")
+    plain = _product_from_oracle(oracle, "tiny")
+    lora = random_lora(oracle.lora_linears(), 16, seed=21, std=0.05)
+    sd = {k: v.to(torch.float16) for k, v in katz_lora_state_dict(lora).items()}   # what the shared memory holds
+    key_match = {}
+    for mod in lora:
+        head, _, leaf = mod.rpartition(".")
+        base = (f"unet.{head}.processor.{leaf}_lora" if leaf in ("to_q", "to_k", "to_v")
+                else f"unet.{mod[:-len('.to_out.0')]}.processor.to_out_lora" if mod.endswith(".to_out.0") else f"unet.{mod}.lora")
+        key_match[mod + ".weight"] = {"lora_down_key": base + ".down.weight", "lora_up_key": base + ".up.weight"}
+    scale = 0.75
+    n = patch_on_lora(merged, sd, key_match, scale=scale)
+    assert n == len(lora)
+    torch.cuda.synchronize()
+    params = dict(merged.named_parameters())
+    for mod in list(lora)[:8] + list(lora)[-4:]:
+        down, up = lora[mod]
+        w0 = dict(oracle.named_parameters())[mod + ".weight"]
+        ref = O.lora_merged_weight(w0, [(down.half().float(), up.half().float(), scale)])
+        assert_close_rel(params[mod + ".weight"], ref, 1e-2, f"merged weight {mod}")
+    # same step, adapter unmerged at the same effective scale (alpha = scale * rank)
+    plain.load_lora_into_unet({k: v.float() for k, v in sd.items()},
+                              network_alphas={k + ".alpha": scale * 16 for k in sd if k.endswith(".down.weight")},
+                              adapter_name="a")
+    plain.set_adapters(["a"], [1.0])
+    x, ctx, added = _inputs(cfg, 2, 32, 77)
+    dev = "cuda:0"
+    with torch.no_grad():
+        a = merged(x.to(dev), torch.tensor([500.0], device=dev), ctx.to(dev), added_cond_kwargs=_to_dev(added)).sample
+        b = plain(x.to(dev), torch.tensor([500.0], device=dev), ctx.to(dev), added_cond_kwargs=_to_dev(added)).sample
+    assert cosine(a, b) >= 0.999, cosine(a, b)

@@ -175,3 +175,49 @@ def test_expand_lora_scales_docstring_example_and_set_adapters():
     assert w("mid_block.attentions.0.proj_in") == 0.25
     assert w("up_blocks.0.attentions.2.transformer_blocks.0.ff.net.2") == 0.3
     assert w("up_blocks.1.attentions.0.transformer_blocks.0.attn2.to_k") == 1.0
+
+
+def test_shm_adapter_segments_roundtrip():
+    """Loader side publishes an adapter into Katz's shared-memory layout; the pipeline side reads it back
+    zero-copy (names "<key>_<loader id>", float16, int8 flag array with states 0 / 1 / 10)."""
+    import json
+    import os
+    import pytest
+    import torch
+    from multiprocessing import shared_memory
+    from katz_amd.shm_adapters import ShmAdapterSegments, LOADED
+
+    golden = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "sdxl_lora_keys.json")))
+    info = {}
+    for wkey in list(golden)[:6]:   # metadata in the reference's schema: {lora key: {"shape", "nbytes"}}
+        e = golden[wkey]
+        for k, shp in ((e["down_key"], e["down"]), (e["up_key"], e["up"])):
+            info[k] = {"shape": shp, "nbytes": shp[0] * shp[1] * 2}
+    prefix = f"katztest{os.getpid()}_"
+    with pytest.raises(FileNotFoundError):
+        ShmAdapterSegments(info, loader_id=0, create=False, name_prefix=prefix)
+    loader = ShmAdapterSegments(info, loader_id=0, n_loaders=2, create=True, name_prefix=prefix)
+    try:
+        reader = ShmAdapterSegments(info, loader_id=0, n_loaders=2, create=False, name_prefix=prefix)
+        assert not reader.loaded()
+        with pytest.raises(RuntimeError):
+            reader.state_dict()
+        reader.request(1)
+        assert int(loader.flags[0]) == 1
+        g = torch.Generator().manual_seed(0)
+        sd = {k: torch.randn(*m["shape"], generator=g).to(torch.float16) for k, m in info.items()}
+        loader.publish(sd)
+        assert reader.loaded() and int(reader.flags[0]) == LOADED
+        got = reader.state_dict()
+        assert set(got) == set(sd) and all(torch.equal(got[k], sd[k]) and got[k].dtype == torch.float16 for k in sd)
+        # the segment of a key is addressable by the reference's name
+        k0 = next(iter(info))
+        seg = shared_memory.SharedMemory(name=f"{prefix}{k0}_0")
+        assert seg.size >= info[k0]["nbytes"]
+        seg.close()
+        reader.clear()
+        assert all(float(a.sum()) == 0 for a in loader.arrays.values())
+        del got
+        reader.close()
+    finally:
+        loader.close()
