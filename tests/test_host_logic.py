@@ -221,3 +221,69 @@ def test_shm_adapter_segments_roundtrip():
         reader.close()
     finally:
         loader.close()
+
+
+def test_kohya_conversion_reproduces_the_reference_key_list():
+    """Kohya / SGM-named keys built by the inverse block arithmetic convert to exactly the 1444 tensor keys (and the
+    alpha naming) the reference holds for its converted adapter (tests/golden/sdxl_lora_keys.json, from
+    lora_info_shm/TheLastBen_Papercut_SDXL*.json), and load into the UNet."""
+    import json
+    import os
+    import re
+    import pytest
+    import torch
+    from katz_amd.lora_conversion import convert_kohya_lora_to_diffusers
+
+    golden = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "sdxl_lora_keys.json")))
+
+    def kohya_name(mod):  # diffusers module path -> sd-scripts name with SGM block numbering (layers_per_block = 2)
+        m = re.match(r"(down_blocks|up_blocks)\.(\d+)\.attentions\.(\d+)\.(.+)", mod)
+        if m:
+            b, l = int(m.group(2)), int(m.group(3))
+            head = f"input_blocks_{b * 3 + l + 1}_1" if m.group(1) == "down_blocks" else f"output_blocks_{b * 3 + l}_1"
+            rest = m.group(4)
+        else:
+            m = re.match(r"mid_block\.attentions\.0\.(.+)", mod)
+            head, rest = "middle_block_1", m.group(1)
+        return "lora_unet_" + head + "_" + rest.replace(".", "_")
+
+    sd, expect_keys, expect_alpha = {}, set(), {}
+    for wkey, e in golden.items():
+        mod = wkey[:-len(".weight")]
+        kn = kohya_name(mod)
+        sd[kn + ".lora_down.weight"] = torch.zeros(e["down"])
+        sd[kn + ".lora_up.weight"] = torch.zeros(e["up"])
+        sd[kn + ".alpha"] = torch.tensor(e["alpha"])
+        expect_keys |= {e["down_key"], e["up_key"]}
+        expect_alpha[e["down_key"] + ".alpha" if ".processor." in e["down_key"] else "unet." + mod + ".alpha"] = e["alpha"]
+    sd["lora_te1_text_model_encoder_layers_0_mlp_fc1.lora_down.weight"] = torch.zeros(4, 8)
+    unet_sd, alphas, rest = convert_kohya_lora_to_diffusers(sd)
+    assert len(expect_keys) == 1444 and set(unet_sd) == expect_keys
+    assert alphas == expect_alpha and len(alphas) == 722
+    assert list(rest) == ["lora_te1_text_model_encoder_layers_0_mlp_fc1.lora_down.weight"]
+    for wkey, e in list(golden.items())[:20]:
+        assert list(unet_sd[e["down_key"]].shape) == e["down"] and list(unet_sd[e["up_key"]].shape) == e["up"]
+    # diffusers-style block names are accepted too; conv targets are refused
+    u2, a2, _ = convert_kohya_lora_to_diffusers({
+        "lora_unet_down_blocks_1_attentions_0_transformer_blocks_0_attn2_to_out_0.lora_down.weight": torch.zeros(4, 640),
+        "lora_unet_down_blocks_1_attentions_0_transformer_blocks_0_attn2_to_out_0.lora_up.weight": torch.zeros(640, 4)})
+    assert set(u2) == {"unet.down_blocks.1.attentions.0.transformer_blocks.0.attn2.processor.to_out_lora.down.weight",
+                       "unet.down_blocks.1.attentions.0.transformer_blocks.0.attn2.processor.to_out_lora.up.weight"}
+    with pytest.raises(NotImplementedError):
+        convert_kohya_lora_to_diffusers({"lora_unet_input_blocks_4_0_in_layers_2.lora_down.weight": torch.zeros(4, 4)})
+    with pytest.raises(ValueError):
+        convert_kohya_lora_to_diffusers({"lora_unet_middle_block_1_proj_in.lora_down.weight": torch.zeros(4, 4)})
+
+    # end to end on the SDXL-shaped module tree: every converted key finds its LoRALinear
+    import katz_amd.layers as L
+    from katz_amd.unet_2d_condition import UNet2DConditionModel, UNetConfig
+    L.SKIP_INIT = True
+    try:
+        unet = UNet2DConditionModel(UNetConfig.sdxl())
+    finally:
+        L.SKIP_INIT = False
+    unet.load_lora_into_unet(unet_sd, network_alphas=alphas, adapter_name="papercut")
+    lin = unet.lora_linears()
+    assert sum("papercut" in m.adapters for m in lin.values()) == 722
+    m = lin["down_blocks.1.attentions.0.transformer_blocks.0.attn1.to_q"]
+    assert m.adapters["papercut"].alpha == 20000.0
