@@ -235,6 +235,62 @@ class Conv3x3(nn.Conv2d):
     def __init__(self, in_channels, out_channels, stride=1, padding=1):
         super().__init__(in_channels, out_channels, 3, stride=stride, padding=padding)
         self._packed = None  # (weight data_ptr, weight version, [Cout,3,3,Cin] copy)
+        # LoRA on the convolution (LoRACompatibleConv + LoRAConv2dLayer, diffusers-hf/src/diffusers/models/lora.py
+        # :258-296, :369-383): down [r,Cin,3,3] with the base conv's stride / padding, up [Cout,r,1,1]
+        self.adapters: Dict[str, Adapter] = {}
+        self.active: List[str] = []
+        self.adapters_enabled = True
+        self._global_scale = 1.0
+        self._lora = None    # (A_cat packed [R,3,3,Cin], B_cat scaled [Cout,R]) of the active adapters
+
+    def add_adapter(self, name: str, down: torch.Tensor, up: torch.Tensor, alpha: Optional[float] = None,
+                    weight: float = 1.0) -> None:
+        up = up.reshape(up.shape[0], up.shape[1])
+        if down.dim() != 4 or tuple(down.shape[1:]) != (self.in_channels, 3, 3) or up.shape != (self.out_channels, down.shape[0]):
+            raise ValueError(f"adapter {name!r}: expected down [r,{self.in_channels},3,3] and up [{self.out_channels},r(,1,1)], "
+                             f"got {tuple(down.shape)} and {tuple(up.shape)}")
+        self.adapters[name] = Adapter(down.detach(), up.detach(), alpha, weight)
+        self._lora = None
+
+    def delete_adapter(self, name: str) -> None:
+        self.adapters.pop(name, None)
+        self.active = [n for n in self.active if n != name]
+        self._lora = None
+
+    def set_active(self, names: Sequence[str], weights: Optional[Sequence[float]] = None) -> None:
+        self.active = [n for n in names if n in self.adapters]
+        if weights is not None:
+            for n, w in zip(names, weights):
+                if n in self.adapters:
+                    self.adapters[n].weight = float(w)
+        self._lora = None
+
+    def set_global_scale(self, scale: float) -> None:
+        if scale != self._global_scale:
+            self._global_scale = float(scale)
+            self._lora = None
+
+    def refresh_adapters(self) -> None:
+        self._lora = None
+
+    def _lora_pack(self):
+        """A_cat: the active down kernels stacked along the rank axis, zero-padded to a multiple of 32, in the conv
+        kernel's [R,3,3,Cin] layout; B_cat [Cout,R] with each adapter's weight * alpha / rank * global scale folded in."""
+        if self._lora is None:
+            names = [n for n in self.active if self.adapters_enabled]
+            if not names:
+                self._lora = (None, None)
+            else:
+                dev, dt = self.weight.device, self.weight.dtype
+                downs = [self.adapters[n].down.to(dev, torch.float32) for n in names]
+                ups = [self.adapters[n].up.to(dev, torch.float32) * self.adapters[n].multiplier(self._global_scale) for n in names]
+                a = torch.cat(downs, dim=0)
+                b = torch.cat(ups, dim=1)
+                pad = -a.shape[0] % 32
+                a = F.pad(a, (0, 0, 0, 0, 0, 0, 0, pad))
+                b = F.pad(b, (0, pad))
+                self._lora = (ops.pack_conv3x3_weight(a.to(dt)), b.to(dt).contiguous())
+        return self._lora
 
     def packed_weight(self) -> torch.Tensor:
         w = self.weight
@@ -245,13 +301,24 @@ class Conv3x3(nn.Conv2d):
     def forward(self, x, residual=None):
         native = (x.is_cuda and x.dtype == torch.bfloat16 and self.weight.dtype == torch.bfloat16
                   and self.padding == (1, 1) and self.in_channels % 32 == 0 and self.out_channels % 8 == 0)
+        a_cat, b_cat = self._lora_pack() if self.adapters else (None, None)
         if not native:
+            if a_cat is not None:
+                raise NotImplementedError("LoRA on a convolution needs the katz_hip conv kernel (bf16 GPU tensors, Cin % 32 == 0)")
             y = super().forward(x)
             return y if residual is None else residual + y
         x = x.contiguous(memory_format=torch.channels_last)   # no copy when the producer already wrote NHWC
         if residual is not None:
             residual = residual.contiguous(memory_format=torch.channels_last)
-        return ops.conv3x3(x, self.packed_weight(), self.bias, stride=self.stride[0], residual=residual)
+        y = ops.conv3x3(x, self.packed_weight(), self.bias, stride=self.stride[0], residual=residual)
+        if a_cat is None:
+            return y
+        # low-rank branch: T = conv3x3(x, A_cat) is [pixels, R]; y += T . B_cat^T as a GEMM with y as its residual
+        t = ops.conv3x3(x, a_cat, None, stride=self.stride[0])
+        nb, co, ho, wo = y.shape
+        y2 = ops.lora_linear(t.permute(0, 2, 3, 1).reshape(nb * ho * wo, t.shape[1]), b_cat, None,
+                             residual=y.permute(0, 2, 3, 1).reshape(nb * ho * wo, co))
+        return y2.view(nb, ho, wo, co).permute(0, 3, 1, 2)
 
 
 class Downsample2D(nn.Module):

@@ -202,13 +202,21 @@ class UNet2DConditionModel(nn.Module):
     def lora_linears(self) -> Dict[str, LoRALinear]:
         return {n: m for n, m in self.named_modules() if isinstance(m, LoRALinear)}
 
+    def lora_convs(self) -> Dict[str, "Conv3x3"]:
+        """3x3 convolutions that can carry a LoRA (resnet conv1 / conv2, down / upsampler convs)."""
+        from .layers import Conv3x3
+        return {n: m for n, m in self.named_modules() if isinstance(m, Conv3x3)}
+
+    def _lora_targets(self) -> Dict[str, Any]:
+        return {**self.lora_linears(), **self.lora_convs()}
+
     def load_lora_into_unet(self, state_dict: Dict[str, torch.Tensor], network_alphas: Optional[Dict[str, float]] = None,
                             adapter_name: Optional[str] = None) -> str:
         """Register one adapter from a LoRA state dict (load_lora_into_unet,
         diffusers-hf/src/diffusers/loaders/lora.py:382-496).  Keys in any spelling parse_lora_key accepts;
         keys of other components (text encoders) are ignored; network_alphas maps
         "<module or down key>.alpha" to alpha (:261-270), default alpha = rank."""
-        lin = self.lora_linears()
+        lin = self._lora_targets()
         pairs: Dict[str, Dict[str, torch.Tensor]] = {}
         for k, v in state_dict.items():
             if k.startswith("text_encoder"):
@@ -226,7 +234,7 @@ class UNet2DConditionModel(nn.Module):
             raise ValueError(f"adapter name {adapter_name!r} is already in use in the UNet")
         for mod, pr in pairs.items():
             if mod not in lin:
-                raise ValueError(f"LoRA targets {mod!r}, which is not a LoRA-able linear of this UNet")
+                raise ValueError(f"LoRA targets {mod!r}, which is not a LoRA-able linear or 3x3 convolution of this UNet")
             if "down" not in pr or "up" not in pr:
                 raise ValueError(f"LoRA for {mod!r} lacks its {'down' if 'down' not in pr else 'up'} matrix")
             alpha = None
@@ -242,7 +250,7 @@ class UNet2DConditionModel(nn.Module):
 
     def adapter_names(self) -> List[str]:
         names: List[str] = []
-        for m in self.lora_linears().values():
+        for m in self._lora_targets().values():
             for n in m.adapters:
                 if n not in names:
                     names.append(n)
@@ -259,7 +267,7 @@ class UNet2DConditionModel(nn.Module):
         if len(weights) != len(names):
             raise ValueError(f"Length of adapter names {len(names)} is not equal to the length of their weights {len(weights)}.")
         weights = [1.0 if w is None else w for w in weights]
-        lin = self.lora_linears()
+        lin = self._lora_targets()
         if any(isinstance(w, dict) for w in weights):
             # per-block scales, e.g. {"down": 0.9, "mid": 1.0, "up": {"block_0": 0.6, "block_1": [0.4, 0.8, 1.0]}}
             # (_maybe_expand_lora_scales, diffusers-hf/src/diffusers/loaders/unet_loader_utils.py:41-58)
@@ -268,19 +276,23 @@ class UNet2DConditionModel(nn.Module):
             tpb = {"down": self.cfg.layers_per_block, "up": self.cfg.layers_per_block + 1}
             weights = [expand_lora_scales_for_one_adapter(w, bwt, tpb, list(lin.keys())) for w in weights]
         for mod_name, m in lin.items():
-            m.set_active(names, [module_weight(w, mod_name) for w in weights])
+            # per-block dictionaries address transformers only; other modules (resnet convs) keep scale 1 under them
+            m.set_active(names, [module_weight(w, mod_name) if (not isinstance(w, dict) or ".attentions." in mod_name) else 1.0
+                                 for w in weights])
 
     def disable_lora(self) -> None:
-        for m in self.lora_linears().values():
+        for m in self._lora_targets().values():
             m.adapters_enabled = False
             m.refresh_adapters()
 
     def enable_lora(self) -> None:
-        for m in self.lora_linears().values():
+        for m in self._lora_targets().values():
             m.adapters_enabled = True
             m.refresh_adapters()
 
     def fuse_lora(self, lora_scale: float = 1.0, adapter_names: Optional[Sequence[str]] = None) -> None:
+        if any(c.adapters for c in self.lora_convs().values()):
+            raise NotImplementedError("fusing adapters that target convolutions is not implemented; run them unfused")
         for m in self.lora_linears().values():
             m.fuse(lora_scale, adapter_names)
 
@@ -295,16 +307,19 @@ class UNet2DConditionModel(nn.Module):
             for n in list(m.adapters):
                 m.delete_adapter(n)
             m.refresh_adapters()
+        for c in self.lora_convs().values():
+            for n in list(c.adapters):
+                c.delete_adapter(n)
 
     def delete_adapters(self, adapter_names: Union[str, Sequence[str]]) -> None:
         names = [adapter_names] if isinstance(adapter_names, str) else list(adapter_names)
-        for m in self.lora_linears().values():
+        for m in self._lora_targets().values():
             for n in names:
                 m.delete_adapter(n)
             m.refresh_adapters()
 
     def scale_lora_layers(self, scale: float) -> None:
-        for m in self.lora_linears().values():
+        for m in self._lora_targets().values():
             m.set_global_scale(scale)
 
     def set_attn_processor(self, processor) -> None:

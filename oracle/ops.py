@@ -42,6 +42,20 @@ def lora_merged_weight(weight, adapters: Sequence[tuple]):
     return w
 
 
+def lora_conv2d(x, weight, bias=None, adapters: Sequence[tuple] = (), stride: int = 1, padding: int = 1):
+    """conv(x, W) + sum_i s_i * conv1x1(conv_k(x, A_i), B_i) with A_i [r, in, k, k], B_i [out, r, 1, 1] (or [out, r]).
+
+    LoRACompatibleConv.forward (diffusers-hf/src/diffusers/models/lora.py:369-383) + LoRAConv2dLayer.forward
+    (:284-296): the down conv has the base conv's kernel, stride and padding, the up conv is 1x1;
+    s_i = weight_i * alpha_i / rank_i.  Equal to the conv with the merged kernel of _fuse_lora (:403-421):
+    W + s * (B.flatten(1) @ A.flatten(1)).reshape(W.shape)."""
+    y = F.conv2d(x, weight, bias, stride=stride, padding=padding)
+    for A, B, s in adapters:
+        t = F.conv2d(x, A, None, stride=stride, padding=padding)
+        y = y + float(s) * F.conv2d(t, B.reshape(B.shape[0], B.shape[1], 1, 1))
+    return y
+
+
 def attention(q, k, v, heads: int, scale: Optional[float] = None):
     """softmax(q k^T * scale) v per head, inputs [B,T,H*d] / [B,S,H*d], output [B,T,H*d].
 

@@ -609,3 +609,45 @@ def test_denoise_loop_matches_oracle_loop(lat_f32):
     cos = torch.nn.functional.cosine_similarity(got.float().cpu().flatten(), ref.float().flatten(), dim=0).item()
     assert cos >= 0.999, cos
     assert_close_rel(got, ref, 1e-2 if lat_f32 else 1e-1, "50-step loop")
+
+
+@pytest.mark.parametrize("stride", [1, 2])
+def test_conv3x3_with_lora_adapters(stride):
+    """Conv3x3 with two active LoRA adapters against the oracle's LoRA conv; scale 0, disable and delete restore the base."""
+    from katz_amd.layers import Conv3x3
+
+    say("conv lora", stride)
+    d = dev()
+    g = torch.Generator().manual_seed(17)
+    cin, cout = 64, 96
+    conv = Conv3x3(cin, cout, stride=stride)
+    with torch.no_grad():
+        conv.weight.copy_(randn(g, cout, cin, 3, 3, std=(9 * cin) ** -0.5).to(BF).float())
+        conv.bias.copy_(randn(g, cout).to(BF).float())
+    w, b = conv.weight.detach().clone(), conv.bias.detach().clone()
+    conv = conv.to(d, BF)
+    ads = [(randn(g, 8, cin, 3, 3, std=0.05).to(BF).float(), randn(g, cout, 8, 1, 1, std=0.05).to(BF).float(), 16.0, 0.8),
+           (randn(g, 4, cin, 3, 3, std=0.05).to(BF).float(), randn(g, cout, 4, 1, 1, std=0.05).to(BF).float(), None, 0.6)]
+    for i, (A, B, alpha, wgt) in enumerate(ads):
+        conv.add_adapter(f"a{i}", A, B, alpha)
+    conv.set_active(["a0", "a1"], [0.8, 0.6])
+    x = randn(g, 2, cin, 12, 10).to(BF)
+    xd = x.to(d).contiguous(memory_format=torch.channels_last)
+    with torch.no_grad():
+        y = conv(xd)
+        ref = O.lora_conv2d(x.float(), w, b, [(ads[0][0], ads[0][1], 0.8 * 16.0 / 8), (ads[1][0], ads[1][1], 0.6)], stride=stride)
+        base = O.lora_conv2d(x.float(), w, b, [], stride=stride)
+        torch.cuda.synchronize()
+        assert y.shape == ref.shape
+        assert_close_rel(y, ref, REL_BF16, "conv + lora")
+        assert (ref - base).abs().max() > 0.05   # the adapters matter at this scale
+        conv.set_active(["a0", "a1"], [0.0, 0.0])
+        assert_close_rel(conv(xd), base, REL_BF16, "conv + lora at scale 0")
+        conv.set_active(["a0", "a1"], [0.8, 0.6])
+        conv.adapters_enabled = False
+        conv.refresh_adapters()
+        y_dis = conv(xd)
+        conv.adapters_enabled = True
+        conv.delete_adapter("a0"); conv.delete_adapter("a1")
+        assert torch.equal(conv(xd), y_dis)
+        assert_close_rel(y_dis, base, REL_BF16, "conv, adapters disabled")

@@ -287,3 +287,41 @@ def test_kohya_conversion_reproduces_the_reference_key_list():
     assert sum("papercut" in m.adapters for m in lin.values()) == 722
     m = lin["down_blocks.1.attentions.0.transformer_blocks.0.attn1.to_q"]
     assert m.adapters["papercut"].alpha == 20000.0
+
+
+def test_unet_lora_surface_reaches_convolutions():
+    """Adapters that target 3x3 convolutions (diffusers key spelling) register on the Conv3x3 modules and follow
+    set_adapters / delete_adapters like the linear ones; fusing them is refused loudly."""
+    import pytest
+    import torch
+    import katz_amd.layers as L
+    from katz_amd.unet_2d_condition import UNet2DConditionModel, UNetConfig
+
+    L.SKIP_INIT = True
+    try:
+        unet = UNet2DConditionModel(UNetConfig.tiny())
+    finally:
+        L.SKIP_INIT = False
+    convs = unet.lora_convs()
+    assert "down_blocks.0.resnets.0.conv1" in convs and "down_blocks.0.downsamplers.0.conv" in convs
+    assert "conv_in" not in convs   # 4 input channels: stays a plain convolution
+    c = convs["down_blocks.0.resnets.0.conv1"]
+    lin_name = "down_blocks.1.attentions.0.transformer_blocks.0.attn1.to_q"
+    lin = unet.lora_linears()[lin_name]
+    sd = {"unet.down_blocks.0.resnets.0.conv1.lora.down.weight": torch.zeros(4, c.in_channels, 3, 3),
+          "unet.down_blocks.0.resnets.0.conv1.lora.up.weight": torch.zeros(c.out_channels, 4, 1, 1),
+          f"unet.{lin_name}.lora.down.weight": torch.zeros(4, lin.in_features),
+          f"unet.{lin_name}.lora.up.weight": torch.zeros(lin.out_features, 4)}
+    unet.load_lora_into_unet(sd, network_alphas={"unet.down_blocks.0.resnets.0.conv1.alpha": 8.0}, adapter_name="locon")
+    assert c.adapters["locon"].alpha == 8.0 and c.active == ["locon"] and lin.active == ["locon"]
+    unet.set_adapters(["locon"], [0.5])
+    assert c.adapters["locon"].weight == 0.5 and c.adapters["locon"].multiplier() == 0.5 * 8.0 / 4
+    unet.set_adapters(["locon"], [{"down": 0.3}])      # block dictionaries address transformers; the conv keeps 1.0
+    assert lin.adapters["locon"].weight == 0.3 and c.adapters["locon"].weight == 1.0
+    with pytest.raises(NotImplementedError):
+        unet.fuse_lora()
+    with pytest.raises(ValueError):
+        unet.load_lora_into_unet({"unet.conv_in.lora.down.weight": torch.zeros(4, 4, 3, 3),
+                                  "unet.conv_in.lora.up.weight": torch.zeros(64, 4, 1, 1)}, adapter_name="bad")
+    unet.delete_adapters("locon")
+    assert not c.adapters and not lin.adapters

@@ -101,3 +101,36 @@ def test_sgmv_is_per_request_lora():
     assert torch.allclose(y[0:3], O.lora_linear(x[0:3], W, None, [ads[1]]), atol=1e-6)
     assert torch.equal(y[3:7], F.linear(x[3:7], W))
     assert torch.allclose(y[7:10], O.lora_linear(x[7:10], W, None, [ads[0]]), atol=1e-6)
+
+
+def test_lora_conv2d_equals_conv_with_merged_kernel():
+    """LoRA on a convolution == the convolution with the fused kernel W + s * (B.flatten(1) @ A.flatten(1)).reshape(W)
+    (diffusers-hf/src/diffusers/models/lora.py:409-421), for stride 1 and 2, two adapters; plus a brute-force pixel."""
+    import torch
+    import torch.nn.functional as F
+    from oracle import ops as O
+
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(2, 6, 9, 7, generator=g, dtype=torch.float64)
+    w = torch.randn(5, 6, 3, 3, generator=g, dtype=torch.float64)
+    b = torch.randn(5, generator=g, dtype=torch.float64)
+    ads = [(torch.randn(4, 6, 3, 3, generator=g, dtype=torch.float64), torch.randn(5, 4, 1, 1, generator=g, dtype=torch.float64), 0.7),
+           (torch.randn(2, 6, 3, 3, generator=g, dtype=torch.float64), torch.randn(5, 2, generator=g, dtype=torch.float64), -1.3)]
+    for stride in (1, 2):
+        got = O.lora_conv2d(x, w, b, ads, stride=stride, padding=1)
+        wm = w.clone()
+        for A, B, s in ads:
+            wm = wm + s * (B.reshape(5, -1) @ A.flatten(1)).reshape(w.shape)
+        assert torch.allclose(got, F.conv2d(x, wm, b, stride=stride, padding=1), atol=1e-10)
+    assert torch.equal(O.lora_conv2d(x, w, b, [(ads[0][0], ads[0][1], 0.0)]), F.conv2d(x, w, b, padding=1))
+    # one output pixel by hand: n=1, co=3, (h, w) = (4, 2), stride 1
+    got = O.lora_conv2d(x, w, b, ads[:1])
+    acc = b[3].clone()
+    for ci in range(6):
+        for kh in range(3):
+            for kw in range(3):
+                hh, ww = 4 + kh - 1, 2 + kw - 1
+                if 0 <= hh < 9 and 0 <= ww < 7:
+                    eff = w[3, ci, kh, kw] + 0.7 * sum(ads[0][1][3, r, 0, 0] * ads[0][0][r, ci, kh, kw] for r in range(4))
+                    acc = acc + eff * x[1, ci, hh, ww]
+    assert abs(got[1, 3, 4, 2] - acc) < 1e-9
