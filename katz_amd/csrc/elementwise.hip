@@ -21,7 +21,7 @@ namespace {
 constexpr int EW_THREADS = 256;
 constexpr int KH_MAX_SRCS = 8;
 
-__device__ __forceinline__ float gelu_erf_f(float x) { return 0.5f * x * (1.f + erff(x * 0.70710678118654752f)); }
+__device__ __forceinline__ float gelu_erf_f(float x) { return kh_gelu_erf(x); }
 __device__ __forceinline__ float gelu_tanh_f(float x) {
   return 0.5f * x * (1.f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
 }

@@ -79,6 +79,17 @@ __device__ __forceinline__ float silu_f(float x) { return x / (1.0f + __expf(-x)
 
 static inline bool kh_aligned16(const void* p) { return (((uintptr_t)p) & 15u) == 0; }
 
+// gelu(x) = 0.5 x (1 + erf(x / sqrt 2)) with erf from Abramowitz & Stegun 7.1.26 (|abs error| <= 1.5e-7, far inside
+// the bf16 rounding the result goes through): a reciprocal, an exp2 and five FMAs instead of the library erff.
+__device__ __forceinline__ float kh_gelu_erf(float x) {
+  const float z = fabsf(x) * 0.70710678118654752f;
+  const float t = __builtin_amdgcn_rcpf(1.0f + 0.3275911f * z);
+  const float poly = t * (0.254829592f + t * (-0.284496736f + t * (1.421413741f + t * (-1.453152027f + t * 1.061405429f))));
+  const float e = poly * __builtin_amdgcn_exp2f(-1.4426950408889634f * z * z);   // 1 - erf(z)
+  const float half_x = 0.5f * x;
+  return x >= 0.f ? half_x * (2.0f - e) : half_x * e;
+}
+
 // Workgroups are dealt round-robin to the 8 XCDs (each with its own L2). Map a
 // hardware block id to a logical tile id such that every XCD walks one
 // contiguous range of logical tiles, so neighbouring tiles share an L2.

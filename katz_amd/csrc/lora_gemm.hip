@@ -285,8 +285,8 @@ __global__ __launch_bounds__(C::NT) void lora_gemm_kernel(const LoraGemmParams p
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
               const float g0 = bf16_lo(gv[e]), g1 = bf16_hi(gv[e]);
-              const float a0 = 0.5f * g0 * (1.f + erff(g0 * 0.70710678118654752f));
-              const float a1 = 0.5f * g1 * (1.f + erff(g1 * 0.70710678118654752f));
+              const float a0 = kh_gelu_erf(g0);
+              const float a1 = kh_gelu_erf(g1);
               // the reference rounds gelu(gate) to the activation dtype before the product
               const float r0 = bf16_lo(pack_bf16x2(a0, 0.f)), r1 = bf16_lo(pack_bf16x2(a1, 0.f));
               o[e] = pack_bf16x2(bf16_lo(hv[e]) * r0, bf16_hi(hv[e]) * r1);

@@ -519,8 +519,8 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
               const float g0 = bf16_lo(gv[e]), g1 = bf16_hi(gv[e]);
-              const float a0 = 0.5f * g0 * (1.f + erff(g0 * 0.70710678118654752f));
-              const float a1 = 0.5f * g1 * (1.f + erff(g1 * 0.70710678118654752f));
+              const float a0 = kh_gelu_erf(g0);
+              const float a1 = kh_gelu_erf(g1);
               const uint32_t ar = pack_bf16x2(a0, a1);  // gelu(gate) rounded to bf16 before the product
               o[e] = pack_bf16x2(bf16_lo(hv[e]) * bf16_lo(ar), bf16_hi(hv[e]) * bf16_hi(ar));
             }
