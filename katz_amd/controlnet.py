@@ -45,7 +45,7 @@ class ControlNetConditioningEmbedding(nn.Module):
     def __init__(self, conditioning_embedding_channels: int, conditioning_channels: int = 3,
                  block_out_channels: Tuple[int, ...] = (16, 32, 96, 256)):
         super().__init__()
-        self.conv_in = nn.Conv2d(conditioning_channels, block_out_channels[0], 3, padding=1)
+        self.conv_in = Conv3x3(conditioning_channels, block_out_channels[0])
         self.blocks = nn.ModuleList()
         for i in range(len(block_out_channels) - 1):
             cin, cout = block_out_channels[i], block_out_channels[i + 1]
@@ -67,7 +67,7 @@ class ControlNetModel(nn.Module):
         self.cfg = cfg
         boc = cfg.block_out_channels
         ted = boc[0] * 4
-        self.conv_in = nn.Conv2d(cfg.in_channels, boc[0], 3, padding=1)
+        self.conv_in = Conv3x3(cfg.in_channels, boc[0])
         self.time_embedding = TimestepEmbedding(boc[0], ted)
         self.add_embedding = TimestepEmbedding(cfg.projection_class_embeddings_input_dim, ted)
         self.controlnet_cond_embedding = ControlNetConditioningEmbedding(boc[0], 3, conditioning_embedding_out_channels)

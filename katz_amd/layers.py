@@ -230,7 +230,8 @@ class Conv3x3(nn.Conv2d):
     """nn.Conv2d(kernel 3, padding 1, stride 1 or 2) whose forward runs the katz_hip implicit-GEMM kernel on
     channels_last bf16 GPU tensors; parameters and state-dict keys are nn.Conv2d's.  forward(x, residual)
     also folds the residual add that follows the convolution (resnet.py:374) into the kernel's epilogue.
-    Shapes the kernel does not take (Cin % 32 != 0, Cout % 8 != 0, other dtypes / layouts) run torch's conv2d."""
+    Channel counts the kernel does not take directly (the 4-channel latent, the 3-channel conditioning image) are
+    zero-padded; other dtypes / devices / paddings run torch's conv2d."""
 
     def __init__(self, in_channels, out_channels, stride=1, padding=1):
         super().__init__(in_channels, out_channels, 3, stride=stride, padding=padding)
@@ -287,30 +288,48 @@ class Conv3x3(nn.Conv2d):
                 a = torch.cat(downs, dim=0)
                 b = torch.cat(ups, dim=1)
                 pad = -a.shape[0] % 32
-                a = F.pad(a, (0, 0, 0, 0, 0, 0, 0, pad))
+                a = F.pad(a, (0, 0, 0, 0, 0, -self.in_channels % 32, 0, pad))
                 b = F.pad(b, (0, pad))
                 self._lora = (ops.pack_conv3x3_weight(a.to(dt)), b.to(dt).contiguous())
         return self._lora
 
-    def packed_weight(self) -> torch.Tensor:
+    def packed_weight(self):
+        """([Cout', 3, 3, Cin'] weight, [Cout'] bias) in the kernel's layout, channel counts zero-padded up to what
+        the kernel takes (Cin' % 32 == 0, Cout' % 8 == 0): padded input channels meet zero weights, padded output
+        channels are dropped by the caller."""
         w = self.weight
         if self._packed is None or self._packed[0] != w.data_ptr() or self._packed[1] != w._version:
-            self._packed = (w.data_ptr(), w._version, ops.pack_conv3x3_weight(w))
-        return self._packed[2]
+            pi, po = -self.in_channels % 32, -self.out_channels % 8
+            wp = w.detach()
+            b = None if self.bias is None else self.bias.detach()
+            if pi or po:
+                wp = F.pad(wp, (0, 0, 0, 0, 0, pi, 0, po))
+                b = None if b is None else F.pad(b, (0, po))
+            self._packed = (w.data_ptr(), w._version, ops.pack_conv3x3_weight(wp), b)
+        return self._packed[2], self._packed[3]
 
     def forward(self, x, residual=None):
-        native = (x.is_cuda and x.dtype == torch.bfloat16 and self.weight.dtype == torch.bfloat16
-                  and self.padding == (1, 1) and self.in_channels % 32 == 0 and self.out_channels % 8 == 0)
+        native = (x.is_cuda and x.dtype == torch.bfloat16 and self.weight.dtype == torch.bfloat16 and self.padding == (1, 1))
         a_cat, b_cat = self._lora_pack() if self.adapters else (None, None)
         if not native:
             if a_cat is not None:
-                raise NotImplementedError("LoRA on a convolution needs the katz_hip conv kernel (bf16 GPU tensors, Cin % 32 == 0)")
+                raise NotImplementedError("LoRA on a convolution needs the katz_hip conv kernel (bf16 GPU tensors, padding 1)")
             y = super().forward(x)
             return y if residual is None else residual + y
+        pi, po = -self.in_channels % 32, -self.out_channels % 8
+        if pi:   # few-channel inputs (the latent, the conditioning image): zero channels up to the kernel's granule
+            x = F.pad(x, (0, 0, 0, 0, 0, pi))
         x = x.contiguous(memory_format=torch.channels_last)   # no copy when the producer already wrote NHWC
+        w_packed, b_packed = self.packed_weight()
+        if po:
+            if a_cat is not None:
+                raise NotImplementedError("LoRA on a convolution whose output channels are not a multiple of 8")
+            y = ops.conv3x3(x, w_packed, b_packed, stride=self.stride[0])[:, :self.out_channels]
+            y = y.contiguous(memory_format=torch.channels_last)
+            return y if residual is None else residual + y
         if residual is not None:
             residual = residual.contiguous(memory_format=torch.channels_last)
-        y = ops.conv3x3(x, self.packed_weight(), self.bias, stride=self.stride[0], residual=residual)
+        y = ops.conv3x3(x, w_packed, b_packed, stride=self.stride[0], residual=residual)
         if a_cat is None:
             return y
         # low-rank branch: T = conv3x3(x, A_cat) is [pixels, R]; y += T . B_cat^T as a GEMM with y as its residual

@@ -25,7 +25,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from . import ops
-from .layers import LoRALinear, TimestepEmbedding, fused_norm_silu
+from .layers import Conv3x3, LoRALinear, TimestepEmbedding, fused_norm_silu
 from .lora import expand_lora_scales_for_one_adapter, module_weight
 from .unet_blocks import (CrossAttnDownBlock2D, CrossAttnUpBlock2D, DownBlock2D, UNetMidBlock2DCrossAttn, UpBlock2D)
 
@@ -117,7 +117,7 @@ class UNet2DConditionModel(nn.Module):
         self.cfg = cfg
         boc = cfg.block_out_channels
         ted = boc[0] * 4
-        self.conv_in = nn.Conv2d(cfg.in_channels, boc[0], 3, padding=1)
+        self.conv_in = Conv3x3(cfg.in_channels, boc[0])
         self.time_embedding = TimestepEmbedding(boc[0], ted)
         self.add_embedding = TimestepEmbedding(cfg.projection_class_embeddings_input_dim, ted)
         n = len(boc)
@@ -159,7 +159,7 @@ class UNet2DConditionModel(nn.Module):
             else:
                 raise ValueError(f"unsupported up block {typ}")
         self.conv_norm_silu = nn.Sequential(*fused_norm_silu(boc[0], cfg.norm_num_groups, cfg.norm_eps))
-        self.conv_out = nn.Conv2d(boc[0], cfg.out_channels, 3, padding=1)
+        self.conv_out = Conv3x3(boc[0], cfg.out_channels)
         self.num_upsamplers = n - 1
         self._ctx_kv = None
         self._register_load_state_dict_pre_hook(self._remap_upstream_keys)

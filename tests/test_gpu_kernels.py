@@ -651,3 +651,33 @@ def test_conv3x3_with_lora_adapters(stride):
         conv.delete_adapter("a0"); conv.delete_adapter("a1")
         assert torch.equal(conv(xd), y_dis)
         assert_close_rel(y_dis, base, REL_BF16, "conv, adapters disabled")
+
+
+@pytest.mark.parametrize("cin,cout", [(4, 64), (64, 4), (3, 16), (16, 32)])
+def test_conv3x3_module_pads_small_channel_counts(cin, cout):
+    """Conv3x3 on the katz_hip kernel for the UNet's conv_in / conv_out and the ControlNet's image embedding:
+    channel counts below the kernel's granule are zero-padded, results match F.conv2d, and are bit-reproducible."""
+    from katz_amd.layers import Conv3x3
+
+    say("conv small channels", cin, cout)
+    d = dev()
+    g = torch.Generator().manual_seed(cin * 100 + cout)
+    conv = Conv3x3(cin, cout)
+    with torch.no_grad():
+        conv.weight.copy_(randn(g, cout, cin, 3, 3, std=(9 * cin) ** -0.5).to(BF).float())
+        conv.bias.copy_(randn(g, cout).to(BF).float())
+    x = randn(g, 2, cin, 20, 12).to(BF)
+    ref = torch.nn.functional.conv2d(x.float(), conv.weight.detach(), conv.bias.detach(), padding=1)
+    conv = conv.to(d, BF)
+    from katz_amd import ops
+    ops.CALL_LOG = []
+    try:
+        with torch.no_grad():
+            y = conv(x.to(d))
+            y2 = conv(x.to(d))
+    finally:
+        log, ops.CALL_LOG = ops.CALL_LOG, None
+    torch.cuda.synchronize()
+    assert [c[0] for c in log] == ["conv3x3", "conv3x3"], "the module must run the katz_hip kernel"
+    assert y.shape == ref.shape and torch.equal(y, y2)
+    assert_close_rel(y, ref, REL_BF16, "conv3x3 with padded channels")

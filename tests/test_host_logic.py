@@ -304,7 +304,7 @@ def test_unet_lora_surface_reaches_convolutions():
         L.SKIP_INIT = False
     convs = unet.lora_convs()
     assert "down_blocks.0.resnets.0.conv1" in convs and "down_blocks.0.downsamplers.0.conv" in convs
-    assert "conv_in" not in convs   # 4 input channels: stays a plain convolution
+    assert "conv_in" in convs and "down_blocks.1.resnets.0.conv_shortcut" not in convs   # 1x1 shortcuts carry no LoRA
     c = convs["down_blocks.0.resnets.0.conv1"]
     lin_name = "down_blocks.1.attentions.0.transformer_blocks.0.attn1.to_q"
     lin = unet.lora_linears()[lin_name]
@@ -321,7 +321,8 @@ def test_unet_lora_surface_reaches_convolutions():
     with pytest.raises(NotImplementedError):
         unet.fuse_lora()
     with pytest.raises(ValueError):
-        unet.load_lora_into_unet({"unet.conv_in.lora.down.weight": torch.zeros(4, 4, 3, 3),
-                                  "unet.conv_in.lora.up.weight": torch.zeros(64, 4, 1, 1)}, adapter_name="bad")
+        unet.load_lora_into_unet({"unet.down_blocks.1.resnets.0.conv_shortcut.lora.down.weight": torch.zeros(4, 64, 1, 1),
+                                  "unet.down_blocks.1.resnets.0.conv_shortcut.lora.up.weight": torch.zeros(128, 4, 1, 1)},
+                                 adapter_name="bad")
     unet.delete_adapters("locon")
     assert not c.adapters and not lin.adapters
