@@ -37,9 +37,11 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
 // and consecutive threads read consecutive 16-byte pieces of a pixel row.
 constexpr int GN_MAX_CPT = 2;
 constexpr int GN_UNROLL = 4;
+constexpr int GN_SUNROLL = 16;  // statistics pass: few, long-lived workgroups keep many loads in flight per thread
 
 struct GnGeom {
-  int N, C, HW, G, Cg, splits;
+  int N, C, HW, G, Cg, splits;   // splits: workgroups per sample of the statistics pass
+  int asplits;                   // workgroups per sample of the apply pass (more, smaller ones)
   int CP;   // 16-byte chunks per pixel (C/8)
   int NTX;  // chunk-threads
   int CPT;  // chunks per thread
@@ -77,13 +79,13 @@ __global__ __launch_bounds__(GN_THREADS) void gn_stats_nhwc(const bf16_t* __rest
       for (int e = 0; e < 8; ++e) s[e] = q[e] = 0.f;
       const bf16_t* base = x + ((size_t)n * g.HW) * g.C + c0;
       int p = p0 + ty;
-      for (; p + (GN_UNROLL - 1) * g.PL < p1; p += GN_UNROLL * g.PL) {
-        u32x4 v[GN_UNROLL];
+      for (; p + (GN_SUNROLL - 1) * g.PL < p1; p += GN_SUNROLL * g.PL) {
+        u32x4 v[GN_SUNROLL];
 #pragma unroll
-        for (int u = 0; u < GN_UNROLL; ++u)
+        for (int u = 0; u < GN_SUNROLL; ++u)
           v[u] = *reinterpret_cast<const u32x4*>(base + (size_t)(p + u * g.PL) * g.C);
 #pragma unroll
-        for (int u = 0; u < GN_UNROLL; ++u) {
+        for (int u = 0; u < GN_SUNROLL; ++u) {
           float f[8];
           unpack8(v[u], f);
 #pragma unroll
@@ -118,21 +120,35 @@ __global__ __launch_bounds__(GN_THREADS) void gn_apply_nhwc(const bf16_t* __rest
                                                             const bf16_t* __restrict__ add_nc,
                                                             const float* __restrict__ ws, const GnGeom g, float eps) {
   __shared__ float s_mean[512], s_rstd[512];
+  __shared__ double s_ps[GN_THREADS], s_pq[GN_THREADS];
   const int n = blockIdx.y, split = blockIdx.x;
   const int tid = threadIdx.x;
   const double cnt = (double)g.Cg * (double)g.HW;
-  for (int i = tid; i < g.G; i += GN_THREADS) {
-    const float* pw = ws + ((size_t)n * g.G + i) * g.splits * 2;
+  // Fold the statistics pass's partial sums of every group (a workgroup needs all groups: a pixel has all channels).
+  // FT threads share a group, each summing every FT-th partial in fp64; their FT sums are then added in a fixed
+  // order, so the result does not depend on scheduling.
+  const int FT = g.G >= GN_THREADS ? 1 : GN_THREADS / g.G;
+  const int gpp = GN_THREADS / FT;   // groups per pass
+  for (int base = 0; base < g.G; base += gpp) {
+    const int grp = base + tid / FT, part = tid % FT;
     double s = 0.0, q = 0.0;
-    for (int k = 0; k < g.splits; ++k) { s += (double)pw[2 * k]; q += (double)pw[2 * k + 1]; }
-    const double mean = s / cnt;
-    double var = q / cnt - mean * mean;
-    var = var > 0.0 ? var : 0.0;
-    s_mean[i] = (float)mean;
-    s_rstd[i] = (float)(1.0 / sqrt(var + (double)eps));
+    if (grp < g.G) {
+      const float2* pw = reinterpret_cast<const float2*>(ws) + ((size_t)n * g.G + grp) * g.splits;
+      for (int k = part; k < g.splits; k += FT) { const float2 v = pw[k]; s += (double)v.x; q += (double)v.y; }
+    }
+    s_ps[tid] = s; s_pq[tid] = q;
+    __syncthreads();
+    if (part == 0 && grp < g.G) {
+      for (int j = 1; j < FT; ++j) { s += s_ps[tid + j]; q += s_pq[tid + j]; }
+      const double mean = s / cnt;
+      double var = q / cnt - mean * mean;
+      var = var > 0.0 ? var : 0.0;
+      s_mean[grp] = (float)mean;
+      s_rstd[grp] = (float)(1.0 / sqrt(var + (double)eps));
+    }
+    __syncthreads();
   }
-  __syncthreads();
-  const int per = (g.HW + g.splits - 1) / g.splits;
+  const int per = (g.HW + g.asplits - 1) / g.asplits;
   const int p0 = split * per, p1 = min(g.HW, p0 + per);
   const int tx = tid % g.NTX, ty = tid / g.NTX;
   if (ty >= g.PL) return;
@@ -255,11 +271,24 @@ __global__ __launch_bounds__(GN_THREADS) void gn_apply_nchw(const bf16_t* __rest
 }
 
 int gn_splits_nhwc(long N, long HW) {
-  long s = HW / 32;  // at least 32 pixels per workgroup
+  // Statistics pass: every workgroup of the apply pass folds all of a sample's partial sums, so there should be
+  // few of them: at most 64 workgroups per sample, each with 16 loads per thread in flight (as many bytes in
+  // flight as four times the workgroups with four loads each), at least 32 pixels per workgroup.
+  long s = HW / 32;
   if (s < 1) s = 1;
-  const long cap = (2048 + N - 1) / N;  // enough workgroups to cover 256 CUs several times
+  const long cap = (256 + N - 1) / N;  // one workgroup per CU is enough at this depth
   if (s > cap) s = cap;
-  if (s > 256) s = 256;
+  if (s > 64) s = 64;
+  return (int)s;
+}
+int gn_apply_splits_nhwc(long N, long HW) {
+  // about 1024 workgroups in all (4 per CU: a latency-bound stream fills HBM by having more of itself in flight),
+  // but at least 4 pixels each
+  long per = (N * HW + 1023) / 1024;
+  if (per < 4) per = 4;
+  long s = (HW + per - 1) / per;
+  if (s < 1) s = 1;
+  if (s > 4096) s = 4096;
   return (int)s;
 }
 int gn_splits_nchw(long rows, long row_len) {
@@ -367,13 +396,14 @@ KH_EXPORT int kh_group_norm_bf16(const void* x, void* y, const void* gamma, cons
     while (g.CP % ntx != 0) --ntx;
     g.NTX = ntx; g.CPT = g.CP / ntx; g.PL = GN_THREADS / ntx;
     if (g.CPT > GN_MAX_CPT) return KH_ERR_UNSUPPORTED;
-    dim3 grid((unsigned)g.splits, (unsigned)N);
+    g.asplits = gn_apply_splits_nhwc(N, HW);
+    dim3 grid((unsigned)g.splits, (unsigned)N), agrid((unsigned)g.asplits, (unsigned)N);
     const size_t lds = (size_t)2 * g.PL * g.C * sizeof(float);
     kh_launch(KH_TAG_GN_STATS, gn_stats_nhwc, grid, dim3(GN_THREADS), lds, s, xp, ap, workspace, g);
     if (activation == 1)
-      kh_launch(KH_TAG_GN_APPLY, gn_apply_nhwc<true>, grid, dim3(GN_THREADS), 0, s, xp, yp, gp, bp, ap, workspace, g, eps);
+      kh_launch(KH_TAG_GN_APPLY, gn_apply_nhwc<true>, agrid, dim3(GN_THREADS), 0, s, xp, yp, gp, bp, ap, workspace, g, eps);
     else
-      kh_launch(KH_TAG_GN_APPLY, gn_apply_nhwc<false>, grid, dim3(GN_THREADS), 0, s, xp, yp, gp, bp, ap, workspace, g, eps);
+      kh_launch(KH_TAG_GN_APPLY, gn_apply_nhwc<false>, agrid, dim3(GN_THREADS), 0, s, xp, yp, gp, bp, ap, workspace, g, eps);
   } else {
     const long Cg = C / G, row_len = Cg * HW, rows = N * G;
     if (HW % 8 != 0) return KH_ERR_UNSUPPORTED;
