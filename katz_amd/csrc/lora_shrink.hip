@@ -170,8 +170,8 @@ KH_EXPORT int kh_lora_shrink_bf16(const void* x, const void* a_cat, const float*
   p.x = (const bf16_t*)x; p.a_cat = (const bf16_t*)a_cat; p.col_scale = col_scale; p.t = (bf16_t*)t;
   p.M = (int)M; p.K = (int)K; p.R = (int)R;
   hipStream_t s = (hipStream_t)stream;
-  // the largest output tile that still gives every CU a workgroup
-  if (R % 64 == 0 && ((M + 63) / 64) * (R / 64) >= 256) return launch_shrink_k<2, 2, 4, 5>(p, s);
+  // the largest output tile that still gives most CUs a workgroup (a 64x64 tile reads half the bytes per output of a 32x64 one)
+  if (R % 64 == 0 && ((M + 63) / 64) * (R / 64) >= 160) return launch_shrink_k<2, 2, 4, 5>(p, s);
   if (R % 64 == 0 && ((M + 31) / 32) * (R / 64) >= 256) return launch_shrink_k<1, 2, 4, 5>(p, s);
   return launch_shrink_k<1, 1, 8, 5>(p, s);
 }
