@@ -606,18 +606,9 @@ int lora_gemm_pipe_launch_grouped(const LoraGemmParams& p, int n_groups, hipStre
 int lora_gemm_pipe_launch(const LoraGemmParams& p, int tile_sel, hipStream_t stream) {
   switch (tile_sel) {
     case 16: return launch_prank<128, 128, 2, 2, 4>(p, stream);
-    case 17: return launch_prank<128, 128, 2, 2, 3>(p, stream);
-    case 18: return launch_prank<128, 128, 2, 2, 2>(p, stream);
     case 20: return deep_stage_ok(p) ? launch_pcfg<PCfg<128, 128, 2, 2, 0, 3, 64>>(p, stream) : KH_ERR_UNSUPPORTED;
-    case 21: return deep_stage_ok(p) ? launch_pcfg<PCfg<128, 128, 2, 2, 0, 2, 64>>(p, stream) : KH_ERR_UNSUPPORTED;
-    case 24: return plain_ok(p) ? launch_pcfg<PCfg<128, 256, 2, 2, 0, 3>>(p, stream) : KH_ERR_UNSUPPORTED;
-    case 25: return plain_ok(p) ? launch_pcfg<PCfg<128, 256, 2, 2, 0, 4>>(p, stream) : KH_ERR_UNSUPPORTED;
-    case 26: return plain_ok(p) ? launch_pcfg<PCfg<256, 128, 2, 2, 0, 3>>(p, stream) : KH_ERR_UNSUPPORTED;
     case 27: return plain_ok(p) ? launch_pcfg<PCfg<256, 128, 4, 2, 0, 4>>(p, stream) : KH_ERR_UNSUPPORTED;
     case 28: return plain_ok(p) ? launch_pcfg<PCfg<128, 256, 2, 4, 0, 4>>(p, stream) : KH_ERR_UNSUPPORTED;
-    case 29: return deep_stage_ok(p) ? launch_pcfg<PCfg<256, 128, 4, 2, 0, 3, 64>>(p, stream) : KH_ERR_UNSUPPORTED;
-    case 30: return plain_ok(p) ? launch_pcfg<PCfg<256, 256, 4, 2, 0, 3>>(p, stream) : KH_ERR_UNSUPPORTED;
-    case 31: return plain_ok(p) ? launch_pcfg<PCfg<256, 256, 4, 2, 0, 4>>(p, stream) : KH_ERR_UNSUPPORTED;
     case 32: return deep_stage_ok(p) ? launch_pcfg<PCfg<128, 128, 2, 4, 0, 3, 64>>(p, stream) : KH_ERR_UNSUPPORTED;
     default: break;
   }

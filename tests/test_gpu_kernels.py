@@ -78,7 +78,7 @@ LORA_SHAPES = [
 ]
 
 
-@pytest.mark.parametrize("tile", [1, 2])
+@pytest.mark.parametrize("tile", [0, 1, 2])
 @pytest.mark.parametrize("case", LORA_SHAPES, ids=lambda c: f"M{c[0]}N{c[1]}K{c[2]}r{'+'.join(map(str, c[3])) or '0'}")
 def test_lora_linear_bf16(case, tile):
     M, N, K, ranks, scales, bias, residual = case
@@ -681,3 +681,30 @@ def test_conv3x3_module_pads_small_channel_counts(cin, cout):
     assert [c[0] for c in log] == ["conv3x3", "conv3x3"], "the module must run the katz_hip kernel"
     assert y.shape == ref.shape and torch.equal(y, y2)
     assert_close_rel(y, ref, REL_BF16, "conv3x3 with padded channels")
+
+
+@pytest.mark.parametrize("tile", [16, 20, 27, 28, 32])
+@pytest.mark.parametrize("shape", [(384, 512, 256, 64), (1000, 328, 640, 0), (2048, 1280, 1280, 128)])
+def test_pipelined_gemm_tile_variants(tile, shape):
+    """Every tile configuration of the pipelined kernel (plain and with the rank columns as extra K tiles, bias,
+    residual, ragged M / N) against the oracle."""
+    from katz_amd import ops
+
+    M, N, K, R = shape
+    say("tile variant", tile, shape)
+    d = dev()
+    g = torch.Generator().manual_seed(tile * 7 + M)
+    x, w, b, res = randn(g, M, K), randn(g, N, K, std=0.03), randn(g, N), randn(g, M, N)
+    xd, wd, bd, rd = (t.to(d, BF) for t in (x, w, b, res))
+    if R == 0:
+        y = ops.lora_linear(xd, wd, bd, residual=rd, tile=tile)
+        ref = O.lora_linear(xd.float().cpu(), wd.float().cpu(), bd.float().cpu(), [], residual=rd.float().cpu())
+    else:
+        A, B = randn(g, R, K, std=0.05), randn(g, N, R, std=0.05)
+        Ad, Bd = A.to(d, BF), B.to(d, BF)
+        t = ops.lora_shrink(xd, Ad, torch.full((R,), 0.7, device=d))
+        y = ops.lora_linear_pre(xd, wd, bd, t, Bd, residual=rd, tile=tile)
+        ref = O.lora_linear(xd.float().cpu(), wd.float().cpu(), bd.float().cpu(), [(Ad.float().cpu(), Bd.float().cpu(), 0.7)],
+                            residual=rd.float().cpu())
+    torch.cuda.synchronize()
+    assert_close_rel(y, ref, REL_BF16, f"tile {tile} {shape}")
