@@ -148,47 +148,99 @@ def cpu_baseline(cores):
     with torch.no_grad():
         blk(x, temb, ctx)  # warm-up
         ts = []
-        for _ in range(3):
+        for _ in range(7):   # ~15 s of CPU work in all
             t0 = time.perf_counter()
             blk(x, temb, ctx)
             ts.append(time.perf_counter() - t0)
     ts.sort()
-    return ts[1], flops
+    return ts[len(ts) // 2], flops
 
 
 # HBM-side bytes of the largest LoRA GEMM launch, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on
-# `bench.py --traffic-probe` and calibrated against a copy of known size (summary under profiles/)
+# `bench.py --kernel-probe` and calibrated against a copy of known size (summary under profiles/)
 GEMM_TRAFFIC_BYTES = 164.7e6
 
 
-def traffic_probe():
-    """Counter calibration run: a device copy of known size (64 MiB read + 64 MiB written), then the largest
-    LoRA linear of the step (GEGLU projection, M 2048, K 1280, N 10240, packed rank 128) as shrink + GEMM,
-    three times.  Under `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE` the copy gives the factor between
-    the counter and bytes; the GEMM rows give its HBM traffic per launch."""
+def kernel_probe():
+    """Counter / trace run of the individual kernels at the shapes of BASELINE.json's configurations, three times
+    each, preceded by a 64 MiB device copy of known size (the calibration of FETCH_SIZE / WRITE_SIZE).
+    Used as  rocprofv3 --kernel-trace --stats -- python3 bench.py --kernel-probe  (durations) and
+    rocprofv3 --pmc <counter> -- python3 bench.py --kernel-probe  (one counter per run).  Prints, as JSON, the
+    algorithmic FLOPs / bytes of every probed launch in launch order."""
     import torch
     from katz_amd import ops
 
     dev = torch.device("cuda:0")
+    bf = torch.bfloat16
     g = torch.Generator(device=dev).manual_seed(0)
+    rn = lambda *s, std=1.0: (torch.randn(*s, device=dev, generator=g) * std).to(bf)
+    cl = lambda t: t.contiguous(memory_format=torch.channels_last)
     src = torch.randn(16 << 20, device=dev, generator=g)            # 64 MiB fp32
     dst = torch.empty_like(src)
-    M, K, N, R = 2048, 1280, 10240, 128
-    x = torch.randn(M, K, device=dev, generator=g).to(torch.bfloat16)
-    w = (torch.randn(N, K, device=dev, generator=g) * 0.02).to(torch.bfloat16)
-    b = torch.randn(N, device=dev, generator=g).to(torch.bfloat16)
-    a_cat = (torch.randn(R, K, device=dev, generator=g) * 0.02).to(torch.bfloat16)
-    b_cat = (torch.randn(N, R, device=dev, generator=g) * 0.02).to(torch.bfloat16)
-    scale = torch.full((R,), 0.8, device=dev)
+    runs, meta = [], []
+
+    def add(name, fn, flops=0.0, nbytes=0.0):
+        runs.append(fn)
+        meta.append({"kernel": name, "algorithmic_flops": flops, "algorithmic_bytes": nbytes})
+
+    # K1: largest LoRA linear (GEGLU projection) and the most frequent one (d x d), as shrink + GEMM
+    for (M, K, N, geglu) in ((2048, 1280, 10240, True), (2048, 1280, 1280, False), (8192, 640, 640, False)):
+        R = 128
+        x, w, b = rn(M, K), rn(N, K, std=0.02), rn(N)
+        a_cat, b_cat = rn(R, K, std=0.02), rn(N, R, std=0.02)
+        scale = torch.full((R,), 0.8, device=dev)
+        tbuf = torch.empty(M, R, device=dev, dtype=bf)
+        nout = N // 2 if geglu else N
+        add(f"lora_shrink M{M} K{K} R{R}", lambda x=x, a=a_cat, s=scale, t=tbuf: ops.lora_shrink(x, a, s, out=t),
+            2.0 * M * K * R, 2.0 * (M * K + R * K + M * R))
+        add(f"lora_gemm M{M} K{K} N{N} R{R}{' geglu' if geglu else ''}",
+            lambda x=x, w=w, b=b, t=tbuf, bc=b_cat, ge=geglu: ops.lora_linear_pre(x, w, b, t, bc, geglu=ge),
+            2.0 * M * N * (K + R), 2.0 * (M * K + K * N + M * nout + R * N + M * R))
+    # K3: attention at the three SDXL shapes
+    for (B, H, T, S) in ((2, 10, 4096, 4096), (2, 20, 1024, 1024), (2, 20, 1024, 77)):
+        q, k, v = rn(B, T, H * 64), rn(B, S, H * 64), rn(B, S, H * 64)
+        add(f"attention B{B} H{H} T{T} S{S}", lambda q=q, k=k, v=v, H=H: ops.attention(q, k, v, H),
+            4.0 * B * H * T * S * 64, 2.0 * 64 * B * H * (2 * T + 2 * S))
+    # K2: segmented shrink / expand, 8 requests x 4096 tokens, d = 640, one adapter each (ranks 8 .. 128)
+    T, dm, RP = 4096, 640, 128
+    ranks = [64, 8, 128, 32, 16, 64, 128, 32]
+    x = rn(8 * T, dm)
+    a_all, b_all = torch.zeros(8, RP, dm, device=dev, dtype=bf), torch.zeros(8, dm, RP, device=dev, dtype=bf)
+    for i, r in enumerate(ranks):
+        a_all[i, :r] = rn(r, dm, std=0.02)
+        b_all[i, :, :r] = rn(dm, r, std=0.02)
+    ss = torch.arange(0, 9 * T, T, dtype=torch.int32, device=dev)
+    sa = torch.arange(8, dtype=torch.int32, device=dev)
+    rp = torch.tensor([(r + 31) // 32 * 32 for r in ranks], dtype=torch.int32, device=dev)
+    sc = torch.full((8,), 0.7, device=dev)
+    y = rn(8 * T, dm)
+    tb = torch.zeros(8 * T, RP, device=dev, dtype=bf)
+    sr = float(sum(ranks))
+    add("sgmv_shrink 8x4096x640", lambda: ops.sgmv_shrink(x, a_all, ss, sa, rp, T, out=tb), 2.0 * T * dm * sr,
+        2.0 * (8 * T * dm + sr * dm + T * sr))
+    add("sgmv_expand 8x4096x640", lambda: ops.sgmv_expand_(y, tb, b_all, ss, sa, rp, sc, T), 2.0 * T * dm * sr,
+        2.0 * (T * sr + sr * dm + 2 * 8 * T * dm))
+    # K4 / K5: norms and the ControlNet residual injection
+    xg, gam, bet = cl(rn(2, 320, 128, 128)), rn(320), rn(320)
+    add("group_norm+silu 2x320x128x128 nhwc", lambda: ops.group_norm(xg, 32, gam, bet, 1e-5, "silu"), 0.0, 4.0 * xg.numel())
+    xl, gl, bl = rn(2048, 1280), rn(1280), rn(1280)
+    add("layer_norm 2048x1280", lambda: ops.layer_norm(xl, gl, bl), 0.0, 4.0 * xl.numel())
+    h, skip, res = cl(rn(2, 320, 128, 128)), cl(rn(2, 320, 128, 128)), cl(rn(2, 320, 128, 128, std=0.1))
+    add("concat_residual 2x(320+320)x128x128", lambda: ops.concat_residual(h, skip, [res]), 0.0, 2.0 * (3 + 2) * h.numel())
+    mid, rmid = cl(rn(2, 1280, 32, 32)), cl(rn(2, 1280, 32, 32, std=0.1))
+    add("residual_add 2x1280x32x32", lambda: ops.residual_add_(mid, [rmid]), 0.0, 2.0 * 3 * mid.numel())
+    # K1c: a 3x3 convolution of the 64x64 level
+    xc, wc, bc = cl(rn(2, 640, 64, 64)), ops.pack_conv3x3_weight(rn(640, 640, 3, 3, std=0.01)), rn(640)
+    add("conv3x3 640->640 @64x64", lambda: ops.conv3x3(xc, wc, bc), 2.0 * 8192 * 640 * 5760,
+        2.0 * (xc.numel() + wc.numel() + 8192 * 640))
     torch.cuda.synchronize()
     for _ in range(3):
         dst.copy_(src)
-        t = ops.lora_shrink(x, a_cat, scale)
-        ops.lora_linear_pre(x, w, b, t, b_cat, geglu=True)
+        for fn in runs:
+            fn()
     torch.cuda.synchronize()
-    print(json.dumps({"traffic_probe": {"copy_bytes_read": src.numel() * 4, "copy_bytes_written": src.numel() * 4,
-                                        "gemm": {"M": M, "N": N, "K": K, "R": R, "geglu": True},
-                                        "algorithmic_bytes": 2 * (M * K + K * N + M * N // 2 + R * (K + N))}}))
+    print(json.dumps({"kernel_probe": {"copy_bytes_read": src.numel() * 4, "copy_bytes_written": src.numel() * 4,
+                                       "launches_per_round": meta, "rounds": 3}}))
 
 
 def main():
@@ -197,8 +249,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--traffic-probe", action="store_true",
-                    help="run only a 64 MiB copy and the dominant LoRA GEMM shape a few times (for rocprofv3 --pmc)")
+    ap.add_argument("--kernel-probe", action="store_true",
+                    help="run only a 64 MiB copy and each kernel at its BASELINE shapes three times (for rocprofv3)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU only (no collectives, no sharding); --gpus must be 1",
@@ -208,8 +260,8 @@ def main():
     import torch
     from katz_amd.graph import GraphedUNetStep
 
-    if args.traffic_probe:
-        traffic_probe()
+    if args.kernel_probe:
+        kernel_probe()
         return
 
     if not torch.cuda.is_available():
@@ -298,7 +350,7 @@ def main():
         "roofline": {"kernel": "lora_gemm_kernel (fused base GEMM + LoRA delta, all launches of one step)",
                      "bound": "mfma", "achieved": round(achieved_tf, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved_tf / PEAK_BF16_TFLOPS, 4), "traffic": GEMM_TRAFFIC_BYTES,
-                     "traffic_note": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of `bench.py --traffic-probe`, largest launch "
+                     "traffic_note": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of `bench.py --kernel-probe`, largest launch "
                                      "(M 2048, K 1280, N 10240, R 128): 143.7 MB read + 21.0 MB written; algorithmic 55.4 MB",
                      "launches_per_step": len(gemm_ms), "shrink_launches_per_step": len(shrink_calls),
                      "shrink_ms_per_step": round(shrink_ms, 3), "avg_launch_us": round(gemm_total_ms / len(gemm_ms) * 1e3, 2),

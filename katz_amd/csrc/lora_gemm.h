@@ -22,6 +22,12 @@ struct LoraGemmParams {
   // tile -> XCD map (xg_n > 0): the 8 XCDs form an xg_m x xg_n grid over the tile matrix, each owning a block of
   // xr_m x xr_n tiles (see launch_pcfg); 0: contiguous ranges of the (m block, n chunk) list per XCD
   int xg_n, xr_m, xr_n;
+  // segmented launch (sg_mode != 0): blockIdx.y = segment s of a batch of requests; rows [sg_start[s], sg_start[s+1])
+  // of x / y, weights of adapter sg_adapter[s] (negative: the segment is skipped) at w + adapter * sg_wstride.
+  // sg_mode 1 (shrink): y = x . W_a^T.  sg_mode 2 (expand): y += sg_scale[a] * (x . W_a^T) over the first
+  // sg_rank[a] K columns (x = the shrink result, row stride K).  M = the longest segment.
+  const int32_t* sg_start; const int32_t* sg_adapter; const int32_t* sg_rank; const float* sg_scale;
+  int sg_mode; long sg_wstride;
   int geglu;                                // 1: W rows are (value,gate) interleaved in 32-column groups, y is [M,N/2]
   // 3x3 convolution as an implicit GEMM (conv_cin > 0): x is an NHWC image [Nb, conv_h, conv_w, conv_cin], row m
   // of the GEMM is output pixel m of [Nb, conv_ho, conv_wo], K = 9 * conv_cin ordered (kh, kw, ci), padding 1
@@ -32,5 +38,7 @@ struct LoraGemmParams {
 int lora_gemm_pipe_launch(const LoraGemmParams& p, int tile_sel, hipStream_t stream);
 // 3x3 convolution (conv_* fields set, R == 0, K == 9 * conv_cin, conv_cin % 32 == 0).
 int lora_gemm_pipe_launch_conv(const LoraGemmParams& p, hipStream_t stream);
+// Segmented multi-adapter form (sg_* fields set; plain GEMM per segment, K % 32 == 0).
+int lora_gemm_pipe_launch_sgmv(const LoraGemmParams& p, int n_segments, hipStream_t stream);
 // Grouped form: grid.y = n_groups, per-group pointers from p.grp; rank columns (p.R > 0) as extra K tiles.
 int lora_gemm_pipe_launch_grouped(const LoraGemmParams& p, int n_groups, hipStream_t stream);

@@ -484,6 +484,7 @@ KH_EXPORT int kh_lora_linear_bf16(const void* x, const void* w, const void* bias
   p.m_tiles = p.n_tiles = p.n_chunk = p.n_chunks = 0;
   p.geglu = geglu ? 1 : 0;
   p.xg_n = p.xr_m = p.xr_n = 0;
+  p.sg_start = p.sg_adapter = p.sg_rank = nullptr; p.sg_scale = nullptr; p.sg_mode = 0; p.sg_wstride = 0;
   p.conv_cin = p.conv_h = p.conv_w = p.conv_ho = p.conv_wo = p.conv_stride = 0;
   p.dbg = (flags >> 16) & 0xff;
   hipStream_t s = (hipStream_t)stream;
@@ -519,6 +520,7 @@ KH_EXPORT int kh_lora_linear_pre_bf16(const void* x, const void* w, const void* 
   p.m_tiles = p.n_tiles = p.n_chunk = p.n_chunks = 0;
   p.geglu = geglu ? 1 : 0;
   p.xg_n = p.xr_m = p.xr_n = 0;
+  p.sg_start = p.sg_adapter = p.sg_rank = nullptr; p.sg_scale = nullptr; p.sg_mode = 0; p.sg_wstride = 0;
   p.conv_cin = p.conv_h = p.conv_w = p.conv_ho = p.conv_wo = p.conv_stride = 0;
   return lora_gemm_pipe_launch(p, (flags >> 8) & 0xff, (hipStream_t)stream);
 }
@@ -544,9 +546,29 @@ KH_EXPORT int kh_conv3x3_nhwc_bf16(const void* x, const void* w, const void* bia
   p.m_tiles = p.n_tiles = p.n_chunk = p.n_chunks = 0;
   p.geglu = 0;
   p.xg_n = p.xr_m = p.xr_n = 0;
+  p.sg_start = p.sg_adapter = p.sg_rank = nullptr; p.sg_scale = nullptr; p.sg_mode = 0; p.sg_wstride = 0;
   p.conv_cin = (int)Cin; p.conv_h = (int)H; p.conv_w = (int)W; p.conv_ho = (int)Ho; p.conv_wo = (int)Wo;
   p.conv_stride = (int)stride;
   return lora_gemm_pipe_launch_conv(p, (hipStream_t)stream);
+}
+
+// The segmented multi-adapter kernels (sgmv.hip) run on the pipelined GEMM when the shapes allow.
+int kh_sgmv_on_gemm(int mode, const void* x, const void* w_all, void* y, const int32_t* seg_start, const int32_t* seg_adapter,
+                    const int32_t* adapter_rank, const float* adapter_scale, int64_t n_segments, int64_t max_seg_rows,
+                    int64_t N, int64_t K, int64_t w_stride, hipStream_t stream) {
+  LoraGemmParams p;
+  p.x = (const bf16_t*)x; p.w = (const bf16_t*)w_all; p.bias = nullptr;
+  p.a_cat = nullptr; p.b_cat = nullptr; p.col_scale = nullptr;
+  p.t_ext = nullptr; p.ldt = 0; p.grp = nullptr; p.dbg = 0; p.t_nsplit = 0;
+  p.res = nullptr; p.y = (bf16_t*)y;
+  p.M = (int)max_seg_rows; p.N = (int)N; p.K = (int)K; p.R = 0;
+  p.m_tiles = p.n_tiles = p.n_chunk = p.n_chunks = 0;
+  p.geglu = 0;
+  p.xg_n = p.xr_m = p.xr_n = 0;
+  p.conv_cin = p.conv_h = p.conv_w = p.conv_ho = p.conv_wo = p.conv_stride = 0;
+  p.sg_start = seg_start; p.sg_adapter = seg_adapter; p.sg_rank = adapter_rank; p.sg_scale = adapter_scale;
+  p.sg_mode = mode; p.sg_wstride = (long)w_stride;
+  return lora_gemm_pipe_launch_sgmv(p, (int)n_segments, stream);
 }
 
 // Many layers that share one input in one launch; see include/katz_hip.h.
@@ -566,6 +588,7 @@ KH_EXPORT int kh_lora_linear_grouped_bf16(const void* x, const uint64_t* table, 
   p.m_tiles = p.n_tiles = p.n_chunk = p.n_chunks = 0;
   p.geglu = 0;
   p.xg_n = p.xr_m = p.xr_n = 0;
+  p.sg_start = p.sg_adapter = p.sg_rank = nullptr; p.sg_scale = nullptr; p.sg_mode = 0; p.sg_wstride = 0;
   p.conv_cin = p.conv_h = p.conv_w = p.conv_ho = p.conv_wo = p.conv_stride = 0;
   return lora_gemm_pipe_launch_grouped(p, (int)n_groups, (hipStream_t)stream);
 }

@@ -270,6 +270,22 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
     p.t_ext = reinterpret_cast<const bf16_t*>(g[3]);
     p.y = reinterpret_cast<bf16_t*>(g[4]);
   }
+  float oscale = 1.f;   // segmented expand: the adapter's scale on the product
+  int k_cols = p.K;     // K columns the loop covers (the row stride stays p.K)
+  if (pin.sg_mode != 0) {
+    const int sg = blockIdx.y;
+    const int r0 = pin.sg_start[sg], r1 = pin.sg_start[sg + 1], ad = pin.sg_adapter[sg];
+    if (ad < 0 || r1 <= r0) return;   // a request without an adapter keeps its base projection untouched
+    p.M = r1 - r0;
+    p.x = pin.x + (size_t)r0 * pin.K;
+    p.w = pin.w + (size_t)ad * pin.sg_wstride;
+    p.y = pin.y + (size_t)r0 * pin.N;
+    if (pin.sg_mode == 2) {
+      p.res = p.y;                    // read-modify-write of y: every element is read and written by one thread
+      oscale = pin.sg_scale[ad];
+      k_cols = pin.sg_rank[ad];
+    }
+  }
   constexpr int BM = C::BM, BN = C::BN, TM = C::TM, TN = C::TN, NRT = C::NRT, R = C::R, NST = C::NST;
   constexpr int SMT = C::SM > 0 ? C::SM : 1, NRTT = NRT > 0 ? NRT : 1;
   bf16_t* sB = reinterpret_cast<bf16_t*>(smem);                // aliases the ring (after the K loop)
@@ -297,9 +313,10 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
     m_blk = logical / p.n_chunks; chunk = logical % p.n_chunks;
   }
   const int m0 = m_blk * BM;
+  if (m0 >= p.M) return;   // segmented launches size the grid for the longest segment
   const int K = p.K, M = p.M, N = p.N;
   constexpr int BKP = C::BKP, ROWB = C::ROWB;
-  const int KT1 = K / BKP;                                             // K tiles of x / W
+  const int KT1 = k_cols / BKP;                                        // K tiles of x / W
   const int KT = KT1 + (p.t_ext != nullptr ? p.R / BKP : 0);           // + rank tiles of T / B_cat (two-launch form)
 
   // DMA geometry of this lane inside a 16-row unit: LDS slot = lane (16 bytes each); it holds row
@@ -485,7 +502,7 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const int row = wm * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
-          sC[row * C::LDC + col] = (bf16_t)(acc[i][j][v] + bv[j]);
+          sC[row * C::LDC + col] = (bf16_t)(acc[i][j][v] * oscale + bv[j]);
         }
       }
       __syncthreads();
@@ -597,6 +614,13 @@ int lora_gemm_pipe_launch_conv(const LoraGemmParams& p, hipStream_t stream) {
   const long tiles = (long)((p.M + 127) / 128) * ((p.N + 127) / 128);
   if (tiles <= 256 && p.conv_cin % 64 == 0) return launch_pcfg<PCfg<128, 128, 2, 4, 0, 3, 64>, true>(p, stream);
   return launch_pcfg<PCfg<128, 128, 2, 2, 0, 4>, true>(p, stream);
+}
+
+int lora_gemm_pipe_launch_sgmv(const LoraGemmParams& p, int n_segments, hipStream_t stream) {
+  // one 128x128 tile column covers all of a shrink's rank columns.  The shrink streams long rows: whole 128-byte
+  // lines per stage and 8 waves per workgroup; the expand's K is the rank (a few 32-column tiles).
+  if (p.sg_mode == 1 && p.K % 64 == 0) return launch_pcfg<PCfg<128, 128, 2, 4, 0, 3, 64>>(p, stream, n_segments);
+  return launch_pcfg<PCfg<128, 128, 2, 2, 0, 4>>(p, stream, n_segments);
 }
 
 int lora_gemm_pipe_launch_grouped(const LoraGemmParams& p, int n_groups, hipStream_t stream) {
