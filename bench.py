@@ -158,7 +158,7 @@ def cpu_baseline(cores):
 
 # HBM-side bytes of the largest LoRA GEMM launch, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on
 # `bench.py --kernel-probe` and calibrated against a copy of known size (summary under profiles/)
-GEMM_TRAFFIC_BYTES = 164.7e6
+GEMM_TRAFFIC_BYTES = 161.0e6
 
 
 def kernel_probe():
@@ -350,8 +350,8 @@ def main():
         "roofline": {"kernel": "lora_gemm_kernel (fused base GEMM + LoRA delta, all launches of one step)",
                      "bound": "mfma", "achieved": round(achieved_tf, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved_tf / PEAK_BF16_TFLOPS, 4), "traffic": GEMM_TRAFFIC_BYTES,
-                     "traffic_note": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of `bench.py --kernel-probe`, largest launch "
-                                     "(M 2048, K 1280, N 10240, R 128): 143.7 MB read + 21.0 MB written; algorithmic 55.4 MB",
+                     "traffic_note": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of `bench.py --kernel-probe` (profiles/), largest launch "
+                                     "(M 2048, K 1280, N 10240, R 128): 140.0 MB read + 21.0 MB written; algorithmic 55.6 MB",
                      "launches_per_step": len(gemm_ms), "shrink_launches_per_step": len(shrink_calls),
                      "shrink_ms_per_step": round(shrink_ms, 3), "avg_launch_us": round(gemm_total_ms / len(gemm_ms) * 1e3, 2),
                      "algorithmic_gflop_per_step": round(gemm_flops / 1e9, 1), "by_shape": shape_rows[:8],
