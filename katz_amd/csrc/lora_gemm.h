@@ -42,3 +42,7 @@ int lora_gemm_pipe_launch_conv(const LoraGemmParams& p, hipStream_t stream);
 int lora_gemm_pipe_launch_sgmv(const LoraGemmParams& p, int n_segments, hipStream_t stream);
 // Grouped form: grid.y = n_groups, per-group pointers from p.grp; rank columns (p.R > 0) as extra K tiles.
 int lora_gemm_pipe_launch_grouped(const LoraGemmParams& p, int n_groups, hipStream_t stream);
+// Narrow-output variant (lora_gemm_ksplit.hip): (32 * row_groups) x 160 tiles, 8 waves as row_groups x k-slices;
+// plain or K-extended GEMM with bias / residual, K % 64 == 0.  row_groups 2 or 4.
+bool lora_gemm_ksplit_ok(const LoraGemmParams& p);
+int lora_gemm_ksplit_launch(const LoraGemmParams& p, int row_groups, hipStream_t stream);

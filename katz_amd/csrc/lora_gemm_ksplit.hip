@@ -1,0 +1,268 @@
+// K1, narrow-output variant: y = [x | T] . [W | B_cat]^T (+ bias, + residual) on bf16 MFMA (gfx950) with
+// (32*WM) x 160 output tiles, for layers whose 128x128 tiles would leave much of the chip idle.
+//
+// Same arithmetic as the two-launch form of lora_gemm_pipe.hip (the reference's LoRA linear,
+// diffusers-hf/src/diffusers/models/lora.py:224-225 after a separate shrink launch): T = the scaled
+// shrink result, so the adapters' rank columns are extra K tiles of the base GEMM.
+//
+// Why another tile shape: N = 1280 = 2^8 * 5.  At M = 2048 the 128x128 tiling has 160 tiles for 256 CUs;
+// 64x160 has exactly 256, 128x160 has 256 at M = 8192 / N = 640.  A factor 5 does not divide over 8
+// waves in M or N, so the waves split K instead: a workgroup's 8 waves form WM row groups of 32 rows times
+// WK = 8 / WM k-slices; a wave owns a 32 x 160 strip of accumulators (5 MFMA tiles) and multiplies only its
+// own 16-column slices of every 64-column stage (1 x fragment + 5 W fragments per 5 MFMAs).  After the K
+// loop the k-slices of a row group meet in LDS and are added in a fixed order (deterministic), then the
+// epilogue is the usual one (bias in fp32, round, transpose through LDS, residual, 16-byte row stores).
+//
+// Operand movement as in lora_gemm_pipe.hip: global -> LDS by global_load_lds (8 rows x 128 bytes per
+// instruction, XOR-swizzled pieces), a ring of 3 stages, loads two stages ahead, one barrier per stage,
+// fragments double-buffered in registers.  (32*WM + 160) / 8 DMA units per stage do not divide by 8 waves:
+// waves below N_HI issue one more than the others, and every wait picks its count by a wave-uniform branch.
+#include "kh_common.h"
+#include "lora_gemm.h"
+
+namespace {
+
+typedef const __attribute__((address_space(1))) void* gptr_t;
+typedef __attribute__((address_space(3))) void* lptr_t;
+
+template <int VM, int LGKM>
+__device__ __forceinline__ void wait_cnt() {  // gfx9 encoding: vmcnt = [15:14|3:0], expcnt = [6:4], lgkmcnt = [11:8]
+  __builtin_amdgcn_s_waitcnt((VM & 15) | (7 << 4) | ((LGKM & 15) << 8) | ((VM >> 4) << 14));
+}
+
+template <int WM_>
+struct KCfg {
+  static constexpr int WM = WM_, WK = 8 / WM_;       // row groups x k-slices = 8 waves
+  static constexpr int BM = 32 * WM, BN = 160, BK = 64, NST = 3, TN = 5;
+  static constexpr int KSW = 4 / WK;                 // 16-column MFMA steps of a stage per wave
+  static constexpr int UNITS = (BM + BN) / 8;        // DMA instructions per stage (8 rows x 128 B each)
+  static constexpr int LPS_LO = UNITS / 8, N_HI = UNITS % 8, LPS_HI = LPS_LO + (N_HI ? 1 : 0);
+  static constexpr int STAGE = (BM + BN) * 128;
+  static constexpr int RING = NST * STAGE;
+  static constexpr int PART = (WK - 1) * WM * 80 * 64 * 4;   // fp32 partial strips of the k-slices 1 .. WK-1
+  static constexpr int LDC = BN + 8;
+  static constexpr int SC = BM * LDC * 2;
+  static constexpr int LDS = RING > PART + SC ? RING : PART + SC;
+  static constexpr int OPC = BM * (BN / 8);          // 16-byte output pieces per tile
+  static constexpr int OPT = (OPC + 511) / 512;      // per thread
+  static_assert(WM == 2 || WM == 4, "row groups");
+  static_assert(LDS <= 160 * 1024, "LDS budget");
+};
+
+template <class C>
+__global__ __launch_bounds__(512, 2) void lora_gemm_ksplit_kernel(const LoraGemmParams p) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  constexpr int BM = C::BM, BN = C::BN, TN = C::TN, KSW = C::KSW, NST = C::NST, STAGE = C::STAGE;
+  constexpr int LPS_LO = C::LPS_LO, LPS_HI = C::LPS_HI, N_HI = C::N_HI;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / C::WK, wk = wave % C::WK;
+  const int l32 = lane & 31, lh = lane >> 5;
+
+  // tile of this workgroup: XCD b % 8 owns a block of xr_m x xr_n tiles (its W rows stay in its L2)
+  const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+  const int m_blk = (xcd / p.xg_n) * p.xr_m + local / p.xr_n;
+  const int n_blk = (xcd % p.xg_n) * p.xr_n + local % p.xr_n;
+  if (local / p.xr_n >= p.xr_m || m_blk >= p.m_tiles || n_blk >= p.n_tiles) return;  // padding of the grid
+  const int m0 = m_blk * BM, n0 = n_blk * BN;
+  const int M = p.M, N = p.N, K = p.K;
+  const int KT1 = K / 64;
+  const int KT = KT1 + (p.t_ext != nullptr ? p.R / 64 : 0);
+  const bool has_hi = wave < N_HI;
+
+  // DMA sources of this lane: unit u = wave + 8*q covers stage rows u*8 .. u*8+7 (x rows first, then W rows);
+  // LDS slot = lane: row lane/8, physical piece lane%8, which holds logical piece (lane%8) ^ ((row/2)%8)
+  const bf16_t* src[LPS_HI];
+  const bf16_t* src2[LPS_HI];
+#pragma unroll
+  for (int q = 0; q < LPS_HI; ++q) {
+    int u = wave + 8 * q;
+    u = u < C::UNITS ? u : C::UNITS - 1;               // never issued (has_hi), keep the address valid
+    const int r = u * 8 + (lane >> 3);
+    const int pc = ((lane & 7) ^ ((r >> 1) & 7)) * 8;
+    if (r < BM) {
+      int row = m0 + r; row = row < M ? row : M - 1;
+      src[q] = p.x + (size_t)row * K + pc;
+      src2[q] = p.t_ext == nullptr ? src[q] : p.t_ext + (size_t)row * p.ldt + pc + (p.t_nsplit > 0 ? (n0 / p.t_nsplit) * p.R : 0);
+    } else {
+      int row = n0 + r - BM; row = row < N ? row : N - 1;
+      src[q] = p.w + (size_t)row * K + pc;
+      src2[q] = p.t_ext == nullptr ? src[q] : p.b_cat + (size_t)row * p.R + pc;
+    }
+  }
+  auto issue = [&](int t, int st) {                    // K tile t into ring stage st
+    char* stage = smem + st * STAGE;
+#pragma unroll
+    for (int q = 0; q < LPS_HI; ++q) {
+      if (q < LPS_LO || has_hi) {
+        const bf16_t* g = t < KT1 ? src[q] + (size_t)t * 64 : src2[q] + (size_t)(t - KT1) * 64;
+        __builtin_amdgcn_global_load_lds((gptr_t)g, (lptr_t)(stage + (wave + 8 * q) * 1024), 16, 0, 0);
+      }
+    }
+  };
+  // wait until at most `tiles` of this wave's younger K tiles are outstanding (and its LDS reads are done)
+  auto wait_tiles1 = [&]() { if (has_hi) wait_cnt<LPS_HI, 0>(); else wait_cnt<LPS_LO, 0>(); };
+  auto wait_tiles0 = [&]() { wait_cnt<0, 0>(); };
+
+  struct Fr { bf16x8 a[KSW]; bf16x8 b[KSW][TN]; };
+  const int sw = (l32 >> 1) & 7;
+  auto read_frags = [&](int st, Fr& f) {
+    const char* s = smem + st * STAGE;
+#pragma unroll
+    for (int k = 0; k < KSW; ++k) {
+      const int po = ((2 * (wk * KSW + k) + lh) ^ sw) * 16;
+      f.a[k] = *reinterpret_cast<const bf16x8*>(s + (wm * 32 + l32) * 128 + po);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) f.b[k][j] = *reinterpret_cast<const bf16x8*>(s + (BM + j * 32 + l32) * 128 + po);
+    }
+  };
+  f32x16 acc[TN];
+#pragma unroll
+  for (int j = 0; j < TN; ++j)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
+  auto mma = [&](const Fr& f) {
+#pragma unroll
+    for (int k = 0; k < KSW; ++k)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a[k], f.b[k][j], acc[j], 0, 0, 0);
+  };
+
+  // bias of this lane's columns, requested before the loop
+  float bv[TN];
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int col = n0 + j * 32 + l32;
+    bv[j] = (p.bias != nullptr && col < N) ? (float)p.bias[col] : 0.f;
+  }
+  wait_cnt<0, 15>();
+
+  // K loop.  Iteration t: tile t is in registers (f_cur); tile t+1 becomes visible at the barrier, after which
+  // every wave has read tile t out of its stage, so that stage takes tile t+3.
+  Fr f0, f1;
+  issue(0, 0);
+  if (KT > 1) issue(1, 1);
+  if (KT > 1) wait_tiles1(); else wait_tiles0();
+  __builtin_amdgcn_s_barrier();
+  if (KT > 2) issue(2, 2);
+  read_frags(0, f0);
+  int st_next = 1, st_fill = 0;                        // stage of tile t+1, stage that tile t+3 refills (= stage of tile t)
+  auto step = [&](int t, const Fr& cur, Fr& nxt) {
+    if (t + 1 < KT) {
+      if (t + 2 < KT) wait_tiles1(); else wait_tiles0();
+      __builtin_amdgcn_s_barrier();
+      if (t + 3 < KT) issue(t + 3, st_fill);
+      read_frags(st_next, nxt);
+    }
+    mma(cur);
+    st_fill = st_next;
+    st_next = st_next + 1 == NST ? 0 : st_next + 1;
+  };
+  int t = 0;
+  for (; t + 1 < KT; t += 2) {
+    step(t, f0, f1);
+    step(t + 1, f1, f0);
+  }
+  if (t < KT) step(t, f0, f1);
+  __syncthreads();   // the ring is dead: partial strips and the staging tile reuse it
+
+  // residual pieces of this thread, requested before the reduction
+  u32x4 rr[C::OPT];
+  if (p.res != nullptr) {
+#pragma unroll
+    for (int q = 0; q < C::OPT; ++q) {
+      const int c = tid + q * 512, srow = c / (BN / 8), ch = c % (BN / 8);
+      const int grow = m0 + srow, gcol = n0 + ch * 8;
+      rr[q] = (c < C::OPC && grow < M && gcol < N) ? *reinterpret_cast<const u32x4*>(p.res + (size_t)grow * N + gcol)
+                                                  : u32x4{0, 0, 0, 0};
+    }
+  }
+  // k-slices 1 .. WK-1 hand their strips to slice 0 of their row group: 20 x 16 bytes per lane, lane-contiguous
+  // (writer lane = reader lane, so the layout is free)
+  f32x4* part = reinterpret_cast<f32x4*>(smem);
+  if (wk > 0) {
+    f32x4* dst = part + ((size_t)((wk - 1) * C::WM + wm) * 20) * 64 + lane;
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+        dst[(j * 4 + g) * 64] = f32x4{acc[j][4 * g], acc[j][4 * g + 1], acc[j][4 * g + 2], acc[j][4 * g + 3]};
+  }
+  __syncthreads();
+  bf16_t* sC = reinterpret_cast<bf16_t*>(smem + C::PART);
+  if (wk == 0) {
+#pragma unroll
+    for (int s = 1; s < C::WK; ++s) {                  // fixed order: deterministic
+      const f32x4* srcp = part + ((size_t)((s - 1) * C::WM + wm) * 20) * 64 + lane;
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const f32x4 v = srcp[(j * 4 + g) * 64];
+          acc[j][4 * g] += v[0]; acc[j][4 * g + 1] += v[1]; acc[j][4 * g + 2] += v[2]; acc[j][4 * g + 3] += v[3];
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int col = j * 32 + l32;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int row = wm * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+        sC[row * C::LDC + col] = (bf16_t)(acc[j][v] + bv[j]);
+      }
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int q = 0; q < C::OPT; ++q) {
+    const int c = tid + q * 512, srow = c / (BN / 8), ch = c % (BN / 8);
+    const int grow = m0 + srow, gcol = n0 + ch * 8;
+    if (c < C::OPC && grow < M && gcol < N) {
+      u32x4 o = *reinterpret_cast<const u32x4*>(sC + srow * C::LDC + ch * 8);
+      if (p.res != nullptr) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          o[e] = pack_bf16x2(bf16_lo(o[e]) + bf16_lo(rr[q][e]), bf16_hi(o[e]) + bf16_hi(rr[q][e]));
+      }
+      *reinterpret_cast<u32x4*>(p.y + (size_t)grow * N + gcol) = o;
+    }
+  }
+}
+
+template <class C>
+int launch_ksplit(LoraGemmParams p, hipStream_t stream) {
+  p.m_tiles = (p.M + C::BM - 1) / C::BM;
+  p.n_tiles = (p.N + C::BN - 1) / C::BN;
+  static bool attr_done = false;  // per template instantiation
+  if (!attr_done) {
+    hipError_t e = hipFuncSetAttribute((const void*)lora_gemm_ksplit_kernel<C>, hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS);
+    if (e != hipSuccess) return (int)e;
+    attr_done = true;
+  }
+  // the XCD grid whose per-XCD block touches the fewest operand rows, padding counted as cost
+  double best = 0;
+  p.xg_n = 0;
+  for (int gm = 1; gm <= 8; gm *= 2) {
+    const int gn = 8 / gm;
+    const int rm = (p.m_tiles + gm - 1) / gm, rn = (p.n_tiles + gn - 1) / gn;
+    const double cost = ((double)rm * C::BM + (double)rn * C::BN) * (8.0 * rm * rn) / ((double)p.m_tiles * p.n_tiles);
+    if (p.xg_n == 0 || cost < best) { best = cost; p.xg_n = gn; p.xr_m = rm; p.xr_n = rn; }
+  }
+  const unsigned grid = 8u * (unsigned)p.xr_m * (unsigned)p.xr_n;
+  kh_launch(KH_TAG_LORA_GEMM, lora_gemm_ksplit_kernel<C>, dim3(grid), dim3(512), C::LDS, stream, p);
+  KH_RETURN_LAST_ERROR();
+}
+
+}  // namespace
+
+bool lora_gemm_ksplit_ok(const LoraGemmParams& p) {
+  const bool plain = p.R == 0 || p.t_ext != nullptr;
+  return plain && p.grp == nullptr && p.sg_mode == 0 && p.conv_cin == 0 && !p.geglu && p.K % 64 == 0 && p.K >= 64 &&
+         (p.t_ext == nullptr || (p.R % 64 == 0 && p.ldt % 8 == 0)) && (p.t_nsplit == 0 || p.t_nsplit % 160 == 0) &&
+         p.N % 8 == 0;
+}
+
+int lora_gemm_ksplit_launch(const LoraGemmParams& p, int row_groups, hipStream_t stream) {
+  if (!lora_gemm_ksplit_ok(p)) return KH_ERR_UNSUPPORTED;
+  return row_groups == 4 ? launch_ksplit<KCfg<4>>(p, stream) : launch_ksplit<KCfg<2>>(p, stream);
+}

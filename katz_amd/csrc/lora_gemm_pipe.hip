@@ -634,6 +634,8 @@ int lora_gemm_pipe_launch(const LoraGemmParams& p, int tile_sel, hipStream_t str
     case 27: return plain_ok(p) ? launch_pcfg<PCfg<256, 128, 4, 2, 0, 4>>(p, stream) : KH_ERR_UNSUPPORTED;
     case 28: return plain_ok(p) ? launch_pcfg<PCfg<128, 256, 2, 4, 0, 4>>(p, stream) : KH_ERR_UNSUPPORTED;
     case 32: return deep_stage_ok(p) ? launch_pcfg<PCfg<128, 128, 2, 4, 0, 3, 64>>(p, stream) : KH_ERR_UNSUPPORTED;
+    case 40: return lora_gemm_ksplit_launch(p, 2, stream);
+    case 41: return lora_gemm_ksplit_launch(p, 4, stream);
     default: break;
   }
   // Default choice.  The limiter is the vector L1 path (every operand byte enters LDS through it), so
@@ -643,6 +645,15 @@ int lora_gemm_pipe_launch(const LoraGemmParams& p, int tile_sel, hipStream_t str
   // two workgroups per CU otherwise.
   if (plain_ok(p)) {
     const long tiles = (long)((p.M + 127) / 128) * ((p.N + 127) / 128);
+    // N a multiple of 160 and a tile count that leaves 128x128 tiles with a ragged last round: 160-column tiles
+    // (8 waves splitting K) give every CU exactly one.  64-row tiles pay for their extra operand traffic only
+    // on long K.
+    if (p.N % 160 == 0 && lora_gemm_ksplit_ok(p)) {
+      const long n160 = p.N / 160;
+      if (tiles > 256 && tiles <= 384 && (long)((p.M + 127) / 128) * n160 <= 256) return lora_gemm_ksplit_launch(p, 4, stream);
+      if (tiles <= 192 && (long)((p.M + 63) / 64) * n160 <= 256 && (long)((p.M + 63) / 64) * n160 > tiles && p.K >= 2560)
+        return lora_gemm_ksplit_launch(p, 2, stream);
+    }
     if (tiles >= 480 && p.K >= 1024 && !p.geglu) return launch_pcfg<PCfg<256, 128, 4, 2, 0, 4>>(p, stream);
     if (tiles <= 256 && p.M >= 1024 && deep_stage_ok(p)) return launch_pcfg<PCfg<128, 128, 2, 4, 0, 3, 64>>(p, stream);
   }

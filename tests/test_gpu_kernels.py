@@ -683,11 +683,13 @@ def test_conv3x3_module_pads_small_channel_counts(cin, cout):
     assert_close_rel(y, ref, REL_BF16, "conv3x3 with padded channels")
 
 
-@pytest.mark.parametrize("tile", [16, 20, 27, 28, 32])
-@pytest.mark.parametrize("shape", [(384, 512, 256, 64), (1000, 328, 640, 0), (2048, 1280, 1280, 128)])
+@pytest.mark.parametrize("tile", [0, 16, 20, 27, 28, 32, 40, 41])
+@pytest.mark.parametrize("shape", [(384, 512, 256, 64), (1000, 328, 640, 0), (2048, 1280, 1280, 128),
+                                   (6600, 640, 640, 128), (1000, 1280, 2560, 64), (70, 168, 64, 0)])
 def test_pipelined_gemm_tile_variants(tile, shape):
-    """Every tile configuration of the pipelined kernel (plain and with the rank columns as extra K tiles, bias,
-    residual, ragged M / N) against the oracle."""
+    """Every tile configuration of the pipelined kernel and of the K-splitting 160-column kernel (codes 40, 41),
+    plain and with the rank columns as extra K tiles, bias, residual, ragged M / N, against the oracle.  Code 0 is
+    the automatic choice: the fourth and fifth shape are ones it sends to the 160-column kernel."""
     from katz_amd import ops
 
     M, N, K, R = shape
