@@ -636,6 +636,7 @@ int lora_gemm_pipe_launch(const LoraGemmParams& p, int tile_sel, hipStream_t str
     case 32: return deep_stage_ok(p) ? launch_pcfg<PCfg<128, 128, 2, 4, 0, 3, 64>>(p, stream) : KH_ERR_UNSUPPORTED;
     case 40: return lora_gemm_ksplit_launch(p, 2, stream);
     case 41: return lora_gemm_ksplit_launch(p, 4, stream);
+    case 42: return lora_gemm_wide_launch(p, stream);
     default: break;
   }
   // Default choice.  The limiter is the vector L1 path (every operand byte enters LDS through it), so
@@ -643,6 +644,12 @@ int lora_gemm_pipe_launch(const LoraGemmParams& p, int tile_sel, hipStream_t str
   // busy with them; when the 128x128 tiles do not even fill one round of 256 CUs, one 8-wave workgroup
   // per CU with 64-column stages (full 128-byte lines) beats two 4-wave ones; 128x128 / 4 waves /
   // two workgroups per CU otherwise.
+  if (lora_gemm_wide_ok(p)) {
+    // 256x320 tiles when they fill (nearly) whole rounds of the 256 CUs: fewer operand bytes per FLOP than any
+    // smaller tile and no ragged last round
+    const long wt = (long)(p.M / 256) * (p.N / 320), rounds = (wt + 255) / 256;
+    if (wt * 8 >= rounds * 256 * 7) return lora_gemm_wide_launch(p, stream);
+  }
   if (plain_ok(p)) {
     const long tiles = (long)((p.M + 127) / 128) * ((p.N + 127) / 128);
     // N a multiple of 160 and a tile count that leaves 128x128 tiles with a ragged last round: 160-column tiles

@@ -1,0 +1,239 @@
+// K1, wide-tile variant: y = [x | T] . [W | B_cat]^T (+ bias, + residual | GEGLU) on bf16 MFMA (gfx950) with
+// 256 x 320 output tiles, for the layers with the most output columns (the GEGLU projection of the feed-forward,
+// diffusers-hf/src/diffusers/models/activations.py:148-149 over attention.py:283-403's ff.net.0.proj).
+//
+// Same arithmetic as the two-launch form of lora_gemm_pipe.hip (T = the scaled shrink result, so the adapters'
+// rank columns are extra K tiles of the base GEMM).  Why another tile shape: N = 10240 at M = 2048 is 640 tiles of
+// 128 x 128, two and a half per CU; 256 x 320 tiles are exactly 256, one per CU, and a tile of that size moves
+// 0.45 times the operand bytes per FLOP through the CU's load path, which is what the smaller tile runs into.
+// The 80 K accumulators of a tile live in the registers of 8 waves (4 row groups x 2 column groups, 64 x 160 =
+// 2 x 5 MFMA tiles = 160 registers per lane); the compiler is held to 256 registers per lane.
+//
+// K loop: 64-column stages (128-byte rows, XOR-swizzled 16-byte pieces), two stages in LDS (144 KB), every wave
+// issues 9 global_load_lds per stage.  Fragments are double-buffered per 16-column MFMA step: the reads of step
+// s+2 are issued before the MFMAs of step s+1, so ten MFMAs cover every read.  The barrier that publishes the
+// next stage sits before the last step of the current one: by then every wave has read all of the current stage,
+// so the loads of the stage after next can refill it at once, a full stage of MFMAs ahead of their use.
+#include "kh_common.h"
+#include "lora_gemm.h"
+
+namespace {
+
+typedef const __attribute__((address_space(1))) void* gptr_t;
+typedef __attribute__((address_space(3))) void* lptr_t;
+
+template <int VM, int LGKM>
+__device__ __forceinline__ void wait_cnt() {  // gfx9 encoding: vmcnt = [15:14|3:0], expcnt = [6:4], lgkmcnt = [11:8]
+  __builtin_amdgcn_s_waitcnt((VM & 15) | (7 << 4) | ((LGKM & 15) << 8) | ((VM >> 4) << 14));
+}
+
+constexpr int WBM = 256, WBN = 320, WTN = 5, WTM = 2;      // tile, MFMA tiles per wave
+constexpr int WSTAGE = (WBM + WBN) * 128;                   // 73728 bytes
+constexpr int WLDS = 2 * WSTAGE;
+constexpr int WLDC = WBN + 8;
+constexpr int WXU = 4, WWU = 5, WLPS = WXU + WWU;           // DMA instructions per wave per stage (x rows, W rows)
+static_assert(128 * WLDC * 2 <= WLDS, "epilogue staging fits the ring");
+
+struct WFr { bf16x8 a[WTM]; bf16x8 b[WTN]; };
+
+__global__ __launch_bounds__(512, 2) void lora_gemm_wide_kernel(const LoraGemmParams p) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int l32 = lane & 31, lh = lane >> 5;
+
+  // tile of this workgroup: XCD b % 8 owns a block of xr_m x xr_n tiles (its W rows stay in its L2)
+  const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+  const int m_blk = (xcd / p.xg_n) * p.xr_m + local / p.xr_n;
+  const int n_blk = (xcd % p.xg_n) * p.xr_n + local % p.xr_n;
+  if (local / p.xr_n >= p.xr_m || m_blk >= p.m_tiles || n_blk >= p.n_tiles) return;  // padding of the grid
+  const int m0 = m_blk * WBM, n0 = n_blk * WBN;
+  const int N = p.N, K = p.K;
+  const int KT1 = K / 64;
+  const int KT = KT1 + (p.t_ext != nullptr ? p.R / 64 : 0);
+
+  // DMA: wave w brings x rows 32w .. 32w+31 (4 instructions of 8 rows) and W rows 40w .. 40w+39 (5) of every stage.
+  // Lane -> row lane/8 of its 8 rows, physical piece lane%8, which holds logical piece (lane%8) ^ ((stage row / 2) % 8).
+  // (stage row / 2) % 8 of instruction q is that of instruction 0 plus 4q mod 8: the piece flips bit 2 for odd q,
+  // so two element offsets (even / odd q) per operand describe all of a lane's sources; M and N are multiples of
+  // the tile (no clamping).
+  const int r8 = lane >> 3;
+  int xo[2], wo[2], xo2[2], wo2[2];
+#pragma unroll
+  for (int par = 0; par < 2; ++par) {
+    const int rx = wave * 32 + par * 8 + r8;                    // stage row of x instruction q = par
+    const int pcx = ((lane & 7) ^ ((rx >> 1) & 7)) * 8;
+    xo[par] = (rx - par * 8) * K + pcx;                         // row of q = 0; the issue adds q * 8 rows
+    xo2[par] = (rx - par * 8) * p.ldt + pcx;
+    const int rw = WBM + wave * 40 + par * 8 + r8;              // stage row of W instruction q = par
+    const int pcw = ((lane & 7) ^ ((rw >> 1) & 7)) * 8;
+    wo[par] = (rw - WBM - par * 8) * K + pcw;
+    wo2[par] = (rw - WBM - par * 8) * p.R + pcw;
+  }
+  const bf16_t* px = p.x + (size_t)m0 * K;
+  const bf16_t* pw = p.w + (size_t)n0 * K;
+  const bf16_t* px2 = p.t_ext != nullptr ? p.t_ext + (size_t)m0 * p.ldt + (p.t_nsplit > 0 ? (n0 / p.t_nsplit) * p.R : 0) : px;
+  const bf16_t* pw2 = p.t_ext != nullptr ? p.b_cat + (size_t)n0 * p.R : pw;
+  const int ldt = p.ldt, R = p.R;
+  auto issue = [&](int t, int st) {                             // K tile t into stage st
+    char* stage = smem + st * WSTAGE;
+    const bool ext = t >= KT1;
+    const bf16_t* bx = ext ? px2 + (t - KT1) * 64 : px + t * 64;
+    const bf16_t* bw = ext ? pw2 + (t - KT1) * 64 : pw + t * 64;
+    const int sx = ext ? ldt : K, sw_ = ext ? R : K;            // row strides
+#pragma unroll
+    for (int q = 0; q < WXU; ++q)
+      __builtin_amdgcn_global_load_lds((gptr_t)(bx + (ext ? xo2[q & 1] : xo[q & 1]) + q * 8 * sx),
+                                       (lptr_t)(stage + (wave * 32 + q * 8) * 128), 16, 0, 0);
+#pragma unroll
+    for (int q = 0; q < WWU; ++q)
+      __builtin_amdgcn_global_load_lds((gptr_t)(bw + (ext ? wo2[q & 1] : wo[q & 1]) + q * 8 * sw_),
+                                       (lptr_t)(stage + (WBM + wave * 40 + q * 8) * 128), 16, 0, 0);
+  };
+  const int sw = (l32 >> 1) & 7;
+  auto read_frags = [&](int st, int ks, WFr& f) {               // MFMA step ks (16 columns) of the stage
+    const char* s = smem + st * WSTAGE;
+    const int po = ((2 * ks + lh) ^ sw) * 16;
+#pragma unroll
+    for (int i = 0; i < WTM; ++i) f.a[i] = *reinterpret_cast<const bf16x8*>(s + (wm * 64 + i * 32 + l32) * 128 + po);
+#pragma unroll
+    for (int j = 0; j < WTN; ++j) f.b[j] = *reinterpret_cast<const bf16x8*>(s + (WBM + wn * 160 + j * 32 + l32) * 128 + po);
+  };
+  f32x16 acc[WTM][WTN];
+#pragma unroll
+  for (int i = 0; i < WTM; ++i)
+#pragma unroll
+    for (int j = 0; j < WTN; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+  auto mma = [&](const WFr& f) {
+#pragma unroll
+    for (int i = 0; i < WTM; ++i)
+#pragma unroll
+      for (int j = 0; j < WTN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a[i], f.b[j], acc[i][j], 0, 0, 0);
+  };
+
+  // bias of this lane's columns, requested before the loop
+  float bv[WTN];
+#pragma unroll
+  for (int j = 0; j < WTN; ++j) {
+    const int col = n0 + wn * 160 + j * 32 + l32;
+    bv[j] = p.bias != nullptr ? (float)p.bias[col] : 0.f;
+  }
+  wait_cnt<0, 15>();
+
+  // K loop over stages t (stage t & 1).  Steps 0..3 of a stage alternate between the fragment buffers fa / fb.
+  WFr fa, fb;
+  issue(0, 0);
+  if (KT > 1) issue(1, 1);
+  if (KT > 1) wait_cnt<WLPS, 15>(); else wait_cnt<0, 15>();
+  __builtin_amdgcn_s_barrier();
+  read_frags(0, 0, fa);
+  read_frags(0, 1, fb);
+  for (int t = 0; t < KT; ++t) {
+    const int st = t & 1;
+    mma(fa);                         // step 0
+    read_frags(st, 2, fa);
+    mma(fb);                         // step 1
+    read_frags(st, 3, fb);
+    mma(fa);                         // step 2
+    if (t + 1 < KT) {
+      // stage t+1 has landed (this wave's share; the barrier collects everyone's); every read of stage t is done
+      wait_cnt<0, 0>();
+      __builtin_amdgcn_s_barrier();
+      if (t + 2 < KT) issue(t + 2, st);
+      read_frags(st ^ 1, 0, fa);
+    }
+    mma(fb);                         // step 3
+    if (t + 1 < KT) read_frags(st ^ 1, 1, fb);
+  }
+  __syncthreads();   // the ring is dead: the staging tile reuses it
+
+  // Epilogue: bias in fp32, round to bf16, transpose through LDS so that every global store is a 16-byte piece of
+  // a contiguous output row; two passes of 128 rows (the waves' upper / lower 32-row MFMA tiles).
+  bf16_t* sC = reinterpret_cast<bf16_t*>(smem);
+  const int out_ld = p.geglu ? (N >> 1) : N;
+  constexpr int CPR = WBN / 8, ECH = 128 * CPR / 512;        // plain: 40 pieces per staged row, 10 per thread
+  constexpr int OPR = WBN / 16, GCH = 128 * OPR / 512;       // GEGLU: 20 output pieces per staged row, 5 per thread
+#pragma unroll
+  for (int i = 0; i < WTM; ++i) {
+#pragma unroll
+    for (int j = 0; j < WTN; ++j) {
+      const int col = wn * 160 + j * 32 + l32;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int row = wm * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+        sC[row * WLDC + col] = (bf16_t)(acc[i][j][v] + bv[j]);
+      }
+    }
+    __syncthreads();
+    if (!p.geglu) {
+#pragma unroll
+      for (int q = 0; q < ECH; ++q) {
+        const int c = tid + q * 512, srow = c / CPR, ch = c % CPR;
+        const size_t g = (size_t)(m0 + (srow >> 5) * 64 + i * 32 + (srow & 31)) * N + n0 + ch * 8;
+        u32x4 o = *reinterpret_cast<const u32x4*>(sC + srow * WLDC + ch * 8);
+        if (p.res != nullptr) {
+          const u32x4 rr = *reinterpret_cast<const u32x4*>(p.res + g);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) o[e] = pack_bf16x2(bf16_lo(o[e]) + bf16_lo(rr[e]), bf16_hi(o[e]) + bf16_hi(rr[e]));
+        }
+        *reinterpret_cast<u32x4*>(p.y + g) = o;
+      }
+    } else {
+      // staged columns come in groups of 64 = 32 value columns then their 32 gate columns
+#pragma unroll
+      for (int q = 0; q < GCH; ++q) {
+        const int c = tid + q * 512, srow = c / OPR, oc = c % OPR;
+        const int grp = oc >> 2, sub = oc & 3;
+        const size_t g = (size_t)(m0 + (srow >> 5) * 64 + i * 32 + (srow & 31)) * out_ld + (n0 >> 1) + grp * 32 + sub * 8;
+        const u32x4 hv = *reinterpret_cast<const u32x4*>(sC + srow * WLDC + grp * 64 + sub * 8);
+        const u32x4 gv = *reinterpret_cast<const u32x4*>(sC + srow * WLDC + grp * 64 + 32 + sub * 8);
+        u32x4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float a0 = kh_gelu_erf(bf16_lo(gv[e])), a1 = kh_gelu_erf(bf16_hi(gv[e]));
+          const uint32_t ar = pack_bf16x2(a0, a1);  // gelu(gate) rounded to bf16 before the product
+          o[e] = pack_bf16x2(bf16_lo(hv[e]) * bf16_lo(ar), bf16_hi(hv[e]) * bf16_hi(ar));
+        }
+        *reinterpret_cast<u32x4*>(p.y + g) = o;
+      }
+    }
+    __syncthreads();
+  }
+}
+
+}  // namespace
+
+bool lora_gemm_wide_ok(const LoraGemmParams& p) {
+  const bool plain = p.R == 0 || p.t_ext != nullptr;
+  return plain && p.grp == nullptr && p.sg_mode == 0 && p.conv_cin == 0 && p.M % WBM == 0 && p.N % WBN == 0 &&
+         p.K % 64 == 0 && p.K >= 64 && (p.t_ext == nullptr || (p.R % 64 == 0 && p.ldt % 8 == 0)) &&
+         (p.t_nsplit == 0 || p.t_nsplit % WBN == 0) && (long)p.M * (p.K > p.ldt ? p.K : p.ldt) < (1L << 31) &&
+         (long)p.N * p.K < (1L << 31);
+}
+
+int lora_gemm_wide_launch(LoraGemmParams p, hipStream_t stream) {
+  if (!lora_gemm_wide_ok(p)) return KH_ERR_UNSUPPORTED;
+  p.m_tiles = p.M / WBM;
+  p.n_tiles = p.N / WBN;
+  static bool attr_done = false;
+  if (!attr_done) {
+    hipError_t e = hipFuncSetAttribute((const void*)lora_gemm_wide_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, WLDS);
+    if (e != hipSuccess) return (int)e;
+    attr_done = true;
+  }
+  // the XCD grid whose per-XCD block touches the fewest operand rows, padding counted as cost
+  double best = 0;
+  p.xg_n = 0;
+  for (int gm = 1; gm <= 8; gm *= 2) {
+    const int gn = 8 / gm;
+    const int rm = (p.m_tiles + gm - 1) / gm, rn = (p.n_tiles + gn - 1) / gn;
+    const double cost = ((double)rm * WBM + (double)rn * WBN) * (8.0 * rm * rn) / ((double)p.m_tiles * p.n_tiles);
+    if (p.xg_n == 0 || cost < best) { best = cost; p.xg_n = gn; p.xr_m = rm; p.xr_n = rn; }
+  }
+  const unsigned grid = 8u * (unsigned)p.xr_m * (unsigned)p.xr_n;
+  kh_launch(KH_TAG_LORA_GEMM, lora_gemm_wide_kernel, dim3(grid), dim3(512), WLDS, stream, p);
+  KH_RETURN_LAST_ERROR();
+}

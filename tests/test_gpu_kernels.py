@@ -710,3 +710,46 @@ def test_pipelined_gemm_tile_variants(tile, shape):
                             residual=rd.float().cpu())
     torch.cuda.synchronize()
     assert_close_rel(y, ref, REL_BF16, f"tile {tile} {shape}")
+
+
+@pytest.mark.parametrize("shape", [(256, 320, 64, 0), (512, 640, 192, 64), (2048, 10240, 1280, 128)])
+@pytest.mark.parametrize("geglu", [False, True])
+def test_wide_tile_gemm(shape, geglu):
+    """The 256x320-tile kernel (code 42; the automatic choice for the third shape): plain and with the rank columns
+    as extra K tiles, bias, residual or the GEGLU epilogue, against the oracle; and bit for bit against the 128x128
+    pipelined kernel, whose summation order per output element it shares."""
+    from katz_amd import ops
+    from katz_amd.lora import interleave_geglu_rows
+
+    M, N, K, R = shape
+    say("wide tile", shape, geglu)
+    d = dev()
+    g = torch.Generator().manual_seed(M + N + int(geglu))
+    x, w, b = randn(g, M, K), randn(g, N, K, std=0.03), randn(g, N)
+    res = None if geglu else randn(g, M, N)
+    xd = x.to(d, BF)
+    wd = (interleave_geglu_rows(w) if geglu else w).to(d, BF)
+    bd = (interleave_geglu_rows(b) if geglu else b).to(d, BF)
+    rd = None if res is None else res.to(d, BF)
+    ads = []
+    if R == 0:
+        run = lambda tile: ops.lora_linear(xd, wd, bd, residual=rd, geglu=geglu, tile=tile)
+    else:
+        A, B = randn(g, R, K, std=0.05), randn(g, N, R, std=0.05)
+        Ad = A.to(d, BF)
+        Bd = (interleave_geglu_rows(B) if geglu else B).to(d, BF)
+        t = ops.lora_shrink(xd, Ad, torch.full((R,), 0.7, device=d))
+        run = lambda tile: ops.lora_linear_pre(xd, wd, bd, t, Bd, residual=rd, geglu=geglu, tile=tile)
+        ads = [(Ad.float().cpu(), B.to(BF).float(), 0.7)]
+    y = run(42)
+    y16 = run(16)
+    y0 = run(0)
+    torch.cuda.synchronize()
+    assert torch.equal(y, y16), "wide tile differs from the 128x128 kernel"
+    assert torch.equal(y0, y16), "automatic choice differs from the 128x128 kernel"
+    xf, wf, bf = xd.float().cpu(), w.to(BF).float(), b.to(BF).float()
+    if geglu:
+        ref = O.geglu(bf16_round(O.lora_linear(xf, wf, bf, ads)))
+    else:
+        ref = O.lora_linear(xf, wf, bf, ads, residual=rd.float().cpu())
+    assert_close_rel(y, ref, REL_BF16, f"wide tile {shape} geglu={geglu}")
