@@ -9,6 +9,9 @@
 // The 80 K accumulators of a tile live in the registers of 8 waves (4 row groups x 2 column groups, 64 x 160 =
 // 2 x 5 MFMA tiles = 160 registers per lane); the compiler is held to 256 registers per lane.
 //
+// The MFMA operands are W first, x second: the accumulators then hold, per lane, one output row and runs of four
+// consecutive columns, so the epilogue's transpose through LDS writes 8 bytes per instruction instead of 2.
+//
 // K loop: 64-column stages (128-byte rows, XOR-swizzled 16-byte pieces), two stages in LDS (144 KB), every wave
 // issues 9 global_load_lds per stage.  Fragments are double-buffered per 16-column MFMA step: the reads of step
 // s+2 are issued before the MFMAs of step s+1, so ten MFMAs cover every read.  The barrier that publishes the
@@ -29,8 +32,15 @@ __device__ __forceinline__ void wait_cnt() {  // gfx9 encoding: vmcnt = [15:14|3
 
 constexpr int WBM = 256, WBN = 320, WTN = 5, WTM = 2;      // tile, MFMA tiles per wave
 constexpr int WSTAGE = (WBM + WBN) * 128;                   // 73728 bytes
-constexpr int WLDS = 2 * WSTAGE;
-constexpr int WLDC = WBN + 8;
+// GEGLU: bf16(gelu(gate)) for every bf16 gate with 2^-15 <= |gate| < 32, built by each workgroup with the same
+// function the direct evaluation uses (so the two agree bit for bit), looked up in the epilogue: the epilogue of a
+// tile this size has 40 K gelu evaluations and nothing to overlap them with
+constexpr int WTAB_LO = 0x3800, WTAB_N = 2560;               // magnitudes 0x3800 .. 0x41ff, per sign
+constexpr int WTAB_OFF = 2 * WSTAGE;
+constexpr int WBIAS_OFF = WTAB_OFF + 2 * WTAB_N * 2;          // the tile's 320 bias values (bf16)
+constexpr int WLDS = WBIAS_OFF + WBN * 2;
+static_assert(WLDS <= 160 * 1024, "LDS budget");
+constexpr int WLDC = WBN + 72;                               // staged row: 196 dwords = 4 mod 64 banks, see the epilogue
 constexpr int WXU = 4, WWU = 5, WLPS = WXU + WWU;           // DMA instructions per wave per stage (x rows, W rows)
 static_assert(128 * WLDC * 2 <= WLDS, "epilogue staging fits the ring");
 
@@ -59,37 +69,33 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_wide_kernel(const LoraGemmPa
   // so two element offsets (even / odd q) per operand describe all of a lane's sources; M and N are multiples of
   // the tile (no clamping).
   const int r8 = lane >> 3;
-  int xo[2], wo[2], xo2[2], wo2[2];
-#pragma unroll
-  for (int par = 0; par < 2; ++par) {
-    const int rx = wave * 32 + par * 8 + r8;                    // stage row of x instruction q = par
-    const int pcx = ((lane & 7) ^ ((rx >> 1) & 7)) * 8;
-    xo[par] = (rx - par * 8) * K + pcx;                         // row of q = 0; the issue adds q * 8 rows
-    xo2[par] = (rx - par * 8) * p.ldt + pcx;
-    const int rw = WBM + wave * 40 + par * 8 + r8;              // stage row of W instruction q = par
-    const int pcw = ((lane & 7) ^ ((rw >> 1) & 7)) * 8;
-    wo[par] = (rw - WBM - par * 8) * K + pcw;
-    wo2[par] = (rw - WBM - par * 8) * p.R + pcw;
-  }
+  const int rx0 = wave * 32 + r8, rx1 = rx0 + 8;               // stage rows of x instructions 0 / 1
+  const int pcx0 = ((lane & 7) ^ ((rx0 >> 1) & 7)) * 8, pcx1 = ((lane & 7) ^ ((rx1 >> 1) & 7)) * 8;
+  const int rw0 = WBM + wave * 40 + r8, rw1 = rw0 + 8;          // stage rows of W instructions 0 / 1
+  const int pcw0 = ((lane & 7) ^ ((rw0 >> 1) & 7)) * 8, pcw1 = ((lane & 7) ^ ((rw1 >> 1) & 7)) * 8;
+  const int wrow = wave * 40 + r8;                              // W row of instruction 0 inside the tile
   const bf16_t* px = p.x + (size_t)m0 * K;
   const bf16_t* pw = p.w + (size_t)n0 * K;
   const bf16_t* px2 = p.t_ext != nullptr ? p.t_ext + (size_t)m0 * p.ldt + (p.t_nsplit > 0 ? (n0 / p.t_nsplit) * p.R : 0) : px;
   const bf16_t* pw2 = p.t_ext != nullptr ? p.b_cat + (size_t)n0 * p.R : pw;
   const int ldt = p.ldt, R = p.R;
-  auto issue = [&](int t, int st) {                             // K tile t into stage st
-    char* stage = smem + st * WSTAGE;
-    const bool ext = t >= KT1;
-    const bf16_t* bx = ext ? px2 + (t - KT1) * 64 : px + t * 64;
-    const bf16_t* bw = ext ? pw2 + (t - KT1) * 64 : pw + t * 64;
-    const int sx = ext ? ldt : K, sw_ = ext ? R : K;            // row strides
+  // one stage from operands with row strides sx / sw_ (elements); bx / bw already point at the stage's first column
+  auto issue_from = [&](const bf16_t* bx, const bf16_t* bw, int sx, int sw_, char* stage) {
+    const bf16_t* gx0 = bx + rx0 * sx + pcx0;                   // row of instruction 0, piece of the even ones
+    const bf16_t* gx1 = bx + rx0 * sx + pcx1;                   // same row, piece of the odd ones
+    const bf16_t* gw0 = bw + wrow * sw_ + pcw0;
+    const bf16_t* gw1 = bw + wrow * sw_ + pcw1;
 #pragma unroll
     for (int q = 0; q < WXU; ++q)
-      __builtin_amdgcn_global_load_lds((gptr_t)(bx + (ext ? xo2[q & 1] : xo[q & 1]) + q * 8 * sx),
-                                       (lptr_t)(stage + (wave * 32 + q * 8) * 128), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((gptr_t)(((q & 1) ? gx1 : gx0) + q * 8 * sx), (lptr_t)(stage + (wave * 32 + q * 8) * 128), 16, 0, 0);
 #pragma unroll
     for (int q = 0; q < WWU; ++q)
-      __builtin_amdgcn_global_load_lds((gptr_t)(bw + (ext ? wo2[q & 1] : wo[q & 1]) + q * 8 * sw_),
-                                       (lptr_t)(stage + (WBM + wave * 40 + q * 8) * 128), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((gptr_t)(((q & 1) ? gw1 : gw0) + q * 8 * sw_), (lptr_t)(stage + (WBM + wave * 40 + q * 8) * 128), 16, 0, 0);
+  };
+  auto issue = [&](int t, int st) {                             // K tile t into stage st
+    char* stage = smem + st * WSTAGE;
+    if (t < KT1) issue_from(px + t * 64, pw + t * 64, K, K, stage);
+    else issue_from(px2 + (t - KT1) * 64, pw2 + (t - KT1) * 64, ldt, R, stage);
   };
   const int sw = (l32 >> 1) & 7;
   auto read_frags = [&](int st, int ks, WFr& f) {               // MFMA step ks (16 columns) of the stage
@@ -111,22 +117,24 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_wide_kernel(const LoraGemmPa
 #pragma unroll
     for (int i = 0; i < WTM; ++i)
 #pragma unroll
-      for (int j = 0; j < WTN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a[i], f.b[j], acc[i][j], 0, 0, 0);
+      for (int j = 0; j < WTN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.b[j], f.a[i], acc[i][j], 0, 0, 0);   // D = W . x^T: lane = row of x
   };
-
-  // bias of this lane's columns, requested before the loop
-  float bv[WTN];
-#pragma unroll
-  for (int j = 0; j < WTN; ++j) {
-    const int col = n0 + wn * 160 + j * 32 + l32;
-    bv[j] = p.bias != nullptr ? (float)p.bias[col] : 0.f;
-  }
-  wait_cnt<0, 15>();
 
   // K loop over stages t (stage t & 1).  Steps 0..3 of a stage alternate between the fragment buffers fa / fb.
   WFr fa, fb;
   issue(0, 0);
   if (KT > 1) issue(1, 1);
+  uint16_t* gtab = reinterpret_cast<uint16_t*>(smem + WTAB_OFF);
+  uint16_t* sbias = reinterpret_cast<uint16_t*>(smem + WBIAS_OFF);   // like the table: written now, read in the epilogue
+  if (tid < WBN) sbias[tid] = p.bias != nullptr ? reinterpret_cast<const uint16_t*>(p.bias)[n0 + tid] : (uint16_t)0;
+  if (p.geglu) {   // published by the barriers of the K loop, read in the epilogue
+#pragma unroll
+    for (int k = 0; k < 2 * WTAB_N / 512; ++k) {
+      const int i = tid + k * 512;
+      const uint32_t bits = (uint32_t)(i >= WTAB_N ? 0x8000 + (i - WTAB_N) : i) + WTAB_LO;
+      gtab[i] = (uint16_t)pack_bf16x2(kh_gelu_erf(bf16_lo(bits)), 0.f);
+    }
+  }
   if (KT > 1) wait_cnt<WLPS, 15>(); else wait_cnt<0, 15>();
   __builtin_amdgcn_s_barrier();
   read_frags(0, 0, fa);
@@ -158,13 +166,19 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_wide_kernel(const LoraGemmPa
   constexpr int OPR = WBN / 16, GCH = 128 * OPR / 512;       // GEGLU: 20 output pieces per staged row, 5 per thread
 #pragma unroll
   for (int i = 0; i < WTM; ++i) {
+    // the MFMA operands are swapped (W rows first), so a lane holds one output row (l32) and, per group of four
+    // accumulator registers, four consecutive columns: 8-byte LDS writes.  With 196-dword rows the 16 rows x 2 halves
+    // of one write phase cover all 64 banks.
 #pragma unroll
     for (int j = 0; j < WTN; ++j) {
-      const int col = wn * 160 + j * 32 + l32;
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int row = wm * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
-        sC[row * WLDC + col] = (bf16_t)(acc[i][j][v] + bv[j]);
+      for (int g4 = 0; g4 < 4; ++g4) {
+        const int col = wn * 160 + j * 32 + 8 * g4 + 4 * lh;
+        const u32x2 bb = *reinterpret_cast<const u32x2*>(sbias + col);
+        u32x2 o;
+        o[0] = pack_bf16x2(acc[i][j][4 * g4] + bf16_lo(bb[0]), acc[i][j][4 * g4 + 1] + bf16_hi(bb[0]));
+        o[1] = pack_bf16x2(acc[i][j][4 * g4 + 2] + bf16_lo(bb[1]), acc[i][j][4 * g4 + 3] + bf16_hi(bb[1]));
+        *reinterpret_cast<u32x2*>(sC + (wm * 32 + l32) * WLDC + col) = o;
       }
     }
     __syncthreads();
@@ -190,13 +204,24 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_wide_kernel(const LoraGemmPa
         const size_t g = (size_t)(m0 + (srow >> 5) * 64 + i * 32 + (srow & 31)) * out_ld + (n0 >> 1) + grp * 32 + sub * 8;
         const u32x4 hv = *reinterpret_cast<const u32x4*>(sC + srow * WLDC + grp * 64 + sub * 8);
         const u32x4 gv = *reinterpret_cast<const u32x4*>(sC + srow * WLDC + grp * 64 + 32 + sub * 8);
-        u32x4 o;
+        u32x4 ar;                                       // gelu(gate) rounded to bf16 before the product
+        bool outside = false;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          const float a0 = kh_gelu_erf(bf16_lo(gv[e])), a1 = kh_gelu_erf(bf16_hi(gv[e]));
-          const uint32_t ar = pack_bf16x2(a0, a1);  // gelu(gate) rounded to bf16 before the product
-          o[e] = pack_bf16x2(bf16_lo(hv[e]) * bf16_lo(ar), bf16_hi(hv[e]) * bf16_hi(ar));
+          const uint32_t lo = gv[e] & 0xffffu, hi = gv[e] >> 16;
+          const uint32_t olo = (lo & 0x7fffu) - WTAB_LO, ohi = (hi & 0x7fffu) - WTAB_LO;
+          outside = outside || olo >= (uint32_t)WTAB_N || ohi >= (uint32_t)WTAB_N;
+          const uint32_t ilo = (olo < (uint32_t)WTAB_N ? olo : 0u) + (lo >> 15) * WTAB_N;
+          const uint32_t ihi = (ohi < (uint32_t)WTAB_N ? ohi : 0u) + (hi >> 15) * WTAB_N;
+          ar[e] = (uint32_t)gtab[ilo] | ((uint32_t)gtab[ihi] << 16);
         }
+        if (outside) {                                  // tiny, huge or non-finite gates: evaluate directly
+#pragma unroll
+          for (int e = 0; e < 4; ++e) ar[e] = pack_bf16x2(kh_gelu_erf(bf16_lo(gv[e])), kh_gelu_erf(bf16_hi(gv[e])));
+        }
+        u32x4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = pack_bf16x2(bf16_lo(hv[e]) * bf16_lo(ar[e]), bf16_hi(hv[e]) * bf16_hi(ar[e]));
         *reinterpret_cast<u32x4*>(p.y + g) = o;
       }
     }

@@ -753,3 +753,31 @@ def test_wide_tile_gemm(shape, geglu):
     else:
         ref = O.lora_linear(xf, wf, bf, ads, residual=rd.float().cpu())
     assert_close_rel(y, ref, REL_BF16, f"wide tile {shape} geglu={geglu}")
+
+
+def test_wide_tile_geglu_gate_range():
+    """GEGLU epilogue of the 256x320-tile kernel on gates outside and at the edges of its lookup table (zero, tiny,
+    2^-15, just below 32, huge, infinite): x = 0, so the projection is the bias."""
+    from katz_amd import ops
+    from katz_amd.lora import interleave_geglu_rows
+
+    say("wide tile geglu gate range")
+    d = dev()
+    M, K, D = 256, 64, 320
+    specials = torch.tensor([0.0, -0.0, 1e-6, -1e-6, 2.0 ** -15, -(2.0 ** -15), 2.0 ** -15 * 0.99, 31.875, -31.875, 32.0,
+                             -32.0, 40.0, -40.0, 1e30, -1e30, float("inf"), -float("inf"), 0.5, -0.5, 3.0, -3.0])
+    g = torch.Generator().manual_seed(3)
+    gate = randn(g, D) * 2.0
+    gate[: specials.numel()] = specials
+    value = randn(g, D)
+    b = torch.cat([value, gate]).to(BF)                       # reference layout: value rows, then gate rows
+    w = torch.zeros(2 * D, K)
+    x = torch.zeros(M, K)
+    wd, bd = interleave_geglu_rows(w).to(d, BF), interleave_geglu_rows(b).to(d, BF)
+    y = ops.lora_linear(x.to(d, BF), wd, bd, geglu=True, tile=42)
+    y16 = ops.lora_linear(x.to(d, BF), wd, bd, geglu=True, tile=16)
+    torch.cuda.synchronize()
+    assert torch.equal(y.view(torch.int16), y16.view(torch.int16)), "lookup differs from the direct evaluation"
+    ref = O.geglu(b.float().unsqueeze(0).expand(M, -1).contiguous())
+    fin = torch.isfinite(ref[0])
+    assert_close_rel(y[:, fin], ref[:, fin], REL_BF16, "wide tile geglu gate range")
