@@ -46,6 +46,8 @@ int lora_gemm_pipe_launch_grouped(const LoraGemmParams& p, int n_groups, hipStre
 // plain or K-extended GEMM with bias / residual, K % 64 == 0.  row_groups 2 or 4.
 bool lora_gemm_ksplit_ok(const LoraGemmParams& p);
 int lora_gemm_ksplit_launch(const LoraGemmParams& p, int row_groups, hipStream_t stream);
+bool lora_gemm_ksplit_conv_ok(const LoraGemmParams& p);
+int lora_gemm_ksplit_launch_conv(const LoraGemmParams& p, int row_groups, hipStream_t stream);
 // Wide-tile variant (lora_gemm_wide.hip): 256 x 320 tiles, 8 waves; plain or K-extended GEMM with bias / residual /
 // GEGLU; M % 256 == 0, N % 320 == 0, K % 64 == 0.
 bool lora_gemm_wide_ok(const LoraGemmParams& p);

@@ -49,7 +49,14 @@ struct KCfg {
   static_assert(LDS <= 160 * 1024, "LDS budget");
 };
 
-template <class C>
+// 16 bytes of zeros (and more): what a 3x3 convolution's DMA reads for taps that fall into the padding
+__device__ __attribute__((aligned(256))) const uint32_t ks_zero_page[64] = {0};
+
+// CONV: x is an NHWC image and row m of the GEMM is output pixel m of a 3x3 convolution with padding 1 (K = 9 * Cin
+// ordered (kh, kw, ci), see lora_gemm_pipe.hip): a stage of 64 K columns is 64 channels of one tap, the x rows of tap
+// (kh, kw) sit (kh * W + kw) * Cin elements after the row's base (the pixel above-left of its window), and rows
+// whose tap falls outside the image read zeros.
+template <class C, bool CONV>
 __global__ __launch_bounds__(512, 2) void lora_gemm_ksplit_kernel(const LoraGemmParams p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   constexpr int BM = C::BM, BN = C::BN, TN = C::TN, KSW = C::KSW, NST = C::NST, STAGE = C::STAGE;
@@ -74,13 +81,27 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_ksplit_kernel(const LoraGemm
   // LDS slot = lane: row lane/8, physical piece lane%8, which holds logical piece (lane%8) ^ ((row/2)%8)
   const bf16_t* src[LPS_HI];
   const bf16_t* src2[LPS_HI];
+  int tapmask[LPS_HI];                                 // CONV, x units: bit t = tap t of this lane's row is inside the image
+  constexpr int XQ = BM / 64;                          // units q < XQ are x rows for every wave, the others W rows
 #pragma unroll
   for (int q = 0; q < LPS_HI; ++q) {
     int u = wave + 8 * q;
     u = u < C::UNITS ? u : C::UNITS - 1;               // never issued (has_hi), keep the address valid
     const int r = u * 8 + (lane >> 3);
     const int pc = ((lane & 7) ^ ((r >> 1) & 7)) * 8;
-    if (r < BM) {
+    tapmask[q] = 0;
+    if (CONV && r < BM) {
+      int row = m0 + r; row = row < M ? row : M - 1;
+      const int wo = row % p.conv_wo, t2 = row / p.conv_wo, ho = t2 % p.conv_ho, nb = t2 / p.conv_ho;
+      const int hi0 = ho * p.conv_stride - 1, wi0 = wo * p.conv_stride - 1;
+#pragma unroll
+      for (int tap = 0; tap < 9; ++tap) {
+        const int hi = hi0 + tap / 3, wi = wi0 + tap % 3;
+        tapmask[q] |= (hi >= 0 && hi < p.conv_h && wi >= 0 && wi < p.conv_w) ? (1 << tap) : 0;
+      }
+      src[q] = p.x + ((long)(nb * p.conv_h + hi0) * p.conv_w + wi0) * p.conv_cin + pc;
+      src2[q] = src[q];
+    } else if (r < BM) {
       int row = m0 + r; row = row < M ? row : M - 1;
       src[q] = p.x + (size_t)row * K + pc;
       src2[q] = p.t_ext == nullptr ? src[q] : p.t_ext + (size_t)row * p.ldt + pc + (p.t_nsplit > 0 ? (n0 / p.t_nsplit) * p.R : 0);
@@ -90,13 +111,26 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_ksplit_kernel(const LoraGemm
       src2[q] = p.t_ext == nullptr ? src[q] : p.b_cat + (size_t)row * p.R + pc;
     }
   }
+  // CONV: K tiles are requested in order, so the tap and the channel offset of the next request are running scalars
+  int cv_tap = 0, cv_kw = 0, cv_c0 = 0, cv_shift = 0, cv_row = 0;
   auto issue = [&](int t, int st) {                    // K tile t into ring stage st
     char* stage = smem + st * STAGE;
 #pragma unroll
     for (int q = 0; q < LPS_HI; ++q) {
       if (q < LPS_LO || has_hi) {
-        const bf16_t* g = t < KT1 ? src[q] + (size_t)t * 64 : src2[q] + (size_t)(t - KT1) * 64;
+        const bf16_t* g;
+        if (CONV && q < XQ)
+          g = ((tapmask[q] >> cv_tap) & 1) ? src[q] + (cv_shift + cv_c0) : reinterpret_cast<const bf16_t*>(ks_zero_page);
+        else
+          g = t < KT1 ? src[q] + (size_t)t * 64 : src2[q] + (size_t)(t - KT1) * 64;
         __builtin_amdgcn_global_load_lds((gptr_t)g, (lptr_t)(stage + (wave + 8 * q) * 1024), 16, 0, 0);
+      }
+    }
+    if (CONV) {
+      cv_c0 += 64;
+      if (cv_c0 == p.conv_cin) {
+        cv_c0 = 0; ++cv_tap; ++cv_kw; cv_shift += p.conv_cin;
+        if (cv_kw == 3) { cv_kw = 0; cv_row += p.conv_w * p.conv_cin; cv_shift = cv_row; }
       }
     }
   };
@@ -229,13 +263,13 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_ksplit_kernel(const LoraGemm
   }
 }
 
-template <class C>
+template <class C, bool CONV = false>
 int launch_ksplit(LoraGemmParams p, hipStream_t stream) {
   p.m_tiles = (p.M + C::BM - 1) / C::BM;
   p.n_tiles = (p.N + C::BN - 1) / C::BN;
   static bool attr_done = false;  // per template instantiation
   if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void*)lora_gemm_ksplit_kernel<C>, hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS);
+    hipError_t e = hipFuncSetAttribute((const void*)lora_gemm_ksplit_kernel<C, CONV>, hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS);
     if (e != hipSuccess) return (int)e;
     attr_done = true;
   }
@@ -249,7 +283,7 @@ int launch_ksplit(LoraGemmParams p, hipStream_t stream) {
     if (p.xg_n == 0 || cost < best) { best = cost; p.xg_n = gn; p.xr_m = rm; p.xr_n = rn; }
   }
   const unsigned grid = 8u * (unsigned)p.xr_m * (unsigned)p.xr_n;
-  kh_launch(KH_TAG_LORA_GEMM, lora_gemm_ksplit_kernel<C>, dim3(grid), dim3(512), C::LDS, stream, p);
+  kh_launch(CONV ? KH_TAG_CONV : KH_TAG_LORA_GEMM, lora_gemm_ksplit_kernel<C, CONV>, dim3(grid), dim3(512), C::LDS, stream, p);
   KH_RETURN_LAST_ERROR();
 }
 
@@ -265,4 +299,15 @@ bool lora_gemm_ksplit_ok(const LoraGemmParams& p) {
 int lora_gemm_ksplit_launch(const LoraGemmParams& p, int row_groups, hipStream_t stream) {
   if (!lora_gemm_ksplit_ok(p)) return KH_ERR_UNSUPPORTED;
   return row_groups == 4 ? launch_ksplit<KCfg<4>>(p, stream) : launch_ksplit<KCfg<2>>(p, stream);
+}
+
+// 3x3 convolution on the same tiles (conv_* fields set, R == 0, K == 9 * conv_cin, conv_cin % 64 == 0).
+bool lora_gemm_ksplit_conv_ok(const LoraGemmParams& p) {
+  return p.conv_cin > 0 && p.conv_cin % 64 == 0 && p.K == 9 * p.conv_cin && p.R == 0 && p.t_ext == nullptr && p.grp == nullptr &&
+         p.sg_mode == 0 && !p.geglu && p.N % 8 == 0;
+}
+
+int lora_gemm_ksplit_launch_conv(const LoraGemmParams& p, int row_groups, hipStream_t stream) {
+  if (!lora_gemm_ksplit_conv_ok(p)) return KH_ERR_UNSUPPORTED;
+  return row_groups == 4 ? launch_ksplit<KCfg<4>, true>(p, stream) : launch_ksplit<KCfg<2>, true>(p, stream);
 }

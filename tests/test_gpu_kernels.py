@@ -507,7 +507,11 @@ def test_fused_qkv_matches_separate_projections():
     (1, 96, 13, 9, 40, 1, True, False),        # ragged: M and Cout not multiples of the tile, Cin = 3 x 32
     (2, 128, 16, 16, 128, 2, True, False),     # Downsample2D
     (1, 64, 15, 11, 72, 2, False, True),       # odd sizes, stride 2
-    (2, 1280, 32, 32, 1280, 1, True, True),    # the deepest SDXL resnet conv (8-wave tile path)
+    (2, 1280, 32, 32, 1280, 1, True, True),    # the deepest SDXL resnet conv (64x160 tiles, waves split K)
+    (2, 640, 64, 64, 640, 1, True, True),      # the middle level (128x160 tiles, waves split K)
+    (1, 640, 60, 67, 640, 1, True, False),     # same tiles, ragged M (4020 pixels), rows crossing image rows
+    (2, 1280, 31, 31, 1280, 1, False, True),   # 64x160 tiles, ragged M (1922 pixels)
+    (2, 640, 50, 80, 640, 1, True, True),      # 128x160 tiles, ragged M (8000 pixels)
 ])
 def test_conv3x3_nhwc_bf16(shape):
     """Implicit-GEMM 3x3 convolution against torch's fp32 conv2d on the same bf16-rounded operands."""
