@@ -615,7 +615,7 @@ int lora_gemm_pipe_launch_conv(const LoraGemmParams& p, hipStream_t stream) {
   // 160-column tiles (lora_gemm_ksplit.hip) by the rules of the linear layers
   if (p.N % 160 == 0 && lora_gemm_ksplit_conv_ok(p)) {
     const long n160 = p.N / 160, m128 = (p.M + 127) / 128, m64 = (p.M + 63) / 64;
-    if (tiles > 256 && tiles <= 384 && m128 * n160 <= 256) return lora_gemm_ksplit_launch_conv(p, 4, stream);
+    if ((tiles > 256 && tiles <= 384 && m128 * n160 <= 256) || (p.N % 128 != 0 && (m128 * n160) % 256 == 0)) return lora_gemm_ksplit_launch_conv(p, 4, stream);
     if (tiles <= 192 && m64 * n160 <= 256 && m64 * n160 > tiles && p.K >= 2560) return lora_gemm_ksplit_launch_conv(p, 2, stream);
   }
   if (tiles <= 256 && p.conv_cin % 64 == 0) return launch_pcfg<PCfg<128, 128, 2, 4, 0, 3, 64>, true>(p, stream);
