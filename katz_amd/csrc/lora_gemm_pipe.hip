@@ -651,10 +651,10 @@ int lora_gemm_pipe_launch(const LoraGemmParams& p, int tile_sel, hipStream_t str
   // per CU with 64-column stages (full 128-byte lines) beats two 4-wave ones; 128x128 / 4 waves /
   // two workgroups per CU otherwise.
   if (lora_gemm_wide_ok(p)) {
-    // 256x320 tiles when they fill (nearly) whole rounds of the 256 CUs: fewer operand bytes per FLOP than any
-    // smaller tile and no ragged last round
+    // 256x320 tiles when they fill at least three quarters of whole rounds of the 256 CUs: fewer operand bytes per
+    // FLOP than any smaller tile and no ragged last round
     const long wt = (long)(p.M / 256) * (p.N / 320), rounds = (wt + 255) / 256;
-    if (wt * 8 >= rounds * 256 * 7) return lora_gemm_wide_launch(p, stream);
+    if (wt * 4 >= rounds * 256 * 3) return lora_gemm_wide_launch(p, stream);
   }
   if (plain_ok(p)) {
     const long tiles = (long)((p.M + 127) / 128) * ((p.N + 127) / 128);

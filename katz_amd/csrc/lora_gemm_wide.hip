@@ -30,24 +30,42 @@ __device__ __forceinline__ void wait_cnt() {  // gfx9 encoding: vmcnt = [15:14|3
   __builtin_amdgcn_s_waitcnt((VM & 15) | (7 << 4) | ((LGKM & 15) << 8) | ((VM >> 4) << 14));
 }
 
-constexpr int WBM = 256, WBN = 320, WTN = 5, WTM = 2;      // tile, MFMA tiles per wave
-constexpr int WSTAGE = (WBM + WBN) * 128;                   // 73728 bytes
 // GEGLU: bf16(gelu(gate)) for every bf16 gate with 2^-15 <= |gate| < 32, built by each workgroup with the same
 // function the direct evaluation uses (so the two agree bit for bit), looked up in the epilogue: the epilogue of a
-// tile this size has 40 K gelu evaluations and nothing to overlap them with
+// tile this size has tens of thousands of gelu evaluations and nothing to overlap them with
 constexpr int WTAB_LO = 0x3800, WTAB_N = 2560;               // magnitudes 0x3800 .. 0x41ff, per sign
-constexpr int WTAB_OFF = 2 * WSTAGE;
-constexpr int WBIAS_OFF = WTAB_OFF + 2 * WTAB_N * 2;          // the tile's 320 bias values (bf16)
-constexpr int WLDS = WBIAS_OFF + WBN * 2;
-static_assert(WLDS <= 160 * 1024, "LDS budget");
-constexpr int WLDC = WBN + 72;                               // staged row: 196 dwords = 4 mod 64 banks, see the epilogue
-constexpr int WXU = 4, WWU = 5, WLPS = WXU + WWU;           // DMA instructions per wave per stage (x rows, W rows)
-static_assert(128 * WLDC * 2 <= WLDS, "epilogue staging fits the ring");
 
-struct WFr { bf16x8 a[WTM]; bf16x8 b[WTN]; };
+// 8 waves = 4 row groups x 2 column groups; a wave owns TM x TN MFMA tiles of 32 x 32: tile (128 TM) x (64 TN).
+// Only 256 x 320 (TM 2, TN 5) is instantiated: 128 x 256, 256 x 256 and 128 x 320 were measured on the SDXL shapes
+// and never beat the tiles of lora_gemm_pipe.hip there.
+template <int TM_, int TN_>
+struct WCfg {
+  static constexpr int TM = TM_, TN = TN_;
+  static constexpr int BM = 128 * TM, BN = 64 * TN;
+  static constexpr int WR = 32 * TM, WC = 32 * TN;            // rows / columns of a wave
+  static constexpr int STAGE = (BM + BN) * 128;               // one 64-column stage
+  static constexpr int TAB_OFF = 2 * STAGE;
+  static constexpr int BIAS_OFF = TAB_OFF + 2 * WTAB_N * 2;   // the tile's bias values (bf16)
+  static constexpr int LDS = BIAS_OFF + BN * 2;
+  static constexpr int XU = 2 * TM, WU = TN, LPS = XU + WU;   // DMA instructions per wave per stage (x rows, W rows)
+  // staged row of the epilogue: (BN + pad) / 2 dwords = 4 mod 64 banks
+  static constexpr int LDC = BN + ((8 + 128 - BN % 128) % 128);
+  static_assert((LDC / 2) % 64 == 4 && LDC >= BN, "staging row stride");
+  static_assert(LDS <= 160 * 1024, "LDS budget");
+  static_assert(128 * LDC * 2 <= 2 * STAGE, "epilogue staging fits the ring");
+  static_assert(BN <= 512 && (128 * (BN / 8)) % 512 == 0 && (128 * (BN / 16)) % 512 == 0, "epilogue split");
+};
 
+template <class C>
+struct WFrT { bf16x8 a[C::TM]; bf16x8 b[C::TN]; };
+
+template <class C>
 __global__ __launch_bounds__(512, 2) void lora_gemm_wide_kernel(const LoraGemmParams p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
+  constexpr int WBM = C::BM, WBN = C::BN, WTM = C::TM, WTN = C::TN, WSTAGE = C::STAGE, WLDC = C::LDC;
+  constexpr int WXU = C::XU, WWU = C::WU, WLPS = C::LPS, WTAB_OFF = C::TAB_OFF, WBIAS_OFF = C::BIAS_OFF;
+  constexpr int WR = C::WR, WC = C::WC;
+  using WFr = WFrT<C>;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
@@ -69,11 +87,11 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_wide_kernel(const LoraGemmPa
   // so two element offsets (even / odd q) per operand describe all of a lane's sources; M and N are multiples of
   // the tile (no clamping).
   const int r8 = lane >> 3;
-  const int rx0 = wave * 32 + r8, rx1 = rx0 + 8;               // stage rows of x instructions 0 / 1
+  const int rx0 = wave * (WBM / 8) + r8, rx1 = rx0 + 8;               // stage rows of x instructions 0 / 1
   const int pcx0 = ((lane & 7) ^ ((rx0 >> 1) & 7)) * 8, pcx1 = ((lane & 7) ^ ((rx1 >> 1) & 7)) * 8;
-  const int rw0 = WBM + wave * 40 + r8, rw1 = rw0 + 8;          // stage rows of W instructions 0 / 1
+  const int rw0 = WBM + wave * (WBN / 8) + r8, rw1 = rw0 + 8;          // stage rows of W instructions 0 / 1
   const int pcw0 = ((lane & 7) ^ ((rw0 >> 1) & 7)) * 8, pcw1 = ((lane & 7) ^ ((rw1 >> 1) & 7)) * 8;
-  const int wrow = wave * 40 + r8;                              // W row of instruction 0 inside the tile
+  const int wrow = wave * (WBN / 8) + r8;                              // W row of instruction 0 inside the tile
   const bf16_t* px = p.x + (size_t)m0 * K;
   const bf16_t* pw = p.w + (size_t)n0 * K;
   const bf16_t* px2 = p.t_ext != nullptr ? p.t_ext + (size_t)m0 * p.ldt + (p.t_nsplit > 0 ? (n0 / p.t_nsplit) * p.R : 0) : px;
@@ -87,10 +105,10 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_wide_kernel(const LoraGemmPa
     const bf16_t* gw1 = bw + wrow * sw_ + pcw1;
 #pragma unroll
     for (int q = 0; q < WXU; ++q)
-      __builtin_amdgcn_global_load_lds((gptr_t)(((q & 1) ? gx1 : gx0) + q * 8 * sx), (lptr_t)(stage + (wave * 32 + q * 8) * 128), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((gptr_t)(((q & 1) ? gx1 : gx0) + q * 8 * sx), (lptr_t)(stage + (wave * (WBM / 8) + q * 8) * 128), 16, 0, 0);
 #pragma unroll
     for (int q = 0; q < WWU; ++q)
-      __builtin_amdgcn_global_load_lds((gptr_t)(((q & 1) ? gw1 : gw0) + q * 8 * sw_), (lptr_t)(stage + (WBM + wave * 40 + q * 8) * 128), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((gptr_t)(((q & 1) ? gw1 : gw0) + q * 8 * sw_), (lptr_t)(stage + (WBM + wave * (WBN / 8) + q * 8) * 128), 16, 0, 0);
   };
   auto issue = [&](int t, int st) {                             // K tile t into stage st
     char* stage = smem + st * WSTAGE;
@@ -102,9 +120,9 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_wide_kernel(const LoraGemmPa
     const char* s = smem + st * WSTAGE;
     const int po = ((2 * ks + lh) ^ sw) * 16;
 #pragma unroll
-    for (int i = 0; i < WTM; ++i) f.a[i] = *reinterpret_cast<const bf16x8*>(s + (wm * 64 + i * 32 + l32) * 128 + po);
+    for (int i = 0; i < WTM; ++i) f.a[i] = *reinterpret_cast<const bf16x8*>(s + (wm * WR + i * 32 + l32) * 128 + po);
 #pragma unroll
-    for (int j = 0; j < WTN; ++j) f.b[j] = *reinterpret_cast<const bf16x8*>(s + (WBM + wn * 160 + j * 32 + l32) * 128 + po);
+    for (int j = 0; j < WTN; ++j) f.b[j] = *reinterpret_cast<const bf16x8*>(s + (WBM + wn * WC + j * 32 + l32) * 128 + po);
   };
   f32x16 acc[WTM][WTN];
 #pragma unroll
@@ -162,8 +180,8 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_wide_kernel(const LoraGemmPa
   // a contiguous output row; two passes of 128 rows (the waves' upper / lower 32-row MFMA tiles).
   bf16_t* sC = reinterpret_cast<bf16_t*>(smem);
   const int out_ld = p.geglu ? (N >> 1) : N;
-  constexpr int CPR = WBN / 8, ECH = 128 * CPR / 512;        // plain: 40 pieces per staged row, 10 per thread
-  constexpr int OPR = WBN / 16, GCH = 128 * OPR / 512;       // GEGLU: 20 output pieces per staged row, 5 per thread
+  constexpr int CPR = WBN / 8, ECH = 128 * CPR / 512;        // plain: pieces per staged row, per thread
+  constexpr int OPR = WBN / 16, GCH = 128 * OPR / 512;       // GEGLU: output pieces per staged row, per thread
 #pragma unroll
   for (int i = 0; i < WTM; ++i) {
     // the MFMA operands are swapped (W rows first), so a lane holds one output row (l32) and, per group of four
@@ -173,7 +191,7 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_wide_kernel(const LoraGemmPa
     for (int j = 0; j < WTN; ++j) {
 #pragma unroll
       for (int g4 = 0; g4 < 4; ++g4) {
-        const int col = wn * 160 + j * 32 + 8 * g4 + 4 * lh;
+        const int col = wn * WC + j * 32 + 8 * g4 + 4 * lh;
         const u32x2 bb = *reinterpret_cast<const u32x2*>(sbias + col);
         u32x2 o;
         o[0] = pack_bf16x2(acc[i][j][4 * g4] + bf16_lo(bb[0]), acc[i][j][4 * g4 + 1] + bf16_hi(bb[0]));
@@ -186,7 +204,7 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_wide_kernel(const LoraGemmPa
 #pragma unroll
       for (int q = 0; q < ECH; ++q) {
         const int c = tid + q * 512, srow = c / CPR, ch = c % CPR;
-        const size_t g = (size_t)(m0 + (srow >> 5) * 64 + i * 32 + (srow & 31)) * N + n0 + ch * 8;
+        const size_t g = (size_t)(m0 + (srow >> 5) * WR + i * 32 + (srow & 31)) * N + n0 + ch * 8;
         u32x4 o = *reinterpret_cast<const u32x4*>(sC + srow * WLDC + ch * 8);
         if (p.res != nullptr) {
           const u32x4 rr = *reinterpret_cast<const u32x4*>(p.res + g);
@@ -201,7 +219,7 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_wide_kernel(const LoraGemmPa
       for (int q = 0; q < GCH; ++q) {
         const int c = tid + q * 512, srow = c / OPR, oc = c % OPR;
         const int grp = oc >> 2, sub = oc & 3;
-        const size_t g = (size_t)(m0 + (srow >> 5) * 64 + i * 32 + (srow & 31)) * out_ld + (n0 >> 1) + grp * 32 + sub * 8;
+        const size_t g = (size_t)(m0 + (srow >> 5) * WR + i * 32 + (srow & 31)) * out_ld + (n0 >> 1) + grp * 32 + sub * 8;
         const u32x4 hv = *reinterpret_cast<const u32x4*>(sC + srow * WLDC + grp * 64 + sub * 8);
         const u32x4 gv = *reinterpret_cast<const u32x4*>(sC + srow * WLDC + grp * 64 + 32 + sub * 8);
         u32x4 ar;                                       // gelu(gate) rounded to bf16 before the product
@@ -229,23 +247,23 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_wide_kernel(const LoraGemmPa
   }
 }
 
-}  // namespace
-
-bool lora_gemm_wide_ok(const LoraGemmParams& p) {
+template <class C>
+bool wide_ok(const LoraGemmParams& p) {
   const bool plain = p.R == 0 || p.t_ext != nullptr;
-  return plain && p.grp == nullptr && p.sg_mode == 0 && p.conv_cin == 0 && p.M % WBM == 0 && p.N % WBN == 0 &&
+  return plain && p.grp == nullptr && p.sg_mode == 0 && p.conv_cin == 0 && p.M % C::BM == 0 && p.N % C::BN == 0 &&
          p.K % 64 == 0 && p.K >= 64 && (p.t_ext == nullptr || (p.R % 64 == 0 && p.ldt % 8 == 0)) &&
-         (p.t_nsplit == 0 || p.t_nsplit % WBN == 0) && (long)p.M * (p.K > p.ldt ? p.K : p.ldt) < (1L << 31) &&
-         (long)p.N * p.K < (1L << 31);
+         (p.t_nsplit == 0 || p.t_nsplit % C::BN == 0) && (long)C::BM * (p.K > p.ldt ? p.K : p.ldt) < (1L << 31) &&
+         (long)C::BN * p.K < (1L << 31);
 }
 
-int lora_gemm_wide_launch(LoraGemmParams p, hipStream_t stream) {
-  if (!lora_gemm_wide_ok(p)) return KH_ERR_UNSUPPORTED;
-  p.m_tiles = p.M / WBM;
-  p.n_tiles = p.N / WBN;
-  static bool attr_done = false;
+template <class C>
+int wide_launch(LoraGemmParams p, hipStream_t stream) {
+  if (!wide_ok<C>(p)) return KH_ERR_UNSUPPORTED;
+  p.m_tiles = p.M / C::BM;
+  p.n_tiles = p.N / C::BN;
+  static bool attr_done = false;  // per template instantiation
   if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void*)lora_gemm_wide_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, WLDS);
+    hipError_t e = hipFuncSetAttribute((const void*)lora_gemm_wide_kernel<C>, hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS);
     if (e != hipSuccess) return (int)e;
     attr_done = true;
   }
@@ -255,10 +273,15 @@ int lora_gemm_wide_launch(LoraGemmParams p, hipStream_t stream) {
   for (int gm = 1; gm <= 8; gm *= 2) {
     const int gn = 8 / gm;
     const int rm = (p.m_tiles + gm - 1) / gm, rn = (p.n_tiles + gn - 1) / gn;
-    const double cost = ((double)rm * WBM + (double)rn * WBN) * (8.0 * rm * rn) / ((double)p.m_tiles * p.n_tiles);
+    const double cost = ((double)rm * C::BM + (double)rn * C::BN) * (8.0 * rm * rn) / ((double)p.m_tiles * p.n_tiles);
     if (p.xg_n == 0 || cost < best) { best = cost; p.xg_n = gn; p.xr_m = rm; p.xr_n = rn; }
   }
   const unsigned grid = 8u * (unsigned)p.xr_m * (unsigned)p.xr_n;
-  kh_launch(KH_TAG_LORA_GEMM, lora_gemm_wide_kernel, dim3(grid), dim3(512), WLDS, stream, p);
+  kh_launch(KH_TAG_LORA_GEMM, lora_gemm_wide_kernel<C>, dim3(grid), dim3(512), C::LDS, stream, p);
   KH_RETURN_LAST_ERROR();
 }
+
+}  // namespace
+
+bool lora_gemm_wide_ok(const LoraGemmParams& p) { return wide_ok<WCfg<2, 5>>(p); }
+int lora_gemm_wide_launch(LoraGemmParams p, hipStream_t stream) { return wide_launch<WCfg<2, 5>>(p, stream); }
