@@ -80,6 +80,26 @@ int kh_lora_shrink_bf16(const void* x, const void* a_cat, const float* col_scale
 int kh_lora_linear_pre_bf16(const void* x, const void* w, const void* bias, const void* t, int64_t ldt,
                             int64_t n_split, const void* b_cat, const void* residual, void* y, int64_t M, int64_t N,
                             int64_t K, int64_t R, int flags, void* stream);
+/* The two-launch form from its unshrunk operands: y = x W^T + b + ((x A_cat^T) * col_scale) B_cat^T (+ residual | GEGLU)
+ * with t_scratch [M,R] bf16 receiving the shrink result (LoRACompatibleLinear.forward, diffusers-hf/src/diffusers/
+ * models/lora.py:224-225 + :423-431, as kh_lora_shrink_bf16 followed by kh_lora_linear_pre_bf16).  Where the base
+ * GEMM's 128x128 tiles leave at least a quarter of the CUs idle (N = 1280 at M = 2048) the shrink runs INSIDE the GEMM
+ * launch on those CUs: its workgroups come first in the grid, store t_scratch write-through and count themselves into
+ * `counters`; the GEMM workgroups read t_scratch (as the last K tiles) only after their row block's count is complete.
+ * Same results as the two launches up to the fp32 summation order of the shrink.
+ * counters: KH_SPLIT_COUNTER_INTS zero-initialised int32 of device memory, owned by the caller and shared by all
+ * calls that do not overlap in time on the device (every launch leaves them zeroed); NULL = always two launches.
+ * counters[KH_SPLIT_COUNTER_INTS - 1] becomes 1 if a bounded wait inside a launch ever ran out (the result of that
+ * call is then undefined).  K % 64 == 0, R % 32 == 0, R <= 128.  flags: bit 0 GEGLU, bits 8..15: 1 = always two
+ * launches. */
+#define KH_SPLIT_MAX_ROW_BLOCKS 2047
+#define KH_SPLIT_COUNTER_INTS (2 * KH_SPLIT_MAX_ROW_BLOCKS + 2)
+int kh_lora_linear_split_bf16(const void* x, const void* w, const void* bias, const void* a_cat, const float* col_scale,
+                              const void* b_cat, void* t_scratch, int32_t* counters, const void* residual, void* y,
+                              int64_t M, int64_t N, int64_t K, int64_t R, int flags, void* stream);
+/* How many kernel launches kh_lora_linear_split_bf16 makes for this shape when counters are given (1 or 2; negative:
+ * KH_ERR_*).  No counterpart in the reference; for callers that account per launch (benchmarks). */
+int kh_lora_linear_split_launches(int64_t M, int64_t N, int64_t K, int64_t R, int flags);
 /* n_groups layers that read the SAME x in one launch (the context K/V projections of every cross-attention
  * of the UNet: 140 GEMMs of 154 rows each, which individually cannot fill the chip):
  *   y_g = x W_g^T + bias_g + t_g B_cat_g^T        g = 0 .. n_groups-1, all with the same M, N, K, R

@@ -32,6 +32,12 @@ struct LoraGemmParams {
   // 3x3 convolution as an implicit GEMM (conv_cin > 0): x is an NHWC image [Nb, conv_h, conv_w, conv_cin], row m
   // of the GEMM is output pixel m of [Nb, conv_ho, conv_wo], K = 9 * conv_cin ordered (kh, kw, ci), padding 1
   int conv_cin, conv_h, conv_w, conv_ho, conv_wo, conv_stride;
+  // shrink inside the GEMM launch (il_blocks > 0): the first il_blocks workgroups compute t_ext = the shrink of x
+  // (a_cat, col_scale) in 64x64 tiles and count themselves into il_cnt[row block]; the GEMM workgroups wait for their
+  // row block's count before they read t_ext.  il_cnt: KH_SPLIT_COUNTER_INTS zero-initialised ints (arrivals, departures,
+  // time-out flag); every launch leaves them zeroed.
+  int il_blocks = 0;
+  int* il_cnt = nullptr;
 };
 
 // Software-pipelined kernel (lora_gemm_pipe.hip); needs K % 32 == 0.  tile_sel: 0 automatic, >= 16 forces a tile.
@@ -42,6 +48,10 @@ int lora_gemm_pipe_launch_conv(const LoraGemmParams& p, hipStream_t stream);
 int lora_gemm_pipe_launch_sgmv(const LoraGemmParams& p, int n_segments, hipStream_t stream);
 // Grouped form: grid.y = n_groups, per-group pointers from p.grp; rank columns (p.R > 0) as extra K tiles.
 int lora_gemm_pipe_launch_grouped(const LoraGemmParams& p, int n_groups, hipStream_t stream);
+// Shrink and GEMM in one launch for shapes whose 128x128 tiles leave CUs idle (p.a_cat / col_scale / b_cat set, p.t_ext =
+// scratch for the shrink result, p.il_cnt = counters); KH_ERR_UNSUPPORTED when the shape does not qualify.
+bool lora_gemm_pipe_il_ok(const LoraGemmParams& p);
+int lora_gemm_pipe_launch_il(const LoraGemmParams& p, hipStream_t stream);
 // Narrow-output variant (lora_gemm_ksplit.hip): (32 * row_groups) x 160 tiles, 8 waves as row_groups x k-slices;
 // plain or K-extended GEMM with bias / residual, K % 64 == 0.  row_groups 2 or 4.
 bool lora_gemm_ksplit_ok(const LoraGemmParams& p);
@@ -52,3 +62,10 @@ int lora_gemm_ksplit_launch_conv(const LoraGemmParams& p, int row_groups, hipStr
 // GEGLU; M % 256 == 0, N % 320 == 0, K % 64 == 0.
 bool lora_gemm_wide_ok(const LoraGemmParams& p);
 int lora_gemm_wide_launch(LoraGemmParams p, hipStream_t stream);
+
+// Counter buffer of kh_lora_linear_split_bf16 (the same numbers as in include/katz_hip.h): arrivals [row block],
+// departures [MAX + row block], the time-out flag last.
+constexpr int KH_SPLIT_MAX_ROW_BLOCKS = 2047;
+constexpr int KH_SPLIT_COUNTER_INTS = 2 * KH_SPLIT_MAX_ROW_BLOCKS + 2;
+extern "C" int kh_lora_shrink_bf16(const void* x, const void* a_cat, const float* col_scale, void* t, int64_t M, int64_t K,
+                                   int64_t R, void* stream);

@@ -525,6 +525,60 @@ KH_EXPORT int kh_lora_linear_pre_bf16(const void* x, const void* w, const void* 
   return lora_gemm_pipe_launch(p, (flags >> 8) & 0xff, (hipStream_t)stream);
 }
 
+// Shrink + base GEMM + expand from the unshrunk operands; one launch where the GEMM leaves CUs idle, two otherwise.
+// See include/katz_hip.h.
+static LoraGemmParams split_params(const void* x, const void* w, const void* bias, const void* a_cat, const float* col_scale,
+                                   const void* b_cat, void* t_scratch, int32_t* counters, const void* residual, void* y,
+                                   int64_t M, int64_t N, int64_t K, int64_t R, bool geglu) {
+  LoraGemmParams p;
+  p.x = (const bf16_t*)x; p.w = (const bf16_t*)w; p.bias = (const bf16_t*)bias;
+  p.a_cat = (const bf16_t*)a_cat; p.b_cat = (const bf16_t*)b_cat; p.col_scale = col_scale;
+  p.t_ext = (const bf16_t*)t_scratch; p.ldt = (int)R; p.grp = nullptr; p.dbg = 0; p.t_nsplit = 0;
+  p.res = (const bf16_t*)residual; p.y = (bf16_t*)y;
+  p.M = (int)M; p.N = (int)N; p.K = (int)K; p.R = (int)R;
+  p.m_tiles = p.n_tiles = p.n_chunk = p.n_chunks = 0;
+  p.geglu = geglu ? 1 : 0;
+  p.xg_n = p.xr_m = p.xr_n = 0;
+  p.sg_start = p.sg_adapter = p.sg_rank = nullptr; p.sg_scale = nullptr; p.sg_mode = 0; p.sg_wstride = 0;
+  p.conv_cin = p.conv_h = p.conv_w = p.conv_ho = p.conv_wo = p.conv_stride = 0;
+  p.il_cnt = counters;
+  return p;
+}
+
+KH_EXPORT int kh_lora_linear_split_launches(int64_t M, int64_t N, int64_t K, int64_t R, int flags) {
+  if (M <= 0 || N <= 0 || K <= 0 || R <= 0 || M > (1 << 24) || N > (1 << 24) || K > (1 << 24)) return KH_ERR_INVALID_ARG;
+  if (((flags >> 8) & 0xff) != 0 || (M + 127) / 128 > KH_SPLIT_MAX_ROW_BLOCKS) return 2;
+  static int32_t dummy_counter;                  // the rule only asks whether counters were given
+  static const char dummy = 0;
+  const LoraGemmParams p = split_params(&dummy, &dummy, nullptr, &dummy, reinterpret_cast<const float*>(&dummy), &dummy,
+                                        const_cast<char*>(&dummy), &dummy_counter, nullptr, const_cast<char*>(&dummy), M, N, K, R,
+                                        (flags & 1) != 0);
+  return lora_gemm_pipe_il_ok(p) ? 1 : 2;
+}
+
+KH_EXPORT int kh_lora_linear_split_bf16(const void* x, const void* w, const void* bias, const void* a_cat,
+                                        const float* col_scale, const void* b_cat, void* t_scratch, int32_t* counters,
+                                        const void* residual, void* y, int64_t M, int64_t N, int64_t K, int64_t R,
+                                        int flags, void* stream) {
+  if (!x || !w || !y || !a_cat || !col_scale || !b_cat || !t_scratch || M <= 0 || N <= 0 || K <= 0 || R <= 0)
+    return KH_ERR_INVALID_ARG;
+  if (K % 64 != 0 || N % 8 != 0 || R % 32 != 0) return KH_ERR_UNSUPPORTED;
+  if (R > 128) return KH_ERR_TOO_LARGE;
+  if (M > (1 << 24) || N > (1 << 24) || K > (1 << 24)) return KH_ERR_TOO_LARGE;
+  const bool geglu = (flags & 1) != 0;
+  if (geglu && (N % 64 != 0 || residual != nullptr)) return KH_ERR_UNSUPPORTED;
+  if (!kh_aligned16(x) || !kh_aligned16(w) || !kh_aligned16(y) || !kh_aligned16(a_cat) || !kh_aligned16(b_cat) ||
+      !kh_aligned16(t_scratch) || (residual && !kh_aligned16(residual)))
+    return KH_ERR_ALIGNMENT;
+  if (counters != nullptr && kh_lora_linear_split_launches(M, N, K, R, flags) == 1) {
+    const LoraGemmParams p = split_params(x, w, bias, a_cat, col_scale, b_cat, t_scratch, counters, residual, y, M, N, K, R, geglu);
+    return lora_gemm_pipe_launch_il(p, (hipStream_t)stream);
+  }
+  const int rc = kh_lora_shrink_bf16(x, a_cat, col_scale, t_scratch, M, K, R, stream);
+  if (rc != KH_OK) return rc;
+  return kh_lora_linear_pre_bf16(x, w, bias, t_scratch, R, 0, b_cat, residual, y, M, N, K, R, flags & 0xff, stream);
+}
+
 // 3x3 convolution, padding 1, NHWC, as an implicit GEMM on the pipelined kernel; see include/katz_hip.h.
 KH_EXPORT int kh_conv3x3_nhwc_bf16(const void* x, const void* w, const void* bias, const void* residual, void* y,
                                    int64_t Nb, int64_t H, int64_t W, int64_t Cin, int64_t Cout, int64_t stride,

@@ -12,6 +12,7 @@
 //     lane fetches, not to where it lands).
 #include "kh_common.h"
 #include "lora_gemm.h"
+#include "lora_shrink_tile.h"
 #include <type_traits>
 
 namespace {
@@ -106,13 +107,14 @@ __device__ __attribute__((aligned(256))) const uint32_t kh_zero_page[64] = {0};
 
 struct ConvGeom { int w, cin; };  // input width and channels (elements)
 
-template <class C, bool SHRINK, int NX, bool CONV, class TailLoads>
+template <class C, bool SHRINK, int NX, bool CONV, class TailLoads, bool IL = false>
 __device__ __forceinline__ void k_loop(char* smem, const Dma<C, SHRINK>& dma, const bf16_t* px, const bf16_t* pw,
                                        const bf16_t* pa, const bf16_t* px2, const bf16_t* pw2, int KT, int KT1,
                                        int lane, int wm, int wn,
                                        int l32, int lh, int sw, f32x16 (&acc)[C::TM][C::TN],
                                        f32x16 (&tacc)[C::SM > 0 ? C::SM : 1][C::NRT > 0 ? C::NRT : 1],
-                                       TailLoads tail_loads, ConvGeom cg, bool nodma = false, bool fixk = false) {
+                                       TailLoads tail_loads, ConvGeom cg, bool nodma = false, bool fixk = false,
+                                       const int* il_cnt = nullptr, int il_target = 0, int* il_err = nullptr) {
   constexpr int TM = C::TM, TN = C::TN, NRT = C::NRT, NST = C::NST;
   constexpr int BKP = C::BKP, ROWB = C::ROWB, KS = C::KS;
   constexpr int PD = NST - 1;  // prefetch distance in K tiles
@@ -141,6 +143,15 @@ __device__ __forceinline__ void k_loop(char* smem, const Dma<C, SHRINK>& dma, co
       }
       return;
     }
+    if (IL && t == KT1) {
+      // first request for T: wait (bounded) until the shrink workgroups of this row block have all arrived
+      if (lane == 0) {
+        int it = 0;
+        while (__hip_atomic_load(il_cnt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < il_target && ++it < (1 << 20))
+          __builtin_amdgcn_s_sleep(8);
+        if (it >= (1 << 20)) __hip_atomic_store(il_err, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
 #pragma unroll
     for (int q = 0; q < D::LPS; ++q) {
       const bool partial = SHRINK && (q == D::LPS - 1) && (D::RA % 16 != 0);
@@ -148,8 +159,12 @@ __device__ __forceinline__ void k_loop(char* smem, const Dma<C, SHRINK>& dma, co
       const bf16_t* base = q < D::XI ? px : (q < D::XI + D::WI ? pw : pa);
       const bf16_t* base2 = q < D::XI ? px2 : pw2;
       const bf16_t* g = (SHRINK || t < KT1) ? base + dma.off[q] + (fixk ? 0 : t * BKP) : base2 + dma.off2[q] + (t - KT1) * BKP;
-      if (!partial || lane < 32)
+      if (IL && t >= KT1 && q < D::XI) {
+        // T was written inside this launch, maybe on another XCD: read past the (non-coherent) L2
+        __builtin_amdgcn_global_load_lds((gptr_t)g, (lptr_t)(stage + dma.dst[q]), 16, 0, 17 /* sc0 sc1 */);
+      } else if (!partial || lane < 32) {
         __builtin_amdgcn_global_load_lds((gptr_t)g, (lptr_t)(stage + dma.dst[q]), 16, 0, 0);
+      }
     }
   };
   auto read_frags = [&](int t, Frags<C, SHRINK>& f) {
@@ -258,10 +273,29 @@ __device__ __forceinline__ void k_loop(char* smem, const Dma<C, SHRINK>& dma, co
   }
 }
 
-template <class C, bool CONV = false>
+template <class C, bool CONV = false, bool IL = false>
 __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const LoraGemmParams pin) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   LoraGemmParams p = pin;
+  if constexpr (IL) {
+    // The first il_blocks workgroups are the shrink: 64x64 tiles of T on 4 of the 8 waves, stored write-through,
+    // then one arrival per tile on the counter of the 128-row block the tile belongs to.  They have the lowest
+    // block ids, so they are resident before any workgroup that waits for them.
+    if ((int)blockIdx.x < pin.il_blocks) {
+      const int gx = (pin.M + 63) / 64, gy = pin.R / 64;
+      if ((int)blockIdx.x >= gx * gy) return;               // padding to a multiple of 8 (the XCD map of the rest)
+      const int bx = blockIdx.x % gx, by = blockIdx.x / gx;
+      ShrinkParams sp;
+      sp.x = pin.x; sp.a_cat = pin.a_cat; sp.col_scale = pin.col_scale; sp.t = const_cast<bf16_t*>(pin.t_ext);
+      sp.M = pin.M; sp.K = pin.K; sp.R = pin.R;
+      lora_shrink_tile<SCfg<4, 2, 2>, true>(sp, bx, by, smem);
+      __builtin_amdgcn_s_waitcnt(0);                          // this thread's write-through stores have completed
+      __syncthreads();
+      if (threadIdx.x == 0) __hip_atomic_fetch_add(pin.il_cnt + bx / 2, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      return;
+    }
+  }
+  const int bid = IL ? (int)blockIdx.x - pin.il_blocks : (int)blockIdx.x;
   if (pin.grp != nullptr) {  // grouped launch: this workgroup's layer
     const uint64_t* g = pin.grp + (size_t)blockIdx.y * 5;
     p.w = reinterpret_cast<const bf16_t*>(g[0]);
@@ -303,13 +337,13 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
     // xg_m x xg_n grid owns the block of xr_m x xr_n tiles at (xm*xr_m, xn*xr_n) and walks it row by row, so
     // the W rows of its xr_n tile columns stay in its L2 while the x rows stream through once.  (With contiguous
     // ranges of a row-major tile list every XCD reads all of W, twice over: 8.6x the algorithmic bytes.)
-    const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+    const int xcd = bid & 7, local = bid >> 3;
     m_blk = (xcd / p.xg_n) * p.xr_m + local / p.xr_n;
     chunk = (xcd % p.xg_n) * p.xr_n + local % p.xr_n;
     if (local / p.xr_n >= p.xr_m || m_blk >= p.m_tiles || chunk >= p.n_chunks) return;  // padding of the grid
   } else {
     const uint32_t total = (uint32_t)p.m_tiles * (uint32_t)p.n_chunks;
-    const uint32_t logical = xcd_remap(blockIdx.x, total);
+    const uint32_t logical = xcd_remap((uint32_t)bid, total);
     m_blk = logical / p.n_chunks; chunk = logical % p.n_chunks;
   }
   const int m0 = m_blk * BM;
@@ -326,7 +360,7 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
   const int sw = (l32 / C::SWR) % C::PPR;
 
   // tuning only: dbg & 16 turns `res` into a timestamp buffer (8 x int64 per workgroup), no residual
-  long long* ts = (p.dbg & 16) ? reinterpret_cast<long long*>(const_cast<bf16_t*>(p.res)) + (size_t)blockIdx.x * 8 : nullptr;
+  long long* ts = (p.dbg & 16) ? reinterpret_cast<long long*>(const_cast<bf16_t*>(p.res)) + (size_t)bid * 8 : nullptr;
   if (p.dbg & 16) p.res = nullptr;
   auto stamp = [&](int i) { if (ts != nullptr && tid == 0) ts[i] = (long long)__builtin_readcyclecounter(); };
   stamp(0);
@@ -430,11 +464,28 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
     } else {
       Dma<C, false> d;
       dma_setup(d);
-      k_loop<C, false, BCH, CONV>(smem, d, p.x, p.w, p.a_cat, p.t_ext, p.b_cat, KT, KT1, lane, wm, wn, l32, lh, sw, acc, tacc, tail_loads, ConvGeom{p.conv_w, p.conv_cin}, (p.dbg & 64) != 0, (p.dbg & 128) != 0);
+      if constexpr (IL) {
+        const int gx = (M + 63) / 64, rt = gx - 2 * m_blk < 2 ? gx - 2 * m_blk : 2;   // 64-row shrink tiles over this row block
+        k_loop<C, false, BCH, CONV, decltype(tail_loads), true>(smem, d, p.x, p.w, p.a_cat, p.t_ext, p.b_cat, KT, KT1, lane, wm, wn, l32, lh, sw, acc, tacc, tail_loads, ConvGeom{0, 0}, false, false,
+                                                                p.il_cnt + m_blk, rt * (p.R / 64), p.il_cnt + (KH_SPLIT_COUNTER_INTS - 1));
+      } else {
+        k_loop<C, false, BCH, CONV>(smem, d, p.x, p.w, p.a_cat, p.t_ext, p.b_cat, KT, KT1, lane, wm, wn, l32, lh, sw, acc, tacc, tail_loads, ConvGeom{p.conv_w, p.conv_cin}, (p.dbg & 64) != 0, (p.dbg & 128) != 0);
+      }
     }
     stamp(2);
     __syncthreads();  // every wave is done reading the ring before sB / sC reuse it
     stamp(3);
+    if constexpr (IL) {
+      // this workgroup has read T: the last of the row block's workgroups to say so zeroes both counters for the
+      // next launch
+      if (tid == 0) {
+        int* dep = p.il_cnt + KH_SPLIT_MAX_ROW_BLOCKS + m_blk;
+        if (__hip_atomic_fetch_add(dep, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == p.n_chunks - 1) {
+          __hip_atomic_store(p.il_cnt + m_blk, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(dep, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+      }
+    }
 
     if constexpr (NRT > 0) {
       if (shrink) {
@@ -609,6 +660,49 @@ bool deep_stage_ok(const LoraGemmParams& p) {
 bool plain_ok(const LoraGemmParams& p) { return p.R == 0 || p.t_ext != nullptr; }
 
 }  // namespace
+
+// Shrink inside the launch: the shapes whose 128x128 tiles leave at least a quarter of the CUs idle, so that the 64x64
+// shrink tiles find CUs of their own next to the GEMM workgroups.  Measured at M 2048 / N 1280 / K 1280: 20 us against
+// 17.8 + 4.6 for the two launches (the GEMM workgroups run 2 us slower beside the shrink, whether or not they have to
+// wait for it); from K = 5120 the 64x160 tiles of the two-launch form win that back, so long K stays with them.
+bool lora_gemm_pipe_il_ok(const LoraGemmParams& p) {
+  const long tiles = (long)((p.M + 127) / 128) * ((p.N + 127) / 128);
+  const long shr = (long)((p.M + 63) / 64) * (p.R / 64);
+  return p.R > 0 && p.R % 64 == 0 && p.K % 64 == 0 && p.t_ext != nullptr && p.a_cat != nullptr && p.col_scale != nullptr &&
+         p.il_cnt != nullptr && p.ldt == p.R && p.t_nsplit == 0 && p.grp == nullptr && p.sg_mode == 0 && p.conv_cin == 0 &&
+         !p.geglu && p.M >= 1024 && p.K <= 2560 && tiles <= 192 && tiles + shr <= 256;
+}
+
+int lora_gemm_pipe_launch_il(const LoraGemmParams& pin, hipStream_t stream) {
+  if (!lora_gemm_pipe_il_ok(pin)) return KH_ERR_UNSUPPORTED;
+  using C = PCfg<128, 128, 2, 4, 0, 3, 64>;
+  using S = SCfg<4, 2, 2>;
+  LoraGemmParams p = pin;
+  p.m_tiles = (p.M + C::BM - 1) / C::BM;
+  p.n_tiles = (p.N + C::BN - 1) / C::BN;
+  p.n_chunk = 1;
+  p.n_chunks = p.n_tiles;
+  constexpr int LDS = (int)C::LDS_BYTES > S::LDS ? (int)C::LDS_BYTES : S::LDS;
+  static bool attr_done = false;
+  if (!attr_done) {
+    hipError_t e = hipFuncSetAttribute((const void*)lora_gemm_pipe_kernel<C, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
+    if (e != hipSuccess) return (int)e;
+    attr_done = true;
+  }
+  double best = 0;
+  p.xg_n = 0;
+  for (int gm = 1; gm <= 8; gm *= 2) {
+    const int gn = 8 / gm;
+    const int rm = (p.m_tiles + gm - 1) / gm, rn = (p.n_tiles + gn - 1) / gn;
+    const double cost = ((double)rm * C::BM + (double)rn * C::BN) * (8.0 * rm * rn) / ((double)p.m_tiles * p.n_tiles);
+    if (p.xg_n == 0 || cost < best) { best = cost; p.xg_n = gn; p.xr_m = rm; p.xr_n = rn; }
+  }
+  const int shr = ((p.M + 63) / 64) * (p.R / 64);
+  p.il_blocks = (shr + 7) / 8 * 8;
+  const unsigned grid = (unsigned)p.il_blocks + 8u * (unsigned)p.xr_m * (unsigned)p.xr_n;
+  kh_launch(KH_TAG_LORA_GEMM, lora_gemm_pipe_kernel<C, false, true>, dim3(grid), dim3(C::NT), (size_t)LDS, stream, p);
+  KH_RETURN_LAST_ERROR();
+}
 
 int lora_gemm_pipe_launch_conv(const LoraGemmParams& p, hipStream_t stream) {
   const long tiles = (long)((p.M + 127) / 128) * ((p.N + 127) / 128);

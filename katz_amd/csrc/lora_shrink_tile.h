@@ -1,0 +1,134 @@
+// Device code of the LoRA shrink tile, shared by the stand-alone kernel (lora_shrink.hip) and by the GEMM launch that
+// runs its shrink on otherwise idle CUs (lora_gemm_pipe.hip).  See lora_shrink.hip for the design.
+#pragma once
+#include "kh_common.h"
+
+namespace {
+
+struct ShrinkParams {
+  const bf16_t* x; const bf16_t* a_cat; const float* col_scale; bf16_t* t;
+  int M, K, R;
+};
+
+typedef const __attribute__((address_space(1))) void* gptr_t;
+typedef __attribute__((address_space(3))) void* lptr_t;
+
+template <int VM>
+__device__ __forceinline__ void wait_vm() {  // vmcnt = VM, other counters unconstrained (gfx9 encoding)
+  __builtin_amdgcn_s_waitcnt((VM & 15) | (7 << 4) | (15 << 8) | ((VM >> 4) << 14));
+}
+__device__ __forceinline__ void wait_lgkm0() { __builtin_amdgcn_s_waitcnt(15 | (7 << 4) | (0 << 8) | (3 << 14)); }
+
+template <int NW_, int TR_, int TC_>
+struct SCfg {
+  static constexpr int NW = NW_, TR = TR_, TC = TC_;
+  static constexpr int NS = 2;                       // stages per wave
+  static constexpr int UNITS = (TR + TC) * 4;        // 8-row DMA units per stage (x rows, then A_cat rows)
+  static constexpr int STAGE = UNITS * 1024;         // 64 K-columns: 128-byte rows (whole cache lines), XOR-swizzled
+  static constexpr int RING = NW * NS * STAGE;
+  static constexpr int LD = TC * 32 + 4;             // padded fp32 row of the partial-sum tile
+  static constexpr int PART = NW * TR * 32 * LD * 4;
+  static constexpr int LDS = RING > PART ? RING : PART;
+  static_assert(LDS <= 160 * 1024 && UNITS < 64, "LDS / vmcnt budget");
+};
+
+// One output tile (bx, by) of t = bf16((x . A_cat^T) * col_scale).  The block may have more waves than C::NW: the extra
+// ones only join the barriers and the final fold.  WT: the results are stored write-through at agent scope (for
+// readers on other XCDs inside the same launch).
+template <class C, bool WT>
+__device__ __forceinline__ void lora_shrink_tile(const ShrinkParams& p, int bx, int by, char* smem) {
+  constexpr int NW = C::NW, TR = C::TR, TC = C::TC, NS = C::NS, UNITS = C::UNITS, STAGE = C::STAGE, LD = C::LD;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31, lh = lane >> 5;
+  const bool active = wave < NW;
+  const int m0 = bx * TR * 32, r0 = by * TC * 32;
+  const int K = p.K, KC = K / 64;                    // 64-column chunks, dealt to the waves round-robin
+  const int n = active ? (KC - wave + NW - 1) / NW : 0;   // chunks wave, wave + NW, ... of this wave
+  char* ring = smem + (active ? wave : 0) * (NS * STAGE);
+
+  // DMA: lane i of a unit lands in LDS slot i = row i/8, physical piece i%8, which holds logical piece
+  // (i%8) ^ ((row/2)%8); the swizzle is applied to the address the lane fetches
+  const bf16_t* src[UNITS];
+#pragma unroll
+  for (int u = 0; u < UNITS; ++u) {
+    const int ru = u * 8 + (lane >> 3);                // row inside the stacked [x rows | A_cat rows] stage
+    const int pc = ((lane & 7) ^ ((ru >> 1) & 7)) * 8;
+    if (u < TR * 4) {
+      int row = m0 + ru; row = row < p.M ? row : p.M - 1;
+      src[u] = p.x + (size_t)row * K + wave * 64 + pc;
+    } else {
+      int row = r0 + ru - TR * 32; row = row < p.R ? row : p.R - 1;
+      src[u] = p.a_cat + (size_t)row * K + wave * 64 + pc;
+    }
+  }
+  auto issue = [&](int i) {                            // this wave's i-th chunk
+    char* st = ring + (i % NS) * STAGE;
+#pragma unroll
+    for (int u = 0; u < UNITS; ++u)
+      __builtin_amdgcn_global_load_lds((gptr_t)(src[u] + (size_t)i * (NW * 64)), (lptr_t)(st + u * 1024), 16, 0, 0);
+  };
+  f32x16 acc[TR][TC];
+#pragma unroll
+  for (int i = 0; i < TR; ++i)
+#pragma unroll
+    for (int j = 0; j < TC; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+  const int sw = (l32 >> 1) & 7;
+
+  if (n > 0) issue(0);
+  if (n > 1) issue(1);
+  for (int i = 0; i < n; ++i) {
+    if (i + 1 < n) wait_vm<UNITS>(); else wait_vm<0>();   // chunk i has landed; chunk i+1 may be in flight
+    const char* st = ring + (i % NS) * STAGE;
+    bf16x8 a[4][TR], b[4][TC];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const int po = ((2 * ks + lh) ^ sw) * 16;
+#pragma unroll
+      for (int r = 0; r < TR; ++r) a[ks][r] = *reinterpret_cast<const bf16x8*>(st + (r * 32 + l32) * 128 + po);
+#pragma unroll
+      for (int c = 0; c < TC; ++c) b[ks][c] = *reinterpret_cast<const bf16x8*>(st + ((TR + c) * 32 + l32) * 128 + po);
+    }
+    wait_lgkm0();                   // fragments are in registers: the stage may be refilled
+    if (i + NS < n) issue(i + NS);
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+      for (int r = 0; r < TR; ++r)
+#pragma unroll
+        for (int c = 0; c < TC; ++c)
+          acc[r][c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ks][r], b[ks][c], acc[r][c], 0, 0, 0);
+  }
+  __syncthreads();                  // every ring is dead: the partial sums reuse the memory
+  float* part = reinterpret_cast<float*>(smem);   // [NW][TR*32][LD]
+  if (active) {
+#pragma unroll
+    for (int i = 0; i < TR; ++i)
+#pragma unroll
+      for (int j = 0; j < TC; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+          part[(wave * TR * 32 + i * 32 + 8 * (v >> 2) + 4 * lh + (v & 3)) * LD + j * 32 + l32] = acc[i][j][v];
+  }
+  __syncthreads();
+  constexpr int COLS = TC * 32, ROWS = TR * 32;
+  for (int i = tid; i < ROWS * COLS / 2; i += (int)blockDim.x) {   // two neighbouring columns per thread
+    const int rr = (2 * i) / COLS, c = (2 * i) % COLS;
+    float s0 = part[rr * LD + c], s1 = part[rr * LD + c + 1];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) {                                  // fixed order: deterministic
+      s0 += part[(w * ROWS + rr) * LD + c];
+      s1 += part[(w * ROWS + rr) * LD + c + 1];
+    }
+    if (m0 + rr < p.M && r0 + c < p.R) {
+      const uint32_t v = pack_bf16x2(s0 * p.col_scale[r0 + c], s1 * p.col_scale[r0 + c + 1]);
+      uint32_t* dst = reinterpret_cast<uint32_t*>(p.t + (size_t)(m0 + rr) * p.R + r0 + c);
+      if (WT) __hip_atomic_store(dst, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      else *dst = v;
+    }
+  }
+}
+
+}  // namespace

@@ -31,6 +31,9 @@ SKIP_INIT = False
 #   "fused": one launch, the rank-R product is computed per output tile and kept in LDS;
 #   "split": kh_lora_shrink_bf16 once per layer input, then the base GEMM + expand reading it from L2.
 LORA_MODE = os.getenv("KATZ_LORA_MODE", "split")
+# split mode: "in_launch" lets kh_lora_linear_split_bf16 run the shrink inside the GEMM launch where the GEMM leaves
+# CUs idle; "separate" always makes two launches (for measurements)
+LORA_SHRINK = os.getenv("KATZ_LORA_SHRINK", "in_launch")
 
 # bumped whenever any layer rebuilds its packed adapter buffers (not on pure scale changes): consumers
 # that cache pointers into those buffers (grouped launches) rebuild when it moves
@@ -171,8 +174,8 @@ class LoRALinear(nn.Module):
         if p is None:
             return ops.lora_linear(x, w, b, residual=residual, geglu=self.geglu)
         if LORA_MODE == "split" and x.dtype == torch.bfloat16 and self.in_features % 64 == 0:
-            t = ops.lora_shrink(x, p.a_cat, p.col_scale)
-            return ops.lora_linear_pre(x, w, b, t, p.b_cat, residual=residual, geglu=self.geglu)
+            return ops.lora_linear_split(x, w, b, p.a_cat, p.col_scale, p.b_cat, residual=residual, geglu=self.geglu,
+                                         two_launches=LORA_SHRINK == "separate")
         return ops.lora_linear(x, w, b, p.a_cat, p.b_cat, p.col_scale, residual=residual, geglu=self.geglu)
 
     def extra_repr(self) -> str:

@@ -155,6 +155,57 @@ def lora_linear_pre(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.
     return out
 
 
+SPLIT_COUNTER_INTS = 2 * 2047 + 2   # KH_SPLIT_COUNTER_INTS of include/katz_hip.h
+_split_counters: dict = {}
+
+
+def split_counters(device) -> torch.Tensor:
+    """The zero-initialised counter buffer kh_lora_linear_split_bf16 synchronises its in-launch shrink with: one per
+    device, shared by every call (calls on one device run one after the other; each leaves the buffer zeroed).  Its
+    last element is set if a bounded wait ever ran out."""
+    key = (device.type, device.index)
+    buf = _split_counters.get(key)
+    if buf is None:
+        buf = torch.zeros(SPLIT_COUNTER_INTS, dtype=torch.int32, device=device)
+        _split_counters[key] = buf
+    return buf
+
+
+def lora_linear_split(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], a_cat: torch.Tensor,
+                      col_scale: torch.Tensor, b_cat: torch.Tensor, residual: Optional[torch.Tensor] = None,
+                      geglu: bool = False, two_launches: bool = False) -> torch.Tensor:
+    """y = x W^T + b + ((x A_cat^T) * col_scale) B_cat^T (+ residual | GEGLU): shrink, base GEMM and expand, with
+    the shrink inside the GEMM launch where the GEMM leaves CUs idle (see kh_lora_linear_split_bf16)."""
+    lib = _lib.load()
+    _req(x, BF16, "x"); _req(weight, BF16, "weight"); _req(a_cat, BF16, "a_cat"); _req(b_cat, BF16, "b_cat")
+    _req(col_scale, torch.float32, "col_scale")
+    K = x.shape[-1]
+    N = weight.shape[0]
+    M = x.numel() // K
+    R = a_cat.shape[0]
+    if weight.shape[1] != K or a_cat.shape != (R, K) or b_cat.shape != (N, R) or col_scale.shape != (R,):
+        raise ValueError("weight / a_cat / b_cat / col_scale do not match x")
+    if bias is not None:
+        _req(bias, BF16, "bias")
+    if residual is not None:
+        _req(residual, BF16, "residual")
+        if residual.numel() != M * N:
+            raise ValueError("residual must have the shape of the output")
+    n_out = N // 2 if geglu else N
+    out = torch.empty(tuple(x.shape[:-1]) + (n_out,), dtype=BF16, device=x.device)
+    t = torch.empty((M, R), dtype=BF16, device=x.device)
+    cnt = split_counters(x.device)
+    flags = (1 if geglu else 0) | ((1 if two_launches else 0) << 8)
+    if CALL_LOG is not None:   # one entry per kernel launch
+        if lib.kh_lora_linear_split_launches(M, N, K, R, flags) == 2:
+            CALL_LOG.append(("lora_shrink", M, K, R))
+        CALL_LOG.append(("lora_linear", M, N, K, R, bool(geglu), residual is not None))
+    rc = lib.kh_lora_linear_split_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(a_cat), _ptr(col_scale), _ptr(b_cat), _ptr(t),
+                                       _ptr(cnt), _ptr(residual), _ptr(out), M, N, K, R, flags, _stream())
+    _lib.check(rc, "kh_lora_linear_split_bf16")
+    return out
+
+
 def lora_linear_grouped(x: torch.Tensor, table: torch.Tensor, M: int, N: int, K: int, R: int, ldt: int) -> None:
     """y_g = x W_g^T + b_g + t_g B_cat_g^T for every row {W, bias, B_cat, t, y} of the int64 device
     `table` [n_groups, 5] in one launch; the caller owns every buffer the table points to."""

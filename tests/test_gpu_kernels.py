@@ -785,3 +785,43 @@ def test_wide_tile_geglu_gate_range():
     ref = O.geglu(b.float().unsqueeze(0).expand(M, -1).contiguous())
     fin = torch.isfinite(ref[0])
     assert_close_rel(y[:, fin], ref[:, fin], REL_BF16, "wide tile geglu gate range")
+
+
+@pytest.mark.parametrize("case", [
+    # (M, N, K, R, residual)
+    (2048, 1280, 1280, 128, True),      # to_out / attn2.to_q at 32x32: 160 GEMM + 64 shrink workgroups in one launch
+    (2048, 1280, 1280, 64, False),
+    (2000, 1280, 640, 64, True),        # ragged rows: the last 128-row block has one 64-row shrink tile
+    (1100, 1000, 1280, 128, True),      # ragged rows and columns
+    (2048, 1280, 5120, 128, True),      # long K: two launches
+    (8192, 640, 640, 128, True),        # every CU busy with the GEMM: two launches
+])
+def test_lora_linear_split(case):
+    """kh_lora_linear_split_bf16 (shrink inside the GEMM launch where the rule allows, else two launches): against the
+    oracle, against the forced two-launch form, repeated calls bit for bit, and the counter buffer left zeroed."""
+    from katz_amd import ops
+
+    M, N, K, R, has_res = case
+    say("lora_linear_split", case)
+    d = dev()
+    g = torch.Generator().manual_seed(M + N + K + R)
+    x, w, b = randn(g, M, K), randn(g, N, K, std=0.03), randn(g, N)
+    A, B = randn(g, R, K, std=0.05), randn(g, N, R, std=0.05)
+    res = randn(g, M, N) if has_res else None
+    xd, wd, bd, Ad, Bd = (t.to(d, BF) for t in (x, w, b, A, B))
+    rd = None if res is None else res.to(d, BF)
+    cs = torch.full((R,), 0.7, device=d)
+    cnt = ops.split_counters(d)
+    ys = [ops.lora_linear_split(xd, wd, bd, Ad, cs, Bd, residual=rd) for _ in range(4)]
+    y2 = ops.lora_linear_split(xd, wd, bd, Ad, cs, Bd, residual=rd, two_launches=True)
+    torch.cuda.synchronize()
+    assert int(cnt.abs().sum()) == 0, "counters not zeroed (or a bounded wait ran out)"
+    for y in ys[1:]:
+        assert torch.equal(y, ys[0])
+    ref = O.lora_linear(xd.float().cpu(), wd.float().cpu(), bd.float().cpu(), [(Ad.float().cpu(), Bd.float().cpu(), 0.7)],
+                        residual=None if rd is None else rd.float().cpu())
+    assert_close_rel(ys[0], ref, REL_BF16, f"split {case}")
+    assert_close_rel(y2, ref, REL_BF16, f"split, two launches {case}")
+    # the two forms differ only by the fp32 summation order inside the shrink: a handful of last-bit differences
+    differing = (ys[0] != y2).float().mean().item()
+    assert differing < 5e-3, differing
