@@ -662,15 +662,16 @@ bool plain_ok(const LoraGemmParams& p) { return p.R == 0 || p.t_ext != nullptr; 
 }  // namespace
 
 // Shrink inside the launch: the shapes whose 128x128 tiles leave at least a quarter of the CUs idle, so that the 64x64
-// shrink tiles find CUs of their own next to the GEMM workgroups.  Measured at M 2048 / N 1280 / K 1280: 20 us against
-// 17.8 + 4.6 for the two launches (the GEMM workgroups run 2 us slower beside the shrink, whether or not they have to
-// wait for it); from K = 5120 the 64x160 tiles of the two-launch form win that back, so long K stays with them.
+// shrink tiles find CUs of their own next to the GEMM workgroups.  Measured alone at M 2048 / N 1280 / K 1280: 20 us
+// against 17.8 + 4.6 for the two launches (the GEMM workgroups run 2 us slower beside the shrink, whether or not they
+// have to wait for it); inside the UNet step, K = 5120: 53 us against 49 + 12 (there the two-launch GEMM would use the
+// 64x160 tiles, which fill every CU and leave the shrink no room).
 bool lora_gemm_pipe_il_ok(const LoraGemmParams& p) {
   const long tiles = (long)((p.M + 127) / 128) * ((p.N + 127) / 128);
   const long shr = (long)((p.M + 63) / 64) * (p.R / 64);
   return p.R > 0 && p.R % 64 == 0 && p.K % 64 == 0 && p.t_ext != nullptr && p.a_cat != nullptr && p.col_scale != nullptr &&
          p.il_cnt != nullptr && p.ldt == p.R && p.t_nsplit == 0 && p.grp == nullptr && p.sg_mode == 0 && p.conv_cin == 0 &&
-         !p.geglu && p.M >= 1024 && p.K <= 2560 && tiles <= 192 && tiles + shr <= 256;
+         !p.geglu && p.M >= 1024 && tiles <= 192 && tiles + shr <= 256;
 }
 
 int lora_gemm_pipe_launch_il(const LoraGemmParams& pin, hipStream_t stream) {

@@ -793,7 +793,7 @@ def test_wide_tile_geglu_gate_range():
     (2048, 1280, 1280, 64, False),
     (2000, 1280, 640, 64, True),        # ragged rows: the last 128-row block has one 64-row shrink tile
     (1100, 1000, 1280, 128, True),      # ragged rows and columns
-    (2048, 1280, 5120, 128, True),      # long K: two launches
+    (2048, 1280, 5120, 128, True),      # ff.net.2
     (8192, 640, 640, 128, True),        # every CU busy with the GEMM: two launches
 ])
 def test_lora_linear_split(case):
