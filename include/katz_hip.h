@@ -90,16 +90,18 @@ int kh_lora_linear_pre_bf16(const void* x, const void* w, const void* bias, cons
  * counters: KH_SPLIT_COUNTER_INTS zero-initialised int32 of device memory, owned by the caller and shared by all
  * calls that do not overlap in time on the device (every launch leaves them zeroed); NULL = always two launches.
  * counters[KH_SPLIT_COUNTER_INTS - 1] becomes 1 if a bounded wait inside a launch ever ran out (the result of that
- * call is then undefined).  K % 64 == 0, R % 32 == 0, R <= 128.  flags: bit 0 GEGLU, bits 8..15: 1 = always two
+ * call is then undefined).  n_split > 0: w / bias / b_cat stack N / n_split layers of n_split rows each (q, k, v of a
+ * self-attention), a_cat / col_scale stack their A matrices ([N / n_split * R, K]) and t_scratch is [M, N / n_split * R],
+ * as for kh_lora_linear_pre_bf16.  K % 64 == 0, R % 32 == 0, R <= 128.  flags: bit 0 GEGLU, bits 8..15: 1 = always two
  * launches. */
 #define KH_SPLIT_MAX_ROW_BLOCKS 2047
 #define KH_SPLIT_COUNTER_INTS (2 * KH_SPLIT_MAX_ROW_BLOCKS + 2)
 int kh_lora_linear_split_bf16(const void* x, const void* w, const void* bias, const void* a_cat, const float* col_scale,
                               const void* b_cat, void* t_scratch, int32_t* counters, const void* residual, void* y,
-                              int64_t M, int64_t N, int64_t K, int64_t R, int flags, void* stream);
+                              int64_t M, int64_t N, int64_t K, int64_t R, int64_t n_split, int flags, void* stream);
 /* How many kernel launches kh_lora_linear_split_bf16 makes for this shape when counters are given (1 or 2; negative:
  * KH_ERR_*).  No counterpart in the reference; for callers that account per launch (benchmarks). */
-int kh_lora_linear_split_launches(int64_t M, int64_t N, int64_t K, int64_t R, int flags);
+int kh_lora_linear_split_launches(int64_t M, int64_t N, int64_t K, int64_t R, int64_t n_split, int flags);
 /* n_groups layers that read the SAME x in one launch (the context K/V projections of every cross-attention
  * of the UNet: 140 GEMMs of 154 rows each, which individually cannot fill the chip):
  *   y_g = x W_g^T + bias_g + t_g B_cat_g^T        g = 0 .. n_groups-1, all with the same M, N, K, R

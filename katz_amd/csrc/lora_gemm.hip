@@ -529,11 +529,12 @@ KH_EXPORT int kh_lora_linear_pre_bf16(const void* x, const void* w, const void* 
 // See include/katz_hip.h.
 static LoraGemmParams split_params(const void* x, const void* w, const void* bias, const void* a_cat, const float* col_scale,
                                    const void* b_cat, void* t_scratch, int32_t* counters, const void* residual, void* y,
-                                   int64_t M, int64_t N, int64_t K, int64_t R, bool geglu) {
+                                   int64_t M, int64_t N, int64_t K, int64_t R, int64_t n_split, bool geglu) {
   LoraGemmParams p;
   p.x = (const bf16_t*)x; p.w = (const bf16_t*)w; p.bias = (const bf16_t*)bias;
   p.a_cat = (const bf16_t*)a_cat; p.b_cat = (const bf16_t*)b_cat; p.col_scale = col_scale;
-  p.t_ext = (const bf16_t*)t_scratch; p.ldt = (int)R; p.grp = nullptr; p.dbg = 0; p.t_nsplit = 0;
+  p.t_ext = (const bf16_t*)t_scratch; p.ldt = (int)(n_split > 0 ? (N / n_split) * R : R); p.grp = nullptr; p.dbg = 0;
+  p.t_nsplit = (int)n_split;
   p.res = (const bf16_t*)residual; p.y = (bf16_t*)y;
   p.M = (int)M; p.N = (int)N; p.K = (int)K; p.R = (int)R;
   p.m_tiles = p.n_tiles = p.n_chunk = p.n_chunks = 0;
@@ -545,23 +546,26 @@ static LoraGemmParams split_params(const void* x, const void* w, const void* bia
   return p;
 }
 
-KH_EXPORT int kh_lora_linear_split_launches(int64_t M, int64_t N, int64_t K, int64_t R, int flags) {
+KH_EXPORT int kh_lora_linear_split_launches(int64_t M, int64_t N, int64_t K, int64_t R, int64_t n_split, int flags) {
   if (M <= 0 || N <= 0 || K <= 0 || R <= 0 || M > (1 << 24) || N > (1 << 24) || K > (1 << 24)) return KH_ERR_INVALID_ARG;
+  if (n_split < 0 || (n_split > 0 && N % n_split != 0)) return KH_ERR_INVALID_ARG;
   if (((flags >> 8) & 0xff) != 0 || (M + 127) / 128 > KH_SPLIT_MAX_ROW_BLOCKS) return 2;
   static int32_t dummy_counter;                  // the rule only asks whether counters were given
   static const char dummy = 0;
   const LoraGemmParams p = split_params(&dummy, &dummy, nullptr, &dummy, reinterpret_cast<const float*>(&dummy), &dummy,
                                         const_cast<char*>(&dummy), &dummy_counter, nullptr, const_cast<char*>(&dummy), M, N, K, R,
-                                        (flags & 1) != 0);
+                                        n_split, (flags & 1) != 0);
   return lora_gemm_pipe_il_ok(p) ? 1 : 2;
 }
 
 KH_EXPORT int kh_lora_linear_split_bf16(const void* x, const void* w, const void* bias, const void* a_cat,
                                         const float* col_scale, const void* b_cat, void* t_scratch, int32_t* counters,
                                         const void* residual, void* y, int64_t M, int64_t N, int64_t K, int64_t R,
-                                        int flags, void* stream) {
+                                        int64_t n_split, int flags, void* stream) {
   if (!x || !w || !y || !a_cat || !col_scale || !b_cat || !t_scratch || M <= 0 || N <= 0 || K <= 0 || R <= 0)
     return KH_ERR_INVALID_ARG;
+  if (n_split < 0 || (n_split > 0 && (n_split % 128 != 0 || N % n_split != 0))) return KH_ERR_INVALID_ARG;
+  const int64_t RT = n_split > 0 ? (N / n_split) * R : R;   // columns of t_scratch / rows of a_cat
   if (K % 64 != 0 || N % 8 != 0 || R % 32 != 0) return KH_ERR_UNSUPPORTED;
   if (R > 128) return KH_ERR_TOO_LARGE;
   if (M > (1 << 24) || N > (1 << 24) || K > (1 << 24)) return KH_ERR_TOO_LARGE;
@@ -570,13 +574,13 @@ KH_EXPORT int kh_lora_linear_split_bf16(const void* x, const void* w, const void
   if (!kh_aligned16(x) || !kh_aligned16(w) || !kh_aligned16(y) || !kh_aligned16(a_cat) || !kh_aligned16(b_cat) ||
       !kh_aligned16(t_scratch) || (residual && !kh_aligned16(residual)))
     return KH_ERR_ALIGNMENT;
-  if (counters != nullptr && kh_lora_linear_split_launches(M, N, K, R, flags) == 1) {
-    const LoraGemmParams p = split_params(x, w, bias, a_cat, col_scale, b_cat, t_scratch, counters, residual, y, M, N, K, R, geglu);
+  if (counters != nullptr && kh_lora_linear_split_launches(M, N, K, R, n_split, flags) == 1) {
+    const LoraGemmParams p = split_params(x, w, bias, a_cat, col_scale, b_cat, t_scratch, counters, residual, y, M, N, K, R, n_split, geglu);
     return lora_gemm_pipe_launch_il(p, (hipStream_t)stream);
   }
-  const int rc = kh_lora_shrink_bf16(x, a_cat, col_scale, t_scratch, M, K, R, stream);
+  const int rc = kh_lora_shrink_bf16(x, a_cat, col_scale, t_scratch, M, K, RT, stream);
   if (rc != KH_OK) return rc;
-  return kh_lora_linear_pre_bf16(x, w, bias, t_scratch, R, 0, b_cat, residual, y, M, N, K, R, flags & 0xff, stream);
+  return kh_lora_linear_pre_bf16(x, w, bias, t_scratch, RT, n_split, b_cat, residual, y, M, N, K, R, flags & 0xff, stream);
 }
 
 // 3x3 convolution, padding 1, NHWC, as an implicit GEMM on the pipelined kernel; see include/katz_hip.h.

@@ -279,19 +279,20 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
   LoraGemmParams p = pin;
   if constexpr (IL) {
     // The first il_blocks workgroups are the shrink: 64x64 tiles of T on 4 of the 8 waves, stored write-through,
-    // then one arrival per tile on the counter of the 128-row block the tile belongs to.  They have the lowest
+    // then one arrival per tile on the counter of the GEMM row block the tile belongs to.  They have the lowest
     // block ids, so they are resident before any workgroup that waits for them.
     if ((int)blockIdx.x < pin.il_blocks) {
-      const int gx = (pin.M + 63) / 64, gy = pin.R / 64;
+      const int gx = (pin.M + 63) / 64, gy = pin.ldt / 64;   // T has ldt columns (several layers' ranks side by side)
       if ((int)blockIdx.x >= gx * gy) return;               // padding to a multiple of 8 (the XCD map of the rest)
       const int bx = blockIdx.x % gx, by = blockIdx.x / gx;
       ShrinkParams sp;
       sp.x = pin.x; sp.a_cat = pin.a_cat; sp.col_scale = pin.col_scale; sp.t = const_cast<bf16_t*>(pin.t_ext);
-      sp.M = pin.M; sp.K = pin.K; sp.R = pin.R;
+      sp.M = pin.M; sp.K = pin.K; sp.R = pin.ldt;
       lora_shrink_tile<SCfg<4, 2, 2>, true>(sp, bx, by, smem);
       __builtin_amdgcn_s_waitcnt(0);                          // this thread's write-through stores have completed
       __syncthreads();
-      if (threadIdx.x == 0) __hip_atomic_fetch_add(pin.il_cnt + bx / 2, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (threadIdx.x == 0)
+        __hip_atomic_fetch_add(pin.il_cnt + (bx * 64) / C::BM, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       return;
     }
   }
@@ -465,9 +466,10 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
       Dma<C, false> d;
       dma_setup(d);
       if constexpr (IL) {
-        const int gx = (M + 63) / 64, rt = gx - 2 * m_blk < 2 ? gx - 2 * m_blk : 2;   // 64-row shrink tiles over this row block
+        constexpr int TPB = BM / 64;                                                   // 64-row shrink tiles per row block
+        const int gx = (M + 63) / 64, rt = gx - TPB * m_blk < TPB ? gx - TPB * m_blk : TPB;
         k_loop<C, false, BCH, CONV, decltype(tail_loads), true>(smem, d, p.x, p.w, p.a_cat, p.t_ext, p.b_cat, KT, KT1, lane, wm, wn, l32, lh, sw, acc, tacc, tail_loads, ConvGeom{0, 0}, false, false,
-                                                                p.il_cnt + m_blk, rt * (p.R / 64), p.il_cnt + (KH_SPLIT_COUNTER_INTS - 1));
+                                                                p.il_cnt + m_blk, rt * (p.ldt / 64), p.il_cnt + (KH_SPLIT_COUNTER_INTS - 1));
       } else {
         k_loop<C, false, BCH, CONV>(smem, d, p.x, p.w, p.a_cat, p.t_ext, p.b_cat, KT, KT1, lane, wm, wn, l32, lh, sw, acc, tacc, tail_loads, ConvGeom{p.conv_w, p.conv_cin}, (p.dbg & 64) != 0, (p.dbg & 128) != 0);
       }
@@ -666,17 +668,25 @@ bool plain_ok(const LoraGemmParams& p) { return p.R == 0 || p.t_ext != nullptr; 
 // against 17.8 + 4.6 for the two launches (the GEMM workgroups run 2 us slower beside the shrink, whether or not they
 // have to wait for it); inside the UNet step, K = 5120: 53 us against 49 + 12 (there the two-launch GEMM would use the
 // 64x160 tiles, which fill every CU and leave the shrink no room).
-bool lora_gemm_pipe_il_ok(const LoraGemmParams& p) {
+// 0: not suited; 1: 128x128 tiles that leave CUs idle; 2: 256x128 tiles for the stacked q/k/v projection (the shrink
+// tiles take a round of CUs first, the GEMM tiles follow as they free up: still shorter than two launches)
+static int il_form(const LoraGemmParams& p) {
   const long tiles = (long)((p.M + 127) / 128) * ((p.N + 127) / 128);
-  const long shr = (long)((p.M + 63) / 64) * (p.R / 64);
-  return p.R > 0 && p.R % 64 == 0 && p.K % 64 == 0 && p.t_ext != nullptr && p.a_cat != nullptr && p.col_scale != nullptr &&
-         p.il_cnt != nullptr && p.ldt == p.R && p.t_nsplit == 0 && p.grp == nullptr && p.sg_mode == 0 && p.conv_cin == 0 &&
-         !p.geglu && p.M >= 1024 && tiles <= 192 && tiles + shr <= 256;
+  const long shr = (long)((p.M + 63) / 64) * (p.ldt / 64);
+  const bool t_ok = p.t_nsplit == 0 ? p.ldt == p.R : (p.N % p.t_nsplit == 0 && p.ldt == (p.N / p.t_nsplit) * p.R && p.t_nsplit % 128 == 0);
+  const bool ok = p.R > 0 && p.R % 64 == 0 && p.ldt % 64 == 0 && p.K % 64 == 0 && p.t_ext != nullptr && p.a_cat != nullptr &&
+                  p.col_scale != nullptr && p.il_cnt != nullptr && t_ok && p.grp == nullptr && p.sg_mode == 0 && p.conv_cin == 0 &&
+                  !p.geglu && p.M >= 1024;
+  if (!ok) return 0;
+  if (tiles <= 192 && tiles + shr <= 256) return 1;
+  if (tiles >= 480 && p.K >= 1024 && (long)((p.M + 255) / 256) * ((p.N + 127) / 128) <= 256 && shr <= 256) return 2;
+  return 0;
 }
 
-int lora_gemm_pipe_launch_il(const LoraGemmParams& pin, hipStream_t stream) {
-  if (!lora_gemm_pipe_il_ok(pin)) return KH_ERR_UNSUPPORTED;
-  using C = PCfg<128, 128, 2, 4, 0, 3, 64>;
+bool lora_gemm_pipe_il_ok(const LoraGemmParams& p) { return il_form(p) != 0; }
+
+template <class C>
+static int launch_il(const LoraGemmParams& pin, hipStream_t stream) {
   using S = SCfg<4, 2, 2>;
   LoraGemmParams p = pin;
   p.m_tiles = (p.M + C::BM - 1) / C::BM;
@@ -684,7 +694,7 @@ int lora_gemm_pipe_launch_il(const LoraGemmParams& pin, hipStream_t stream) {
   p.n_chunk = 1;
   p.n_chunks = p.n_tiles;
   constexpr int LDS = (int)C::LDS_BYTES > S::LDS ? (int)C::LDS_BYTES : S::LDS;
-  static bool attr_done = false;
+  static bool attr_done = false;  // per template instantiation
   if (!attr_done) {
     hipError_t e = hipFuncSetAttribute((const void*)lora_gemm_pipe_kernel<C, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
     if (e != hipSuccess) return (int)e;
@@ -698,11 +708,19 @@ int lora_gemm_pipe_launch_il(const LoraGemmParams& pin, hipStream_t stream) {
     const double cost = ((double)rm * C::BM + (double)rn * C::BN) * (8.0 * rm * rn) / ((double)p.m_tiles * p.n_tiles);
     if (p.xg_n == 0 || cost < best) { best = cost; p.xg_n = gn; p.xr_m = rm; p.xr_n = rn; }
   }
-  const int shr = ((p.M + 63) / 64) * (p.R / 64);
+  const int shr = ((p.M + 63) / 64) * (p.ldt / 64);
   p.il_blocks = (shr + 7) / 8 * 8;
   const unsigned grid = (unsigned)p.il_blocks + 8u * (unsigned)p.xr_m * (unsigned)p.xr_n;
   kh_launch(KH_TAG_LORA_GEMM, lora_gemm_pipe_kernel<C, false, true>, dim3(grid), dim3(C::NT), (size_t)LDS, stream, p);
   KH_RETURN_LAST_ERROR();
+}
+
+int lora_gemm_pipe_launch_il(const LoraGemmParams& p, hipStream_t stream) {
+  switch (il_form(p)) {
+    case 1: return launch_il<PCfg<128, 128, 2, 4, 0, 3, 64>>(p, stream);
+    case 2: return launch_il<PCfg<256, 128, 4, 2, 0, 4>>(p, stream);
+    default: return KH_ERR_UNSUPPORTED;
+  }
 }
 
 int lora_gemm_pipe_launch_conv(const LoraGemmParams& p, hipStream_t stream) {

@@ -485,8 +485,8 @@ class Attention(nn.Module):
         if not st["ok"]:
             return None
         if st["R"]:
-            t = ops.lora_shrink(x, st["a"], st["s"])
-            y = ops.lora_linear_pre(x, st["w"], None, t, st["b"], n_split=N)
+            y = ops.lora_linear_split(x, st["w"], None, st["a"], st["s"], st["b"], n_split=N,
+                                      two_launches=LORA_SHRINK == "separate")
         else:
             y = ops.lora_linear(x, st["w"], None)
         return y.split(N, dim=-1)

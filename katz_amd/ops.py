@@ -173,17 +173,23 @@ def split_counters(device) -> torch.Tensor:
 
 def lora_linear_split(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], a_cat: torch.Tensor,
                       col_scale: torch.Tensor, b_cat: torch.Tensor, residual: Optional[torch.Tensor] = None,
-                      geglu: bool = False, two_launches: bool = False) -> torch.Tensor:
+                      geglu: bool = False, two_launches: bool = False, n_split: int = 0) -> torch.Tensor:
     """y = x W^T + b + ((x A_cat^T) * col_scale) B_cat^T (+ residual | GEGLU): shrink, base GEMM and expand, with
-    the shrink inside the GEMM launch where the GEMM leaves CUs idle (see kh_lora_linear_split_bf16)."""
+    the shrink inside the GEMM launch where that pays (see kh_lora_linear_split_bf16).  n_split > 0: weight / bias /
+    b_cat stack several layers of n_split rows each and a_cat / col_scale stack their A matrices."""
     lib = _lib.load()
     _req(x, BF16, "x"); _req(weight, BF16, "weight"); _req(a_cat, BF16, "a_cat"); _req(b_cat, BF16, "b_cat")
     _req(col_scale, torch.float32, "col_scale")
     K = x.shape[-1]
     N = weight.shape[0]
     M = x.numel() // K
-    R = a_cat.shape[0]
-    if weight.shape[1] != K or a_cat.shape != (R, K) or b_cat.shape != (N, R) or col_scale.shape != (R,):
+    RT = a_cat.shape[0]
+    R = b_cat.shape[1]
+    if n_split and (N % n_split or RT != (N // n_split) * R):
+        raise ValueError("stacked layers: a_cat must have N / n_split * R rows")
+    if not n_split and RT != R:
+        raise ValueError("a_cat and b_cat disagree on the rank")
+    if weight.shape[1] != K or a_cat.shape != (RT, K) or b_cat.shape != (N, R) or col_scale.shape != (RT,):
         raise ValueError("weight / a_cat / b_cat / col_scale do not match x")
     if bias is not None:
         _req(bias, BF16, "bias")
@@ -193,15 +199,15 @@ def lora_linear_split(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torc
             raise ValueError("residual must have the shape of the output")
     n_out = N // 2 if geglu else N
     out = torch.empty(tuple(x.shape[:-1]) + (n_out,), dtype=BF16, device=x.device)
-    t = torch.empty((M, R), dtype=BF16, device=x.device)
+    t = torch.empty((M, RT), dtype=BF16, device=x.device)
     cnt = split_counters(x.device)
     flags = (1 if geglu else 0) | ((1 if two_launches else 0) << 8)
     if CALL_LOG is not None:   # one entry per kernel launch
-        if lib.kh_lora_linear_split_launches(M, N, K, R, flags) == 2:
-            CALL_LOG.append(("lora_shrink", M, K, R))
+        if lib.kh_lora_linear_split_launches(M, N, K, R, n_split, flags) == 2:
+            CALL_LOG.append(("lora_shrink", M, K, RT))
         CALL_LOG.append(("lora_linear", M, N, K, R, bool(geglu), residual is not None))
     rc = lib.kh_lora_linear_split_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(a_cat), _ptr(col_scale), _ptr(b_cat), _ptr(t),
-                                       _ptr(cnt), _ptr(residual), _ptr(out), M, N, K, R, flags, _stream())
+                                       _ptr(cnt), _ptr(residual), _ptr(out), M, N, K, R, n_split, flags, _stream())
     _lib.check(rc, "kh_lora_linear_split_bf16")
     return out
 

@@ -788,40 +788,48 @@ def test_wide_tile_geglu_gate_range():
 
 
 @pytest.mark.parametrize("case", [
-    # (M, N, K, R, residual)
-    (2048, 1280, 1280, 128, True),      # to_out / attn2.to_q at 32x32: 160 GEMM + 64 shrink workgroups in one launch
-    (2048, 1280, 1280, 64, False),
-    (2000, 1280, 640, 64, True),        # ragged rows: the last 128-row block has one 64-row shrink tile
-    (1100, 1000, 1280, 128, True),      # ragged rows and columns
-    (2048, 1280, 5120, 128, True),      # ff.net.2
-    (8192, 640, 640, 128, True),        # every CU busy with the GEMM: two launches
+    # (M, N, K, R, residual, n_split)
+    (2048, 1280, 1280, 128, True, 0),      # to_out / attn2.to_q at 32x32: 160 GEMM + 64 shrink workgroups in one launch
+    (2048, 1280, 1280, 64, False, 0),
+    (2000, 1280, 640, 64, True, 0),        # ragged rows: the last 128-row block has one 64-row shrink tile
+    (1100, 1000, 1280, 128, True, 0),      # ragged rows and columns
+    (2048, 1280, 5120, 128, True, 0),      # ff.net.2
+    (2048, 3840, 1280, 128, False, 1280),  # stacked q / k / v: one launch on 256x128 tiles, T = [M, 3R]
+    (1900, 3840, 1280, 64, False, 1280),   # the same, ragged rows (the last 256-row block has 2 of 4 shrink tiles)
+    (8192, 640, 640, 128, True, 0),        # every CU busy with the GEMM: two launches
 ])
 def test_lora_linear_split(case):
     """kh_lora_linear_split_bf16 (shrink inside the GEMM launch where the rule allows, else two launches): against the
     oracle, against the forced two-launch form, repeated calls bit for bit, and the counter buffer left zeroed."""
     from katz_amd import ops
 
-    M, N, K, R, has_res = case
+    M, N, K, R, has_res, n_split = case
     say("lora_linear_split", case)
     d = dev()
     g = torch.Generator().manual_seed(M + N + K + R)
+    parts = N // n_split if n_split else 1
     x, w, b = randn(g, M, K), randn(g, N, K, std=0.03), randn(g, N)
-    A, B = randn(g, R, K, std=0.05), randn(g, N, R, std=0.05)
+    A, B = randn(g, parts * R, K, std=0.05), randn(g, N, R, std=0.05)
     res = randn(g, M, N) if has_res else None
     xd, wd, bd, Ad, Bd = (t.to(d, BF) for t in (x, w, b, A, B))
     rd = None if res is None else res.to(d, BF)
-    cs = torch.full((R,), 0.7, device=d)
+    cs = torch.full((parts * R,), 0.7, device=d)
     cnt = ops.split_counters(d)
-    ys = [ops.lora_linear_split(xd, wd, bd, Ad, cs, Bd, residual=rd) for _ in range(4)]
-    y2 = ops.lora_linear_split(xd, wd, bd, Ad, cs, Bd, residual=rd, two_launches=True)
+    run = lambda **kw: ops.lora_linear_split(xd, wd, bd, Ad, cs, Bd, residual=rd, n_split=n_split, **kw)
+    ys = [run() for _ in range(4)]
+    y2 = run(two_launches=True)
     torch.cuda.synchronize()
     assert int(cnt.abs().sum()) == 0, "counters not zeroed (or a bounded wait ran out)"
     for y in ys[1:]:
         assert torch.equal(y, ys[0])
-    ref = O.lora_linear(xd.float().cpu(), wd.float().cpu(), bd.float().cpu(), [(Ad.float().cpu(), Bd.float().cpu(), 0.7)],
-                        residual=None if rd is None else rd.float().cpu())
-    assert_close_rel(ys[0], ref, REL_BF16, f"split {case}")
-    assert_close_rel(y2, ref, REL_BF16, f"split, two launches {case}")
+    xf, wf, bfl, Af, Bf = (t.float().cpu() for t in (xd, wd, bd, Ad, Bd))
+    step = n_split if n_split else N
+    for j in range(parts):   # every stacked layer against the oracle with its own A / B
+        rows = slice(j * step, (j + 1) * step)
+        ref = O.lora_linear(xf, wf[rows], bfl[rows], [(Af[j * R:(j + 1) * R], Bf[rows], 0.7)],
+                            residual=None if rd is None else rd.float().cpu()[:, rows])
+        assert_close_rel(ys[0][:, rows], ref, REL_BF16, f"split {case} part {j}")
+        assert_close_rel(y2[:, rows], ref, REL_BF16, f"split, two launches {case} part {j}")
     # the two forms differ only by the fp32 summation order inside the shrink: a handful of last-bit differences
     differing = (ys[0] != y2).float().mean().item()
     assert differing < 5e-3, differing
