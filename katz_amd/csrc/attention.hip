@@ -193,7 +193,6 @@ __global__ __launch_bounds__(NW * 64, 2) void attention_kernel(const AttnParams 
         for (int v = 0; v < 16; ++v) oacc[dt][v] *= alpha;
     }
     const float mb = m_run * p.scale_log2e;
-    float rs = 0.f;
     bf16x8 pf[2][2];
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt)
@@ -201,19 +200,23 @@ __global__ __launch_bounds__(NW * 64, 2) void attention_kernel(const AttnParams 
       for (int v = 0; v < 16; v += 2) {
         const float e0 = __builtin_amdgcn_exp2f(st[kt][v] * p.scale_log2e - mb);
         const float e1 = __builtin_amdgcn_exp2f(st[kt][v + 1] * p.scale_log2e - mb);
-        rs += e0 + e1;
         pf[kt][v >> 3][v & 7] = (bf16_t)e0;
         pf[kt][v >> 3][(v & 7) + 1] = (bf16_t)e1;
       }
-    l_run += rs;
-
-    // O^T += V^T . P^T : A fragment row d = dt*32 + l32, element e <-> key kt*32 + 8*(2s + e/4) + 4*lh + e%4
+    // O^T += V^T . P^T : A fragment row d = dt*32 + l32, element e <-> key kt*32 + 8*(2s + e/4) + 4*lh + e%4.
+    // Row sums ride along on the matrix pipe, which has cycles to spare here (the vector ALU does not):
+    // ones^T . P^T puts sum_k P[k][q] of all 64 keys (both lane halves) into every row of column q, i.e. into every
+    // register of the lanes of query q.  The denominator is then the sum of the same rounded P values the numerator
+    // uses.  Its MFMAs sit between those of the two output tiles, so nothing waits on their dependency chain.
+    const bf16_t one = (bf16_t)1.0f;
+    const bf16x8 ones = {one, one, one, one, one, one, one, one};
+    f32x16 rsum = zero;
 #pragma unroll
-    for (int dt = 0; dt < 2; ++dt)
+    for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
+      for (int s = 0; s < 2; ++s) {
 #pragma unroll
-        for (int s = 0; s < 2; ++s) {
+        for (int dt = 0; dt < 2; ++dt) {
           const bf16_t* base = &sVt[buf][(dt * 32 + l32) * LDV + kt * 32 + 16 * s + 4 * lh];
           const bf16x4 v0 = *reinterpret_cast<const bf16x4*>(base);
           const bf16x4 v1 = *reinterpret_cast<const bf16x4*>(base + 8);
@@ -222,6 +225,9 @@ __global__ __launch_bounds__(NW * 64, 2) void attention_kernel(const AttnParams 
           for (int e = 0; e < 4; ++e) { vf[e] = v0[e]; vf[4 + e] = v1[e]; }
           oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[kt][s], oacc[dt], 0, 0, 0);
         }
+        rsum = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pf[kt][s], rsum, 0, 0, 0);
+      }
+    l_run += rsum[0];
 
     if (t + 1 < n_tiles) store_tile(buf ^ 1);
     __syncthreads();
@@ -230,8 +236,7 @@ __global__ __launch_bounds__(NW * 64, 2) void attention_kernel(const AttnParams 
   for (int t = 0; t < full_tiles; ++t) tile_step(t, std::false_type{});
   if (full_tiles < n_tiles) tile_step(full_tiles, std::true_type{});
 
-  const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
-  const float inv = 1.0f / l_tot;
+  const float inv = 1.0f / l_run;   // the MFMA row sums already cover the keys of both lane halves
   if (qrow < p.T) {
 #pragma unroll
     for (int dt = 0; dt < 2; ++dt)
