@@ -30,7 +30,7 @@ class GraphedUNetStep:
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side), torch.no_grad():
-            for _ in range(warmup):   # MIOpen kernel selection, workspace growth, lazy packing: all before capture
+            for _ in range(warmup):   # workspace and counter allocation, lazy packing: all before capture
                 self._run()
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()

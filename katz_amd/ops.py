@@ -166,6 +166,10 @@ def split_counters(device) -> torch.Tensor:
     key = (device.type, device.index)
     buf = _split_counters.get(key)
     if buf is None:
+        if torch.cuda.is_current_stream_capturing():
+            # memory allocated during a capture belongs to the graph's pool and dies with the graph
+            raise RuntimeError("katz_amd: run the step once eagerly before capturing it (the LoRA counter buffer is "
+                               "allocated on first use and must outlive the graph)")
         buf = torch.zeros(SPLIT_COUNTER_INTS, dtype=torch.int32, device=device)
         _split_counters[key] = buf
     return buf
@@ -299,6 +303,9 @@ def _workspace(nbytes: int, device) -> torch.Tensor:
     key = (device.type, device.index)
     buf = _gn_workspace.get(key)
     if buf is None or buf.numel() * 4 < nbytes:
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError("katz_amd: run the step once eagerly before capturing it (the GroupNorm workspace grows "
+                               "on first use and must outlive the graph)")
         buf = torch.empty(max(nbytes // 4, 1 << 16), dtype=torch.float32, device=device)
         _gn_workspace[key] = buf
     return buf
