@@ -218,6 +218,7 @@ ATTN_SHAPES = [
     # B, H, T, S
     (1, 2, 4096, 4096),   # self-attention at 64x64 (two of the ten heads)
     (2, 20, 1024, 1024),  # self-attention at 32x32, full head count
+    (3, 16, 1000, 384),   # ragged last query block, six full key tiles
     (2, 10, 4096, 77),    # cross-attention at 64x64
     (2, 20, 1024, 77),    # cross-attention at 32x32
     (1, 1, 100, 77),      # ragged query block and key tile
