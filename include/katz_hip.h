@@ -87,15 +87,15 @@ int kh_lora_linear_pre_bf16(const void* x, const void* w, const void* bias, cons
  * launch on those CUs: its workgroups come first in the grid, store t_scratch write-through and count themselves into
  * `counters`; the GEMM workgroups read t_scratch (as the last K tiles) only after their row block's count is complete.
  * Same results as the two launches up to the fp32 summation order of the shrink.
- * counters: KH_SPLIT_COUNTER_INTS zero-initialised int32 of device memory, owned by the caller and shared by all
- * calls that do not overlap in time on the device (every launch leaves them zeroed); NULL = always two launches.
- * counters[KH_SPLIT_COUNTER_INTS - 1] becomes 1 if a bounded wait inside a launch ever ran out (the result of that
+ * counters: KH_SPLIT_COUNTER_INTS(M) int32 of device memory owned by the caller, ZERO when the call is enqueued;
+ * the launch leaves its arrival counts in them, so the caller clears them (a fill kernel; in a HIP graph, one fill
+ * over all call sites' counters at the start of the step) before the same memory serves another call.  NULL = always
+ * two launches.  The last of them becomes 1 if a bounded wait inside the launch ever ran out (the result of that
  * call is then undefined).  n_split > 0: w / bias / b_cat stack N / n_split layers of n_split rows each (q, k, v of a
  * self-attention), a_cat / col_scale stack their A matrices ([N / n_split * R, K]) and t_scratch is [M, N / n_split * R],
  * as for kh_lora_linear_pre_bf16.  K % 64 == 0, R % 32 == 0, R <= 128.  flags: bit 0 GEGLU, bits 8..15: 1 = always two
  * launches. */
-#define KH_SPLIT_MAX_ROW_BLOCKS 2047
-#define KH_SPLIT_COUNTER_INTS (2 * KH_SPLIT_MAX_ROW_BLOCKS + 2)
+#define KH_SPLIT_COUNTER_INTS(M) (((M) + 127) / 128 + 1)
 int kh_lora_linear_split_bf16(const void* x, const void* w, const void* bias, const void* a_cat, const float* col_scale,
                               const void* b_cat, void* t_scratch, int32_t* counters, const void* residual, void* y,
                               int64_t M, int64_t N, int64_t K, int64_t R, int64_t n_split, int flags, void* stream);

@@ -134,6 +134,8 @@ class ControlNetModel(nn.Module):
             sample = sample.to(torch.bfloat16).contiguous(memory_format=torch.channels_last)
         cond = controlnet_cond.to(torch.bfloat16).contiguous(memory_format=torch.channels_last)
         ctx = encoder_hidden_states.to(torch.bfloat16).contiguous()
+        if sample.is_cuda:
+            ops.split_counters_reset(sample.device)   # one fill per step clears the in-launch shrinks' counters
         if self._ctx_kv is None:
             self.prepare()
         self._ctx_kv.run(ctx)

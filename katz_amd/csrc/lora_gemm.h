@@ -34,8 +34,8 @@ struct LoraGemmParams {
   int conv_cin, conv_h, conv_w, conv_ho, conv_wo, conv_stride;
   // shrink inside the GEMM launch (il_blocks > 0): the first il_blocks workgroups compute t_ext = the shrink of x
   // (a_cat, col_scale) in 64x64 tiles and count themselves into il_cnt[row block]; the GEMM workgroups wait for their
-  // row block's count before they read t_ext.  il_cnt: KH_SPLIT_COUNTER_INTS zero-initialised ints (arrivals, departures,
-  // time-out flag); every launch leaves them zeroed.
+  // row block's count before they read t_ext.  il_cnt: ceil(M / 128) + 1 ints, zero when the launch starts (arrivals
+  // per row block, then a time-out flag); the launch leaves the arrivals in them.
   int il_blocks = 0;
   int* il_cnt = nullptr;
 };
@@ -63,9 +63,5 @@ int lora_gemm_ksplit_launch_conv(const LoraGemmParams& p, int row_groups, hipStr
 bool lora_gemm_wide_ok(const LoraGemmParams& p);
 int lora_gemm_wide_launch(LoraGemmParams p, hipStream_t stream);
 
-// Counter buffer of kh_lora_linear_split_bf16 (the same numbers as in include/katz_hip.h): arrivals [row block],
-// departures [MAX + row block], the time-out flag last.
-constexpr int KH_SPLIT_MAX_ROW_BLOCKS = 2047;
-constexpr int KH_SPLIT_COUNTER_INTS = 2 * KH_SPLIT_MAX_ROW_BLOCKS + 2;
 extern "C" int kh_lora_shrink_bf16(const void* x, const void* a_cat, const float* col_scale, void* t, int64_t M, int64_t K,
                                    int64_t R, void* stream);

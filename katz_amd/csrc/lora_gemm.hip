@@ -549,7 +549,7 @@ static LoraGemmParams split_params(const void* x, const void* w, const void* bia
 KH_EXPORT int kh_lora_linear_split_launches(int64_t M, int64_t N, int64_t K, int64_t R, int64_t n_split, int flags) {
   if (M <= 0 || N <= 0 || K <= 0 || R <= 0 || M > (1 << 24) || N > (1 << 24) || K > (1 << 24)) return KH_ERR_INVALID_ARG;
   if (n_split < 0 || (n_split > 0 && N % n_split != 0)) return KH_ERR_INVALID_ARG;
-  if (((flags >> 8) & 0xff) != 0 || (M + 127) / 128 > KH_SPLIT_MAX_ROW_BLOCKS) return 2;
+  if (((flags >> 8) & 0xff) != 0) return 2;
   static int32_t dummy_counter;                  // the rule only asks whether counters were given
   static const char dummy = 0;
   const LoraGemmParams p = split_params(&dummy, &dummy, nullptr, &dummy, reinterpret_cast<const float*>(&dummy), &dummy,

@@ -469,7 +469,7 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
         constexpr int TPB = BM / 64;                                                   // 64-row shrink tiles per row block
         const int gx = (M + 63) / 64, rt = gx - TPB * m_blk < TPB ? gx - TPB * m_blk : TPB;
         k_loop<C, false, BCH, CONV, decltype(tail_loads), true>(smem, d, p.x, p.w, p.a_cat, p.t_ext, p.b_cat, KT, KT1, lane, wm, wn, l32, lh, sw, acc, tacc, tail_loads, ConvGeom{0, 0}, false, false,
-                                                                p.il_cnt + m_blk, rt * (p.ldt / 64), p.il_cnt + (KH_SPLIT_COUNTER_INTS - 1));
+                                                                p.il_cnt + m_blk, rt * (p.ldt / 64), p.il_cnt + (p.M + 127) / 128);
       } else {
         k_loop<C, false, BCH, CONV>(smem, d, p.x, p.w, p.a_cat, p.t_ext, p.b_cat, KT, KT1, lane, wm, wn, l32, lh, sw, acc, tacc, tail_loads, ConvGeom{p.conv_w, p.conv_cin}, (p.dbg & 64) != 0, (p.dbg & 128) != 0);
       }
@@ -477,18 +477,6 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
     stamp(2);
     __syncthreads();  // every wave is done reading the ring before sB / sC reuse it
     stamp(3);
-    if constexpr (IL) {
-      // this workgroup has read T: the last of the row block's workgroups to say so zeroes both counters for the
-      // next launch
-      if (tid == 0) {
-        int* dep = p.il_cnt + KH_SPLIT_MAX_ROW_BLOCKS + m_blk;
-        if (__hip_atomic_fetch_add(dep, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == p.n_chunks - 1) {
-          __hip_atomic_store(p.il_cnt + m_blk, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          __hip_atomic_store(dep, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-      }
-    }
-
     if constexpr (NRT > 0) {
       if (shrink) {
 #pragma unroll

@@ -155,24 +155,51 @@ def lora_linear_pre(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.
     return out
 
 
-SPLIT_COUNTER_INTS = 2 * 2047 + 2   # KH_SPLIT_COUNTER_INTS of include/katz_hip.h
-_split_counters: dict = {}
+# Counters of kh_lora_linear_split_bf16's in-launch shrink.  Every call needs ceil(M / 128) + 1 zeroed int32 and leaves
+# them dirty, so they come from one arena per device: calls take consecutive slices, and `split_counters_reset`
+# clears what has been handed out with ONE fill kernel and starts over.  The UNet / ControlNet forward resets at its
+# start (inside a captured graph that is one fill node per step and the same slices on every replay); a caller that
+# never resets is served until the arena is full, then it is reset for him.  One stream per device: a reset must not
+# overtake launches that still use their slices.
+SPLIT_ARENA_INTS = 1 << 16
+_split_arena: dict = {}     # (device type, index) -> [buffer, ints handed out, last slice]
 
 
-def split_counters(device) -> torch.Tensor:
-    """The zero-initialised counter buffer kh_lora_linear_split_bf16 synchronises its in-launch shrink with: one per
-    device, shared by every call (calls on one device run one after the other; each leaves the buffer zeroed).  Its
-    last element is set if a bounded wait ever ran out."""
+def _arena(device):
     key = (device.type, device.index)
-    buf = _split_counters.get(key)
-    if buf is None:
+    st = _split_arena.get(key)
+    if st is None:
         if torch.cuda.is_current_stream_capturing():
             # memory allocated during a capture belongs to the graph's pool and dies with the graph
-            raise RuntimeError("katz_amd: run the step once eagerly before capturing it (the LoRA counter buffer is "
+            raise RuntimeError("katz_amd: run the step once eagerly before capturing it (the LoRA counter arena is "
                                "allocated on first use and must outlive the graph)")
-        buf = torch.zeros(SPLIT_COUNTER_INTS, dtype=torch.int32, device=device)
-        _split_counters[key] = buf
-    return buf
+        st = [torch.zeros(SPLIT_ARENA_INTS, dtype=torch.int32, device=device), 0, None]
+        _split_arena[key] = st
+    return st
+
+
+def split_counters_reset(device) -> None:
+    """Clear the counters handed out since the last reset (one fill kernel; nothing when none were)."""
+    st = _arena(device)
+    if st[1]:
+        st[0][:st[1]].zero_()
+        st[1] = 0
+
+
+def _split_counters(device, M: int) -> torch.Tensor:
+    n = (M + 127) // 128 + 1   # KH_SPLIT_COUNTER_INTS(M)
+    st = _arena(device)
+    if st[1] + n > SPLIT_ARENA_INTS:
+        split_counters_reset(device)
+    st[2] = st[0][st[1]:st[1] + n]
+    st[1] += n
+    return st[2]
+
+
+def split_counters_last(device) -> Optional[torch.Tensor]:
+    """The counters of the most recent lora_linear_split call on this device (for tests: arrivals per row block, then
+    the time-out flag)."""
+    return _arena(device)[2]
 
 
 def lora_linear_split(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], a_cat: torch.Tensor,
@@ -204,7 +231,7 @@ def lora_linear_split(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torc
     n_out = N // 2 if geglu else N
     out = torch.empty(tuple(x.shape[:-1]) + (n_out,), dtype=BF16, device=x.device)
     t = torch.empty((M, RT), dtype=BF16, device=x.device)
-    cnt = split_counters(x.device)
+    cnt = _split_counters(x.device, M)
     flags = (1 if geglu else 0) | ((1 if two_launches else 0) << 8)
     if CALL_LOG is not None:   # one entry per kernel launch
         if lib.kh_lora_linear_split_launches(M, N, K, R, n_split, flags) == 2:

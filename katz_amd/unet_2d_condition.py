@@ -386,6 +386,8 @@ class UNet2DConditionModel(nn.Module):
         if sample.dtype != torch.bfloat16 or not sample.is_contiguous(memory_format=torch.channels_last):
             sample = sample.to(torch.bfloat16).contiguous(memory_format=torch.channels_last)
         ctx = encoder_hidden_states.to(torch.bfloat16).contiguous()
+        if sample.is_cuda:
+            ops.split_counters_reset(sample.device)   # one fill per step clears the in-launch shrinks' counters
 
         if self._ctx_kv is None:
             self.prepare()
