@@ -1,6 +1,7 @@
 // Shared device/host helpers for the katz_hip kernels (gfx950 / CDNA4 only).
 #pragma once
 #include <hip/hip_runtime.h>
+#include <atomic>
 #include <hip/hip_ext.h>
 #include <stdint.h>
 
@@ -19,6 +20,20 @@
     hipError_t e__ = hipGetLastError();             \
     return e__ == hipSuccess ? KH_OK : (int)e__;    \
   } while (0)
+
+// hipFuncAttributeMaxDynamicSharedMemorySize is a setting per device: remembered per kernel and device, so a process
+// that drives several GPUs sets it on each (devices beyond 63: set on every launch).
+template <auto Kernel>
+inline hipError_t kh_allow_lds(int bytes) {
+  static std::atomic<uint64_t> done{0};
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev >= 0 && dev < 64 && ((done.load(std::memory_order_relaxed) >> dev) & 1)) return hipSuccess;
+  e = hipFuncSetAttribute((const void*)Kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e == hipSuccess && dev >= 0 && dev < 64) done.fetch_or(1ull << dev, std::memory_order_relaxed);
+  return e;
+}
 
 // ---- optional per-launch timing (host) -----------------------------------------------------------
 // While profiling is on (kh_profile_begin .. kh_profile_end) every kernel goes out through

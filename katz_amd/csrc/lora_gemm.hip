@@ -312,13 +312,7 @@ int launch_cfg(LoraGemmParams p, hipStream_t stream) {
   }
   p.n_chunk = nc;
   p.n_chunks = (p.n_tiles + nc - 1) / nc;
-  static bool attr_done = false;  // per template instantiation
-  if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void*)lora_gemm_kernel<C>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)C::LDS_BYTES);
-    if (e != hipSuccess) return (int)e;
-    attr_done = true;
-  }
+  if (hipError_t e = kh_allow_lds<lora_gemm_kernel<C>>((int)C::LDS_BYTES); e != hipSuccess) return (int)e;
   const unsigned grid = (unsigned)(p.m_tiles * p.n_chunks);
   kh_launch(KH_TAG_LORA_GEMM, lora_gemm_kernel<C>, dim3(grid), dim3(C::NT), C::LDS_BYTES, stream, p);
   KH_RETURN_LAST_ERROR();

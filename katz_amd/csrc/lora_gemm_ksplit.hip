@@ -267,12 +267,7 @@ template <class C, bool CONV = false>
 int launch_ksplit(LoraGemmParams p, hipStream_t stream) {
   p.m_tiles = (p.M + C::BM - 1) / C::BM;
   p.n_tiles = (p.N + C::BN - 1) / C::BN;
-  static bool attr_done = false;  // per template instantiation
-  if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void*)lora_gemm_ksplit_kernel<C, CONV>, hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS);
-    if (e != hipSuccess) return (int)e;
-    attr_done = true;
-  }
+  if (hipError_t e = kh_allow_lds<lora_gemm_ksplit_kernel<C, CONV>>(C::LDS); e != hipSuccess) return (int)e;
   // the XCD grid whose per-XCD block touches the fewest operand rows, padding counted as cost
   double best = 0;
   p.xg_n = 0;

@@ -603,13 +603,7 @@ int launch_pcfg(LoraGemmParams p, hipStream_t stream, int n_groups = 1) {
   }
   p.n_chunk = nc;
   p.n_chunks = (p.n_tiles + nc - 1) / nc;
-  static bool attr_done = false;  // per template instantiation
-  if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void*)lora_gemm_pipe_kernel<C, CONV>,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)C::LDS_BYTES);
-    if (e != hipSuccess) return (int)e;
-    attr_done = true;
-  }
+  if (hipError_t e = kh_allow_lds<lora_gemm_pipe_kernel<C, CONV>>((int)C::LDS_BYTES); e != hipSuccess) return (int)e;
   unsigned grid = (unsigned)(p.m_tiles * p.n_chunks);
   p.xg_n = p.xr_m = p.xr_n = 0;
   if (C::NRT == 0 && (p.dbg & 8) == 0) {
@@ -682,12 +676,7 @@ static int launch_il(const LoraGemmParams& pin, hipStream_t stream) {
   p.n_chunk = 1;
   p.n_chunks = p.n_tiles;
   constexpr int LDS = (int)C::LDS_BYTES > S::LDS ? (int)C::LDS_BYTES : S::LDS;
-  static bool attr_done = false;  // per template instantiation
-  if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void*)lora_gemm_pipe_kernel<C, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS);
-    if (e != hipSuccess) return (int)e;
-    attr_done = true;
-  }
+  if (hipError_t e = kh_allow_lds<lora_gemm_pipe_kernel<C, false, true>>(LDS); e != hipSuccess) return (int)e;
   double best = 0;
   p.xg_n = 0;
   for (int gm = 1; gm <= 8; gm *= 2) {

@@ -261,12 +261,7 @@ int wide_launch(LoraGemmParams p, hipStream_t stream) {
   if (!wide_ok<C>(p)) return KH_ERR_UNSUPPORTED;
   p.m_tiles = p.M / C::BM;
   p.n_tiles = p.N / C::BN;
-  static bool attr_done = false;  // per template instantiation
-  if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void*)lora_gemm_wide_kernel<C>, hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS);
-    if (e != hipSuccess) return (int)e;
-    attr_done = true;
-  }
+  if (hipError_t e = kh_allow_lds<lora_gemm_wide_kernel<C>>(C::LDS); e != hipSuccess) return (int)e;
   // the XCD grid whose per-XCD block touches the fewest operand rows, padding counted as cost
   double best = 0;
   p.xg_n = 0;

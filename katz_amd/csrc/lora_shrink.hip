@@ -32,12 +32,7 @@ __global__ __launch_bounds__(C::NW * 64) void lora_shrink_kernel(const ShrinkPar
 
 template <class C>
 int launch_shrink(const ShrinkParams& p, hipStream_t stream) {
-  static bool attr_done = false;
-  if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute((const void*)lora_shrink_kernel<C>, hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS);
-    if (e != hipSuccess) return (int)e;
-    attr_done = true;
-  }
+  if (hipError_t e = kh_allow_lds<lora_shrink_kernel<C>>(C::LDS); e != hipSuccess) return (int)e;
   dim3 grid((unsigned)((p.M + C::TR * 32 - 1) / (C::TR * 32)), (unsigned)((p.R + C::TC * 32 - 1) / (C::TC * 32)));
   kh_launch(KH_TAG_LORA_SHRINK, lora_shrink_kernel<C>, grid, dim3(C::NW * 64), C::LDS, stream, p);
   KH_RETURN_LAST_ERROR();
