@@ -141,6 +141,7 @@ class ControlNetModel(nn.Module):
         self._ctx_kv.run(ctx)
         emb = self._embed(sample, timestep, added_cond_kwargs)
         temb_act = F.silu(emb)
+        self._temb_proj.run(temb_act)   # time_emb_proj of all resnets, batched per width
         sample = self.conv_in(sample)
         sample = sample + self.controlnet_cond_embedding(cond)
         skips = (sample,)

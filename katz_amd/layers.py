@@ -382,6 +382,7 @@ class ResnetBlock2D(nn.Module):
         self.norm_silu2 = nn.Sequential(*fused_norm_silu(out_channels, groups, eps))
         self.conv2 = Conv3x3(out_channels, out_channels)
         self.conv_shortcut = nn.Conv2d(in_channels, out_channels, 1) if in_channels != out_channels else None
+        self.temb_proj = None   # this step's time_emb_proj(temb_act), when a TimeEmbProjector computed it ahead
 
     def _shortcut(self, x):
         """1x1 convolution = a linear layer over the channels of every pixel (NHWC rows)."""
@@ -398,13 +399,49 @@ class ResnetBlock2D(nn.Module):
         h = self.norm_silu1(input_tensor)
         h = self.conv1(h)
         # hidden_states + temb[:, :, None, None] rides inside the second norm (no separate pass)
-        h = self.norm_silu2[0](h, add_nc=self.time_emb_proj(temb_act))
+        tp, self.temb_proj = self.temb_proj, None
+        h = self.norm_silu2[0](h, add_nc=self.time_emb_proj(temb_act) if tp is None else tp)
         if self.conv_shortcut is not None:
             input_tensor = self._shortcut(input_tensor)
         out = self.conv2(h, residual=input_tensor)   # input_tensor + conv2(h), the add in the conv's epilogue
         if self.output_scale_factor != 1.0:
             out = out / self.output_scale_factor
         return out
+
+
+class TimeEmbProjector:
+    """time_emb_proj(silu(temb)) of EVERY resnet of the model at the start of the step, one batched launch per output
+    width instead of one two-row GEMM per resnet inside the chain of big kernels (the reference computes each where
+    it is used, resnet.py:381-390).  Same arithmetic, same inputs; nothing is kept across steps."""
+
+    def __init__(self, resnets: Sequence["ResnetBlock2D"]):
+        self.groups: Dict[int, List[ResnetBlock2D]] = {}
+        for r in resnets:
+            self.groups.setdefault(r.time_emb_proj.out_features, []).append(r)
+        self._stacked: Dict[int, tuple] = {}   # width -> (key, W [G,C,K], b [G,1,C])
+
+    @staticmethod
+    def _key(rs):
+        return tuple((r.time_emb_proj.weight.data_ptr(), r.time_emb_proj.weight._version, r.time_emb_proj.bias._version)
+                     for r in rs)
+
+    def run(self, temb_act: torch.Tensor) -> None:
+        for width, rs in self.groups.items():
+            key = self._key(rs)
+            st = self._stacked.get(width)
+            if st is None or st[0] != key:
+                if temb_act.is_cuda and torch.cuda.is_current_stream_capturing():
+                    raise RuntimeError("katz_amd: run the step once eagerly before capturing it (stacked time_emb_proj weights)")
+                with torch.no_grad():
+                    w = torch.stack([r.time_emb_proj.weight.detach() for r in rs]).contiguous()
+                    b = torch.stack([r.time_emb_proj.bias.detach() for r in rs]).unsqueeze(1).contiguous()
+                st = (key, w, b)
+                self._stacked[width] = st
+            _, w, b = st
+            x = temb_act.to(w.dtype).unsqueeze(0).expand(len(rs), -1, -1)
+            y = torch.baddbmm(b, x, w.transpose(1, 2))          # [G, N, C], every resnet's [N, C] contiguous
+            for i, r in enumerate(rs):
+                r.temb_proj = y[i]
 
 
 class KatzAttnProcessor:

@@ -63,13 +63,27 @@ class UNet2DConditionOutput:
     sample: torch.Tensor
 
 
+_freq_tables: Dict[tuple, torch.Tensor] = {}
+
+
+def _frequencies(half: int, downscale_freq_shift: float, max_period: int, device) -> torch.Tensor:
+    """exp(-ln(max_period) * arange(half) / (half - shift)) (embeddings.py:50-55): constants of the model, computed
+    once per device with the reference's own sequence of operations instead of in every step."""
+    key = (half, float(downscale_freq_shift), int(max_period), device.type, device.index)
+    t = _freq_tables.get(key)
+    if t is None:
+        exponent = -math.log(max_period) * torch.arange(0, half, dtype=torch.float32, device=device)
+        t = torch.exp(exponent / (half - downscale_freq_shift))
+        if not (device.type == "cuda" and torch.cuda.is_current_stream_capturing()):
+            _freq_tables[key] = t   # a tensor made during graph capture lives in the graph's pool: do not keep it
+    return t
+
+
 def get_timestep_embedding(timesteps, embedding_dim, flip_sin_to_cos=False, downscale_freq_shift=1.0, scale=1.0,
                            max_period=10000):
     """diffusers-hf/src/diffusers/models/embeddings.py:26-66, evaluated on the device of `timesteps`."""
     half = embedding_dim // 2
-    exponent = -math.log(max_period) * torch.arange(0, half, dtype=torch.float32, device=timesteps.device)
-    exponent = exponent / (half - downscale_freq_shift)
-    emb = scale * timesteps[:, None].float() * torch.exp(exponent)[None, :]
+    emb = scale * timesteps[:, None].float() * _frequencies(half, downscale_freq_shift, max_period, timesteps.device)[None, :]
     emb = torch.cat([torch.sin(emb), torch.cos(emb)], dim=-1)
     if flip_sin_to_cos:
         emb = torch.cat([emb[:, half:], emb[:, :half]], dim=-1)
@@ -195,8 +209,9 @@ class UNet2DConditionModel(nn.Module):
         for m in self.lora_linears().values():
             m.prepare()
         if self._ctx_kv is None:
-            from .layers import Attention, ContextKVProjector
+            from .layers import Attention, ContextKVProjector, ResnetBlock2D, TimeEmbProjector
             self._ctx_kv = ContextKVProjector([m for m in self.modules() if isinstance(m, Attention)])
+            self._temb_proj = TimeEmbProjector([m for m in self.modules() if isinstance(m, ResnetBlock2D)])
 
     # ---- LoRA surface ----------------------------------------------------------------------------
     def lora_linears(self) -> Dict[str, LoRALinear]:
@@ -394,6 +409,7 @@ class UNet2DConditionModel(nn.Module):
         self._ctx_kv.run(ctx)  # K/V projections of all cross-attentions, grouped
         emb = self._embed(sample, timestep, added_cond_kwargs)
         temb_act = F.silu(emb)
+        self._temb_proj.run(temb_act)   # time_emb_proj of all resnets, batched per width
         sample = self.conv_in(sample)
         skips = (sample,)
         for blk in self.down_blocks:

@@ -176,6 +176,33 @@ def test_tiny_unet_step_with_lora_and_controlnet(tiny_pair):
             m.adapters.clear(); m.active = []
 
 
+def test_time_emb_projector_matches_per_resnet_linear(tiny_pair):
+    """The batched time_emb_proj of all resnets equals each resnet's own nn.Linear on the same input (bf16 rounding of
+    one GEMM against another), is handed out once per run, and follows in-place weight changes."""
+    from katz_amd.layers import ResnetBlock2D
+
+    cfg, oracle, prod = tiny_pair
+    say("time emb projector")
+    resnets = [m for m in prod.modules() if isinstance(m, ResnetBlock2D)]
+    assert len(resnets) >= 6 and len({r.time_emb_proj.out_features for r in resnets}) >= 2
+    g = torch.Generator().manual_seed(3)
+    temb = torch.randn(2, resnets[0].time_emb_proj.in_features, generator=g).to("cuda:0", BF)
+    with torch.no_grad():
+        prod._temb_proj.run(temb)
+        for r in resnets:
+            assert r.temb_proj is not None and r.temb_proj.is_contiguous()
+            assert_close_rel(r.temb_proj, r.time_emb_proj(temb).float().cpu(), 2e-2, "batched time_emb_proj")
+        first = resnets[0]
+        before = first.temb_proj.clone()
+        first.time_emb_proj.weight.mul_(2.0)                     # in place: same storage, new version
+        prod._temb_proj.run(temb)
+        assert_close_rel(first.temb_proj, first.time_emb_proj(temb).float().cpu(), 2e-2, "after an in-place change")
+        assert not torch.equal(first.temb_proj, before)
+        first.time_emb_proj.weight.mul_(0.5)
+        for r in resnets:
+            r.temb_proj = None
+
+
 def test_tiny_unet_graph_replay_matches_eager(tiny_pair):
     """The captured step reproduces eager results over several replays with fresh inputs."""
     from katz_amd.graph import GraphedUNetStep
