@@ -41,7 +41,7 @@ const char* kh_error_string(int code);
  * kh_profile_begin and kh_profile_end every kernel of this library is launched with its own HIP
  * start/stop event pair on the launch stream.  kh_profile_end waits for them and writes, in launch
  * order, a kernel tag (1 lora_gemm, 2 lora_gemm_f32, 3 attention, 4 group_norm stats, 5 group_norm apply,
- * 6 layer_norm, 7 geglu, 8 residual_add, 9 concat_residual, 10 sgmv_shrink, 11 sgmv_expand, 12 lora_shrink, 13 conv3x3, 14 cfg_euler) and the
+ * 6 layer_norm, 7 geglu, 8 residual_add, 9 concat_residual, 10 sgmv_shrink, 11 sgmv_expand, 12 lora_shrink, 13 conv3x3, 14 cfg_euler, 15 upsample) and the
  * duration in ms into HOST arrays; returns the number of launches (or -hipError_t).  Do not use under
  * graph capture. */
 int kh_profile_begin(void);
@@ -181,6 +181,10 @@ int kh_residual_add_bf16(void* dst, const void* const* srcs, int n_srcs, float i
  * residuals: HOST array of n_residuals (0..8) device pointers; C1 % 8 == 0, C2 % 8 == 0. */
 int kh_concat_residual_bf16(const void* h, const void* skip, const void* const* residuals, int n_residuals,
                             float inv_count, void* out, int64_t rows, int64_t C1, int64_t C2, void* stream);
+/* Nearest-neighbour 2x upsampling of an NHWC tensor: y[n, h, w, :] = x[n, h/2, w/2, :], y is [N, 2H, 2W, C].
+ * Replaces F.interpolate(hidden_states, scale_factor=2.0, mode="nearest") of Upsample2D.forward
+ * (diffusers-hf/src/diffusers/models/upsampling.py:169-171) in front of the upsampler's convolution.  C % 8 == 0. */
+int kh_upsample_nearest2x_nhwc_bf16(const void* x, void* y, int64_t N, int64_t H, int64_t W, int64_t C, void* stream);
 
 /* ---- 3x3 convolution of the residual blocks ------------------------------------------------------------
  * y[n,ho,wo,co] = bias[co] + sum_{kh,kw,ci} x[n, ho*stride+kh-1, wo*stride+kw-1, ci] * w[co,kh,kw,ci]

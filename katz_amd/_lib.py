@@ -37,6 +37,7 @@ SIGNATURES = {
     "kh_gelu_mul_bf16": (c_int, [_P, _P, _P, _I, c_int, _P]),
     "kh_residual_add_bf16": (c_int, [_P, _P, c_int, c_float, _I, _P]),
     "kh_concat_residual_bf16": (c_int, [_P, _P, _P, c_int, c_float, _P, _I, _I, _I, _P]),
+    "kh_upsample_nearest2x_nhwc_bf16": (c_int, [_P, _P, _I, _I, _I, _I, _P]),
     "kh_cfg_euler_step_bf16": (c_int, [_P, _P, _P, _P, _I, c_float, _P, c_int, _P]),
     "kh_conv3x3_nhwc_bf16": (c_int, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]),
 }

@@ -132,6 +132,22 @@ __global__ __launch_bounds__(EW_THREADS) void concat_residual_kernel(const bf16_
   }
 }
 
+// nearest-neighbour 2x upsampling, NHWC: out pixel (h, w) = in pixel (h / 2, w / 2); one 16-byte channel chunk per item
+__global__ __launch_bounds__(EW_THREADS) void upsample2x_kernel(const bf16_t* __restrict__ x, bf16_t* __restrict__ y,
+                                                                int N, int H, int W, int C) {
+  const int cp = C / 8, W2 = 2 * W, H2 = 2 * H;
+  const long total = (long)N * H2 * W2 * cp;
+  for (long i = (long)blockIdx.x * EW_THREADS + threadIdx.x; i < total; i += (long)gridDim.x * EW_THREADS) {
+    const int c = (int)(i % cp);
+    long p = i / cp;
+    const int w = (int)(p % W2); p /= W2;
+    const int h = (int)(p % H2);
+    const long n = p / H2;
+    const u32x4 v = *reinterpret_cast<const u32x4*>(x + ((n * H + (h >> 1)) * W + (w >> 1)) * C + c * 8);
+    *reinterpret_cast<u32x4*>(y + i * 8) = v;
+  }
+}
+
 unsigned ew_grid(long work_items) {
   long b = (work_items + EW_THREADS - 1) / EW_THREADS;
   const long cap = 256L * 16;  // 16 workgroups per CU, grid-stride beyond that
@@ -280,5 +296,16 @@ KH_EXPORT int kh_concat_residual_bf16(const void* h, const void* skip, const voi
   kh_launch(KH_TAG_CONCAT_RESIDUAL, concat_residual_kernel, dim3(ew_grid(rows * ((C1 + C2) / 8))), dim3(EW_THREADS), 0,
                      (hipStream_t)stream, (const bf16_t*)h, (const bf16_t*)skip, s, (bf16_t*)out, (long)rows, (int)C1,
                      (int)C2);
+  KH_RETURN_LAST_ERROR();
+}
+
+// Upsample2D's interpolation, see include/katz_hip.h.
+KH_EXPORT int kh_upsample_nearest2x_nhwc_bf16(const void* x, void* y, int64_t N, int64_t H, int64_t W, int64_t C, void* stream) {
+  if (!x || !y || N <= 0 || H <= 0 || W <= 0 || C <= 0) return KH_ERR_INVALID_ARG;
+  if (C % 8 != 0) return KH_ERR_UNSUPPORTED;
+  if (N > (1 << 20) || H > (1 << 14) || W > (1 << 14) || C > (1 << 20)) return KH_ERR_TOO_LARGE;
+  if (!kh_aligned16(x) || !kh_aligned16(y)) return KH_ERR_ALIGNMENT;
+  kh_launch(KH_TAG_UPSAMPLE, upsample2x_kernel, dim3(ew_grid(N * 4 * H * W * (C / 8))), dim3(EW_THREADS), 0, (hipStream_t)stream,
+            (const bf16_t*)x, (bf16_t*)y, (int)N, (int)H, (int)W, (int)C);
   KH_RETURN_LAST_ERROR();
 }

@@ -362,7 +362,11 @@ class Upsample2D(nn.Module):
 
     def forward(self, x, output_size=None):
         if output_size is None:
-            x = F.interpolate(x, scale_factor=2.0, mode="nearest")
+            if (x.is_cuda and x.dtype == torch.bfloat16 and x.shape[1] % 8 == 0
+                    and x.is_contiguous(memory_format=torch.channels_last)):
+                x = ops.upsample_nearest2x(x)
+            else:
+                x = F.interpolate(x, scale_factor=2.0, mode="nearest")
         else:
             x = F.interpolate(x, size=output_size, mode="nearest")
         return self.conv(x)

@@ -455,6 +455,18 @@ def concat_residual(h: torch.Tensor, skip: torch.Tensor, residuals: Sequence[tor
     return out
 
 
+def upsample_nearest2x(x: torch.Tensor) -> torch.Tensor:
+    """F.interpolate(x, scale_factor=2.0, mode="nearest") for a channels_last bfloat16 [N,C,H,W] tensor."""
+    lib = _lib.load()
+    if not x.is_cuda or x.dtype != BF16 or x.dim() != 4 or not x.is_contiguous(memory_format=torch.channels_last):
+        raise ValueError("x must be a channels_last bfloat16 GPU tensor")
+    N, C, H, W = x.shape
+    out = torch.empty((N, C, 2 * H, 2 * W), dtype=BF16, device=x.device, memory_format=torch.channels_last)
+    rc = lib.kh_upsample_nearest2x_nhwc_bf16(_ptr(x), _ptr(out), N, H, W, C, _stream())
+    _lib.check(rc, "kh_upsample_nearest2x_nhwc_bf16")
+    return out
+
+
 def pack_conv3x3_weight(weight: torch.Tensor) -> torch.Tensor:
     """nn.Conv2d weight [Cout,Cin,3,3] -> the [Cout,3,3,Cin] layout kh_conv3x3_nhwc_bf16 reads (a copy)."""
     if weight.dim() != 4 or weight.shape[2:] != (3, 3):
@@ -518,7 +530,7 @@ def cfg_euler_step(noise_pred: torch.Tensor, latents: torch.Tensor, coef: torch.
 # --------------------------------------------------------------------------------------- per-launch timing
 KERNEL_TAGS = {1: "lora_gemm", 2: "lora_gemm_f32", 3: "attention", 4: "group_norm_stats", 5: "group_norm_apply",
                6: "layer_norm", 7: "geglu", 8: "residual_add", 9: "concat_residual", 10: "sgmv_shrink",
-               11: "sgmv_expand", 12: "lora_shrink", 13: "conv3x3", 14: "cfg_euler"}
+               11: "sgmv_expand", 12: "lora_shrink", 13: "conv3x3", 14: "cfg_euler", 15: "upsample"}
 
 
 def profile_begin() -> None:

@@ -19,7 +19,7 @@ def test_header_declares_the_expected_entry_points():
     for must in ("kh_lora_linear_bf16", "kh_lora_linear_f32", "kh_lora_shrink_bf16", "kh_lora_linear_pre_bf16",
                  "kh_sgmv_shrink_bf16", "kh_sgmv_expand_bf16", "kh_attention_bf16", "kh_group_norm_bf16",
                  "kh_layer_norm_bf16", "kh_geglu_bf16", "kh_gelu_mul_bf16", "kh_residual_add_bf16",
-                 "kh_concat_residual_bf16", "kh_version", "kh_error_string"):
+                 "kh_concat_residual_bf16", "kh_upsample_nearest2x_nhwc_bf16", "kh_version", "kh_error_string"):
         assert must in syms
 
 

@@ -430,6 +430,22 @@ def test_concat_residual_bf16(k):
     assert_close_rel(out, ref, REL_BF16, "concat_residual")
 
 
+@pytest.mark.parametrize("shape", [(2, 1280, 32, 32), (2, 640, 64, 64), (1, 8, 1, 1), (3, 24, 5, 7)], ids=str)
+def test_upsample_nearest2x(shape):
+    """Upsample2D's interpolation (upsampling.py:169-171) is a copy: bit equality with F.interpolate on the same bf16
+    values (the oracle's upsampler calls the same function)."""
+    from katz_amd import ops
+
+    say("upsample_nearest2x", shape)
+    g = torch.Generator().manual_seed(sum(shape))
+    x = randn(g, *shape).to(BF)
+    out = ops.upsample_nearest2x(x.to(dev()).contiguous(memory_format=torch.channels_last))
+    torch.cuda.synchronize()
+    N, C, H, W = shape
+    assert out.shape == (N, C, 2 * H, 2 * W) and out.is_contiguous(memory_format=torch.channels_last)
+    assert torch.equal(out.cpu(), torch.nn.functional.interpolate(x, scale_factor=2.0, mode="nearest"))
+
+
 # ------------------------------------------------------------------------------------------- K2
 @pytest.mark.parametrize("T,dm", [(1024, 1280), (4096, 640), (77, 640)], ids=str)
 def test_sgmv_heterogeneous_batch(T, dm):
