@@ -157,12 +157,14 @@ def lora_linear_pre(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.
 
 # Counters of kh_lora_linear_split_bf16's in-launch shrink.  Every call needs ceil(M / 128) + 1 zeroed int32 and leaves
 # them dirty, so they come from one arena per device: calls take consecutive slices, and `split_counters_reset`
-# clears what has been handed out with ONE fill kernel and starts over.  The UNet / ControlNet forward resets at its
-# start (inside a captured graph that is one fill node per step and the same slices on every replay); a caller that
-# never resets is served until the arena is full, then it is reset for him.  One stream per device: a reset must not
-# overtake launches that still use their slices.
+# clears the WHOLE arena with one fill kernel (256 KB: as cheap as any fill) and starts over.  The whole arena, not
+# just what the host handed out since the last reset: a reset recorded into a HIP graph runs at replay time, when the
+# host's count says nothing about what eager forwards or other graphs have dirtied in between.  The UNet / ControlNet
+# forward resets at its start (inside a captured graph that is one fill node per step and the same slices on every
+# replay); a caller that never resets is served until the arena is full, then it is reset for him.  One stream per
+# device: a reset must not overtake launches that still use their slices.
 SPLIT_ARENA_INTS = 1 << 16
-_split_arena: dict = {}     # (device type, index) -> [buffer, ints handed out, last slice]
+_split_arena: dict = {}     # (device type, index) -> [buffer, ints handed out, last slice, ever used]
 
 
 def _arena(device):
@@ -173,17 +175,17 @@ def _arena(device):
             # memory allocated during a capture belongs to the graph's pool and dies with the graph
             raise RuntimeError("katz_amd: run the step once eagerly before capturing it (the LoRA counter arena is "
                                "allocated on first use and must outlive the graph)")
-        st = [torch.zeros(SPLIT_ARENA_INTS, dtype=torch.int32, device=device), 0, None]
+        st = [torch.zeros(SPLIT_ARENA_INTS, dtype=torch.int32, device=device), 0, None, False]
         _split_arena[key] = st
     return st
 
 
 def split_counters_reset(device) -> None:
-    """Clear the counters handed out since the last reset (one fill kernel; nothing when none were)."""
+    """Clear every counter of the device's arena (one fill kernel; nothing while no counter has ever been handed out)."""
     st = _arena(device)
-    if st[1]:
-        st[0][:st[1]].zero_()
-        st[1] = 0
+    if st[3]:
+        st[0].zero_()
+    st[1] = 0
 
 
 def _split_counters(device, M: int) -> torch.Tensor:
@@ -193,6 +195,7 @@ def _split_counters(device, M: int) -> torch.Tensor:
         split_counters_reset(device)
     st[2] = st[0][st[1]:st[1] + n]
     st[1] += n
+    st[3] = True
     return st[2]
 
 

@@ -855,3 +855,48 @@ def test_lora_linear_split(case):
     # the two forms differ only by the fp32 summation order inside the shrink: a handful of last-bit differences
     differing = (ys[0] != y2).float().mean().item()
     assert differing < 5e-3, differing
+
+
+def test_split_counters_after_a_reset_that_was_only_recorded():
+    """A reset recorded into a HIP graph does not run at capture time.  Counters that eager calls dirtied before the
+    capture must still be clear when later eager calls reach them: every slice shows exactly its own arrivals (a slice
+    that was not cleared would show them on top of the old ones) and the results repeat bit for bit."""
+    from katz_amd import ops
+
+    say("split counters: recorded reset")
+    d = dev()
+    g = torch.Generator().manual_seed(77)
+    M, N, K, R = 2048, 1280, 1280, 64
+    x, w, b = randn(g, M, K).to(d, BF), randn(g, N, K, std=0.03).to(d, BF), randn(g, N).to(d, BF)
+    A, B = randn(g, R, K, std=0.05).to(d, BF), randn(g, N, R, std=0.05).to(d, BF)
+    cs = torch.full((R,), 0.7, device=d)
+    call = lambda rows: ops.lora_linear_split(x[:rows], w, b, A, cs, B)
+    assert ops._lib.load().kh_lora_linear_split_launches(M, N, K, R, 0, 0) == 1, "shape no longer runs as one launch"
+
+    def burst(n_calls):
+        outs, cnts = [], []
+        for _ in range(n_calls):
+            outs.append(call(M))
+            cnts.append(ops.split_counters_last(d).clone())
+        return outs, cnts
+
+    ops.split_counters_reset(d)
+    ref_outs, ref_cnts = burst(6)                      # dirties six slices
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):     # records a reset and ONE call: nothing of it runs now
+            ops.split_counters_reset(d)
+            y_graph = call(M)
+    torch.cuda.current_stream().wait_stream(side)
+    ops.split_counters_reset(d)                        # the next eager "step"
+    outs, cnts = burst(6)                              # reaches the slices the capture's reset never cleared
+    graph.replay()
+    torch.cuda.synchronize()
+    for o, c, rc in zip(outs, cnts, ref_cnts):
+        assert torch.equal(c, rc), f"counters {c.tolist()} instead of {rc.tolist()}"
+        assert int(c[-1]) == 0
+        assert torch.equal(o, ref_outs[0])
+    assert torch.equal(y_graph, ref_outs[0])
+    ops.split_counters_reset(d)
