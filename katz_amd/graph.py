@@ -15,6 +15,17 @@ import torch
 
 
 class GraphedUNetStep:
+    """One captured step with static input / output tensors.
+
+    The graph holds device addresses: of the weights, of the kernel-side weight copies (stacked q/k/v, interleaved
+    GEGLU rows, packed convolution weights, stacked time_emb_proj), of the packed adapters and of the scratch buffers.
+    It stays valid across everything that is written IN PLACE -- new inputs, adapter weights and the global LoRA scale
+    (`set_adapters` with the same adapter set, `cross_attention_kwargs["scale"]`: only `col_scale` of the linear layers is
+    rewritten; adapters on 3x3 convolutions repack on any change).
+    After anything that repacks or re-derives buffers -- a different set of active adapters, `load_lora_into_unet` /
+    `unload_lora`, `fuse_lora` / `unfuse_lora`, `patch_on_lora`, `load_state_dict`, another batch size or resolution --
+    build a new GraphedUNetStep; replaying the old one would compute with the old buffers."""
+
     def __init__(self, unet, sample, timestep, encoder_hidden_states, added_cond_kwargs,
                  down_block_additional_residuals: Optional[Sequence[torch.Tensor]] = None,
                  mid_block_additional_residual: Optional[torch.Tensor] = None, warmup: int = 2):

@@ -326,6 +326,7 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, heads: int, sca
 
 # --------------------------------------------------------------------------------------- K4
 _gn_workspace: dict = {}
+_gn_retired: list = []     # outgrown workspaces, kept alive for graphs captured while they were current
 
 
 def _workspace(nbytes: int, device) -> torch.Tensor:
@@ -336,6 +337,8 @@ def _workspace(nbytes: int, device) -> torch.Tensor:
         if torch.cuda.is_current_stream_capturing():
             raise RuntimeError("katz_amd: run the step once eagerly before capturing it (the GroupNorm workspace grows "
                                "on first use and must outlive the graph)")
+        if buf is not None:
+            _gn_retired.append(buf)   # a captured graph may still write its partial sums there: never hand it back
         buf = torch.empty(max(nbytes // 4, 1 << 16), dtype=torch.float32, device=device)
         _gn_workspace[key] = buf
     return buf
