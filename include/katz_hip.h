@@ -74,7 +74,10 @@ int kh_lora_linear_bf16(const void* x, const void* w, const void* bias, const vo
  * (lora.py:222-232: up(down(x)) * scale).  K % 32 == 0, R <= 128, flags as for kh_lora_linear_bf16.
  * n_split > 0 fuses several layers with one input into one GEMM (to_q/to_k/to_v): W, bias, B_cat are the
  * layers stacked along N in blocks of n_split rows (n_split % 128 == 0) and block j takes T columns
- * [j*R, (j+1)*R) of the shared shrink result; 0 = a single layer. */
+ * [j*R, (j+1)*R) of the shared shrink result; 0 = a single layer.
+ * flags bits 16..23 (kh_lora_linear_pre_bf16, kh_lora_linear_split_bf16): r_used / 16, a promise that the rank columns
+ * >= r_used of every layer's t block and B_cat are all zero (the padding of R = sum of the adapters' ranks up to a
+ * multiple of 64); the kernels then skip products that could only add zeros.  0 = no promise. */
 int kh_lora_shrink_bf16(const void* x, const void* a_cat, const float* col_scale, void* t, int64_t M, int64_t K,
                         int64_t R, void* stream);
 int kh_lora_linear_pre_bf16(const void* x, const void* w, const void* bias, const void* t, int64_t ldt,
@@ -94,7 +97,7 @@ int kh_lora_linear_pre_bf16(const void* x, const void* w, const void* bias, cons
  * call is then undefined).  n_split > 0: w / bias / b_cat stack N / n_split layers of n_split rows each (q, k, v of a
  * self-attention), a_cat / col_scale stack their A matrices ([N / n_split * R, K]) and t_scratch is [M, N / n_split * R],
  * as for kh_lora_linear_pre_bf16.  K % 64 == 0, R % 32 == 0, R <= 128.  flags: bit 0 GEGLU, bits 8..15: 1 = always two
- * launches. */
+ * launches, bits 16..23: r_used / 16 as above. */
 #define KH_SPLIT_COUNTER_INTS(M) (((M) + 127) / 128 + 1)
 int kh_lora_linear_split_bf16(const void* x, const void* w, const void* bias, const void* a_cat, const float* col_scale,
                               const void* b_cat, void* t_scratch, int32_t* counters, const void* residual, void* y,

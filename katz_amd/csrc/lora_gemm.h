@@ -38,6 +38,9 @@ struct LoraGemmParams {
   // per row block, then a time-out flag); the launch leaves the arrivals in them.
   int il_blocks = 0;
   int* il_cnt = nullptr;
+  // two-launch / in-launch forms: rank columns >= r_used of t_ext and b_cat are all zero (0: unknown, use R); the
+  // 128x128 / 256x128 and 256x320 kernels then skip the MFMA steps that would only add zeros
+  int r_used = 0;
 };
 
 // Software-pipelined kernel (lora_gemm_pipe.hip); needs K % 32 == 0.  tile_sel: 0 automatic, >= 16 forces a tile.

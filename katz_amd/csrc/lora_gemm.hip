@@ -516,6 +516,8 @@ KH_EXPORT int kh_lora_linear_pre_bf16(const void* x, const void* w, const void* 
   p.xg_n = p.xr_m = p.xr_n = 0;
   p.sg_start = p.sg_adapter = p.sg_rank = nullptr; p.sg_scale = nullptr; p.sg_mode = 0; p.sg_wstride = 0;
   p.conv_cin = p.conv_h = p.conv_w = p.conv_ho = p.conv_wo = p.conv_stride = 0;
+  p.r_used = ((flags >> 16) & 0xff) * 16;
+  if (p.r_used > p.R) return KH_ERR_INVALID_ARG;
   return lora_gemm_pipe_launch(p, (flags >> 8) & 0xff, (hipStream_t)stream);
 }
 
@@ -565,16 +567,18 @@ KH_EXPORT int kh_lora_linear_split_bf16(const void* x, const void* w, const void
   if (M > (1 << 24) || N > (1 << 24) || K > (1 << 24)) return KH_ERR_TOO_LARGE;
   const bool geglu = (flags & 1) != 0;
   if (geglu && (N % 64 != 0 || residual != nullptr)) return KH_ERR_UNSUPPORTED;
+  if (((flags >> 16) & 0xff) * 16 > R) return KH_ERR_INVALID_ARG;
   if (!kh_aligned16(x) || !kh_aligned16(w) || !kh_aligned16(y) || !kh_aligned16(a_cat) || !kh_aligned16(b_cat) ||
       !kh_aligned16(t_scratch) || (residual && !kh_aligned16(residual)))
     return KH_ERR_ALIGNMENT;
   if (counters != nullptr && kh_lora_linear_split_launches(M, N, K, R, n_split, flags) == 1) {
-    const LoraGemmParams p = split_params(x, w, bias, a_cat, col_scale, b_cat, t_scratch, counters, residual, y, M, N, K, R, n_split, geglu);
+    LoraGemmParams p = split_params(x, w, bias, a_cat, col_scale, b_cat, t_scratch, counters, residual, y, M, N, K, R, n_split, geglu);
+    p.r_used = ((flags >> 16) & 0xff) * 16;
     return lora_gemm_pipe_launch_il(p, (hipStream_t)stream);
   }
   const int rc = kh_lora_shrink_bf16(x, a_cat, col_scale, t_scratch, M, K, RT, stream);
   if (rc != KH_OK) return rc;
-  return kh_lora_linear_pre_bf16(x, w, bias, t_scratch, RT, n_split, b_cat, residual, y, M, N, K, R, flags & 0xff, stream);
+  return kh_lora_linear_pre_bf16(x, w, bias, t_scratch, RT, n_split, b_cat, residual, y, M, N, K, R, flags & 0xff00ff, stream);
 }
 
 // 3x3 convolution, padding 1, NHWC, as an implicit GEMM on the pipelined kernel; see include/katz_hip.h.

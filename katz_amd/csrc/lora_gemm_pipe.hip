@@ -114,7 +114,8 @@ __device__ __forceinline__ void k_loop(char* smem, const Dma<C, SHRINK>& dma, co
                                        int l32, int lh, int sw, f32x16 (&acc)[C::TM][C::TN],
                                        f32x16 (&tacc)[C::SM > 0 ? C::SM : 1][C::NRT > 0 ? C::NRT : 1],
                                        TailLoads tail_loads, ConvGeom cg, bool nodma = false, bool fixk = false,
-                                       const int* il_cnt = nullptr, int il_target = 0, int* il_err = nullptr) {
+                                       const int* il_cnt = nullptr, int il_target = 0, int* il_err = nullptr,
+                                       bool half_last = false) {   // the upper half of the last K tile is all zeros
   constexpr int TM = C::TM, TN = C::TN, NRT = C::NRT, NST = C::NST;
   constexpr int BKP = C::BKP, ROWB = C::ROWB, KS = C::KS;
   constexpr int PD = NST - 1;  // prefetch distance in K tiles
@@ -258,7 +259,7 @@ __device__ __forceinline__ void k_loop(char* smem, const Dma<C, SHRINK>& dma, co
     }
     const Frags<C, SHRINK>& last = (PD & 1) ? f1 : f0;
     mma(last, 0);
-    mma(last, 1);
+    if (!half_last) mma(last, 1);
   } else {
     // fewer K tiles than ring stages (tiny K): request everything, wait for everything
     for (int t = 0; t < KT; ++t) issue(t);
@@ -268,7 +269,7 @@ __device__ __forceinline__ void k_loop(char* smem, const Dma<C, SHRINK>& dma, co
     for (int t = 0; t < KT; ++t) {
       read_frags(t, f0);
       mma(f0, 0);
-      mma(f0, 1);
+      if (!(half_last && t == KT - 1)) mma(f0, 1);
     }
   }
 }
@@ -352,7 +353,11 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
   const int K = p.K, M = p.M, N = p.N;
   constexpr int BKP = C::BKP, ROWB = C::ROWB;
   const int KT1 = k_cols / BKP;                                        // K tiles of x / W
-  const int KT = KT1 + (p.t_ext != nullptr ? p.R / BKP : 0);           // + rank tiles of T / B_cat (two-launch form)
+  // + rank tiles of T / B_cat (two-launch form).  Only the first r_used rank columns can be non-zero: tiles beyond
+  // them are not visited, and of a last tile that they fill at most half only that half is multiplied.
+  const int r_used = (p.r_used > 0 && p.r_used < p.R) ? p.r_used : p.R;
+  const int KT = KT1 + (p.t_ext != nullptr ? (r_used + BKP - 1) / BKP : 0);
+  const bool half_last = p.t_ext != nullptr && (r_used % BKP) != 0 && (r_used % BKP) <= BKP / 2;
 
   // DMA geometry of this lane inside a 16-row unit: LDS slot = lane (16 bytes each); it holds row
   // lane/4, physical piece lane%4, which stores logical piece (lane%4) ^ ((row/4)%4).
@@ -469,9 +474,10 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
         constexpr int TPB = BM / 64;                                                   // 64-row shrink tiles per row block
         const int gx = (M + 63) / 64, rt = gx - TPB * m_blk < TPB ? gx - TPB * m_blk : TPB;
         k_loop<C, false, BCH, CONV, decltype(tail_loads), true>(smem, d, p.x, p.w, p.a_cat, p.t_ext, p.b_cat, KT, KT1, lane, wm, wn, l32, lh, sw, acc, tacc, tail_loads, ConvGeom{0, 0}, false, false,
-                                                                p.il_cnt + m_blk, rt * (p.ldt / 64), p.il_cnt + (p.M + 127) / 128);
+                                                                p.il_cnt + m_blk, rt * (p.ldt / 64), p.il_cnt + (p.M + 127) / 128, half_last);
       } else {
-        k_loop<C, false, BCH, CONV>(smem, d, p.x, p.w, p.a_cat, p.t_ext, p.b_cat, KT, KT1, lane, wm, wn, l32, lh, sw, acc, tacc, tail_loads, ConvGeom{p.conv_w, p.conv_cin}, (p.dbg & 64) != 0, (p.dbg & 128) != 0);
+        k_loop<C, false, BCH, CONV>(smem, d, p.x, p.w, p.a_cat, p.t_ext, p.b_cat, KT, KT1, lane, wm, wn, l32, lh, sw, acc, tacc, tail_loads, ConvGeom{p.conv_w, p.conv_cin}, (p.dbg & 64) != 0, (p.dbg & 128) != 0,
+                                    nullptr, 0, nullptr, half_last);
       }
     }
     stamp(2);

@@ -79,7 +79,11 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_wide_kernel(const LoraGemmPa
   const int m0 = m_blk * WBM, n0 = n_blk * WBN;
   const int N = p.N, K = p.K;
   const int KT1 = K / 64;
-  const int KT = KT1 + (p.t_ext != nullptr ? p.R / 64 : 0);
+  // only the first r_used rank columns of T / B_cat can be non-zero: stages beyond them are not visited, and of a
+  // last stage that they fill at most half only the first two MFMA steps run
+  const int r_used = (p.r_used > 0 && p.r_used < p.R) ? p.r_used : p.R;
+  const int KT = KT1 + (p.t_ext != nullptr ? (r_used + 63) / 64 : 0);
+  const bool half_last = p.t_ext != nullptr && (r_used & 63) != 0 && (r_used & 63) <= 32;
 
   // DMA: wave w brings x rows 32w .. 32w+31 (4 instructions of 8 rows) and W rows 40w .. 40w+39 (5) of every stage.
   // Lane -> row lane/8 of its 8 rows, physical piece lane%8, which holds logical piece (lane%8) ^ ((stage row / 2) % 8).
@@ -157,22 +161,31 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_wide_kernel(const LoraGemmPa
   __builtin_amdgcn_s_barrier();
   read_frags(0, 0, fa);
   read_frags(0, 1, fb);
-  for (int t = 0; t < KT; ++t) {
+  for (int t = 0; t + 1 < KT; ++t) {   // every stage but the last
     const int st = t & 1;
     mma(fa);                         // step 0
     read_frags(st, 2, fa);
     mma(fb);                         // step 1
     read_frags(st, 3, fb);
     mma(fa);                         // step 2
-    if (t + 1 < KT) {
-      // stage t+1 has landed (this wave's share; the barrier collects everyone's); every read of stage t is done
-      wait_cnt<0, 0>();
-      __builtin_amdgcn_s_barrier();
-      if (t + 2 < KT) issue(t + 2, st);
-      read_frags(st ^ 1, 0, fa);
-    }
+    // stage t+1 has landed (this wave's share; the barrier collects everyone's); every read of stage t is done
+    wait_cnt<0, 0>();
+    __builtin_amdgcn_s_barrier();
+    if (t + 2 < KT) issue(t + 2, st);
+    read_frags(st ^ 1, 0, fa);
     mma(fb);                         // step 3
-    if (t + 1 < KT) read_frags(st ^ 1, 1, fb);
+    read_frags(st ^ 1, 1, fb);
+  }
+  {                                  // the last stage: all four steps, or two when its upper half is zero padding
+    const int st = (KT - 1) & 1;
+    mma(fa);
+    if (!half_last) read_frags(st, 2, fa);
+    mma(fb);
+    if (!half_last) {
+      read_frags(st, 3, fb);
+      mma(fa);
+      mma(fb);
+    }
   }
   __syncthreads();   // the ring is dead: the staging tile reuses it
 

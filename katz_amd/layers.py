@@ -175,7 +175,7 @@ class LoRALinear(nn.Module):
             return ops.lora_linear(x, w, b, residual=residual, geglu=self.geglu)
         if LORA_MODE == "split" and x.dtype == torch.bfloat16 and self.in_features % 64 == 0:
             return ops.lora_linear_split(x, w, b, p.a_cat, p.col_scale, p.b_cat, residual=residual, geglu=self.geglu,
-                                         two_launches=LORA_SHRINK == "separate")
+                                         two_launches=LORA_SHRINK == "separate", r_used=p.r_used)
         return ops.lora_linear(x, w, b, p.a_cat, p.b_cat, p.col_scale, residual=residual, geglu=self.geglu)
 
     def extra_repr(self) -> str:
@@ -517,6 +517,7 @@ class Attention(nn.Module):
                 st["R"] = 0 if packs[0] is None else packs[0].R
                 if st["R"]:
                     R = st["R"]
+                    st["r_used"] = max(p.r_used for p in packs)
                     st["a"] = torch.cat([p.a_cat for p in packs], dim=0).contiguous()
                     st["s"] = torch.cat([p.col_scale for p in packs], dim=0).contiguous()
                     st["b"] = torch.cat([p.b_cat for p in packs], dim=0).contiguous()
@@ -527,7 +528,7 @@ class Attention(nn.Module):
             return None
         if st["R"]:
             y = ops.lora_linear_split(x, st["w"], None, st["a"], st["s"], st["b"], n_split=N,
-                                      two_launches=LORA_SHRINK == "separate")
+                                      two_launches=LORA_SHRINK == "separate", r_used=st["r_used"])
         else:
             y = ops.lora_linear(x, st["w"], None)
         return y.split(N, dim=-1)

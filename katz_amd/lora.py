@@ -54,6 +54,13 @@ class PackedAdapters:
     def R(self) -> int:
         return self.a_cat.shape[0]
 
+    @property
+    def r_used(self) -> int:
+        """Rank columns that can be non-zero (the adapters' ranks side by side), rounded up to the 16 columns of one
+        MFMA step; the columns from there to R are zero padding."""
+        used = max((c + r for _, c, r in self.spans), default=0)
+        return min(self.R, (used + 15) // 16 * 16)
+
 
 def interleave_geglu_rows(t: torch.Tensor) -> torch.Tensor:
     """Reorder the output-feature axis (dim 0) of a GEGLU projection tensor from

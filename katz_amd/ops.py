@@ -121,12 +121,19 @@ def lora_shrink(x: torch.Tensor, a_cat: torch.Tensor, col_scale: torch.Tensor, o
     return out
 
 
+def _r_used_bits(r_used: int, R: int) -> int:
+    if r_used < 0 or r_used > R or r_used % 16:
+        raise ValueError(f"r_used must be a multiple of 16 in [0, {R}], got {r_used}")
+    return r_used // 16
+
+
 def lora_linear_pre(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], t: torch.Tensor,
                     b_cat: torch.Tensor, residual: Optional[torch.Tensor] = None, geglu: bool = False,
-                    tile: int = 0, n_split: int = 0) -> torch.Tensor:
+                    tile: int = 0, n_split: int = 0, r_used: int = 0) -> torch.Tensor:
     """y = x W^T + b + t B_cat^T (+ residual | GEGLU) with t = lora_shrink(x, ...)[:, cols] (a column
     slice of a wider shrink result is fine: only its last axis must be contiguous).  n_split > 0: weight /
-    bias / b_cat stack several layers of n_split rows each and t holds their shrink results side by side."""
+    bias / b_cat stack several layers of n_split rows each and t holds their shrink results side by side.
+    r_used > 0 (a multiple of 16): rank columns >= r_used of t and b_cat are all zero (padding)."""
     lib = _lib.load()
     _req(x, BF16, "x"); _req(weight, BF16, "weight"); _req(b_cat, BF16, "b_cat")
     K = x.shape[-1]
@@ -148,7 +155,7 @@ def lora_linear_pre(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.
     out = torch.empty(tuple(x.shape[:-1]) + (n_out,), dtype=BF16, device=x.device)
     if CALL_LOG is not None:
         CALL_LOG.append(("lora_linear", M, N, K, R, bool(geglu), residual is not None))
-    flags = (1 if geglu else 0) | ((tile & 0xFF) << 8)
+    flags = (1 if geglu else 0) | ((tile & 0xFF) << 8) | (_r_used_bits(r_used, R) << 16)
     rc = lib.kh_lora_linear_pre_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(t), t.stride(0), n_split, _ptr(b_cat),
                                      _ptr(residual), _ptr(out), M, N, K, R, flags, _stream())
     _lib.check(rc, "kh_lora_linear_pre_bf16")
@@ -207,7 +214,7 @@ def split_counters_last(device) -> Optional[torch.Tensor]:
 
 def lora_linear_split(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], a_cat: torch.Tensor,
                       col_scale: torch.Tensor, b_cat: torch.Tensor, residual: Optional[torch.Tensor] = None,
-                      geglu: bool = False, two_launches: bool = False, n_split: int = 0) -> torch.Tensor:
+                      geglu: bool = False, two_launches: bool = False, n_split: int = 0, r_used: int = 0) -> torch.Tensor:
     """y = x W^T + b + ((x A_cat^T) * col_scale) B_cat^T (+ residual | GEGLU): shrink, base GEMM and expand, with
     the shrink inside the GEMM launch where that pays (see kh_lora_linear_split_bf16).  n_split > 0: weight / bias /
     b_cat stack several layers of n_split rows each and a_cat / col_scale stack their A matrices."""
@@ -235,7 +242,7 @@ def lora_linear_split(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torc
     out = torch.empty(tuple(x.shape[:-1]) + (n_out,), dtype=BF16, device=x.device)
     t = torch.empty((M, RT), dtype=BF16, device=x.device)
     cnt = _split_counters(x.device, M)
-    flags = (1 if geglu else 0) | ((1 if two_launches else 0) << 8)
+    flags = (1 if geglu else 0) | ((1 if two_launches else 0) << 8) | (_r_used_bits(r_used, R) << 16)
     if CALL_LOG is not None:   # one entry per kernel launch
         if lib.kh_lora_linear_split_launches(M, N, K, R, n_split, flags) == 2:
             CALL_LOG.append(("lora_shrink", M, K, RT))

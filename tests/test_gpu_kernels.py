@@ -900,3 +900,56 @@ def test_split_counters_after_a_reset_that_was_only_recorded():
         assert torch.equal(o, ref_outs[0])
     assert torch.equal(y_graph, ref_outs[0])
     ops.split_counters_reset(d)
+
+
+@pytest.mark.parametrize("case", [
+    # (M, N, K, R, r_used, geglu, n_split)
+    (2048, 10240, 1280, 128, 96, True, 0),     # 256x320 tiles: the last 64-column stage runs two of its four steps
+    (2048, 1280, 1280, 128, 96, False, 0),     # in-launch form on 128x128 tiles
+    (2048, 3840, 1280, 128, 96, False, 1280),  # stacked q / k / v on 256x128 tiles
+    (2048, 1280, 1280, 128, 48, False, 0),     # a whole stage of padding: one K tile fewer
+    (1100, 1000, 640, 64, 16, False, 0),       # ragged shape on the 4-wave tiles (32-column stages)
+    (8192, 640, 640, 128, 96, False, 0),       # 160-column tiles: the promise is accepted and not used
+], ids=str)
+def test_lora_linear_split_rank_padding_promise(case):
+    """r_used: with the rank columns >= r_used of A_cat / B_cat zero (the padding of the packed adapters), the result is
+    bit-identical with and without the promise, in one launch and in two, and matches the oracle."""
+    from katz_amd import ops
+
+    from katz_amd.lora import interleave_geglu_rows
+
+    M, N, K, R, r_used, geglu, n_split = case
+    say("lora_linear_split r_used", case)
+    d = dev()
+    g = torch.Generator().manual_seed(M + N + K + R + r_used)
+    parts = N // n_split if n_split else 1
+    x, w = randn(g, M, K), randn(g, N, K, std=0.03)
+    A, B = randn(g, parts, R, K, std=0.05), randn(g, N, R, std=0.05)
+    A[:, r_used:] = 0
+    B[:, r_used:] = 0
+    xd, wd, Ad, Bd = x.to(d, BF), w.to(d, BF), A.reshape(parts * R, K).to(d, BF), B.to(d, BF)
+    if geglu:
+        wd, Bd = interleave_geglu_rows(wd), interleave_geglu_rows(Bd)
+    cs = torch.full((parts * R,), 0.7, device=d)
+    outs = {}
+    for two in (False, True):
+        for ru in (0, r_used):
+            ops.split_counters_reset(d)
+            outs[two, ru] = ops.lora_linear_split(xd, wd, None, Ad, cs, Bd, geglu=geglu, two_launches=two,
+                                                  n_split=n_split, r_used=ru)
+    torch.cuda.synchronize()
+    for two in (False, True):
+        assert torch.equal(outs[two, 0], outs[two, r_used]), f"two_launches={two}: the promise changed the result"
+    xf, wf, Af, Bf = (t.float().cpu() for t in (x.to(BF), w.to(BF), A.to(BF), B.to(BF)))
+    step = n_split if n_split else N
+    for j in range(parts):
+        rows = slice(j * step, (j + 1) * step)
+        ref = O.lora_linear(xf, wf[rows], None, [(Af[j], Bf[rows], 0.7)])
+        if geglu:
+            ref = O.geglu(ref)
+            assert_close_rel(outs[False, r_used], ref, REL_BF16, f"r_used {case}")
+        else:
+            assert_close_rel(outs[False, r_used][:, rows], ref, REL_BF16, f"r_used {case} part {j}")
+    with pytest.raises(Exception):
+        ops.lora_linear_split(xd, wd, None, Ad, cs, Bd, geglu=geglu, n_split=n_split, r_used=R + 16)
+    ops.split_counters_reset(d)

@@ -73,6 +73,8 @@ def test_pack_adapters_layout_and_rescale():
     assert pk.R == 64 and pk.a_cat.shape == (64, 16) and pk.b_cat.shape == (64, 64)
     assert torch.equal(pk.a_cat[:4], ads["b"].down) and torch.equal(pk.a_cat[4:12], ads["a"].down)
     assert torch.all(pk.a_cat[12:] == 0) and torch.all(pk.b_cat[:, 12:] == 0)
+    # 12 rank columns in use -> the kernels are promised zeros from column 16 on
+    assert pk.r_used == 16 and torch.all(pk.a_cat[pk.r_used:] == 0) and torch.all(pk.b_cat[:, pk.r_used:] == 0)
     assert torch.allclose(pk.col_scale[:4], torch.tensor(2.0 * 1.0 * 0.5))          # alpha = rank
     assert torch.allclose(pk.col_scale[4:12], torch.tensor(0.5 * 16.0 / 8 * 0.5))   # weight * alpha / rank * scale
     # the packed product equals the sum over adapters
