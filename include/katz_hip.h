@@ -158,6 +158,18 @@ int64_t kh_group_norm_workspace_bytes(int64_t N, int64_t C, int64_t HW, int64_t 
 int kh_group_norm_bf16(const void* x, void* y, const void* gamma, const void* beta, const void* add_nc,
                        float* workspace, int64_t N, int64_t C, int64_t HW, int64_t G, float eps, int activation,
                        int channels_last, void* stream);
+/* kh_group_norm_bf16 for callers that cannot allocate device memory (code under HIP graph capture whose allocator is
+ * out of reach, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference (its op
+ * allocates two tensors per call, group_norm.cu:240-242).  Same arguments without `workspace`; same kernels, same
+ * results bit for bit.  The partial statistics go to a 256 KiB array that the library holds in the memory of every GPU
+ * it runs on until the process ends; shapes whose kh_group_norm_workspace_bytes(...) exceeds 256 KiB (none of the
+ * SDXL UNet / ControlNet norms: they need <= 33 KiB) return KH_ERR_TOO_LARGE.  The call allocates nothing.  All calls
+ * on one GPU share the array: calls that can overlap on one GPU (different streams, several host threads) race; calls
+ * on one stream are ordered.  The first call on a device looks up the array's address (no allocation, no launch);
+ * make that call outside graph capture. */
+int kh_group_norm_static_bf16(const void* x, void* y, const void* gamma, const void* beta, const void* add_nc,
+                              int64_t N, int64_t C, int64_t HW, int64_t G, float eps, int activation,
+                              int channels_last, void* stream);
 /* nn.LayerNorm over the last axis (norm1/2/3 of BasicTransformerBlock,
  * diffusers-hf/src/diffusers/models/attention.py:195,225,253); D % 8 == 0, D <= 2048. */
 int kh_layer_norm_bf16(const void* x, void* y, const void* gamma, const void* beta, int64_t M, int64_t D, float eps,

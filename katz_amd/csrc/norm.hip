@@ -13,6 +13,13 @@
 // eps 1e-5, affine) keeps one row per wave in registers: one read, one write.
 #include "kh_common.h"
 
+#include <mutex>
+
+// Partial statistics of kh_group_norm_static_bf16: one array per GPU, held until the process ends.  In host code this
+// name is only a handle for hipGetSymbolAddress; kernels get the address that call returns.
+constexpr size_t GN_STATIC_WS_BYTES = 256 * 1024;
+static __device__ __align__(256) float scratch[GN_STATIC_WS_BYTES / sizeof(float)];
+
 namespace {
 
 constexpr int GN_THREADS = 256;
@@ -420,6 +427,40 @@ KH_EXPORT int kh_group_norm_bf16(const void* x, void* y, const void* gamma, cons
                          splits, (int)G, (int)Cg, (int)HW, eps);
   }
   KH_RETURN_LAST_ERROR();
+}
+
+// Device address of `scratch` on the current device, resolved once per device.
+static int gn_static_workspace(float** out) {
+  constexpr int MAX_DEV = 64;
+  static std::mutex mu;
+  static float* ptr[MAX_DEV] = {};
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= MAX_DEV) return KH_ERR_UNSUPPORTED;
+  std::lock_guard<std::mutex> lk(mu);
+  if (!ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (!p) return (int)hipErrorInvalidSymbol;
+    ptr[dev] = (float*)p;
+  }
+  *out = ptr[dev];
+  return KH_OK;
+}
+
+KH_EXPORT int kh_group_norm_static_bf16(const void* x, void* y, const void* gamma, const void* beta, const void* add_nc,
+                                        int64_t N, int64_t C, int64_t HW, int64_t G, float eps, int activation,
+                                        int channels_last, void* stream) {
+  const int64_t need = kh_group_norm_workspace_bytes(N, C, HW, G, channels_last);
+  if (need < 0) return (int)need;
+  if ((uint64_t)need > GN_STATIC_WS_BYTES) return KH_ERR_TOO_LARGE;
+  float* ws = nullptr;
+  const int rc = gn_static_workspace(&ws);
+  if (rc != KH_OK) return rc;
+  // The statistics pass overwrites every partial sum the apply pass reads, so nothing has to start at zero.
+  return kh_group_norm_bf16(x, y, gamma, beta, add_nc, ws, N, C, HW, G, eps, activation, channels_last, stream);
 }
 
 KH_EXPORT int kh_layer_norm_bf16(const void* x, void* y, const void* gamma, const void* beta, int64_t M, int64_t D,
