@@ -61,7 +61,8 @@ int kh_profile_end(int32_t* tags, float* ms, int capacity);
  * flags bit 0: GEGLU epilogue -- W/bias/B_cat rows are permuted so that every 64 consecutive rows are
  *   32 value rows followed by their 32 gate rows; y is [M, N/2] = value * gelu_erf(gate)
  *   (GEGLU.forward, diffusers-hf/src/diffusers/models/activations.py:139-149); N % 64 == 0, no residual.
- * flags bits 8..15: tile override for tuning (0 = automatic). */
+ * flags bits 8..15: tile override for tuning (0 = automatic).  Every other bit must be zero (KH_ERR_INVALID_ARG);
+ * in particular the r_used promise of the sibling entry points below (bits 16..23) has no meaning here. */
 int kh_lora_linear_bf16(const void* x, const void* w, const void* bias, const void* a_cat, const void* b_cat,
                         const float* col_scale, const void* residual, void* y, int64_t M, int64_t N, int64_t K,
                         int64_t R, int flags, void* stream);
@@ -102,6 +103,14 @@ int kh_lora_linear_pre_bf16(const void* x, const void* w, const void* bias, cons
 int kh_lora_linear_split_bf16(const void* x, const void* w, const void* bias, const void* a_cat, const float* col_scale,
                               const void* b_cat, void* t_scratch, int32_t* counters, const void* residual, void* y,
                               int64_t M, int64_t N, int64_t K, int64_t R, int64_t n_split, int flags, void* stream);
+/* Bounded waits of kh_lora_linear_split_bf16's in-launch shrink that have run out on the current device since the
+ * process started (or since the last call with clear != 0): writes the number to *count (HOST pointer).  A GEMM workgroup
+ * of that launch waits for the shrink workgroups of the same launch, which have lower workgroup ids and are therefore
+ * dispatched first; the wait gives up after 2^20 polls (about a quarter of a second) and the result of that call is then
+ * undefined.  The flag word in `counters` says so per call but is wiped by the caller's next reset; this count is not.
+ * A non-zero value means results since the last check cannot be trusted.  Blocks until the device's earlier work is
+ * done (a 4-byte copy on the null stream); not under graph capture.  No counterpart in the reference. */
+int kh_lora_split_timeouts(int32_t* count, int clear);
 /* How many kernel launches kh_lora_linear_split_bf16 makes for this shape when counters are given (1 or 2; negative:
  * KH_ERR_*).  No counterpart in the reference; for callers that account per launch (benchmarks). */
 int kh_lora_linear_split_launches(int64_t M, int64_t N, int64_t K, int64_t R, int64_t n_split, int flags);

@@ -14,7 +14,7 @@ struct LoraGemmParams {
   int t_nsplit;            // > 0: W rows come in blocks of t_nsplit rows; block j uses T columns [j*R, (j+1)*R)
   // grouped launch: blockIdx.y selects a row {w, bias, b_cat, t_ext, y} of this device table (null: single layer)
   const uint64_t* grp;
-  int dbg;  // tuning experiments only (flags bits 16..23); 0 in production
+  int dbg;  // always 0 unless the library is built with -DKH_TUNING (kernel experiments; not part of the C ABI)
   const bf16_t* res;       // [M,N] residual added in the epilogue, may be null
   bf16_t* y;
   int M, N, K, R;
@@ -68,3 +68,11 @@ int lora_gemm_wide_launch(LoraGemmParams p, hipStream_t stream);
 
 extern "C" int kh_lora_shrink_bf16(const void* x, const void* a_cat, const float* col_scale, void* t, int64_t M, int64_t K,
                                    int64_t R, void* stream);
+
+// Kernel experiments (timestamps, frozen operands, alternative tile maps) exist only in builds with -DKH_TUNING; the
+// shipped library compiles them out and its entry points reject the flag bits that would select them.
+#ifdef KH_TUNING
+#define KH_DBG(p, bit) (((p).dbg & (bit)) != 0)
+#else
+#define KH_DBG(p, bit) false
+#endif

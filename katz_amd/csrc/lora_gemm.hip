@@ -480,7 +480,11 @@ KH_EXPORT int kh_lora_linear_bf16(const void* x, const void* w, const void* bias
   p.xg_n = p.xr_m = p.xr_n = 0;
   p.sg_start = p.sg_adapter = p.sg_rank = nullptr; p.sg_scale = nullptr; p.sg_mode = 0; p.sg_wstride = 0;
   p.conv_cin = p.conv_h = p.conv_w = p.conv_ho = p.conv_wo = p.conv_stride = 0;
+#ifdef KH_TUNING
   p.dbg = (flags >> 16) & 0xff;
+#else
+  if ((flags >> 16) != 0) return KH_ERR_INVALID_ARG;   // no meaning on this entry point
+#endif
   hipStream_t s = (hipStream_t)stream;
   const int tile_sel = (flags >> 8) & 0xff;  // 0 = automatic
   // K % 32 == 0 (every SDXL layer): the software-pipelined kernel; tile_sel 1/2 force the simple kernel

@@ -15,6 +15,11 @@
 #include "lora_shrink_tile.h"
 #include <type_traits>
 
+// How many bounded waits of the in-launch shrink (kh_lora_linear_split_bf16) have ever run out on this GPU.  Unlike the
+// flag word at the end of a call's counters it is never cleared by the caller's counter resets; read and cleared by
+// kh_lora_split_timeouts.
+static __device__ int kh_split_timeout_count;
+
 namespace {
 
 // K columns per stage (BKP) are a template parameter: 32 (64-byte LDS rows) or 64 (128-byte rows).
@@ -150,7 +155,10 @@ __device__ __forceinline__ void k_loop(char* smem, const Dma<C, SHRINK>& dma, co
         int it = 0;
         while (__hip_atomic_load(il_cnt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < il_target && ++it < (1 << 20))
           __builtin_amdgcn_s_sleep(8);
-        if (it >= (1 << 20)) __hip_atomic_store(il_err, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (it >= (1 << 20)) {
+          __hip_atomic_store(il_err, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_fetch_add(&kh_split_timeout_count, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
       }
     }
 #pragma unroll
@@ -365,10 +373,14 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
   // fragment read: logical piece (2*ks + lh) of row (.. + l32) sits at physical piece ^ ((l32/SWR) % PPR)
   const int sw = (l32 / C::SWR) % C::PPR;
 
-  // tuning only: dbg & 16 turns `res` into a timestamp buffer (8 x int64 per workgroup), no residual
+#ifdef KH_TUNING
+  // tuning builds only: dbg & 16 turns `res` into a timestamp buffer (8 x int64 per workgroup), no residual
   long long* ts = (p.dbg & 16) ? reinterpret_cast<long long*>(const_cast<bf16_t*>(p.res)) + (size_t)bid * 8 : nullptr;
   if (p.dbg & 16) p.res = nullptr;
   auto stamp = [&](int i) { if (ts != nullptr && tid == 0) ts[i] = (long long)__builtin_readcyclecounter(); };
+#else
+  auto stamp = [](int) {};
+#endif
   stamp(0);
   for (int jt = 0; jt < p.n_chunk; ++jt) {
     const int n_tile = chunk * p.n_chunk + jt;
@@ -384,7 +396,7 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
       for (int i = 0; i < D::XI; ++i, ++q) {
         const int r = (wave * D::XI + i) * C::UROWS + u_row;  // row inside the x tile
         const int pc = ((lane % C::PPR) ^ ((r / C::SWR) % C::PPR)) * 8;
-        int row = ((p.dbg & 32) ? 0 : m0) + r; row = row < M ? row : M - 1;
+        int row = (KH_DBG(p, 32) ? 0 : m0) + r; row = row < M ? row : M - 1;
         if constexpr (CONV) {
           // output pixel -> the input pixel above-left of its 3x3 window, and which taps are inside the image
           const int wo = row % p.conv_wo, t2 = row / p.conv_wo, ho = t2 % p.conv_ho, nb = t2 / p.conv_ho;
@@ -407,7 +419,7 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
       for (int i = 0; i < D::WI; ++i, ++q) {
         const int r = (wave * D::WI + i) * C::UROWS + u_row;
         const int pc = ((lane % C::PPR) ^ ((r / C::SWR) % C::PPR)) * 8;
-        int row = ((p.dbg & 32) ? 0 : n0) + r; row = row < N ? row : N - 1;
+        int row = (KH_DBG(p, 32) ? 0 : n0) + r; row = row < N ? row : N - 1;
         d.off[q] = (long)row * K + pc;
         d.off2[q] = row * p.R + pc;
         d.dst[q] = C::SW_OFF + (wave * D::WI + i) * 1024;
@@ -476,7 +488,7 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
         k_loop<C, false, BCH, CONV, decltype(tail_loads), true>(smem, d, p.x, p.w, p.a_cat, p.t_ext, p.b_cat, KT, KT1, lane, wm, wn, l32, lh, sw, acc, tacc, tail_loads, ConvGeom{0, 0}, false, false,
                                                                 p.il_cnt + m_blk, rt * (p.ldt / 64), p.il_cnt + (p.M + 127) / 128, half_last);
       } else {
-        k_loop<C, false, BCH, CONV>(smem, d, p.x, p.w, p.a_cat, p.t_ext, p.b_cat, KT, KT1, lane, wm, wn, l32, lh, sw, acc, tacc, tail_loads, ConvGeom{p.conv_w, p.conv_cin}, (p.dbg & 64) != 0, (p.dbg & 128) != 0,
+        k_loop<C, false, BCH, CONV>(smem, d, p.x, p.w, p.a_cat, p.t_ext, p.b_cat, KT, KT1, lane, wm, wn, l32, lh, sw, acc, tacc, tail_loads, ConvGeom{p.conv_w, p.conv_cin}, KH_DBG(p, 64), KH_DBG(p, 128),
                                     nullptr, 0, nullptr, half_last);
       }
     }
@@ -612,7 +624,7 @@ int launch_pcfg(LoraGemmParams p, hipStream_t stream, int n_groups = 1) {
   if (hipError_t e = kh_allow_lds<lora_gemm_pipe_kernel<C, CONV>>((int)C::LDS_BYTES); e != hipSuccess) return (int)e;
   unsigned grid = (unsigned)(p.m_tiles * p.n_chunks);
   p.xg_n = p.xr_m = p.xr_n = 0;
-  if (C::NRT == 0 && (p.dbg & 8) == 0) {
+  if (C::NRT == 0 && !KH_DBG(p, 8)) {
     // choose the XCD grid whose per-XCD block touches the fewest operand rows, padding counted as cost
     double best = 0;
     for (int gm = 1; gm <= 8; gm *= 2) {
@@ -672,6 +684,21 @@ static int il_form(const LoraGemmParams& p) {
 }
 
 bool lora_gemm_pipe_il_ok(const LoraGemmParams& p) { return il_form(p) != 0; }
+
+// See include/katz_hip.h.  Synchronous (a blocking 4-byte copy on the null stream of the current device).
+KH_EXPORT int kh_lora_split_timeouts(int32_t* count, int clear) {
+  if (!count) return KH_ERR_INVALID_ARG;
+  int v = 0;
+  hipError_t e = hipMemcpyFromSymbol(&v, HIP_SYMBOL(kh_split_timeout_count), sizeof(int), 0, hipMemcpyDeviceToHost);
+  if (e != hipSuccess) return (int)e;
+  *count = v;
+  if (clear && v != 0) {
+    const int zero = 0;
+    e = hipMemcpyToSymbol(HIP_SYMBOL(kh_split_timeout_count), &zero, sizeof(int), 0, hipMemcpyHostToDevice);
+    if (e != hipSuccess) return (int)e;
+  }
+  return KH_OK;
+}
 
 template <class C>
 static int launch_il(const LoraGemmParams& pin, hipStream_t stream) {

@@ -73,3 +73,10 @@ class GraphedUNetStep:
             self.mid.copy_(mid_block_additional_residual)
         self.graph.replay()
         return self.out
+
+    def check(self) -> None:
+        """Wait for the replays issued so far and raise ops.SplitTimeoutError if a bounded wait inside one of the
+        step's LoRA launches ran out (the output of such a step is not trustworthy)."""
+        from . import ops
+
+        ops.check_split_timeouts(self.sample.device)

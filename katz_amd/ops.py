@@ -50,7 +50,6 @@ def lora_linear(
     geglu: bool = False,
     tile: int = 0,
     out: Optional[torch.Tensor] = None,
-    dbg: int = 0,
 ) -> torch.Tensor:
     """y = x W^T + b + ((x A_cat^T) * col_scale) B_cat^T (+ residual); bf16 or fp32 by x.dtype.
 
@@ -89,7 +88,7 @@ def lora_linear(
     if CALL_LOG is not None:
         CALL_LOG.append(("lora_linear", M, N, K, R, bool(geglu), residual is not None))
     if dt == BF16:
-        flags = (1 if geglu else 0) | ((tile & 0xFF) << 8) | ((dbg & 0xFF) << 16)
+        flags = (1 if geglu else 0) | ((tile & 0xFF) << 8)
         rc = lib.kh_lora_linear_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(a_cat), _ptr(b_cat), _ptr(col_scale),
                                      _ptr(residual), _ptr(out), M, N, K, R, flags, _stream())
     elif dt == torch.float32:
@@ -188,11 +187,39 @@ def _arena(device):
 
 
 def split_counters_reset(device) -> None:
-    """Clear every counter of the device's arena (one fill kernel; nothing while no counter has ever been handed out)."""
+    """Clear every counter of the device's arena with one fill kernel.  Outside graph capture the fill is skipped
+    while no counter has ever been handed out; under capture it is always recorded, because by the time the graph is
+    replayed other forwards may have dirtied the arena."""
     st = _arena(device)
-    if st[3]:
+    if st[3] or torch.cuda.is_current_stream_capturing():
         st[0].zero_()
     st[1] = 0
+
+
+class SplitTimeoutError(_lib.KatzHipError):
+    """A bounded wait inside kh_lora_linear_split_bf16 ran out: results since the last check are not trustworthy."""
+
+
+def split_timeouts(device=None, clear: bool = False) -> int:
+    """How many in-launch waits of lora_linear_split have run out on `device` since the last clearing call.
+    Synchronises with the device."""
+    import ctypes
+
+    lib = _lib.load()
+    n = ctypes.c_int32(0)
+    with torch.cuda.device(device if device is not None else torch.cuda.current_device()):
+        rc = lib.kh_lora_split_timeouts(ctypes.byref(n), 1 if clear else 0)
+    _lib.check(rc, "kh_lora_split_timeouts")
+    return int(n.value)
+
+
+def check_split_timeouts(device=None) -> None:
+    """Raise SplitTimeoutError if any in-launch wait has run out since the last check (and clear the count).  Call it
+    where the host synchronises anyway: after a denoise loop, after a benchmark's timed region, in tests."""
+    n = split_timeouts(device, clear=True)
+    if n:
+        raise SplitTimeoutError(f"{n} in-launch shrink wait(s) of kh_lora_linear_split_bf16 timed out on {device}: "
+                                "the LoRA linears of the affected steps read an incomplete shrink result")
 
 
 def _split_counters(device, M: int) -> torch.Tensor:

@@ -104,12 +104,14 @@ class EulerDiscreteScheduler:
 
 
 def denoise_loop(model: Callable[[torch.Tensor, torch.Tensor], torch.Tensor], scheduler: EulerDiscreteScheduler,
-                 latents: torch.Tensor, guidance_scale: float, latents_fp32: bool = False) -> torch.Tensor:
+                 latents: torch.Tensor, guidance_scale: float, latents_fp32: bool = False,
+                 check: bool = True) -> torch.Tensor:
     """The guided denoise loop of the reference (pipeline_controlnet_sd_xl_katz.py:1509-1658) around
     model(latent_model_input [2B,...] bf16, t) -> noise_pred [2B,...] bf16, with guidance, the Euler update and
     the next step's input scaling fused into one kernel per step.  `latents` must already be scaled by
     init_noise_sigma (prepare_latents, :872-887).  latents_fp32 keeps the latents in fp32 between steps
-    instead of the model dtype the reference casts them to."""
+    instead of the model dtype the reference casts them to.  check: wait for the loop at its end and raise if a
+    bounded in-launch wait of the LoRA linears ran out on the way (ops.check_split_timeouts)."""
     dev = latents.device
     coef = scheduler.coef_table(dev)
     lat = latents.to(torch.float32 if latents_fp32 else torch.bfloat16).contiguous()
@@ -123,4 +125,6 @@ def denoise_loop(model: Callable[[torch.Tensor, torch.Tensor], torch.Tensor], sc
         ops.cfg_euler_step(noise_pred.contiguous(), lat, coef[i], guidance_scale, latents_out=lat_out, model_input_next=nxt)
         lat, lat_out = lat_out, lat
         model_input, nxt = nxt, model_input
+    if check and dev.type == "cuda":
+        ops.check_split_timeouts(dev)
     return lat

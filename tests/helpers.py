@@ -62,3 +62,69 @@ def cosine(a, b):
     a = a.detach().float().flatten().cpu()
     b = b.detach().float().flatten().cpu()
     return (torch.dot(a, b) / (a.norm() * b.norm()).clamp_min(1e-30)).item()
+
+
+# ---- deterministic tensors for the committed reference fixtures -----------------------------------------------
+# tests/golden/make_unet_tiny_fixture.py (run once, in the build container, against the reference's own modules) and
+# the tests that read its output must hold identical weights and inputs without storing them: every tensor is a
+# function of its name and shape only.
+
+def det_tensor(name: str, shape, std: float = 1.0, mean: float = 0.0) -> torch.Tensor:
+    """fp32 tensor of the given shape, N(mean, std), from a numpy PCG64 stream seeded by crc32(name)."""
+    import zlib
+
+    import numpy as np
+
+    rng = np.random.Generator(np.random.PCG64(zlib.crc32(name.encode())))
+    n = 1
+    for s in shape:
+        n *= int(s)
+    a = rng.standard_normal(n).astype(np.float32) * np.float32(std) + np.float32(mean)
+    return torch.from_numpy(a).reshape(tuple(int(s) for s in shape))
+
+
+def det_state_dict(shapes, prefix: str = ""):
+    """{key: tensor} for a {key: shape} map: weights of >= 2 dims ~ N(0, 1/fan_in), norm scales ~ 1 + 0.1 N(0,1), every
+    other 1-D tensor (biases) ~ 0.1 N(0,1).  A norm scale is a 1-D `weight` (GroupNorm / LayerNorm)."""
+    out = {}
+    for k, shape in shapes.items():
+        shape = tuple(shape)
+        if len(shape) >= 2:
+            fan_in = 1
+            for s in shape[1:]:
+                fan_in *= s
+            out[k] = det_tensor(prefix + k, shape, std=fan_in ** -0.5)
+        elif k.endswith("weight"):
+            out[k] = det_tensor(prefix + k, shape, std=0.1, mean=1.0)
+        else:
+            out[k] = det_tensor(prefix + k, shape, std=0.1)
+    return out
+
+
+FIXTURE_UNET = dict(block_out_channels=(64, 128, 256), transformer_layers_per_block=(1, 2, 3),
+                    num_attention_heads=(1, 2, 4), cross_attention_dim=128, addition_time_embed_dim=32,
+                    projection_class_embeddings_input_dim=64 + 6 * 32)
+
+
+def fixture_unet_inputs(latent: int):
+    """Inputs of the reference-fixture runs at a `latent` x `latent` resolution (batch 2, 7 context tokens)."""
+    B = 2
+    time_ids = torch.tensor([[8.0 * latent, 8.0 * latent, 0, 0, 8.0 * latent, 8.0 * latent],
+                             [8.0 * latent, 6.0 * latent, 4, 8, 8.0 * latent, 8.0 * latent]])
+    return dict(sample=det_tensor(f"in.sample.{latent}", (B, 4, latent, latent)),
+                timestep=500.0,
+                encoder_hidden_states=det_tensor("in.context", (B, 7, 128)),
+                text_embeds=det_tensor("in.text_embeds", (B, 64)),
+                time_ids=time_ids,
+                controlnet_cond=det_tensor(f"in.cond.{latent}", (B, 3, 8 * latent, 8 * latent), std=0.3, mean=0.5))
+
+
+def fixture_residuals(latent: int, std: float = 0.3):
+    """9 down residuals + 1 mid residual with the skip shapes of the fixture UNet (unet_2d_condition.py:539-563 scaled)."""
+    c = FIXTURE_UNET["block_out_channels"]
+    H = latent
+    shapes = [(c[0], H), (c[0], H), (c[0], H), (c[0], H // 2), (c[1], H // 2), (c[1], H // 2), (c[1], H // 4),
+              (c[2], H // 4), (c[2], H // 4)]
+    down = [det_tensor(f"in.res.{i}.{latent}", (2, ch, h, h), std=std) for i, (ch, h) in enumerate(shapes)]
+    mid = det_tensor(f"in.res.mid.{latent}", (2, c[2], H // 4, H // 4), std=std)
+    return down, mid

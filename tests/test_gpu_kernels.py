@@ -857,6 +857,41 @@ def test_lora_linear_split(case):
     assert differing < 5e-3, differing
 
 
+def test_split_time_out_is_reported_and_survives_the_counter_reset():
+    """A bounded in-launch wait that runs out must not pass silently.  Forced from the host: the row-block counters
+    start at -1000 instead of zero, so the arrivals of the shrink workgroups never reach the target; every GEMM
+    workgroup gives up after its 2^20 polls (about a quarter of a second) and the kernel ends normally.  The call's flag
+    word says so, the per-device count says so after the arena has been reset, and check_split_timeouts raises once."""
+    from katz_amd import _lib, ops
+
+    say("lora_linear_split time-out")
+    d = dev()
+    M, N, K, R = 2048, 1280, 1280, 64
+    lib = _lib.load()
+    assert lib.kh_lora_linear_split_launches(M, N, K, R, 0, 0) == 1    # the shrink runs inside the launch
+    g = torch.Generator().manual_seed(5)
+    x, w = randn(g, M, K).to(d, BF), randn(g, N, K, std=0.03).to(d, BF)
+    A, B = randn(g, R, K, std=0.05).to(d, BF), randn(g, N, R, std=0.05).to(d, BF)
+    cs = torch.ones(R, device=d)
+    t = torch.empty(M, R, dtype=BF, device=d)
+    y = torch.empty(M, N, dtype=BF, device=d)
+    torch.cuda.synchronize()
+    ops.split_timeouts(d, clear=True)
+    cnt = torch.full(((M + 127) // 128 + 1,), -1000, dtype=torch.int32, device=d)
+    cnt[-1] = 0
+    rc = lib.kh_lora_linear_split_bf16(x.data_ptr(), w.data_ptr(), None, A.data_ptr(), cs.data_ptr(), B.data_ptr(),
+                                       t.data_ptr(), cnt.data_ptr(), None, y.data_ptr(), M, N, K, R, 0, 0,
+                                       torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert int(cnt[-1]) == 1
+    ops.split_counters_reset(d)                       # the next step's reset does not wipe the evidence
+    assert ops.split_timeouts(d) >= 1
+    with pytest.raises(ops.SplitTimeoutError):
+        ops.check_split_timeouts(d)
+    ops.check_split_timeouts(d)                       # cleared by the raising check
+
+
 def test_split_counters_after_a_reset_that_was_only_recorded():
     """A reset recorded into a HIP graph does not run at capture time.  Counters that eager calls dirtied before the
     capture must still be clear when later eager calls reach them: every slice shows exactly its own arrivals (a slice

@@ -70,3 +70,31 @@ def test_conditioning_image_enters_after_conv_in():
     e = cn.controlnet_cond_embedding(cond)
     assert e.shape == (2, cfg.block_out_channels[0], 16, 16)
     assert torch.allclose(d1[0], cn.controlnet_down_blocks[0](cn.conv_in(sample) + e), atol=1e-6)
+
+
+def test_controlnet_forward_matches_reference_fixture():
+    """oracle.controlnet.ControlNetModel.forward == the reference's ControlNetModel.forward (controlnet.py:687-847,
+    built with from_unet :432-506) on identical weights (random, non-zero zero-convs and conditioning embedding) and
+    inputs, <= 1e-4; default conditioning_scale 0.5 (:693) and 1.0.  Fixture: tests/golden/make_unet_tiny_fixture.py."""
+    from pathlib import Path
+
+    from safetensors.torch import load_file
+
+    from helpers import FIXTURE_UNET, det_state_dict, fixture_unet_inputs
+
+    gold = load_file(str(Path(__file__).resolve().parent / "golden" / "unet_tiny_reference.safetensors"))
+    cn = ControlNetModel(UNetConfig(**FIXTURE_UNET)).eval()
+    cn.load_state_dict(det_state_dict({k: v.shape for k, v in cn.state_dict().items()}, "controlnet."))
+    i = fixture_unet_inputs(8)
+    added = dict(text_embeds=i["text_embeds"], time_ids=i["time_ids"])
+    with torch.no_grad():
+        down, mid = cn(i["sample"], i["timestep"], i["encoder_hidden_states"], i["controlnet_cond"],
+                       added_cond_kwargs=added)
+        _, mid1 = cn(i["sample"], i["timestep"], i["encoder_hidden_states"], i["controlnet_cond"], 1.0, added)
+    assert len(down) == 9
+    for j, d in enumerate(down):
+        ref = gold[f"controlnet.down.{j}"]
+        assert d.shape == ref.shape
+        assert (d - ref).abs().max().item() <= 1e-4 * max(1.0, ref.abs().max().item()), j
+    assert (mid - gold["controlnet.mid"]).abs().max().item() <= 1e-4 * gold["controlnet.mid"].abs().max().item()
+    assert (mid1 - gold["controlnet.mid_scale1"]).abs().max().item() <= 1e-4 * gold["controlnet.mid_scale1"].abs().max().item()

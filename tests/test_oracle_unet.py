@@ -66,3 +66,65 @@ def test_tiny_unet_forward_shapes_and_skip_order():
     assert y0.shape == (B, 4, H, H)
     assert torch.equal(y0, y1)
     assert not torch.allclose(y0, y2)
+
+
+# ---- numerical pin of the wiring: the reference's own UNet2DConditionModel on a tiny SDXL-topology configuration ----
+FIXTURE = Path(__file__).resolve().parent / "golden" / "unet_tiny_reference.safetensors"
+
+
+def _fixture_unet():
+    from helpers import FIXTURE_UNET, det_state_dict
+
+    m = UNet2DConditionModel(UNetConfig(**FIXTURE_UNET)).eval()
+    m.load_state_dict(det_state_dict({k: v.shape for k, v in m.state_dict().items()}, "unet."))
+    return m
+
+
+def test_unet_forward_matches_reference_fixture():
+    """oracle.unet_sdxl.UNet2DConditionModel.forward == the reference's forward (unet_2d_condition.py:1955-2075,
+    residual run through :1127-1341) on identical weights and inputs, <= 1e-4.  The fixture was written by
+    tests/golden/make_unet_tiny_fixture.py from the reference's modules; depths (1, 2, 3), two different time_ids
+    rows and three distinct same-shape skips make transposed wiring (skip order, text/time concat order, embedding
+    flip / shift, emb + aug_emb) change the output."""
+    from safetensors.torch import load_file
+
+    from helpers import fixture_residuals, fixture_unet_inputs
+
+    gold = load_file(str(FIXTURE))
+    m = _fixture_unet()
+    i = fixture_unet_inputs(16)
+    added = dict(text_embeds=i["text_embeds"], time_ids=i["time_ids"])
+    down, mid = fixture_residuals(16)
+    with torch.no_grad():
+        y0 = m(i["sample"], i["timestep"], i["encoder_hidden_states"], added)
+        y1 = m(i["sample"], i["timestep"], i["encoder_hidden_states"], added, down, mid)
+        y_mid_only = m(i["sample"], i["timestep"], i["encoder_hidden_states"], added, None, mid)
+    assert (y0 - gold["unet.out_plain"]).abs().max().item() <= 1e-4
+    assert (y1 - gold["unet.out_residuals"]).abs().max().item() <= 1e-4
+    # the residuals matter at this tolerance, so the comparison above is not vacuous
+    assert (gold["unet.out_plain"] - gold["unet.out_residuals"]).abs().max().item() > 1e-2
+    # the reference's eager forward (graphs off) applies the mid residual only (unet_2d_condition.py:1886-1898)
+    assert (y_mid_only - gold["unet.out_residuals_eager"]).abs().max().item() <= 1e-4
+
+
+def test_unet_fixture_detects_wiring_mistakes():
+    """Each plausible wiring mistake moves the output by far more than the 1e-4 tolerance of the pin."""
+    from safetensors.torch import load_file
+
+    from helpers import fixture_residuals, fixture_unet_inputs
+
+    gold = load_file(str(FIXTURE))
+    m = _fixture_unet()
+    i = fixture_unet_inputs(16)
+    added = dict(text_embeds=i["text_embeds"], time_ids=i["time_ids"])
+    down, mid = fixture_residuals(16)
+    with torch.no_grad():
+        swapped = list(down)
+        swapped[1], swapped[2] = swapped[2], swapped[1]          # two of the three same-shape skips
+        y = m(i["sample"], i["timestep"], i["encoder_hidden_states"], added, swapped, mid)
+        assert (y - gold["unet.out_residuals"]).abs().max().item() > 1e-2
+        ids = i["time_ids"][:, [1, 0, 2, 3, 4, 5]]               # order of the size conditioning
+        y = m(i["sample"], i["timestep"], i["encoder_hidden_states"], dict(text_embeds=i["text_embeds"], time_ids=ids))
+        assert (y - gold["unet.out_plain"]).abs().max().item() > 1e-3
+        y = m(i["sample"], 499.0, i["encoder_hidden_states"], added)
+        assert (y - gold["unet.out_plain"]).abs().max().item() > 1e-4
