@@ -9,9 +9,11 @@ residual set (9 down + 1 mid, ~N(0,0.1)).  A step = one HIP-graph replay of the 
 resident in HBM.
 
 Prints ONE JSON line: ms per step (value), the adapter-free step beside it, a `roofline` object for the
-dominant kernel (the fused LoRA GEMM: algorithmic FLOPs of all its launches in a step / the sum of their
-durations, each launch timed with its own HIP event pair on the launch stream) and a `cpu_baseline`
-object (the fp32 CPU oracle timed on a bounded sample and scaled by FLOPs).
+dominant kernel (the fused LoRA GEMM: algorithmic FLOPs of all its launches in a step, counted on the adapters'
+true ranks, / the sum of their durations, each launch timed with its own HIP event pair on the launch stream),
+`rooflines` for the other kernels of the path (attention and convolution against the MFMA peak; GroupNorm,
+LayerNorm, residual injection and the segmented shrink / expand against the HBM peak) and a `cpu_baseline`
+object (the fp32 CPU oracle timed on a bounded sample and extrapolated by FLOPs).
 """
 from __future__ import annotations
 
@@ -43,7 +45,10 @@ def build_product(device, seed=0):
     return unet.to_runtime(device, torch.bfloat16)
 
 
-def add_random_loras(unet, device, specs=(("r64", 64, 0.8), ("r32", 32, 0.6)), seed=10):
+LORA_SPECS = (("r64", 64, 0.8), ("r32", 32, 0.6))   # (adapter name, rank, weight): BASELINE.json configs[2]
+
+
+def add_random_loras(unet, device, specs=LORA_SPECS, seed=10):
     import torch
 
     g = torch.Generator(device=device).manual_seed(seed)
@@ -117,6 +122,77 @@ def instrumented_step(unet, inputs):
     return launches, log, conv_flops[0]
 
 
+def host_cores():
+    """Threads for the CPU baseline: the share of the host this job has been given (OMP_NUM_THREADS, which the GPU
+    boxes set to their per-GPU share of cores), never more than the CPUs visible."""
+    n = os.cpu_count() or 1
+    try:
+        n = min(n, int(os.environ.get("OMP_NUM_THREADS", n)))
+    except ValueError:
+        pass
+    return max(n, 1)
+
+
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def sgmv_rooflines(dev):
+    """Segmented shrink / expand (BASELINE.json configs[3]: 8 requests, one adapter each, ranks from {8..128}) at the
+    two SDXL widths, timed per launch with HIP events; algorithmic bytes: shrink 2(sum T K + sum r K + sum T r), expand
+    2(sum T r + sum r N + 2 sum T N) (y is read, updated and written)."""
+    import torch
+    from katz_amd import ops
+
+    bf = torch.bfloat16
+    g = torch.Generator(device=dev).manual_seed(2)
+    rn = lambda *s, std=1.0: (torch.randn(*s, device=dev, generator=g) * std).to(bf)
+    ranks = [64, 8, 128, 32, 16, 64, 128, 32]
+    rows = {"shrink": [], "expand": []}
+    for T, K, N in ((4096, 640, 640), (1024, 1280, 1280), (77, 2048, 1280)):
+        RP = 128
+        x = rn(8 * T, K)
+        a_all = torch.zeros(8, RP, K, device=dev, dtype=bf)
+        b_all = torch.zeros(8, N, RP, device=dev, dtype=bf)
+        for i, r in enumerate(ranks):
+            a_all[i, :r] = rn(r, K, std=0.02)
+            b_all[i, :, :r] = rn(N, r, std=0.02)
+        ss = torch.arange(0, 9 * T, T, dtype=torch.int32, device=dev)
+        sa = torch.arange(8, dtype=torch.int32, device=dev)
+        rp = torch.tensor([(r + 31) // 32 * 32 for r in ranks], dtype=torch.int32, device=dev)
+        sc = torch.full((8,), 0.7, device=dev)
+        y = rn(8 * T, N)
+        tb = torch.zeros(8 * T, RP, device=dev, dtype=bf)
+        sr = float(sum(ranks))
+        for _ in range(3):
+            ops.sgmv_shrink(x, a_all, ss, sa, rp, T, out=tb); ops.sgmv_expand_(y, tb, b_all, ss, sa, rp, sc, T)
+        torch.cuda.synchronize()
+        ops.profile_begin()
+        for _ in range(10):
+            ops.sgmv_shrink(x, a_all, ss, sa, rp, T, out=tb); ops.sgmv_expand_(y, tb, b_all, ss, sa, rp, sc, T)
+        ls = ops.profile_end()
+        assert len(ls) == 20, len(ls)    # one launch per call
+        for kind, nbytes in (("shrink", 2.0 * (8 * T * K + sr * K + T * sr)), ("expand", 2.0 * (T * sr + sr * N + 2 * 8 * T * N))):
+            ds = sorted(d for i, (_, d) in enumerate(ls) if (i % 2 == 0) == (kind == "shrink"))   # launches alternate
+            med = ds[len(ds) // 2]
+            rows[kind].append({"shape": f"8 requests x {T} rows, K{K} N{N}, ranks {ranks}", "avg_us": round(med * 1e3, 2),
+                               "achieved": round(nbytes / (med * 1e-3) / 1e9, 1),
+                               "frac": round(nbytes / (med * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)})
+    out = []
+    for kind in ("shrink", "expand"):
+        best = rows[kind][0]
+        out.append({"kernel": f"segmented multi-adapter {kind} (kh_sgmv_{kind}_bf16), median of 10 launches per shape",
+                    "bound": "hbm", "achieved": best["achieved"], "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": best["frac"],
+                    "by_shape": rows[kind]})
+    return out
+
+
 def cpu_baseline(cores):
     """fp32 CPU oracle on a bounded sample: the UNet mid block (resnet, 10 transformer blocks with both
     LoRAs, resnet; batch 2, 32x32 latent) -- scaled to a whole step by algorithmic FLOPs."""
@@ -156,9 +232,24 @@ def cpu_baseline(cores):
     return ts[len(ts) // 2], flops
 
 
-# HBM-side bytes of the largest LoRA GEMM launch, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on
-# `bench.py --kernel-probe` and calibrated against a copy of known size (summary under profiles/)
-GEMM_TRAFFIC_BYTES = 96.5e6
+PROFILE_SUMMARY = ROOT / "profiles" / "kernels_at_baseline_shapes_mfma_busy_and_hbm_traffic.txt"
+
+
+def traffic_from_profiles(kernel_prefix):
+    """HBM-side bytes per launch (read + written) of the first row of the committed counter summary whose name starts
+    with `kernel_prefix`, with the row it came from; (None, reason) when the summary or the row is missing.  The
+    summary is written from two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE) of `bench.py --kernel-probe`, each
+    calibrated against a copy of known size; it is a record of that run, not a measurement of this one."""
+    import re
+
+    if not PROFILE_SUMMARY.exists():
+        return None, f"{PROFILE_SUMMARY.name} not found"
+    for line in PROFILE_SUMMARY.read_text().splitlines():
+        if line.startswith(kernel_prefix):
+            m = re.search(r"hbm rd\s+([0-9.]+)\s+wr\s+([0-9.]+)\s+MB", line)
+            if m:
+                return (float(m.group(1)) + float(m.group(2))) * 1e6, " ".join(line.split())
+    return None, f"no row {kernel_prefix!r} in {PROFILE_SUMMARY.name}"
 
 
 def kernel_probe():
@@ -295,8 +386,13 @@ def main():
         del g1
         launches, log, conv_flops = instrumented_step(unet, inputs)
 
-    # per-kernel accounting of the instrumented step
-    by_kernel = {}
+    from katz_amd import ops
+
+    ops.check_split_timeouts(dev)   # a bounded in-launch wait that ran out would make every number below meaningless
+
+    # ---- per-kernel accounting of the instrumented step --------------------------------------------------------
+    true_rank = sum(r for _, r, _ in LORA_SPECS)       # 64 + 32: FLOPs are counted on the adapters' ranks, not on the
+    by_kernel = {}                                     # 128 columns they are padded to (the kernels skip the padding)
     for name, dur in launches:
         e = by_kernel.setdefault(name, [0, 0.0])
         e[0] += 1
@@ -314,25 +410,71 @@ def main():
         e = shrink_shapes.setdefault(tuple(c[1:4]), [0, 0.0])
         e[0] += 1
         e[1] += d
-    shrink_rows = [{"M": M, "K": K, "R": R, "launches": cnt, "avg_us": round(tot / cnt, 2)}
+    shrink_rows = [{"M": M, "K": K, "R_padded": R, "launches": cnt, "avg_us": round(tot / cnt, 2)}
                    for (M, K, R), (cnt, tot) in sorted(shrink_shapes.items(), key=lambda kv: -kv[1][1])]
     n_layers = lambda c: c[5] if c[0] == "lora_linear_grouped" else 1
-    gemm_flops = sum(n_layers(c) * lora_linear_flops(c[1], c[2], c[3], c[4]) for c in gemm_calls)
+    rank_of = lambda c: true_rank if c[4] > 0 else 0
+    gemm_flops = sum(n_layers(c) * lora_linear_flops(c[1], c[2], c[3], rank_of(c)) for c in gemm_calls)
     gemm_total_ms = sum(gemm_ms) + shrink_ms
     attn_flops = sum(4.0 * c[1] * c[2] * c[3] * c[4] * c[5] for c in log if c[0] == "attention")
     step_flops = gemm_flops + attn_flops + conv_flops
     achieved_tf = gemm_flops / (gemm_total_ms * 1e-3) / 1e12
-    # the largest fused-LoRA GEMM shape class, for the headline "fused LoRA-GEMM TFLOP/s"
     by_shape = {}
     for c, d in zip(gemm_calls, gemm_ms):
-        e = by_shape.setdefault(tuple(c[1:5]) + (n_layers(c),), [0, 0.0])
+        e = by_shape.setdefault(tuple(c[1:4]) + (rank_of(c), n_layers(c)), [0, 0.0])
         e[0] += 1
         e[1] += d
     shape_rows = []
     for (M, N, K, R, G), (cnt, tot) in sorted(by_shape.items(), key=lambda kv: -kv[1][1]):
         fl = G * lora_linear_flops(M, N, K, R)
-        shape_rows.append({"M": M, "N": N, "K": K, "R": R, "layers_per_launch": G, "launches": cnt, "avg_us": round(tot / cnt * 1e3, 2),
-                           "tflops": round(fl / (tot / cnt * 1e-3) / 1e12, 1)})
+        tf = fl / (tot / cnt * 1e-3) / 1e12
+        shape_rows.append({"M": M, "N": N, "K": K, "rank": R, "layers_per_launch": G, "launches": cnt,
+                           "avg_us": round(tot / cnt * 1e3, 2), "ms_per_step": round(tot, 3), "tflops": round(tf, 1),
+                           "frac": round(tf / PEAK_BF16_TFLOPS, 3)})
+    traffic, traffic_src = traffic_from_profiles("lora_gemm M2048 K1280 N10240")
+
+    # ---- the other kernels of the path against their own rooflines ----------------------------------------------
+    def pair(kernel_names, call_name, work_of):
+        """(launch durations, algorithmic work) of one kernel family, matched in launch order with the call log."""
+        durs = [d for n, d in launches if n in kernel_names]
+        calls = [c for c in log if c[0] == call_name]
+        per_call = len(kernel_names)
+        assert len(durs) == per_call * len(calls), (call_name, len(durs), len(calls))
+        return [(sum(durs[i * per_call:(i + 1) * per_call]), work_of(c), c) for i, c in enumerate(calls)]
+
+    def roofline_rows(name, bound, rows, key_of):
+        peak, unit, scale = (PEAK_BF16_TFLOPS, "TFLOP/s", 1e12) if bound == "mfma" else (PEAK_HBM_GBS, "GB/s", 1e9)
+        tot_ms = sum(r[0] for r in rows)
+        tot_work = sum(r[1] for r in rows)
+        groups = {}
+        for ms_, work, c in rows:
+            e = groups.setdefault(key_of(c), [0, 0.0, 0.0])
+            e[0] += 1; e[1] += ms_; e[2] += work
+        ach = tot_work / (tot_ms * 1e-3) / scale if tot_ms > 0 else 0.0
+        return {"kernel": name, "bound": bound, "achieved": round(ach, 1), "peak": peak, "unit": unit,
+                "frac": round(ach / peak, 4), "launches_per_step": len(rows), "ms_per_step": round(tot_ms, 3),
+                "by_shape": [{"shape": k, "launches": n, "avg_us": round(ms_ / n * 1e3, 2),
+                              "achieved": round(w / (ms_ * 1e-3) / scale, 1), "frac": round(w / (ms_ * 1e-3) / scale / peak, 4)}
+                             for k, (n, ms_, w) in sorted(groups.items(), key=lambda kv: -kv[1][1])[:6]]}
+
+    rooflines = [
+        roofline_rows("attention (kh_attention_bf16)", "mfma",
+                      pair(("attention",), "attention", lambda c: 4.0 * c[1] * c[2] * c[3] * c[4] * c[5]),
+                      lambda c: f"B{c[1]} H{c[2]} T{c[3]} S{c[4]}"),
+        roofline_rows("conv3x3 implicit GEMM (kh_conv3x3_nhwc_bf16)", "mfma",
+                      pair(("conv3x3",), "conv3x3", lambda c: 2.0 * c[1] * c[2] * c[3]),
+                      lambda c: f"M{c[1]} Cout{c[2]} K{c[3]} stride{c[4]}"),
+        roofline_rows("GroupNorm(+SiLU), statistics + apply launches (kh_group_norm_bf16); bytes = one read + one write",
+                      "hbm", pair(("group_norm_stats", "group_norm_apply"), "group_norm", lambda c: 4.0 * c[1] * c[2] * c[3]),
+                      lambda c: f"N{c[1]} C{c[2]} HW{c[3]}"),
+        roofline_rows("LayerNorm (kh_layer_norm_bf16)", "hbm",
+                      pair(("layer_norm",), "layer_norm", lambda c: 4.0 * c[1] * c[2]), lambda c: f"M{c[1]} D{c[2]}"),
+        roofline_rows("ControlNet residual injection folded into the up-block concat (kh_concat_residual_bf16)", "hbm",
+                      pair(("concat_residual",), "concat_residual",
+                           lambda c: 2.0 * c[1] * (c[2] + c[3] * (1 + c[4]) + c[2] + c[3])),
+                      lambda c: f"rows{c[1]} C{c[2]}+{c[3]}"),
+    ]
+    rooflines += sgmv_rooflines(dev)
 
     result = {
         "metric": "unet_step_ms_1024_2lora_1cn",
@@ -357,23 +499,26 @@ def main():
         "output_finite": finite,
         "roofline": {"kernel": "LoRA linear GEMM kernels lora_gemm_pipe / _wide / _ksplit (base GEMM + LoRA delta, all launches of one step, shrink launches included)",
                      "bound": "mfma", "achieved": round(achieved_tf, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved_tf / PEAK_BF16_TFLOPS, 4), "traffic": GEMM_TRAFFIC_BYTES,
-                     "traffic_note": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of `bench.py --kernel-probe` (profiles/), largest launch "
-                                     "(M 2048, K 1280, N 10240, R 128): 75.5 MB read + 21.0 MB written; algorithmic 55.6 MB",
+                     "frac": round(achieved_tf / PEAK_BF16_TFLOPS, 4), "traffic": traffic,
+                     "traffic_note": "NOT measured by this run: HBM-side bytes (read + written) of the largest launch as recorded in "
+                                     f"profiles/{PROFILE_SUMMARY.name} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of `bench.py --kernel-probe`); row: {traffic_src}",
+                     "rank_counted": true_rank,
                      "launches_per_step": len(gemm_ms), "shrink_launches_per_step": len(shrink_calls),
                      "shrink_ms_per_step": round(shrink_ms, 3), "avg_launch_us": round(gemm_total_ms / len(gemm_ms) * 1e3, 2),
-                     "algorithmic_gflop_per_step": round(gemm_flops / 1e9, 1), "by_shape": shape_rows[:8],
+                     "algorithmic_gflop_per_step": round(gemm_flops / 1e9, 1), "by_shape": shape_rows[:10],
                      "shrink_by_shape": shrink_rows[:6]},
+        "rooflines": rooflines,
         "kernel_ms_per_step": {k: {"launches": v[0], "ms": round(v[1], 3)} for k, v in sorted(by_kernel.items())},
     }
     if not args.no_cpu_baseline:
-        cores = min(16, os.cpu_count() or 1)
+        cores = host_cores()
         sec, sample_flops = cpu_baseline(cores)
         est_ms = sec * 1e3 * step_flops / sample_flops
-        result["cpu_baseline"] = {"value": round(est_ms, 1), "unit": "ms", "cores": cores, "kind": "port",
+        result["cpu_baseline"] = {"value": round(est_ms, 1), "unit": "ms", "cores": cores, "kind": "port, extrapolated",
+                                  "cpu": cpu_model(), "host_cpus_visible": os.cpu_count(),
                                   "sample": f"fp32 oracle, UNet mid block (2 resnets + 10 transformer blocks with both "
-                                            f"LoRAs, batch 2, 32x32) = {sample_flops / 1e12:.3f} TFLOP in {sec:.2f} s, "
-                                            f"scaled by FLOPs to the {step_flops / 1e12:.2f} TFLOP step"}
+                                            f"LoRAs, batch 2, 32x32) = {sample_flops / 1e12:.3f} TFLOP in {sec:.2f} s "
+                                            f"(median of 7) on {cores} threads, EXTRAPOLATED by FLOPs to the {step_flops / 1e12:.2f} TFLOP step"}
     print(json.dumps(result))
 
 

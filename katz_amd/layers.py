@@ -125,19 +125,35 @@ class LoRALinear(nn.Module):
         """W += sum_i (lora_scale * m_i) B_i A_i in fp32, cast back -- _fuse_lora,
         diffusers-hf/src/diffusers/models/lora.py:403-433 (Katz: pipeline_controlnet_sd_xl_katz.py:1737-1747)."""
         names = list(self.active if names is None else names)
+        merged = self._fuse_candidate(lora_scale, names)
+        if merged is not None:
+            self._fuse_commit(*merged)
+
+    def _fuse_candidate(self, lora_scale: float, names: Sequence[str]):
+        """(merged fp32 weight, {adapter: multiplier}) without touching any state, or None when there is nothing to
+        fuse.  Raises if the merged weight is not finite: like the reference (lora.py:416-421) the layer is then left
+        exactly as it was."""
+        todo = {}
         with torch.no_grad():
             w = self.weight.float()
+            dev = self.weight.device
             for n in names:
-                if n in self._fused or n not in self.adapters:
+                if n in self._fused or n in todo or n not in self.adapters:
                     continue
                 ad = self.adapters[n]
                 m = lora_scale * ad.multiplier(1.0)
-                dev = self.weight.device
                 w = w + m * (ad.up.to(dev).float() @ ad.down.to(dev).float())
-                self._fused[n] = m
+                todo[n] = m
+            if not todo:
+                return None
             if not torch.isfinite(w).all():
                 raise ValueError("fusing produced non-finite weights; LoRA left unfused")
+        return w, todo
+
+    def _fuse_commit(self, w: torch.Tensor, todo: Dict[str, float]) -> None:
+        with torch.no_grad():
             self.weight.copy_(w.to(self.weight.dtype))
+        self._fused.update(todo)
         self.refresh_adapters()
 
     def unfuse(self) -> None:

@@ -114,49 +114,51 @@ def rescale_(packed: PackedAdapters, adapters: Dict[str, Adapter], global_scale:
 
 
 # ---- per-block adapter scales -------------------------------------------------------------------------------------
-def _translate_into_actual_layer_name(name: str) -> str:
-    """'mid' -> 'mid_block.attentions.0'; 'down.block_1.0' -> 'down_blocks.1.attentions.0'
-    (diffusers-hf/src/diffusers/loaders/unet_loader_utils.py:28-38)."""
-    if name == "mid":
-        return "mid_block.attentions.0"
-    updown, block, attn = name.split(".")
-    updown = updown.replace("down", "down_blocks").replace("up", "up_blocks")
-    return ".".join((updown, block.replace("block_", ""), "attentions." + attn))
+# A per-adapter weight may be one number or a nested description of the UNet's transformers (the surface of
+# diffusers-hf/src/diffusers/loaders/unet_loader_utils.py:41-141):
+#     {"down": 2, "mid": 3, "up": {"block_0": 4, "block_1": [5, 6, 7]}}
+# "mid" is one number; "down" / "up" are a number for the whole half, or a dict per block ("block_<i>") whose value is
+# a number for the block or a list with one number per transformer of the block; whatever is left out counts as 1.
+# The result maps the module path of every transformer ("up_blocks.1.attentions.2") to its number.
+
+def _transformer_slots(blocks_with_transformer, transformer_per_block):
+    """(user spelling, module path, half, block index, transformer index) of every Transformer2DModel, the order the
+    reference's result dict has: mid, then up, then down."""
+    slots = [("mid", "mid_block.attentions.0", "mid", None, None)]
+    for half in ("up", "down"):
+        for blk in blocks_with_transformer[half]:
+            for j in range(transformer_per_block[half]):
+                slots.append((f"{half}.block_{blk}.{j}", f"{half}_blocks.{blk}.attentions.{j}", half, blk, j))
+    return slots
+
+
+def _scale_of_slot(spec: dict, half: str, blk, j):
+    node = spec.get(half, 1)
+    if half == "mid":
+        return node
+    if isinstance(node, dict):
+        node = node[f"block_{blk}"]      # a per-block dict must name every block that has transformers (KeyError)
+    if isinstance(node, list):
+        node = node[j]
+    return node
 
 
 def expand_lora_scales_for_one_adapter(scales, blocks_with_transformer: Dict[str, List[int]],
                                        transformer_per_block: Dict[str, int], module_names: Optional[Sequence[str]] = None):
-    """A float stays a float; a dict like {"down": 2, "mid": 3, "up": {"block_0": 4, "block_1": [5, 6, 7]}} becomes
-    {actual layer name: scale} for every transformer of the UNet, missing parts defaulting to 1
-    (_maybe_expand_lora_scales_for_one_adapter, unet_loader_utils.py:61-141).  module_names: when given, every
-    expanded layer must be a substring of at least one of them (the reference checks the state-dict keys)."""
-    import copy
-    if sorted(blocks_with_transformer.keys()) != ["down", "up"]:
-        raise ValueError("blocks_with_transformer needs to be a dict with keys `'down' and `'up'`")
-    if sorted(transformer_per_block.keys()) != ["down", "up"]:
-        raise ValueError("transformer_per_block needs to be a dict with keys `'down' and `'up'`")
+    """Number in, number out; nested description in, {transformer module path: scale} out (see above).
+    module_names: when given, every transformer path must occur inside at least one of them (the reference checks
+    against the state-dict keys, unet_loader_utils.py:135-139), else ValueError."""
+    for what, d in (("blocks_with_transformer", blocks_with_transformer), ("transformer_per_block", transformer_per_block)):
+        if set(d) != {"down", "up"}:
+            raise ValueError(f"{what} needs to be a dict with keys `'down' and `'up'`")
     if not isinstance(scales, dict):
         return scales
-    scales = copy.deepcopy(scales)
-    scales.setdefault("mid", 1)
-    for updown in ("up", "down"):
-        scales.setdefault(updown, 1)
-        if not isinstance(scales[updown], dict):
-            scales[updown] = {f"block_{i}": scales[updown] for i in blocks_with_transformer[updown]}
-        for i in blocks_with_transformer[updown]:
-            block = f"block_{i}"
-            if not isinstance(scales[updown][block], list):
-                scales[updown][block] = [scales[updown][block]] * transformer_per_block[updown]
-        for i in blocks_with_transformer[updown]:
-            block = f"block_{i}"
-            for tf_idx, value in enumerate(scales[updown][block]):
-                scales[f"{updown}.{block}.{tf_idx}"] = value
-        del scales[updown]
-    out = {_translate_into_actual_layer_name(k): v for k, v in scales.items()}
-    if module_names is not None:
-        for user, layer in zip(scales.keys(), out.keys()):
-            if not any(layer in m for m in module_names):
-                raise ValueError(f"Can't set lora scale for layer {user}. It either doesn't exist in this unet or it has no attentions.")
+    out = {}
+    for user_name, path, half, blk, j in _transformer_slots(blocks_with_transformer, transformer_per_block):
+        if module_names is not None and not any(path in m for m in module_names):
+            raise ValueError(f"Can't set lora scale for layer {user_name}. It either doesn't exist in this unet or "
+                             "it has no attentions.")
+        out[path] = _scale_of_slot(scales, half, blk, j)
     return out
 
 

@@ -409,6 +409,8 @@ def group_norm(x: torch.Tensor, num_groups: int, weight: Optional[torch.Tensor],
         _req(add_nc, BF16, "add_nc")
         if add_nc.shape != (N, C):
             raise ValueError(f"add_nc must be [N,C] = [{N},{C}], got {tuple(add_nc.shape)}")
+    if CALL_LOG is not None:
+        CALL_LOG.append(("group_norm", N, C, H * W))
     rc = lib.kh_group_norm_bf16(_ptr(x), _ptr(out), _ptr(weight), _ptr(bias), _ptr(add_nc), _ptr(ws), N, C, H * W, num_groups,
                                 float(eps), 1 if activation == "silu" else 0, cl, _stream())
     _lib.check(rc, "kh_group_norm_bf16")
@@ -423,6 +425,8 @@ def layer_norm(x: torch.Tensor, weight: Optional[torch.Tensor], bias: Optional[t
     M = x.numel() // D
     if out is None:
         out = torch.empty_like(x)
+    if CALL_LOG is not None:
+        CALL_LOG.append(("layer_norm", M, D))
     rc = lib.kh_layer_norm_bf16(_ptr(x), _ptr(out), _ptr(weight), _ptr(bias), M, D, float(eps), _stream())
     _lib.check(rc, "kh_layer_norm_bf16")
     return out
@@ -470,6 +474,8 @@ def residual_add_(dst: torch.Tensor, residuals: Sequence[torch.Tensor]) -> torch
     for r in residuals:
         if r.shape != dst.shape or r.stride() != dst.stride() or r.dtype != BF16:
             raise ValueError("every residual must match dst in shape, strides and dtype")
+    if CALL_LOG is not None:
+        CALL_LOG.append(("residual_add", dst.numel(), len(residuals)))
     rc = lib.kh_residual_add_bf16(_ptr(dst), _ptr_array(residuals), len(residuals), 1.0 / len(residuals),
                                   dst.numel(), _stream())
     _lib.check(rc, "kh_residual_add_bf16")
@@ -489,6 +495,8 @@ def concat_residual(h: torch.Tensor, skip: torch.Tensor, residuals: Sequence[tor
             raise ValueError("residuals must have the shape of skip")
     out = torch.empty((N, C1 + C2, H, W), dtype=BF16, device=h.device, memory_format=torch.channels_last)
     inv = 1.0 / len(residuals) if residuals else 1.0
+    if CALL_LOG is not None:
+        CALL_LOG.append(("concat_residual", N * H * W, C1, C2, len(residuals)))
     rc = lib.kh_concat_residual_bf16(_ptr(h), _ptr(skip), _ptr_array(residuals), len(residuals), inv, _ptr(out),
                                      N * H * W, C1, C2, _stream())
     _lib.check(rc, "kh_concat_residual_bf16")

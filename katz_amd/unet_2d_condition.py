@@ -308,8 +308,23 @@ class UNet2DConditionModel(nn.Module):
     def fuse_lora(self, lora_scale: float = 1.0, adapter_names: Optional[Sequence[str]] = None) -> None:
         if any(c.adapters for c in self.lora_convs().values()):
             raise NotImplementedError("fusing adapters that target convolutions is not implemented; run them unfused")
-        for m in self.lora_linears().values():
-            m.fuse(lora_scale, adapter_names)
+        # all layers or none: a layer whose merged weight is not finite raises (the reference's safe_fusing check,
+        # models/lora.py:416-421); the layers merged before it get their weights back bit for bit
+        done = []
+        try:
+            for m in self.lora_linears().values():
+                names = list(m.active if adapter_names is None else adapter_names)
+                cand = m._fuse_candidate(lora_scale, names)
+                if cand is not None:
+                    done.append((m, m.weight.detach().clone(), dict(m._fused)))
+                    m._fuse_commit(*cand)
+        except Exception:
+            with torch.no_grad():
+                for m, w0, fused0 in reversed(done):
+                    m.weight.copy_(w0)
+                    m._fused = fused0
+                    m.refresh_adapters()
+            raise
 
     def unfuse_lora(self) -> None:
         for m in self.lora_linears().values():

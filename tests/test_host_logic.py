@@ -328,3 +328,41 @@ def test_unet_lora_surface_reaches_convolutions():
                                  adapter_name="bad")
     unet.delete_adapters("locon")
     assert not c.adapters and not lin.adapters
+
+
+def test_fuse_that_fails_leaves_everything_as_it_was():
+    """A non-finite merged weight raises (the reference's safe_fusing, models/lora.py:416-421) and neither the layer
+    that failed nor the layers merged before it keep any trace: weights bit for bit, no adapter marked as fused."""
+    import pytest
+    import torch
+    import katz_amd.layers as L
+    from katz_amd.unet_2d_condition import UNet2DConditionModel, UNetConfig
+
+    torch.manual_seed(0)
+    unet = UNet2DConditionModel(UNetConfig.tiny())
+    lin = unet.lora_linears()
+    g = torch.Generator().manual_seed(1)
+    names = list(lin)
+    for n in names:
+        m = lin[n]
+        m.add_adapter("a", torch.randn(4, m.in_features, generator=g) * 0.1, torch.randn(m.out_features, 4, generator=g) * 0.1)
+    bad = names[len(names) // 2]
+    lin[bad].adapters["a"].up[0, 0] = float("inf")
+    for m in lin.values():
+        m.active = ["a"]
+    before = {n: lin[n].weight.detach().clone() for n in names}
+    with pytest.raises(ValueError):
+        unet.fuse_lora()
+    for n in names:
+        assert torch.equal(lin[n].weight, before[n]), n
+        assert not lin[n]._fused, n
+    # one layer on its own: same guarantee
+    with pytest.raises(ValueError):
+        lin[bad].fuse()
+    assert torch.equal(lin[bad].weight, before[bad]) and not lin[bad]._fused
+    # and with the bad adapter repaired the whole model fuses and unfuses
+    lin[bad].adapters["a"].up[0, 0] = 0.0
+    unet.fuse_lora()
+    assert all(m._fused for m in lin.values())
+    unet.unfuse_lora()
+    assert max((lin[n].weight - before[n]).abs().max().item() for n in names) < 1e-5
