@@ -560,15 +560,32 @@ class Attention(nn.Module):
                               attention_mask=attention_mask, **cross_attention_kwargs)
 
 
+def env_flag(name: str) -> bool:
+    """The reference's switches are environment variables read when a module is built, "1" = on
+    (ENABLE_FUSED_GEGLU diffusers-hf/src/diffusers/models/activations.py:123, ENABLE_FUSED_NORM_SILU
+    normalization.py:31, ENABLE_CHANNELS_LAST resnet.py:330, ENABLE_CUDA_GRAPH unets/unet_2d_condition.py:511)."""
+    import os
+
+    return os.getenv(name, "0") == "1"
+
+
 class GEGLU(nn.Module):
     """`proj` holds the reference's [2*inner, dim] weight (value rows then gate rows); the kernel reads a
-    row-interleaved copy and applies value * gelu(gate) in the GEMM epilogue."""
+    row-interleaved copy and applies value * gelu(gate) in the GEMM epilogue.
+
+    ENABLE_FUSED_GEGLU=1 (read at construction, like activations.py:123) selects the arithmetic of the reference's
+    fused op instead: value * gelu_tanh(gate) (fast_gelu_mul_fp16(proj_2(x), proj_1(x)), activations.py:145,
+    csrc/gelu.cuh:29-42) -- the projection then runs without the epilogue and kh_geglu_bf16 applies the tanh form.
+    Off (the default) is the exact erf form of the unfused branch (:148-149)."""
 
     def __init__(self, dim_in, dim_out):
         super().__init__()
-        self.proj = LoRALinear(dim_in, dim_out * 2, geglu=True)
+        self.enable_fused_geglu = env_flag("ENABLE_FUSED_GEGLU")
+        self.proj = LoRALinear(dim_in, dim_out * 2, geglu=not self.enable_fused_geglu)
 
     def forward(self, x):
+        if self.enable_fused_geglu:
+            return ops.geglu(self.proj(x), approximate="tanh")
         return self.proj(x)
 
 

@@ -176,6 +176,16 @@ class UNet2DConditionModel(nn.Module):
         self.conv_out = Conv3x3(boc[0], cfg.out_channels)
         self.num_upsamplers = n - 1
         self._ctx_kv = None
+        # The reference's switches (read at construction, unet_2d_condition.py:511, resnet.py:330, normalization.py:31).
+        # ENABLE_CUDA_GRAPH=1: forward replays a captured HIP graph of the step (see _forward_graphed).
+        # ENABLE_FUSED_NORM_SILU / ENABLE_CHANNELS_LAST: accepted and recorded; this build always runs the fused
+        # GroupNorm+SiLU kernel on NHWC memory, which is what the reference does with both switched on, so they change
+        # nothing here.  ENABLE_FUSED_GEGLU is read by layers.GEGLU.
+        from .layers import env_flag
+        self.enable_cuda_graph = env_flag("ENABLE_CUDA_GRAPH")
+        self.enable_fused_norm_silu = env_flag("ENABLE_FUSED_NORM_SILU")
+        self.enable_channels_last = env_flag("ENABLE_CHANNELS_LAST")
+        self._graphs: Dict[tuple, Any] = {}
         self._register_load_state_dict_pre_hook(self._remap_upstream_keys)
 
     # ---- checkpoints ---------------------------------------------------------------------------
@@ -400,11 +410,49 @@ class UNet2DConditionModel(nn.Module):
             per_skip = [[r] for r in res]
         return [[r.to(torch.bfloat16).contiguous(memory_format=torch.channels_last) for r in rs] for rs in per_skip]
 
+    def _forward_graphed(self, sample, timestep, ctx, cross_attention_kwargs, added, down, mid):
+        """ENABLE_CUDA_GRAPH=1: the step as a captured graph, built on the first call with a given signature (input
+        shapes, which residuals are given, the packed-adapter generation, the global LoRA scale) and replayed with
+        refreshed static inputs afterwards -- what _forward_w_separate_cuda_graph does with its two graphs
+        (unet_2d_condition.py:1344-1526, static inputs refreshed by recursive_copy :64-78).  The returned tensor is
+        the graph's static output: it is overwritten by the next call with the same signature."""
+        from . import layers as L
+        from .graph import GraphedUNetStep
+
+        scale = 1.0 if cross_attention_kwargs is None else float(cross_attention_kwargs.get("scale", 1.0))
+        self.scale_lora_layers(scale)
+        multi = bool(down) and isinstance(down[0], (list, tuple))
+        if multi or isinstance(mid, (list, tuple)):
+            raise NotImplementedError("ENABLE_CUDA_GRAPH=1 takes one ControlNet residual set; average several first")
+        key = (tuple(sample.shape), tuple(ctx.shape), None if down is None else len(down), mid is not None,
+               L._pack_epoch, scale, tuple(sorted((k, tuple(v.shape)) for k, v in added.items())))
+        g = self._graphs.get(key)
+        if g is None:
+            if len(self._graphs) >= 4:      # adapters changed or a new resolution: old graphs hold dead buffers
+                self._graphs.clear()
+            self._building_graph = True
+            try:
+                with torch.no_grad():
+                    g = GraphedUNetStep(self, sample, timestep, ctx, added, down, mid)
+            finally:
+                self._building_graph = False
+            self._graphs[key] = g
+        out = g(sample, timestep, ctx, added, down, mid)
+        if cross_attention_kwargs is not None:
+            self.scale_lora_layers(1.0)
+        return out
+
     def forward(self, sample, timestep, encoder_hidden_states, class_labels=None, timestep_cond=None,
                 attention_mask=None, cross_attention_kwargs=None, added_cond_kwargs=None,
                 down_block_additional_residuals=None, mid_block_additional_residual=None,
                 down_intrablock_additional_residuals=None, encoder_attention_mask=None, return_dict: bool = True,
                 controlnet_skt=None, serve_mode=None, time_stats=None, controlnet_num=None):
+        if (self.enable_cuda_graph and sample.is_cuda and not torch.cuda.is_current_stream_capturing()
+                and not getattr(self, "_building_graph", False)):
+            out = self._forward_graphed(sample, timestep, encoder_hidden_states, cross_attention_kwargs,
+                                        added_cond_kwargs, down_block_additional_residuals,
+                                        mid_block_additional_residual)
+            return (out,) if not return_dict else UNet2DConditionOutput(sample=out)
         for name, val in (("class_labels", class_labels), ("timestep_cond", timestep_cond),
                           ("attention_mask", attention_mask), ("encoder_attention_mask", encoder_attention_mask),
                           ("down_intrablock_additional_residuals", down_intrablock_additional_residuals),

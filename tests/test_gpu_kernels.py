@@ -447,19 +447,22 @@ def test_upsample_nearest2x(shape):
 
 
 # ------------------------------------------------------------------------------------------- K2
-@pytest.mark.parametrize("T,dm", [(1024, 1280), (4096, 640), (77, 640)], ids=str)
-def test_sgmv_heterogeneous_batch(T, dm):
-    """BASELINE config 4: 8 requests, each with its own adapter, ranks drawn (seed 2) from {8,16,32,64,128}."""
+@pytest.mark.parametrize("T,K,N", [(1024, 1280, 1280), (4096, 640, 640), (77, 640, 640),
+                                   (77, 2048, 640), (77, 2048, 1280),        # cross-attention to_k / to_v (context 2048)
+                                   (1024, 1280, 10240), (1024, 5120, 1280)], ids=str)   # feed-forward in / out
+def test_sgmv_heterogeneous_batch(T, K, N):
+    """BASELINE config 4: 8 requests, each with its own adapter, ranks drawn (seed 2) from {8,16,32,64,128}, on every
+    shape class of the SDXL attention linears (self-attention and to_out d x d, cross-attention to_k / to_v 2048 -> d)
+    plus the feed-forward widths."""
     from katz_amd import ops
 
-    say("sgmv", T, dm)
+    say("sgmv", T, K, N)
     g = torch.Generator().manual_seed(2)
     n_req = 8
     choices = [8, 16, 32, 64, 128]
     ranks = [choices[i] for i in torch.randint(0, 5, (n_req,), generator=g).tolist()]
     seg_adapter = torch.randperm(n_req, generator=g).tolist()
     seg_adapter[3] = -1  # one request without an adapter
-    K = N = dm
     x = randn(g, n_req * T, K)
     w = randn(g, N, K, std=0.02)
     adapters = [(randn(g, r, K, std=0.02), randn(g, N, r, std=0.02), 0.5 + 0.1 * i) for i, r in enumerate(ranks)]

@@ -327,3 +327,110 @@ def test_patch_on_lora_merge_matches_unmerged_adapter():
         a = merged(x.to(dev), torch.tensor([500.0], device=dev), ctx.to(dev), added_cond_kwargs=_to_dev(added)).sample
         b = plain(x.to(dev), torch.tensor([500.0], device=dev), ctx.to(dev), added_cond_kwargs=_to_dev(added)).sample
     assert cosine(a, b) >= 0.999, cosine(a, b)
+
+
+def test_reference_env_flags(monkeypatch):
+    """ENABLE_FUSED_GEGLU=1 switches the feed-forward to the reference's fused arithmetic (tanh GELU, gelu.cuh:29-42),
+    ENABLE_CUDA_GRAPH=1 makes forward() replay a captured graph (unet_2d_condition.py:511, :2030-2050); the other two
+    switches are recorded.  Compared with the oracle evaluated with the tanh form, and with the eager product."""
+    import katz_amd.layers as L
+    from katz_amd.unet_2d_condition import UNet2DConditionModel, UNetConfig
+    from oracle import ops as OO
+
+    say("env flags")
+    for k in ("ENABLE_FUSED_GEGLU", "ENABLE_CUDA_GRAPH", "ENABLE_FUSED_NORM_SILU", "ENABLE_CHANNELS_LAST"):
+        monkeypatch.setenv(k, "1")
+    torch.manual_seed(0)
+    cfg = OracleCfg.tiny()
+    oracle = round_module_to_bf16_(OracleUNet(cfg).eval())
+    L.SKIP_INIT = True
+    try:
+        prod = UNet2DConditionModel(UNetConfig.tiny())
+    finally:
+        L.SKIP_INIT = False
+    assert prod.enable_cuda_graph and prod.enable_fused_norm_silu and prod.enable_channels_last
+    assert all(m.enable_fused_geglu for m in prod.modules() if isinstance(m, L.GEGLU))
+    prod.load_state_dict(oracle.state_dict(), strict=True)
+    prod = prod.to_runtime("cuda:0", BF)
+    x, ctx, added = _inputs(cfg, 2, 16, 7, seed=9)
+    down, midr = _tiny_residuals(oracle, x, ctx, added, 4)
+    dev = "cuda:0"
+    kw = dict(added_cond_kwargs=_to_dev(added), down_block_additional_residuals=[d.to(dev) for d in down],
+              mid_block_additional_residual=midr.to(dev))
+    t = torch.tensor([500.0], device=dev)
+    with torch.no_grad():
+        monkeypatch.setattr(OO, "geglu", lambda proj, approximate="none": OO.gelu(proj.chunk(2, -1)[1], "tanh") * proj.chunk(2, -1)[0])
+        ref_tanh = oracle(x, 500, ctx, added, down, midr)
+        monkeypatch.undo()
+        ref_erf = oracle(x, 500, ctx, added, down, midr)
+        got = prod(x.to(dev), t, ctx.to(dev), **kw).sample.clone()            # builds the graph, replays it
+        got2 = prod(x.to(dev), t, ctx.to(dev), **kw).sample.clone()           # replay only
+        assert len(prod._graphs) == 1
+        prod.enable_cuda_graph = False
+        eager = prod(x.to(dev), t, ctx.to(dev), **kw).sample
+        torch.cuda.synchronize()
+    assert torch.equal(got, got2) and torch.equal(got, eager)
+    assert cosine(got, ref_tanh) >= 0.999 and cosine(got, ref_erf) >= 0.999   # the two forms differ below bf16 noise here
+    # so that the tanh form is what ran is checked on the calls: every feed-forward went through kh_geglu_bf16(tanh)
+    from katz_amd import ops
+    seen = []
+    real = ops.geglu
+    monkeypatch.setattr(ops, "geglu", lambda proj, approximate="none": (seen.append(approximate), real(proj, approximate))[1])
+    with torch.no_grad():
+        prod(x.to(dev), t, ctx.to(dev), **kw)
+    n_ff = sum(1 for m in prod.modules() if isinstance(m, L.GEGLU))
+    assert seen == ["tanh"] * n_ff and n_ff > 0
+
+
+def test_kohya_named_adapter_to_step(tiny_pair):
+    """A kohya / SGM-named adapter file (lora_unet_input_blocks_4_1_..., .lora_down / .lora_up / .alpha) goes through
+    convert_kohya_lora_to_diffusers -> load_lora_into_unet -> one step, against the oracle given the same matrices
+    under their module names (conversion: diffusers-hf/src/diffusers/loaders/lora_conversion_utils.py:126-287)."""
+    import re
+
+    from katz_amd.lora_conversion import convert_kohya_lora_to_diffusers
+
+    cfg, oracle, prod = tiny_pair
+    say("kohya adapter -> step")
+
+    def kohya_name(mod):   # diffusers module path -> sd-scripts name with SGM block numbering (layers_per_block = 2)
+        m = re.match(r"(down_blocks|up_blocks)\.(\d+)\.attentions\.(\d+)\.(.+)", mod)
+        if m:
+            b, l = int(m.group(2)), int(m.group(3))
+            head = f"input_blocks_{b * 3 + l + 1}_1" if m.group(1) == "down_blocks" else f"output_blocks_{b * 3 + l}_1"
+            rest = m.group(4)
+        else:
+            head, rest = "middle_block_1", re.match(r"mid_block\.attentions\.0\.(.+)", mod).group(1)
+        return "lora_unet_" + head + "_" + rest.replace(".", "_")
+
+    rank, alpha = 16, 8.0
+    lora = random_lora(oracle.lora_linears(), rank, seed=21, std=0.05)
+    file_sd = {}
+    for mod, (down, up) in lora.items():
+        kn = kohya_name(mod)
+        file_sd[kn + ".lora_down.weight"] = down
+        file_sd[kn + ".lora_up.weight"] = up
+        file_sd[kn + ".alpha"] = torch.tensor(alpha)
+    unet_sd, alphas, rest = convert_kohya_lora_to_diffusers(file_sd)
+    assert not rest and len(unet_sd) == 2 * len(lora) and len(alphas) == len(lora)
+    prod.load_lora_into_unet(unet_sd, network_alphas=alphas, adapter_name="kohya")
+    oracle.add_adapter("kohya", lora, alpha=alpha)
+    x, ctx, added = _inputs(cfg, 2, 16, 77, seed=12)
+    dev = "cuda:0"
+    try:
+        with torch.no_grad():
+            oracle.set_adapters(["kohya"], [0.9]); prod.set_adapters(["kohya"], [0.9])
+            ref = oracle(x, 500, ctx, added)
+            got = prod(x.to(dev), torch.tensor([500.0], device=dev), ctx.to(dev), added_cond_kwargs=_to_dev(added)).sample
+            prod.set_adapters([], [])
+            base = prod(x.to(dev), torch.tensor([500.0], device=dev), ctx.to(dev), added_cond_kwargs=_to_dev(added)).sample
+            torch.cuda.synchronize()
+        assert cosine(got, ref) >= 0.999, cosine(got, ref)
+        assert_close_rel(got, ref, 6e-2, "kohya adapter step")
+        assert (got.float() - base.float()).abs().max().item() > 1e-2     # the adapter (alpha / rank = 0.5) matters
+        lin = prod.lora_linears()
+        assert all(m.adapters["kohya"].alpha == alpha for m in lin.values())
+    finally:
+        prod.unload_lora()
+        for m in oracle.lora_linears().values():
+            m.adapters.clear(); m.active = []
