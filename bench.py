@@ -342,12 +342,108 @@ def kernel_probe():
                                        "launches_per_round": meta, "rounds": 3}}))
 
 
+def loop_bench(args):
+    """BASELINE.json configs[4]: the 50-step guided denoise loop at 1024x1024 -- random-init SDXL UNet with the two
+    LoRAs, random-init SDXL-size ControlNet (from_unet, conditioning image [2,3,1024,1024] uniform[0,1], scale 0.5),
+    Euler discrete scheduler (SDXL schedule), guidance 7.5, seeded latents x init_noise_sigma; every step is one replay
+    of one captured graph holding ControlNet -> UNet -> guidance + Euler.  Prints one JSON line: end-to-end ms of the
+    loop, ms per step, and the per-kernel breakdown of one step (per-launch HIP events on an eager step)."""
+    import torch
+    from katz_amd import ops
+    from katz_amd.controlnet import ControlNetModel
+    from katz_amd.graph import GraphedDenoiseStep
+    from katz_amd.scheduler import EulerDiscreteScheduler
+
+    dev = torch.device("cuda:0")
+    bf = torch.bfloat16
+    torch.manual_seed(0)
+    with torch.device(dev):
+        from katz_amd.unet_2d_condition import UNet2DConditionModel, UNetConfig
+        unet = UNet2DConditionModel(UNetConfig.sdxl())
+        cn = ControlNetModel.from_unet(unet)
+        g = torch.Generator(device=dev).manual_seed(3)
+        with torch.no_grad():   # a trained ControlNet's "zero" convolutions are not zero: small random ones
+            for m in [cn.controlnet_cond_embedding.conv_out, cn.controlnet_mid_block, *cn.controlnet_down_blocks]:
+                m.weight.copy_(torch.randn(m.weight.shape, generator=g, device=dev) * (0.1 / m.weight[0].numel() ** 0.5))
+    unet, cn = unet.to_runtime(dev, bf), cn.to_runtime(dev, bf)
+    names, weights = add_random_loras(unet, dev)
+    unet.set_adapters(names, weights)
+    sample, t, ctx, added, _, _ = make_inputs(dev)
+    cond = torch.rand(2, 3, 1024, 1024, generator=g, device=dev).to(bf)
+    sch = EulerDiscreteScheduler(beta_start=0.00085, beta_end=0.012, beta_schedule="scaled_linear",
+                                 timestep_spacing="leading", steps_offset=1)
+    sch.set_timesteps(args.loop_steps, device=dev)
+    lat0 = (torch.randn(1, 4, 128, 128, generator=g, device=dev) * sch.init_noise_sigma).to(bf)
+    with torch.no_grad():
+        step = GraphedDenoiseStep(unet, cn, lat0, ctx, added, cond, 7.5, 0.5)
+        for _ in range(args.warmup_loops):
+            out = step.run(lat0, sch)
+        torch.cuda.synchronize()
+        times = []
+        for _ in range(args.loops):
+            t0 = time.perf_counter()
+            out = step.run(lat0, sch, check=False)
+            torch.cuda.synchronize()
+            times.append((time.perf_counter() - t0) * 1e3)
+        ops.check_split_timeouts(dev)
+        finite = bool(torch.isfinite(out.float()).all())
+        # the same loop with the UNet alone (zero-cost ControlNet): what the ControlNet adds per step
+        # per-kernel breakdown of one eager step
+        model_input = torch.cat([lat0] * 2).contiguous(memory_format=torch.channels_last)
+        emb = cn.embed_condition(cond)
+        torch.cuda.synchronize()
+        torch.cuda._sleep(int(0.1 * 2.4e9))
+        ops.profile_begin()
+        try:
+            d, m = cn(model_input, t, ctx, cond, 0.5, added_cond_kwargs=added, cond_embedding=emb)
+            n_cn = None
+            eps = unet(model_input, t, ctx, added_cond_kwargs=added, down_block_additional_residuals=d,
+                       mid_block_additional_residual=m).sample
+            ops.cfg_euler_step(eps, lat0.contiguous(memory_format=torch.channels_last), sch.coef_table(dev)[0], 7.5)
+        finally:
+            launches = ops.profile_end()
+        torch.cuda.synchronize()
+        torch.cuda._sleep(int(0.1 * 2.4e9))
+        ops.profile_begin()
+        try:
+            cn.embed_condition(cond)
+        finally:
+            emb_launches = ops.profile_end()
+    by_kernel = {}
+    for name, dur in launches:
+        e = by_kernel.setdefault(name, [0, 0.0])
+        e[0] += 1
+        e[1] += dur
+    times.sort()
+    med = times[len(times) // 2]
+    result = {
+        "metric": "denoise_loop_ms_1024_2lora_1cn", "value": round(med, 2), "unit": "ms", "n_gpus": 1,
+        "loops_timed": args.loops, "loop_steps": args.loop_steps, "ms_per_step": round(med / args.loop_steps, 3),
+        "higher_is_better": False, "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic (random-init SDXL UNet and ControlNet, seeded latents, conditioning image uniform[0,1])",
+        "config": {"workload": f"{args.loop_steps}-step SDXL denoise loop at 1024x1024: per step ControlNet (SDXL arch, image "
+                               "[2,3,1024,1024], scale 0.5) -> UNet (2 LoRAs r64 s0.8 + r32 s0.6, CFG batch 2) -> guidance 7.5 + "
+                               "Euler discrete; one HIP graph replay per step; conditioning embedding computed once per loop",
+                   "global_batch": 2, "parallelism": "single GPU"},
+        "loop_ms_all": [round(x, 2) for x in times], "output_finite": finite,
+        "kernel_ms_per_step": {k: {"launches": v[0], "ms": round(v[1], 3)} for k, v in sorted(by_kernel.items())},
+        "kernel_ms_sum_per_step": round(sum(v[1] for v in by_kernel.values()), 3),
+        "cond_embedding_once_per_loop_ms": round(sum(d for _, d in emb_launches), 3),
+    }
+    print(json.dumps(result))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--loop", action="store_true",
+                    help="BASELINE configs[4]: the 50-step ControlNet + UNet + Euler denoise loop, end-to-end ms")
+    ap.add_argument("--loop-steps", type=int, default=50)
+    ap.add_argument("--loops", type=int, default=3)
+    ap.add_argument("--warmup-loops", type=int, default=1)
     ap.add_argument("--kernel-probe", action="store_true",
                     help="run only a 64 MiB copy and each kernel at its BASELINE shapes three times (for rocprofv3)")
     args = ap.parse_args()
@@ -361,6 +457,12 @@ def main():
 
     if args.kernel_probe:
         kernel_probe()
+        return
+    if args.loop:
+        if not torch.cuda.is_available():
+            print("bench.py: no GPU visible; the katz_hip kernels have no CPU path", file=sys.stderr)
+            sys.exit(1)
+        loop_bench(args)
         return
 
     if not torch.cuda.is_available():

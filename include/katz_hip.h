@@ -231,7 +231,8 @@ int kh_conv3x3_nhwc_bf16(const void* x, const void* w, const void* bias, const v
  * in one pass over the latents, fp32 arithmetic in that order.  noise_pred [2,n] bf16; latents / latents_out [n]
  * bf16 (the reference casts prev_sample to the model dtype, :530) or fp32 when latents_f32 != 0; model_input_next
  * [2,n] bf16 or NULL.  coef: DEVICE pointer to {sigma, sigma_next, next_scale = sqrt(sigma_next^2 + 1)} so that a
- * captured graph can be replayed for every step with the three floats rewritten between replays.  n % 8 == 0. */
+ * captured graph can be replayed for every step with the three floats rewritten between replays.  n % 8 == 0.
+ * latents_out may equal latents (update in place); model_input_next must not overlap noise_pred. */
 int kh_cfg_euler_step_bf16(const void* noise_pred, const void* latents, void* latents_out, void* model_input_next,
                            int64_t n, float guidance_scale, const float* coef, int latents_f32, void* stream);
 

@@ -29,13 +29,26 @@ def zero_module(m: nn.Module) -> nn.Module:
     return m
 
 
-def conv1x1_scaled(x: torch.Tensor, conv: nn.Conv2d, scale: float) -> torch.Tensor:
-    """(1x1 convolution of a channels_last tensor) * scale: a linear layer over the channels of every pixel."""
+def conv1x1_scaled(x: torch.Tensor, conv: nn.Conv2d, scale: float, cache: Optional[dict] = None) -> torch.Tensor:
+    """(1x1 convolution of a channels_last tensor) * scale: a linear layer over the channels of every pixel, with the
+    scale folded into the layer, scale * (W x + b) = (scale W) x + scale b, so the residual leaves the GEMM epilogue
+    finished (controlnet.py:818-824 followed by the `sample * conditioning_scale` of :833-835).  Exact for powers of
+    two (Katz's default 0.5, upstream's 1.0); otherwise the scaled weights are rounded to bf16 once instead of the
+    output twice.  cache: {id(conv): (key, weight, bias)} kept by the caller, rebuilt when scale or weights change."""
     nb, c, hh, ww = x.shape
     x = x.contiguous(memory_format=torch.channels_last)
-    y = ops.lora_linear(x.permute(0, 2, 3, 1).reshape(nb * hh * ww, c), conv.weight.reshape(conv.out_channels, c), conv.bias)
+    w, b = conv.weight.reshape(conv.out_channels, c), conv.bias
     if scale != 1.0:
-        y.mul_(scale)
+        key = (float(scale), conv.weight._version, conv.weight.data_ptr(), None if b is None else b._version)
+        hit = None if cache is None else cache.get(id(conv))
+        if hit is None or hit[0] != key:
+            with torch.no_grad():
+                hit = (key, (w.float() * scale).to(w.dtype).contiguous(),
+                       None if b is None else (b.float() * scale).to(b.dtype))
+            if cache is not None and not (x.is_cuda and torch.cuda.is_current_stream_capturing()):
+                cache[id(conv)] = hit     # tensors made during a capture belong to that graph: do not keep them
+        w, b = hit[1], hit[2]
+    y = ops.lora_linear(x.permute(0, 2, 3, 1).reshape(nb * hh * ww, c), w, b)
     return y.view(nb, hh, ww, conv.out_channels).permute(0, 3, 1, 2)
 
 
@@ -98,6 +111,7 @@ class ControlNetModel(nn.Module):
             resnet_eps=cfg.norm_eps, resnet_groups=cfg.norm_num_groups, num_attention_heads=cfg.num_attention_heads[-1],
             cross_attention_dim=cfg.cross_attention_dim, use_linear_projection=cfg.use_linear_projection)
         self._ctx_kv = None
+        self._zero_conv_cache: Dict[int, tuple] = {}
         self._register_load_state_dict_pre_hook(UNet2DConditionModel._remap_upstream_keys)
 
     @classmethod
@@ -116,6 +130,11 @@ class ControlNetModel(nn.Module):
         self.prepare()
         return self.eval()
 
+    def embed_condition(self, controlnet_cond: torch.Tensor) -> torch.Tensor:
+        """controlnet_cond_embedding(image) (:84-126, applied at :780), channels_last bf16."""
+        cond = controlnet_cond.to(torch.bfloat16).contiguous(memory_format=torch.channels_last)
+        return self.controlnet_cond_embedding(cond).contiguous(memory_format=torch.channels_last)
+
     prepare = UNet2DConditionModel.prepare
     lora_linears = UNet2DConditionModel.lora_linears
     _embed = UNet2DConditionModel._embed
@@ -124,7 +143,9 @@ class ControlNetModel(nn.Module):
                 class_labels=None, timestep_cond=None, attention_mask=None,
                 added_cond_kwargs: Optional[Dict[str, torch.Tensor]] = None,
                 cross_attention_kwargs: Optional[Dict[str, Any]] = None, guess_mode: bool = False,
-                return_dict: bool = False):
+                return_dict: bool = False, cond_embedding: Optional[torch.Tensor] = None):
+        """controlnet.py:687-847.  cond_embedding (not in the reference): the result of embed_condition(controlnet_cond)
+        computed earlier -- in a denoise loop the image, and so its embedding, is the same in every step."""
         for name, val in (("class_labels", class_labels), ("timestep_cond", timestep_cond), ("attention_mask", attention_mask)):
             if val is not None:
                 raise NotImplementedError(f"`{name}` is not used on the SDXL ControlNet path and is not implemented")
@@ -132,7 +153,6 @@ class ControlNetModel(nn.Module):
             raise NotImplementedError("guess_mode (logspace residual scales, controlnet.py:827-831) is not implemented")
         if sample.dtype != torch.bfloat16 or not sample.is_contiguous(memory_format=torch.channels_last):
             sample = sample.to(torch.bfloat16).contiguous(memory_format=torch.channels_last)
-        cond = controlnet_cond.to(torch.bfloat16).contiguous(memory_format=torch.channels_last)
         ctx = encoder_hidden_states.to(torch.bfloat16).contiguous()
         if sample.is_cuda:
             ops.split_counters_reset(sample.device)   # one fill per step clears the in-launch shrinks' counters
@@ -142,15 +162,18 @@ class ControlNetModel(nn.Module):
         emb = self._embed(sample, timestep, added_cond_kwargs)
         temb_act = F.silu(emb)
         self._temb_proj.run(temb_act)   # time_emb_proj of all resnets, batched per width
-        sample = self.conv_in(sample)
-        sample = sample + self.controlnet_cond_embedding(cond)
+        if cond_embedding is None:
+            cond_embedding = self.embed_condition(controlnet_cond)
+        # conv_in(sample) + embedding (:780-783): the add runs in the convolution's epilogue
+        sample = self.conv_in(sample, residual=cond_embedding)
         skips = (sample,)
         for blk in self.down_blocks:
             sample, res = blk(sample, temb_act, ctx)
             skips += res
         sample = self.mid_block(sample, temb_act, ctx)
-        down = [conv1x1_scaled(s, zc, conditioning_scale) for s, zc in zip(skips, self.controlnet_down_blocks)]
-        mid = conv1x1_scaled(sample, self.controlnet_mid_block, conditioning_scale)
+        zc_cache = self._zero_conv_cache
+        down = [conv1x1_scaled(s, zc, conditioning_scale, zc_cache) for s, zc in zip(skips, self.controlnet_down_blocks)]
+        mid = conv1x1_scaled(sample, self.controlnet_mid_block, conditioning_scale, zc_cache)
         if not return_dict:
             return (down, mid)
         return {"down_block_res_samples": down, "mid_block_res_sample": mid}

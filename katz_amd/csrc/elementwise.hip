@@ -175,8 +175,9 @@ namespace {
 // One thread: 8 latent elements.  Arithmetic in fp32 in the reference's order (epsilon prediction, no churn):
 //   eps = u + g*(t - u); x0 = x - sigma*eps; d = (x - x0)/sigma; x' = x + d*(sigma_next - sigma).
 template <bool LAT_F32>
-__global__ __launch_bounds__(EW_THREADS) void cfg_euler_kernel(const bf16_t* __restrict__ noise, const void* __restrict__ lat_in,
-                                                               void* __restrict__ lat_out, bf16_t* __restrict__ next_in,
+// lat_out may be lat_in (a thread reads its eight elements before it writes them): no __restrict__ on the two.
+__global__ __launch_bounds__(EW_THREADS) void cfg_euler_kernel(const bf16_t* __restrict__ noise, const void* lat_in,
+                                                               void* lat_out, bf16_t* __restrict__ next_in,
                                                                long n, float g, const float* __restrict__ coef) {
   const float sigma = coef[0], dt = coef[1] - coef[0], den = coef[2];
   const long chunks = n / 8;

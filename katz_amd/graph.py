@@ -80,3 +80,90 @@ class GraphedUNetStep:
         from . import ops
 
         ops.check_split_timeouts(self.sample.device)
+
+
+class GraphedDenoiseStep:
+    """One step of the guided ControlNet loop -- ControlNet -> UNet with its residuals -> guidance + Euler update + the
+    next step's scaled, duplicated input -- as ONE captured graph (the body of the reference's loop,
+    diffusers-hf/src/diffusers/pipelines/controlnet/pipeline_controlnet_sd_xl_katz.py:1509-1675; the reference splits
+    it over processes and two graphs per UNet because its ControlNets run elsewhere, unet_2d_condition.py:1344-1526).
+
+    Static state: the latents [B,4,H,W], the model input [2B,4,H,W] (both updated in place by the last kernel of the
+    graph) and one fp32 row {sigma_i, sigma_{i+1}, sqrt(sigma_{i+1}^2 + 1), sqrt(sigma_i^2 + 1), timestep_i} that
+    `run` rewrites before every replay; so one graph serves all steps of a schedule.
+
+    hoist_cond_embedding: the ControlNet's conditioning embedding depends on the image only, which is the same in every
+    step; it is computed once per `run` instead of inside the graph (the reference recomputes it every step,
+    controlnet.py:780-783; same value, bit for bit).  Everything the notes on GraphedUNetStep say about rebuilding after
+    adapters are repacked applies here too."""
+
+    def __init__(self, unet, controlnet, latents, encoder_hidden_states, added_cond_kwargs, controlnet_cond,
+                 guidance_scale: float, conditioning_scale: float = 0.5, hoist_cond_embedding: bool = True,
+                 warmup: int = 2):
+        from . import ops
+
+        self.unet, self.controlnet = unet, controlnet
+        self.guidance_scale, self.conditioning_scale = float(guidance_scale), float(conditioning_scale)
+        dev = latents.device
+        bf = torch.bfloat16
+        cl = lambda t: t.detach().to(bf).contiguous(memory_format=torch.channels_last).clone()
+        self.latents = cl(latents)
+        self.model_input = cl(torch.cat([latents] * 2))
+        self.ctx = encoder_hidden_states.detach().to(bf).contiguous().clone()
+        self.added = {k: v.detach().clone() for k, v in added_cond_kwargs.items()}
+        self.cond = cl(controlnet_cond)
+        self.row = torch.zeros(5, dtype=torch.float32, device=dev)
+        self.row[:4] = torch.tensor([1.0, 0.5, 1.0, 1.0])     # harmless values for the warm-up runs
+        self.row[4] = 500.0
+        self.hoist = hoist_cond_embedding
+        self.cond_emb = None
+        unet.prepare()
+        controlnet.prepare()
+        keep = (self.latents.clone(), self.model_input.clone())
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side), torch.no_grad():
+            if self.hoist:
+                self.cond_emb = controlnet.embed_condition(self.cond)
+            for _ in range(warmup):
+                self._step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        self.latents.copy_(keep[0]); self.model_input.copy_(keep[1])
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph), torch.no_grad():
+            self._step()
+        self.latents.copy_(keep[0]); self.model_input.copy_(keep[1])
+        self._ops = ops
+
+    def _step(self):
+        from . import ops
+
+        t = self.row[4:5]
+        down, mid = self.controlnet(self.model_input, t, self.ctx, self.cond, self.conditioning_scale,
+                                    added_cond_kwargs=self.added, cond_embedding=self.cond_emb)
+        eps = self.unet(self.model_input, t, self.ctx, added_cond_kwargs=self.added,
+                        down_block_additional_residuals=down, mid_block_additional_residual=mid, return_dict=False)[0]
+        ops.cfg_euler_step(eps, self.latents, self.row, self.guidance_scale, latents_out=self.latents,
+                           model_input_next=self.model_input)
+
+    def run(self, latents: torch.Tensor, scheduler, controlnet_cond: Optional[torch.Tensor] = None,
+            check: bool = True) -> torch.Tensor:
+        """The whole loop: `latents` already scaled by init_noise_sigma (prepare_latents, pipeline :872-887);
+        scheduler.set_timesteps(...) done.  Returns the final latents (a copy, in the model dtype like the reference's
+        scheduler output, scheduling_euler_discrete.py:530)."""
+        dev = self.latents.device
+        table = torch.cat([scheduler.coef_table(dev), scheduler.timesteps.to(dev, torch.float32)[:, None]], dim=1).contiguous()
+        with torch.no_grad():
+            if controlnet_cond is not None:
+                self.cond.copy_(controlnet_cond)
+                if self.hoist:
+                    self.cond_emb.copy_(self.controlnet.embed_condition(self.cond))
+            self.latents.copy_(latents)
+            self.model_input.copy_((torch.cat([latents] * 2).float() / table[0, 3]).to(torch.bfloat16))
+            for i in range(table.shape[0]):
+                self.row.copy_(table[i])
+                self.graph.replay()
+        if check:
+            self._ops.check_split_timeouts(dev)
+        return self.latents.clone()

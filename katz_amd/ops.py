@@ -552,22 +552,33 @@ def cfg_euler_step(noise_pred: torch.Tensor, latents: torch.Tensor, coef: torch.
                    latents_out: Optional[torch.Tensor] = None, model_input_next: Optional[torch.Tensor] = None):
     """Guidance + Euler step (+ the next step's scaled, duplicated model input) in one kernel.
     noise_pred [2B,...] bf16 (uncond rows first), latents [B,...] bf16 or fp32, coef: fp32 GPU tensor
-    {sigma, sigma_next, sqrt(sigma_next^2+1)}.  Returns latents_out (allocated unless given)."""
+    {sigma, sigma_next, sqrt(sigma_next^2+1)}.  All tensors dense in one memory format (contiguous, or channels_last as
+    the UNet returns its output).  latents_out may be latents itself.  Returns latents_out (allocated unless given)."""
     lib = _lib.load()
-    _req(noise_pred, BF16, "noise_pred")
-    if latents.dtype not in (BF16, torch.float32) or not latents.is_cuda or not latents.is_contiguous():
-        raise ValueError("latents must be a contiguous bfloat16 or float32 GPU tensor")
-    if not noise_pred.is_contiguous() or noise_pred.numel() != 2 * latents.numel():
-        raise ValueError("noise_pred must be contiguous with twice the elements of latents")
+    if not noise_pred.is_cuda or noise_pred.dtype != BF16:
+        raise _lib.KatzHipError("noise_pred must be a bfloat16 GPU tensor; katz_hip has no CPU path")
+
+    def layout(t):   # the op is elementwise per batch row: every tensor must be dense in ONE memory format
+        if t.is_contiguous():
+            return "rows"
+        if t.dim() == 4 and t.is_contiguous(memory_format=torch.channels_last):
+            return "nhwc"
+        return None
+
+    kind = layout(noise_pred)
+    if kind is None or noise_pred.numel() != 2 * latents.numel():
+        raise ValueError("noise_pred must be dense (contiguous or channels_last) with twice the elements of latents")
+    if latents.dtype not in (BF16, torch.float32) or not latents.is_cuda or layout(latents) != kind:
+        raise ValueError("latents must be a bfloat16 or float32 GPU tensor in the memory format of noise_pred")
     if coef.dtype != torch.float32 or not coef.is_cuda or coef.numel() < 3:
         raise ValueError("coef must be a float32 GPU tensor of at least 3 elements")
     if latents_out is None:
         latents_out = torch.empty_like(latents)
-    if latents_out.dtype != latents.dtype or latents_out.shape != latents.shape or not latents_out.is_contiguous():
+    if latents_out.dtype != latents.dtype or latents_out.shape != latents.shape or layout(latents_out) != kind:
         raise ValueError("latents_out must match latents")
-    if model_input_next is not None and (model_input_next.dtype != BF16 or not model_input_next.is_contiguous()
+    if model_input_next is not None and (model_input_next.dtype != BF16 or layout(model_input_next) != kind
                                          or model_input_next.numel() != noise_pred.numel()):
-        raise ValueError("model_input_next must be a contiguous bfloat16 tensor of noise_pred's size")
+        raise ValueError("model_input_next must be a bfloat16 tensor of noise_pred's size and memory format")
     rc = lib.kh_cfg_euler_step_bf16(_ptr(noise_pred), _ptr(latents), _ptr(latents_out), _ptr(model_input_next),
                                     latents.numel(), float(guidance_scale), _ptr(coef),
                                     1 if latents.dtype == torch.float32 else 0, _stream())

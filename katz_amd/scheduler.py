@@ -116,7 +116,9 @@ def denoise_loop(model: Callable[[torch.Tensor, torch.Tensor], torch.Tensor], sc
     coef = scheduler.coef_table(dev)
     lat = latents.to(torch.float32 if latents_fp32 else torch.bfloat16).contiguous()
     x = torch.cat([lat] * 2).to(torch.bfloat16)
-    model_input = (x / coef[0, 3]).contiguous()   # first scale_model_input; later ones come out of the fused kernel
+    # first scale_model_input (later ones come out of the fused kernel): the division in fp32, as the reference's
+    # `sample / ((sigma**2 + 1) ** 0.5)` with its CPU-resident sigma evaluates it (scheduling_euler_discrete.py:292-296)
+    model_input = (x.float() / coef[0, 3]).to(torch.bfloat16).contiguous()
     nxt = torch.empty_like(model_input)
     lat_out = torch.empty_like(lat)
     timesteps = scheduler.timesteps.to(dev)
