@@ -342,6 +342,54 @@ def kernel_probe():
                                        "launches_per_round": meta, "rounds": 3}}))
 
 
+def merge_probe():
+    """Katz's per-request merge (patch_on_lora, pipeline_controlnet_sd_xl_katz.py:1730-1770: 0.090 / 0.123 s on H800
+    in the reference's logs) on the SDXL UNet: a rank-64 adapter on all 722 linears merged by the batched merge kernel.
+    Timed three ways: adapters in pageable host memory as float16 (what the shared-memory segments are; the upload is
+    part of the time, as in the reference), adapters already resident on the GPU, and the merge launch alone (HIP
+    events).  Prints one JSON line."""
+    import torch
+    from katz_amd import ops
+    from katz_amd.shm_adapters import KATZ_MERGE_SCALE, patch_on_lora
+
+    dev = torch.device("cuda:0")
+    unet = build_product(dev)
+    lin = unet.lora_linears()
+    g = torch.Generator().manual_seed(4)
+    host_sd, key_match = {}, {}
+    for name, m in lin.items():
+        host_sd[name + ".down"] = (torch.randn(64, m.in_features, generator=g) * 1e-3).to(torch.float16)
+        host_sd[name + ".up"] = (torch.randn(m.out_features, 64, generator=g) * 1e-3).to(torch.float16)
+        key_match[name + ".weight"] = {"lora_down_key": name + ".down", "lora_up_key": name + ".up"}
+    dev_sd = {k: v.to(dev) for k, v in host_sd.items()}
+    n_bytes = sum(v.numel() * 2 for v in host_sd.values())
+    w_bytes = sum(m.weight.numel() * 2 for m in lin.values())
+
+    def timed(sd, sign):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        n = patch_on_lora(unet, sd, key_match, scale=sign * KATZ_MERGE_SCALE)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3, n
+
+    timed(dev_sd, 1.0); timed(dev_sd, -1.0)   # warm-up
+    host_ms = [timed(host_sd, s)[0] for s in (1.0, -1.0, 1.0, -1.0)]
+    dev_ms = [timed(dev_sd, s)[0] for s in (1.0, -1.0, 1.0, -1.0)]
+    ops.profile_begin()
+    timed(dev_sd, 1.0); timed(dev_sd, -1.0)
+    kernel_ms = [d for n, d in ops.profile_end() if n == "lora_merge"]
+    finite = all(bool(torch.isfinite(m.weight).all()) for m in list(lin.values())[:20])
+    print(json.dumps({
+        "metric": "patch_on_lora_ms_sdxl_722_linears_rank64", "unit": "ms",
+        "value_adapters_in_pageable_host_memory": round(min(host_ms), 2),
+        "value_adapters_resident_on_gpu": round(min(dev_ms), 2),
+        "merge_kernel_ms": round(min(kernel_ms), 3), "layers": len(lin),
+        "adapter_bytes": n_bytes, "weight_bytes_read_plus_written": 2 * w_bytes,
+        "merge_kernel_GBps": round((2 * w_bytes + n_bytes) / (min(kernel_ms) * 1e-3) / 1e9, 1),
+        "reference_h800_s": [0.090, 0.123], "all_runs_ms": {"host": [round(x, 2) for x in host_ms], "gpu": [round(x, 2) for x in dev_ms]},
+        "weights_finite": finite}))
+
+
 def loop_bench(args):
     """BASELINE.json configs[4]: the 50-step guided denoise loop at 1024x1024 -- random-init SDXL UNet with the two
     LoRAs, random-init SDXL-size ControlNet (from_unet, conditioning image [2,3,1024,1024] uniform[0,1], scale 0.5),
@@ -441,6 +489,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--loop", action="store_true",
                     help="BASELINE configs[4]: the 50-step ControlNet + UNet + Euler denoise loop, end-to-end ms")
+    ap.add_argument("--merge-probe", action="store_true",
+                    help="time Katz's patch_on_lora (merge of a rank-64 adapter into all 722 SDXL linears)")
     ap.add_argument("--loop-steps", type=int, default=50)
     ap.add_argument("--loops", type=int, default=3)
     ap.add_argument("--warmup-loops", type=int, default=1)
@@ -457,6 +507,9 @@ def main():
 
     if args.kernel_probe:
         kernel_probe()
+        return
+    if args.merge_probe:
+        merge_probe()
         return
     if args.loop:
         if not torch.cuda.is_available():

@@ -41,7 +41,7 @@ const char* kh_error_string(int code);
  * kh_profile_begin and kh_profile_end every kernel of this library is launched with its own HIP
  * start/stop event pair on the launch stream.  kh_profile_end waits for them and writes, in launch
  * order, a kernel tag (1 lora_gemm, 2 lora_gemm_f32, 3 attention, 4 group_norm stats, 5 group_norm apply,
- * 6 layer_norm, 7 geglu, 8 residual_add, 9 concat_residual, 10 sgmv_shrink, 11 sgmv_expand, 12 lora_shrink, 13 conv3x3, 14 cfg_euler, 15 upsample) and the
+ * 6 layer_norm, 7 geglu, 8 residual_add, 9 concat_residual, 10 sgmv_shrink, 11 sgmv_expand, 12 lora_shrink, 13 conv3x3, 14 cfg_euler, 15 upsample, 16 lora_merge) and the
  * duration in ms into HOST arrays; returns the number of launches (or -hipError_t).  Do not use under
  * graph capture. */
 int kh_profile_begin(void);
@@ -123,6 +123,20 @@ int kh_lora_linear_split_launches(int64_t M, int64_t N, int64_t K, int64_t R, in
  * attention_processor.py:1260-1262).  K % 32 == 0, R <= 128, no GEGLU / residual. */
 int kh_lora_linear_grouped_bf16(const void* x, const uint64_t* table, int64_t n_groups, int64_t ldt, int64_t M,
                                 int64_t N, int64_t K, int64_t R, int flags, void* stream);
+/* Merge adapters into the weights of MANY layers in one launch:  W_l += scale * layer_scale[l] * up_l . down_l.
+ * Replaces the per-layer loop of Katz's patch_on_lora, `unet_state_dict[key] += cur_up @ cur_down * scale`
+ * (diffusers-hf/src/diffusers/pipelines/controlnet/pipeline_controlnet_sd_xl_katz.py:1737-1747), and the per-module
+ * _fuse_lora of diffusers-hf/src/diffusers/models/lora.py:403-433; the product is accumulated in fp32 and the sum
+ * rounded once.  table: DEVICE array of n_layers rows of six 64-bit words {W, up, down, N, K, r}: device addresses of
+ * W [N,K] (bf16, updated in place), up [N,r], down [r,K], then the three sizes as int64.  up / down are bf16 storage,
+ * or float16 when operands_fp16 != 0 (the dtype of Katz's shared-memory adapter arrays, load_lora_shm_multi.py:49-61).
+ * tile_start: DEVICE int32 [n_layers + 1], tile_start[l] = sum over layers before l of ceil(N/128) * ceil(K/128);
+ * total_tiles = tile_start[n_layers] (sizes the grid).  layer_scale: DEVICE float [n_layers] or NULL (all 1).
+ * max_rank: the largest r in the table (<= 128; sizes the kernel's LDS).  A negative scale undoes a merge up to
+ * rounding.  The same W must not appear in two rows. */
+int kh_lora_merge_grouped_bf16(const uint64_t* table, const int32_t* tile_start, const float* layer_scale,
+                               int64_t n_layers, int64_t total_tiles, int64_t max_rank, float scale, int operands_fp16,
+                               void* stream);
 /* fp32 variant of the same formula (fp32 parity path); R <= 128, any M/N/K. */
 int kh_lora_linear_f32(const float* x, const float* w, const float* bias, const float* a_cat, const float* b_cat,
                        const float* col_scale, const float* residual, float* y, int64_t M, int64_t N, int64_t K,

@@ -24,6 +24,7 @@ SIGNATURES = {
     "kh_lora_shrink_bf16": (c_int, [_P, _P, _P, _P, _I, _I, _I, _P]),
     "kh_lora_linear_pre_bf16": (c_int, [_P, _P, _P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, c_int, _P]),
     "kh_lora_linear_grouped_bf16": (c_int, [_P, _P, _I, _I, _I, _I, _I, _I, c_int, _P]),
+    "kh_lora_merge_grouped_bf16": (c_int, [_P, _P, _P, _I, _I, _I, c_float, c_int, _P]),
     "kh_lora_linear_f32": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
     "kh_sgmv_shrink_bf16": (c_int, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
     "kh_sgmv_expand_bf16": (c_int, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),

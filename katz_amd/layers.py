@@ -245,7 +245,58 @@ class TimestepEmbedding(nn.Module):
         return self.linear_2(F.silu(self.linear_1(sample)))
 
 
-class Conv3x3(nn.Conv2d):
+class _ConvLoRAFuse:
+    """W += sum_i (lora_scale * m_i) * (up_i . down_i) for a convolution, through the merged-kernel identity of the
+    reference: the [Cout, r] x [r, Cin*kh*kw] product reshaped to the weight's shape (_fuse_lora of LoRACompatibleConv,
+    diffusers-hf/src/diffusers/models/lora.py:403-421; _unfuse_lora :423-441), fp32 then cast back.  Shared by the 3x3
+    and the 1x1 convolution; same all-or-nothing contract as LoRALinear.fuse."""
+
+    def _delta(self, ad: Adapter, m: float) -> torch.Tensor:
+        dev = self.weight.device
+        up = ad.up.to(dev).float().reshape(ad.up.shape[0], -1)
+        down = ad.down.to(dev).float().reshape(ad.down.shape[0], -1)
+        return (m * (up @ down)).reshape(self.weight.shape)
+
+    def _fuse_candidate(self, lora_scale: float, names: Sequence[str]):
+        todo = {}
+        with torch.no_grad():
+            w = self.weight.float()
+            for n in names:
+                if n in self._fused or n in todo or n not in self.adapters:
+                    continue
+                m = lora_scale * self.adapters[n].multiplier(1.0)
+                w = w + self._delta(self.adapters[n], m)
+                todo[n] = m
+            if not todo:
+                return None
+            if not torch.isfinite(w).all():
+                raise ValueError("fusing produced non-finite weights; LoRA left unfused")
+        return w, todo
+
+    def _fuse_commit(self, w: torch.Tensor, todo: Dict[str, float]) -> None:
+        with torch.no_grad():
+            self.weight.copy_(w.to(self.weight.dtype))
+        self._fused.update(todo)
+        self.refresh_adapters()
+
+    def fuse(self, lora_scale: float = 1.0, names: Optional[Sequence[str]] = None) -> None:
+        merged = self._fuse_candidate(lora_scale, list(self.active if names is None else names))
+        if merged is not None:
+            self._fuse_commit(*merged)
+
+    def unfuse(self) -> None:
+        if not self._fused:
+            return
+        with torch.no_grad():
+            w = self.weight.float()
+            for n, m in self._fused.items():
+                w = w - self._delta(self.adapters[n], m)
+            self.weight.copy_(w.to(self.weight.dtype))
+        self._fused.clear()
+        self.refresh_adapters()
+
+
+class Conv3x3(_ConvLoRAFuse, nn.Conv2d):
     """nn.Conv2d(kernel 3, padding 1, stride 1 or 2) whose forward runs the katz_hip implicit-GEMM kernel on
     channels_last bf16 GPU tensors; parameters and state-dict keys are nn.Conv2d's.  forward(x, residual)
     also folds the residual add that follows the convolution (resnet.py:374) into the kernel's epilogue.
@@ -262,6 +313,7 @@ class Conv3x3(nn.Conv2d):
         self.adapters_enabled = True
         self._global_scale = 1.0
         self._lora = None    # (A_cat packed [R,3,3,Cin], B_cat scaled [Cout,R]) of the active adapters
+        self._fused: Dict[str, float] = {}   # adapter name -> multiplier merged into weight
 
     def add_adapter(self, name: str, down: torch.Tensor, up: torch.Tensor, alpha: Optional[float] = None,
                     weight: float = 1.0) -> None:
@@ -297,7 +349,7 @@ class Conv3x3(nn.Conv2d):
         """A_cat: the active down kernels stacked along the rank axis, zero-padded to a multiple of 32, in the conv
         kernel's [R,3,3,Cin] layout; B_cat [Cout,R] with each adapter's weight * alpha / rank * global scale folded in."""
         if self._lora is None:
-            names = [n for n in self.active if self.adapters_enabled]
+            names = [n for n in self.active if self.adapters_enabled and n not in self._fused]
             if not names:
                 self._lora = (None, None)
             else:
@@ -359,6 +411,77 @@ class Conv3x3(nn.Conv2d):
         return y2.view(nb, ho, wo, co).permute(0, 3, 1, 2)
 
 
+class Conv1x1(_ConvLoRAFuse, nn.Conv2d):
+    """1x1 convolution (the resnets' conv_shortcut) with the reference's LoRA on it: down [r,Cin,1,1], up [Cout,r,1,1]
+    (LoRAConv2dLayer, diffusers-hf/src/diffusers/models/lora.py:258-296; LoRACompatibleConv.forward :369-383).  On
+    channels_last bf16 GPU tensors it is a linear layer over the channels of every pixel and runs on the LoRA linear
+    kernel, adapters included; parameters and state-dict keys are nn.Conv2d's."""
+
+    def __init__(self, in_channels, out_channels):
+        super().__init__(in_channels, out_channels, 1)
+        self.adapters: Dict[str, Adapter] = {}
+        self.active: List[str] = []
+        self.adapters_enabled = True
+        self._global_scale = 1.0
+        self._packed = None       # PackedAdapters of the active adapters, False = none active
+        self._fused: Dict[str, float] = {}
+
+    def add_adapter(self, name: str, down: torch.Tensor, up: torch.Tensor, alpha: Optional[float] = None,
+                    weight: float = 1.0) -> None:
+        r = down.shape[0]
+        if down.numel() != r * self.in_channels or up.numel() != self.out_channels * r or up.shape[0] != self.out_channels:
+            raise ValueError(f"adapter {name!r}: expected down [r,{self.in_channels}(,1,1)] and up [{self.out_channels},r(,1,1)], "
+                             f"got {tuple(down.shape)} and {tuple(up.shape)}")
+        self.adapters[name] = Adapter(down.detach().reshape(r, self.in_channels), up.detach().reshape(self.out_channels, r),
+                                      alpha, weight)
+        self._packed = None
+
+    def delete_adapter(self, name: str) -> None:
+        self.adapters.pop(name, None)
+        self.active = [n for n in self.active if n != name]
+        self._packed = None
+
+    def set_active(self, names: Sequence[str], weights: Optional[Sequence[float]] = None) -> None:
+        self.active = [n for n in names if n in self.adapters]
+        if weights is not None:
+            for n, w in zip(names, weights):
+                if n in self.adapters:
+                    self.adapters[n].weight = float(w)
+        self._packed = None
+
+    def set_global_scale(self, scale: float) -> None:
+        if scale != self._global_scale:
+            self._global_scale = float(scale)
+            self._packed = None
+
+    def refresh_adapters(self) -> None:
+        self._packed = None
+
+    def _pack(self):
+        if self._packed is None:
+            names = [n for n in self.active if self.adapters_enabled and n not in self._fused]
+            self._packed = pack_adapters(self.adapters, names, self.in_channels, self.out_channels, self.weight.dtype,
+                                         self.weight.device, self._global_scale) if names else False
+        return self._packed or None
+
+    def forward(self, x):
+        if not (x.is_cuda and x.dtype == torch.bfloat16 and self.weight.dtype == torch.bfloat16
+                and self.in_channels % 32 == 0 and self.out_channels % 8 == 0):
+            if self.adapters and self.active:
+                raise NotImplementedError("LoRA on a 1x1 convolution needs the katz_hip kernels (bf16 GPU tensors)")
+            return super().forward(x)
+        x = x.contiguous(memory_format=torch.channels_last)
+        nb, c, hh, ww = x.shape
+        p = self._pack() if self.adapters else None
+        x2 = x.permute(0, 2, 3, 1).reshape(nb * hh * ww, c)
+        w2 = self.weight.reshape(self.out_channels, c)
+        if p is None:
+            y = ops.lora_linear(x2, w2, self.bias)
+        else:
+            y = ops.lora_linear(x2, w2, self.bias, p.a_cat, p.b_cat, p.col_scale)
+        return y.view(nb, hh, ww, self.out_channels).permute(0, 3, 1, 2)
+
+
 class Downsample2D(nn.Module):
     def __init__(self, channels, use_conv=True, out_channels=None, padding=1, name="op"):
         super().__init__()
@@ -401,18 +524,8 @@ class ResnetBlock2D(nn.Module):
         self.time_emb_proj = nn.Linear(temb_channels, out_channels)
         self.norm_silu2 = nn.Sequential(*fused_norm_silu(out_channels, groups, eps))
         self.conv2 = Conv3x3(out_channels, out_channels)
-        self.conv_shortcut = nn.Conv2d(in_channels, out_channels, 1) if in_channels != out_channels else None
+        self.conv_shortcut = Conv1x1(in_channels, out_channels) if in_channels != out_channels else None
         self.temb_proj = None   # this step's time_emb_proj(temb_act), when a TimeEmbProjector computed it ahead
-
-    def _shortcut(self, x):
-        """1x1 convolution = a linear layer over the channels of every pixel (NHWC rows)."""
-        sc = self.conv_shortcut
-        if not (x.is_cuda and x.dtype == torch.bfloat16 and x.is_contiguous(memory_format=torch.channels_last)
-                and sc.in_channels % 32 == 0 and sc.out_channels % 8 == 0):
-            return sc(x)
-        nb, c, hh, ww = x.shape
-        y = ops.lora_linear(x.permute(0, 2, 3, 1).reshape(nb * hh * ww, c), sc.weight.reshape(sc.out_channels, c), sc.bias)
-        return y.view(nb, hh, ww, sc.out_channels).permute(0, 3, 1, 2)
 
     def forward(self, input_tensor, temb_act):
         """temb_act = silu(temb), computed once per step by the caller."""
@@ -422,7 +535,7 @@ class ResnetBlock2D(nn.Module):
         tp, self.temb_proj = self.temb_proj, None
         h = self.norm_silu2[0](h, add_nc=self.time_emb_proj(temb_act) if tp is None else tp)
         if self.conv_shortcut is not None:
-            input_tensor = self._shortcut(input_tensor)
+            input_tensor = self.conv_shortcut(input_tensor)
         out = self.conv2(h, residual=input_tensor)   # input_tensor + conv2(h), the add in the conv's epilogue
         if self.output_scale_factor != 1.0:
             out = out / self.output_scale_factor

@@ -280,6 +280,51 @@ def lora_linear_split(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torc
     return out
 
 
+def lora_merge_grouped(weights: Sequence[torch.Tensor], ups: Sequence[torch.Tensor], downs: Sequence[torch.Tensor],
+                       scale: float = 1.0, layer_scales: Optional[Sequence[float]] = None) -> None:
+    """W_l += scale * layer_scales[l] * up_l @ down_l for all layers in ONE launch, in place (kh_lora_merge_grouped_bf16).
+    weights: contiguous bf16 [N,K] GPU tensors, each at most once; ups [N,r] / downs [r,K]: contiguous GPU tensors, all
+    bfloat16 or all float16, r <= 128.  Tensors derived from a weight notice the change through its version counter,
+    which is bumped here as an in-place torch op would."""
+    lib = _lib.load()
+    n = len(weights)
+    if n == 0:
+        return
+    if len(ups) != n or len(downs) != n or (layer_scales is not None and len(layer_scales) != n):
+        raise ValueError("weights, ups, downs (and layer_scales) must have one entry per layer")
+    dev = weights[0].device
+    op_dtype = ups[0].dtype
+    if op_dtype not in (BF16, torch.float16):
+        raise TypeError("adapter matrices must be bfloat16 or float16")
+    rows, starts, max_rank, seen = [], [0], 0, set()
+    for w, u, d in zip(weights, ups, downs):
+        if not w.is_cuda or w.dtype != BF16 or w.dim() != 2 or not w.is_contiguous() or w.device != dev:
+            raise ValueError("every weight must be a contiguous 2-D bfloat16 tensor on one GPU")
+        N, K = w.shape
+        r = d.shape[0]
+        for t, shape, name in ((u, (N, r), "up"), (d, (r, K), "down")):
+            if not t.is_cuda or t.device != dev or t.dtype != op_dtype or not t.is_contiguous() or tuple(t.shape) != shape:
+                raise ValueError(f"{name} must be a contiguous {op_dtype} {shape} tensor on {dev}, got {t.dtype} {tuple(t.shape)}")
+        if r < 1 or r > 128:
+            raise ValueError(f"rank {r} outside 1..128")
+        if w.data_ptr() in seen:
+            raise ValueError("a weight appears twice in one merge (the tiles of the two rows would race)")
+        seen.add(w.data_ptr())
+        rows.append((w.data_ptr(), u.data_ptr(), d.data_ptr(), N, K, r))
+        starts.append(starts[-1] + ((N + 127) // 128) * ((K + 127) // 128))
+        max_rank = max(max_rank, r)
+    table = torch.tensor(rows, dtype=torch.int64).to(dev, non_blocking=True)
+    tile_start = torch.tensor(starts, dtype=torch.int32).to(dev, non_blocking=True)
+    ls = None if layer_scales is None else torch.tensor(list(layer_scales), dtype=torch.float32).to(dev, non_blocking=True)
+    rc = lib.kh_lora_merge_grouped_bf16(_ptr(table), _ptr(tile_start), _ptr(ls), n, starts[-1], max_rank, float(scale),
+                                        1 if op_dtype == torch.float16 else 0, _stream())
+    _lib.check(rc, "kh_lora_merge_grouped_bf16")
+    for w in weights:
+        torch.autograd.graph.increment_version(w)
+    # the table tensors are freed when this returns: torch's caching allocator keeps the memory valid for work already
+    # enqueued on the current stream, which is where the kernel runs
+
+
 def lora_linear_grouped(x: torch.Tensor, table: torch.Tensor, M: int, N: int, K: int, R: int, ldt: int) -> None:
     """y_g = x W_g^T + b_g + t_g B_cat_g^T for every row {W, bias, B_cat, t, y} of the int64 device
     `table` [n_groups, 5] in one launch; the caller owns every buffer the table points to."""
@@ -589,7 +634,7 @@ def cfg_euler_step(noise_pred: torch.Tensor, latents: torch.Tensor, coef: torch.
 # --------------------------------------------------------------------------------------- per-launch timing
 KERNEL_TAGS = {1: "lora_gemm", 2: "lora_gemm_f32", 3: "attention", 4: "group_norm_stats", 5: "group_norm_apply",
                6: "layer_norm", 7: "geglu", 8: "residual_add", 9: "concat_residual", 10: "sgmv_shrink",
-               11: "sgmv_expand", 12: "lora_shrink", 13: "conv3x3", 14: "cfg_euler", 15: "upsample"}
+               11: "sgmv_expand", 12: "lora_shrink", 13: "conv3x3", 14: "cfg_euler", 15: "upsample", 16: "lora_merge"}
 
 
 def profile_begin() -> None:

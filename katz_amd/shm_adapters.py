@@ -108,29 +108,31 @@ KATZ_MERGE_SCALE = 20000.0 / 64.0   # alpha / rank, hard-coded in the reference 
 def patch_on_lora(unet, lora_state_dict: Mapping[str, torch.Tensor], key_match: Mapping[str, Mapping[str, str]],
                   scale: float = KATZ_MERGE_SCALE) -> int:
     """Katz's merge: for every matched UNet weight, W += (up @ down) * scale
-    (pipeline_controlnet_sd_xl_katz.py:1730-1747) on the GPU weights.  Each update is one launch of the LoRA GEMM
-    kernel with M = out, N = in, K = rank and the weight as the epilogue's residual, then a copy back into the
-    parameter (which also tells every cache derived from the weight that it changed).  The product is accumulated
-    in fp32 and rounded once (the reference rounds up @ down and the scaled product to fp16 first).
-    Returns the number of patched weights."""
+    (pipeline_controlnet_sd_xl_katz.py:1730-1747), in place on the GPU weights.  The adapter matrices are uploaded as
+    they are (float16 in Katz's shared-memory layout, or bfloat16) and ALL layers are merged by one launch of the
+    batched merge kernel (kh_lora_merge_grouped_bf16): products on the matrix cores in the adapters' own dtype, fp32
+    accumulation, W + scale * product rounded once (the reference rounds up @ down and the scaled product to fp16
+    first, and writes the result back with load_state_dict).  Returns the number of patched weights."""
     params = dict(unet.named_parameters())
-    done = 0
+    ws, ups, downs = [], [], []
+    for wkey, m in key_match.items():
+        if wkey not in params:
+            raise KeyError(f"{wkey} is not a parameter of the UNet")
+        w = params[wkey]
+        if not w.is_cuda or w.dtype != torch.bfloat16 or w.dim() != 2 or not w.is_contiguous():
+            raise ValueError(f"{wkey}: patch_on_lora needs a contiguous 2-D bfloat16 GPU weight")
+        down, up = lora_state_dict[m["lora_down_key"]], lora_state_dict[m["lora_up_key"]]
+        n_out, n_in = w.shape
+        r = down.shape[0]
+        if down.shape != (r, n_in) or up.shape != (n_out, r):
+            raise ValueError(f"{wkey}: adapter shapes {tuple(up.shape)} x {tuple(down.shape)} do not match {tuple(w.shape)}")
+        if down.dtype not in (torch.float16, torch.bfloat16):
+            down, up = down.to(torch.bfloat16), up.to(torch.bfloat16)
+        ws.append(w.data)
+        downs.append(down.to(w.device, non_blocking=True).contiguous())
+        ups.append(up.to(w.device, non_blocking=True).contiguous())
     with torch.no_grad():
-        for wkey, m in key_match.items():
-            if wkey not in params:
-                raise KeyError(f"{wkey} is not a parameter of the UNet")
-            w = params[wkey]
-            if not w.is_cuda or w.dtype != torch.bfloat16 or w.dim() != 2 or not w.is_contiguous():
-                raise ValueError(f"{wkey}: patch_on_lora needs a contiguous 2-D bfloat16 GPU weight")
-            down = lora_state_dict[m["lora_down_key"]].to(w.device, non_blocking=True)
-            up = lora_state_dict[m["lora_up_key"]].to(w.device, non_blocking=True)
-            n_out, n_in = w.shape
-            r = down.shape[0]
-            if down.shape != (r, n_in) or up.shape != (n_out, r):
-                raise ValueError(f"{wkey}: adapter shapes {tuple(up.shape)} x {tuple(down.shape)} do not match {tuple(w.shape)}")
-            pad = -r % 32
-            x = torch.nn.functional.pad(up.float() * scale, (0, pad)).to(torch.bfloat16).contiguous()       # [out, r']
-            bt = torch.nn.functional.pad(down.t().float(), (0, pad)).to(torch.bfloat16).contiguous()         # [in, r']
-            w.copy_(ops.lora_linear(x, bt, None, residual=w.data))
-            done += 1
-    return done
+        ops.lora_merge_grouped(ws, ups, downs, scale=scale)
+    for wkey in key_match:
+        torch.autograd.graph.increment_version(params[wkey])   # `.data` above is a separate version counter
+    return len(ws)

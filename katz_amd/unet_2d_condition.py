@@ -227,10 +227,11 @@ class UNet2DConditionModel(nn.Module):
     def lora_linears(self) -> Dict[str, LoRALinear]:
         return {n: m for n, m in self.named_modules() if isinstance(m, LoRALinear)}
 
-    def lora_convs(self) -> Dict[str, "Conv3x3"]:
-        """3x3 convolutions that can carry a LoRA (resnet conv1 / conv2, down / upsampler convs)."""
-        from .layers import Conv3x3
-        return {n: m for n, m in self.named_modules() if isinstance(m, Conv3x3)}
+    def lora_convs(self) -> Dict[str, Any]:
+        """Convolutions that can carry a LoRA: 3x3 (resnet conv1 / conv2, down / upsampler convs) and the resnets' 1x1
+        conv_shortcut."""
+        from .layers import Conv1x1, Conv3x3
+        return {n: m for n, m in self.named_modules() if isinstance(m, (Conv3x3, Conv1x1))}
 
     def _lora_targets(self) -> Dict[str, Any]:
         return {**self.lora_linears(), **self.lora_convs()}
@@ -315,14 +316,21 @@ class UNet2DConditionModel(nn.Module):
             m.adapters_enabled = True
             m.refresh_adapters()
 
-    def fuse_lora(self, lora_scale: float = 1.0, adapter_names: Optional[Sequence[str]] = None) -> None:
-        if any(c.adapters for c in self.lora_convs().values()):
-            raise NotImplementedError("fusing adapters that target convolutions is not implemented; run them unfused")
-        # all layers or none: a layer whose merged weight is not finite raises (the reference's safe_fusing check,
-        # models/lora.py:416-421); the layers merged before it get their weights back bit for bit
+    def fuse_lora(self, lora_scale: float = 1.0, adapter_names: Optional[Sequence[str]] = None,
+                  safe_fusing: bool = False) -> None:
+        """W += lora_scale * weight_i * alpha_i / rank_i * B_i A_i for the named (default: active) adapters of every
+        target (fuse_lora, diffusers-hf/src/diffusers/loaders/unet.py:514-550 -> _fuse_lora, models/lora.py:403-433,
+        :258-296 for convolutions).  safe_fusing=False (the reference's default): all linear layers in one launch per
+        adapter of the batched merge kernel.  safe_fusing=True: layer by layer in fp32 with the reference's finite
+        check (:416-421), all layers or none -- a layer that fails raises and the layers merged before it get their
+        weights back bit for bit."""
+        if not safe_fusing and self._merge_grouped(lora_scale, adapter_names):
+            for c in self.lora_convs().values():
+                c.fuse(lora_scale, adapter_names)
+            return
         done = []
         try:
-            for m in self.lora_linears().values():
+            for m in self._lora_targets().values():
                 names = list(m.active if adapter_names is None else adapter_names)
                 cand = m._fuse_candidate(lora_scale, names)
                 if cand is not None:
@@ -336,8 +344,52 @@ class UNet2DConditionModel(nn.Module):
                     m.refresh_adapters()
             raise
 
+    def _merge_grouped(self, lora_scale: float, adapter_names: Optional[Sequence[str]], undo: bool = False) -> bool:
+        """Fuse (or, with undo, unfuse) the adapters of all LoRALinear layers with the batched merge kernel; False when
+        the weights are not bf16 on a GPU (the caller then takes the per-layer path)."""
+        lin = list(self.lora_linears().values())
+        if not lin or any((not m.weight.is_cuda) or m.weight.dtype != torch.bfloat16 for m in lin):
+            return False
+        rounds: List[List[tuple]] = []      # round k: the k-th adapter to merge of every layer (a weight once per launch)
+        for m in lin:
+            if undo:
+                todo = list(m._fused.items())
+            else:
+                names = list(m.active if adapter_names is None else adapter_names)
+                todo, seen = [], set()
+                for n in names:
+                    if n in m.adapters and n not in m._fused and n not in seen:
+                        todo.append((n, lora_scale * m.adapters[n].multiplier(1.0)))
+                        seen.add(n)
+            for k, (n, mult) in enumerate(todo):
+                if len(rounds) <= k:
+                    rounds.append([])
+                rounds[k].append((m, n, mult))
+        dev = lin[0].weight.device
+        with torch.no_grad():
+            for rnd in rounds:
+                ops.lora_merge_grouped([m.weight.data for m, _, _ in rnd],
+                                       [m.adapters[n].up.to(dev, torch.bfloat16).contiguous() for m, n, _ in rnd],
+                                       [m.adapters[n].down.to(dev, torch.bfloat16).contiguous() for m, n, _ in rnd],
+                                       scale=-1.0 if undo else 1.0, layer_scales=[mult for _, _, mult in rnd])
+        for m in lin:
+            torch.autograd.graph.increment_version(m.weight)
+        for rnd in rounds:
+            for m, n, mult in rnd:
+                if undo:
+                    m._fused.pop(n, None)
+                else:
+                    m._fused[n] = mult
+        for m in lin:
+            m.refresh_adapters()
+        return True
+
     def unfuse_lora(self) -> None:
-        for m in self.lora_linears().values():
+        if self._merge_grouped(1.0, None, undo=True):
+            for c in self.lora_convs().values():
+                c.unfuse()
+            return
+        for m in self._lora_targets().values():
             m.unfuse()
 
     def unload_lora(self) -> None:
@@ -348,6 +400,8 @@ class UNet2DConditionModel(nn.Module):
                 m.delete_adapter(n)
             m.refresh_adapters()
         for c in self.lora_convs().values():
+            if c._fused:
+                c.unfuse()
             for n in list(c.adapters):
                 c.delete_adapter(n)
 

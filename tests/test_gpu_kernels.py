@@ -677,6 +677,49 @@ def test_conv3x3_with_lora_adapters(stride):
         assert_close_rel(y_dis, base, REL_BF16, "conv, adapters disabled")
 
 
+def test_conv1x1_with_lora_and_conv_fuse():
+    """The resnets' 1x1 conv_shortcut with two LoRA adapters (LoRAConv2dLayer, models/lora.py:258-296) against the
+    oracle, and fuse / unfuse of 1x1 and 3x3 conv adapters (merged kernel, :403-441): fused == unfused == oracle."""
+    from katz_amd.layers import Conv1x1, Conv3x3
+
+    say("conv1x1 lora + conv fuse")
+    d = dev()
+    g = torch.Generator().manual_seed(23)
+    cin, cout = 64, 128
+    x = randn(g, 2, cin, 12, 10).to(BF)
+    xd = x.to(d).contiguous(memory_format=torch.channels_last)
+    for cls, k in ((Conv1x1, 1), (Conv3x3, 3)):
+        conv = cls(cin, cout)
+        with torch.no_grad():
+            conv.weight.copy_(randn(g, cout, cin, k, k, std=(k * k * cin) ** -0.5).to(BF).float())
+            conv.bias.copy_(randn(g, cout).to(BF).float())
+        w, b = conv.weight.detach().clone(), conv.bias.detach().clone()
+        conv = conv.to(d, BF)
+        ads = [(randn(g, 8, cin, k, k, std=0.08).to(BF).float(), randn(g, cout, 8, 1, 1, std=0.08).to(BF).float(), 16.0, 0.8),
+               (randn(g, 4, cin, k, k, std=0.08).to(BF).float(), randn(g, cout, 4, 1, 1, std=0.08).to(BF).float(), None, 0.6)]
+        for i, (A, B, alpha, wgt) in enumerate(ads):
+            conv.add_adapter(f"a{i}", A, B, alpha)
+        conv.set_active(["a0", "a1"], [0.8, 0.6])
+        oracle_ads = [(ads[0][0], ads[0][1], 0.8 * 16.0 / 8), (ads[1][0], ads[1][1], 0.6)]
+        with torch.no_grad():
+            ref = O.lora_conv2d(x.float(), w, b, oracle_ads, padding=k // 2)
+            base = O.lora_conv2d(x.float(), w, b, [], padding=k // 2)
+            y = conv(xd)
+            assert_close_rel(y, ref, REL_BF16, f"conv{k}x{k} + lora")
+            assert (ref - base).abs().max() > 0.05
+            conv.fuse()
+            assert set(conv._fused) == {"a0", "a1"}
+            merged = w + sum(s * (B.reshape(cout, -1) @ A.reshape(A.shape[0], -1)).reshape(w.shape) for A, B, s in oracle_ads)
+            assert_close_rel(conv.weight.float().cpu(), merged, 1e-2, "merged conv weight")
+            yf = conv(xd)
+            assert_close_rel(yf, ref, REL_BF16, f"conv{k}x{k} fused")
+            conv.unfuse()
+            assert_close_rel(conv.weight.float().cpu(), w, 1e-2, "unfused conv weight")
+            assert_close_rel(conv(xd), ref, REL_BF16, f"conv{k}x{k} unfused again")
+            conv.set_active([])
+            assert_close_rel(conv(xd), base, REL_BF16, f"conv{k}x{k} without adapters")
+
+
 @pytest.mark.parametrize("cin,cout", [(4, 64), (64, 4), (3, 16), (16, 32)])
 def test_conv3x3_module_pads_small_channel_counts(cin, cout):
     """Conv3x3 on the katz_hip kernel for the UNet's conv_in / conv_out and the ControlNet's image embedding:
@@ -991,3 +1034,78 @@ def test_lora_linear_split_rank_padding_promise(case):
     with pytest.raises(Exception):
         ops.lora_linear_split(xd, wd, None, Ad, cs, Bd, geglu=geglu, n_split=n_split, r_used=R + 16)
     ops.split_counters_reset(d)
+
+
+# ------------------------------------------------------------------------------------------- batched merge
+@pytest.mark.parametrize("op_dtype", [torch.float16, torch.bfloat16], ids=str)
+def test_lora_merge_grouped(op_dtype):
+    """kh_lora_merge_grouped_bf16: W_l += scale * s_l * up_l @ down_l for several layers of different shapes and ranks in
+    one launch, against the oracle's merged weight (models/lora.py:409-425; Katz's patch_on_lora,
+    pipeline_controlnet_sd_xl_katz.py:1743-1746); ragged sizes, rank 4 .. 128, fp16 (Katz's shared-memory dtype) and
+    bf16 operands; a negative scale undoes the merge up to one rounding; weights not in the table are untouched."""
+    from katz_amd import ops
+
+    say("lora_merge_grouped", op_dtype)
+    d = dev()
+    g = torch.Generator().manual_seed(77)
+    shapes = [(1280, 1280, 64), (640, 2048, 16), (10240, 1280, 128), (1280, 5120, 4), (200, 136, 24), (130, 60, 7), (64, 64, 64)]
+    ws, ups, downs, scales = [], [], [], []
+    for N, K, r in shapes:
+        ws.append(randn(g, N, K, std=0.03).to(BF))
+        ups.append(randn(g, N, r, std=0.2).to(op_dtype))
+        downs.append(randn(g, r, K, std=0.2).to(op_dtype))
+        scales.append(0.25 + 0.5 * len(scales))
+    bystander = randn(g, 256, 256).to(d, BF)
+    keep = bystander.clone()
+    wd = [w.to(d).clone() for w in ws]
+    v0 = [w._version for w in wd]
+    ops.lora_merge_grouped(wd, [u.to(d) for u in ups], [x.to(d) for x in downs], scale=0.7, layer_scales=scales)
+    torch.cuda.synchronize()
+    assert all(w._version > v for w, v in zip(wd, v0))
+    for w0, w1, u, x, s in zip(ws, wd, ups, downs, scales):
+        ref = O.lora_merged_weight(w0.float(), [(x.float(), u.float(), 0.7 * s)])
+        assert_close_rel(w1, ref, 4e-3, f"merged weight {tuple(w0.shape)}")     # one bf16 rounding of the sum
+        assert (ref - w0.float()).abs().max() > 0.05
+    assert torch.equal(bystander, keep)
+    ops.lora_merge_grouped(wd, [u.to(d) for u in ups], [x.to(d) for x in downs], scale=-0.7, layer_scales=scales)
+    torch.cuda.synchronize()
+    for w0, w1, u, x, sc in zip(ws, wd, ups, downs, scales):
+        # the merged weight was rounded to bf16 at ITS magnitude: undoing restores W up to that rounding
+        merged_max = O.lora_merged_weight(w0.float(), [(x.float(), u.float(), 0.7 * sc)]).abs().max().item()
+        assert (w1.float().cpu() - w0.float()).abs().max().item() <= 2.0 ** -7 * merged_max, tuple(w0.shape)
+    with pytest.raises(ValueError):
+        ops.lora_merge_grouped([wd[0], wd[0]], [ups[0].to(d)] * 2, [downs[0].to(d)] * 2)
+    with pytest.raises(ValueError):
+        ops.lora_merge_grouped([wd[0]], [ups[1].to(d)], [downs[0].to(d)])
+
+
+def test_unet_fuse_lora_through_the_batched_merge():
+    """UNet.fuse_lora / unfuse_lora on the GPU (safe_fusing=False: one merge launch per adapter over all linear layers)
+    give the weights of the per-layer fp32 path (safe_fusing=True) and mark the same adapters as fused."""
+    import katz_amd.layers as L
+    from katz_amd.unet_2d_condition import UNet2DConditionModel, UNetConfig
+
+    say("fuse_lora grouped")
+    torch.manual_seed(0)
+    unet = UNet2DConditionModel(UNetConfig.tiny()).to_runtime(dev(), BF)
+    g = torch.Generator().manual_seed(5)
+    lin = unet.lora_linears()
+    for name, rank in (("a", 8), ("b", 4)):
+        for m in lin.values():
+            m.add_adapter(name, randn(g, rank, m.in_features, std=0.05).to(dev(), BF), randn(g, m.out_features, rank, std=0.05).to(dev(), BF), alpha=2.0 * rank)
+    unet.set_adapters(["a", "b"], [0.8, 0.6])
+    w0 = {n: m.weight.detach().clone() for n, m in lin.items()}
+    unet.fuse_lora(0.5)
+    fast = {n: m.weight.detach().clone() for n, m in lin.items()}
+    assert all(m._fused == {"a": 0.5 * 0.8 * 2.0, "b": 0.5 * 0.6 * 2.0} for m in lin.values())
+    assert all(m._packed is None for m in lin.values())          # fused adapters are not applied a second time
+    unet.unfuse_lora()
+    assert not any(m._fused for m in lin.values())
+    for n, m in lin.items():
+        assert_close_rel(m.weight, w0[n].float().cpu(), 2e-2, f"unfused {n}")   # two bf16 roundings of the merged weight
+        with torch.no_grad():
+            m.weight.copy_(w0[n])
+    unet.fuse_lora(0.5, safe_fusing=True)
+    for n, m in lin.items():
+        assert_close_rel(fast[n], m.weight.float().cpu(), 8e-3, f"grouped vs per-layer fuse {n}")
+        assert (m.weight.float() - w0[n].float()).abs().max() > 1e-3

@@ -271,8 +271,23 @@ def test_kohya_conversion_reproduces_the_reference_key_list():
         "lora_unet_down_blocks_1_attentions_0_transformer_blocks_0_attn2_to_out_0.lora_up.weight": torch.zeros(640, 4)})
     assert set(u2) == {"unet.down_blocks.1.attentions.0.transformer_blocks.0.attn2.processor.to_out_lora.down.weight",
                        "unet.down_blocks.1.attentions.0.transformer_blocks.0.attn2.processor.to_out_lora.up.weight"}
-    with pytest.raises(NotImplementedError):
-        convert_kohya_lora_to_diffusers({"lora_unet_input_blocks_4_0_in_layers_2.lora_down.weight": torch.zeros(4, 4)})
+    # convolution targets: the renames of lora_conversion_utils.py:78-118 (block numbering) and :178-186 (layer names)
+    conv_names = {"input_blocks_4_0_in_layers_2": "down_blocks.1.resnets.0.conv1",
+                  "input_blocks_5_0_out_layers_3": "down_blocks.1.resnets.1.conv2",
+                  "input_blocks_4_0_skip_connection": "down_blocks.1.resnets.0.conv_shortcut",
+                  "input_blocks_3_0_op": "down_blocks.0.downsamplers.0.conv",
+                  "output_blocks_2_2_conv": "up_blocks.0.upsamplers.0.conv",
+                  "output_blocks_5_0_skip_connection": "up_blocks.1.resnets.2.conv_shortcut",
+                  "middle_block_0_in_layers_2": "mid_block.resnets.0.conv1",
+                  "middle_block_2_out_layers_3": "mid_block.resnets.1.conv2"}
+    csd = {}
+    for kn in conv_names:
+        csd[f"lora_unet_{kn}.lora_down.weight"] = torch.zeros(4, 4)
+        csd[f"lora_unet_{kn}.lora_up.weight"] = torch.zeros(4, 4)
+    u3, _, _ = convert_kohya_lora_to_diffusers(csd)
+    assert set(u3) == {f"unet.{v}.lora.{w}.weight" for v in conv_names.values() for w in ("down", "up")}
+    with pytest.raises(NotImplementedError):   # a resnet's time_emb_proj carries no LoRA here
+        convert_kohya_lora_to_diffusers({"lora_unet_input_blocks_4_0_emb_layers_1.lora_down.weight": torch.zeros(4, 4)})
     with pytest.raises(ValueError):
         convert_kohya_lora_to_diffusers({"lora_unet_middle_block_1_proj_in.lora_down.weight": torch.zeros(4, 4)})
 
@@ -292,21 +307,18 @@ def test_kohya_conversion_reproduces_the_reference_key_list():
 
 
 def test_unet_lora_surface_reaches_convolutions():
-    """Adapters that target 3x3 convolutions (diffusers key spelling) register on the Conv3x3 modules and follow
-    set_adapters / delete_adapters like the linear ones; fusing them is refused loudly."""
+    """Adapters that target convolutions (diffusers key spelling; 3x3 and the 1x1 conv_shortcut) register on the
+    Conv3x3 / Conv1x1 modules and follow set_adapters / fuse_lora / delete_adapters like the linear ones."""
     import pytest
     import torch
     import katz_amd.layers as L
     from katz_amd.unet_2d_condition import UNet2DConditionModel, UNetConfig
 
-    L.SKIP_INIT = True
-    try:
-        unet = UNet2DConditionModel(UNetConfig.tiny())
-    finally:
-        L.SKIP_INIT = False
+    torch.manual_seed(0)
+    unet = UNet2DConditionModel(UNetConfig.tiny())     # initialised weights: fuse checks the merged weights are finite
     convs = unet.lora_convs()
     assert "down_blocks.0.resnets.0.conv1" in convs and "down_blocks.0.downsamplers.0.conv" in convs
-    assert "conv_in" in convs and "down_blocks.1.resnets.0.conv_shortcut" not in convs   # 1x1 shortcuts carry no LoRA
+    assert "conv_in" in convs and "down_blocks.1.resnets.0.conv_shortcut" in convs
     c = convs["down_blocks.0.resnets.0.conv1"]
     lin_name = "down_blocks.1.attentions.0.transformer_blocks.0.attn1.to_q"
     lin = unet.lora_linears()[lin_name]
@@ -320,14 +332,35 @@ def test_unet_lora_surface_reaches_convolutions():
     assert c.adapters["locon"].weight == 0.5 and c.adapters["locon"].multiplier() == 0.5 * 8.0 / 4
     unet.set_adapters(["locon"], [{"down": 0.3}])      # block dictionaries address transformers; the conv keeps 1.0
     assert lin.adapters["locon"].weight == 0.3 and c.adapters["locon"].weight == 1.0
-    with pytest.raises(NotImplementedError):
-        unet.fuse_lora()
+    # the 1x1 shortcut takes [r,Cin,1,1] / [Cout,r,1,1] (LoRAConv2dLayer, models/lora.py:258-296); wrong shapes are refused
+    sc = convs["down_blocks.1.resnets.0.conv_shortcut"]
+    g = torch.Generator().manual_seed(0)
+    unet.load_lora_into_unet({"unet.down_blocks.1.resnets.0.conv_shortcut.lora.down.weight": torch.randn(4, 64, 1, 1, generator=g),
+                              "unet.down_blocks.1.resnets.0.conv_shortcut.lora.up.weight": torch.randn(128, 4, 1, 1, generator=g)},
+                             adapter_name="short")
+    assert sc.active == ["short"] and sc.adapters["short"].down.shape == (4, 64)
     with pytest.raises(ValueError):
-        unet.load_lora_into_unet({"unet.down_blocks.1.resnets.0.conv_shortcut.lora.down.weight": torch.zeros(4, 64, 1, 1),
+        unet.load_lora_into_unet({"unet.down_blocks.1.resnets.0.conv_shortcut.lora.down.weight": torch.zeros(4, 32, 1, 1),
                                   "unet.down_blocks.1.resnets.0.conv_shortcut.lora.up.weight": torch.zeros(128, 4, 1, 1)},
                                  adapter_name="bad")
-    unet.delete_adapters("locon")
-    assert not c.adapters and not lin.adapters
+    # fusing merges conv adapters through the merged-kernel identity (models/lora.py:403-421) and unfusing restores
+    with torch.no_grad():
+        c.adapters["locon"].down.copy_(torch.randn(c.adapters["locon"].down.shape, generator=g) * 0.1)
+        c.adapters["locon"].up.copy_(torch.randn(c.adapters["locon"].up.shape, generator=g) * 0.1)
+    unet.set_adapters(["locon", "short"], [0.5, 2.0])
+    w_c, w_sc = c.weight.detach().clone(), sc.weight.detach().clone()
+    unet.fuse_lora(lora_scale=0.7)
+    ad = c.adapters["locon"]
+    want = w_c + 0.7 * 0.5 * 8.0 / 4 * (ad.up.reshape(c.out_channels, -1) @ ad.down.reshape(4, -1)).reshape(w_c.shape)
+    assert torch.allclose(c.weight, want, atol=1e-5) and c._fused == {"locon": 0.7 * 0.5 * 8.0 / 4}
+    ads = sc.adapters["short"]
+    want = w_sc + 0.7 * 2.0 * (ads.up @ ads.down).reshape(w_sc.shape)
+    assert torch.allclose(sc.weight, want, atol=1e-5)
+    assert c._lora_pack() == (None, None) and sc._pack() is None       # fused adapters are not applied a second time
+    unet.unfuse_lora()
+    assert torch.allclose(c.weight, w_c, atol=1e-5) and torch.allclose(sc.weight, w_sc, atol=1e-5) and not c._fused
+    unet.delete_adapters(["locon", "short"])
+    assert not c.adapters and not lin.adapters and not sc.adapters
 
 
 def test_fuse_that_fails_leaves_everything_as_it_was():
