@@ -149,7 +149,8 @@ int kh_lora_linear_f32(const float* x, const float* w, const float* bias, const 
  * t [rows_total, RP]; adapter_rank[a] = rank rounded up to a multiple of 32 (zero padded), RP <= 128.
  * seg_start (n_segments+1), seg_adapter, adapter_rank: device int32; adapter_scale: device float.
  * max_seg_rows = longest segment (sizes the grid).
- *   shrink: t[rows, 0:r] = x[rows,:] A_a^T          expand: y[rows,:] += scale_a * t[rows,0:r] B_a^T */
+ *   shrink: t[rows, 0:r] = x[rows,:] A_a^T          expand: y[rows,:] += scale_a * t[rows,0:r] B_a^T
+ * with r = adapter_rank[a]; the shrink leaves the columns t[rows, r:RP] as they were (the expand never reads them). */
 int kh_sgmv_shrink_bf16(const void* x, const void* a_all, void* t, const int32_t* seg_start,
                         const int32_t* seg_adapter, const int32_t* adapter_rank, int64_t n_segments,
                         int64_t max_seg_rows, int64_t K, int64_t RP, void* stream);

@@ -316,6 +316,7 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
   }
   float oscale = 1.f;   // segmented expand: the adapter's scale on the product
   int k_cols = p.K;     // K columns the loop covers (the row stride stays p.K)
+  int n_store = p.N;    // output columns that are written (segmented shrink: the adapter's rank, not the padded maximum)
   if (pin.sg_mode != 0) {
     const int sg = blockIdx.y;
     const int r0 = pin.sg_start[sg], r1 = pin.sg_start[sg + 1], ad = pin.sg_adapter[sg];
@@ -328,6 +329,8 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
       p.res = p.y;                    // read-modify-write of y: every element is read and written by one thread
       oscale = pin.sg_scale[ad];
       k_cols = pin.sg_rank[ad];
+    } else {
+      n_store = pin.sg_rank[ad] < p.N ? pin.sg_rank[ad] : p.N;   // the expand reads t[:, 0:rank] only
     }
   }
   constexpr int BM = C::BM, BN = C::BN, TM = C::TM, TN = C::TN, NRT = C::NRT, R = C::R, NST = C::NST;
@@ -570,7 +573,7 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
         for (int q = 0; q < ECH; ++q) {
           const int c = tid + q * C::NT, srow = c / CPR, ch = c % CPR;
           const int grow = m0 + (srow >> 5) * C::WTM + i * 32 + (srow & 31), gcol = n0 + ch * 8;
-          if (grow < M && gcol < N) {
+          if (grow < M && gcol < n_store) {
             u32x4 o = *reinterpret_cast<const u32x4*>(sC + srow * C::LDC + ch * 8);
             if (p.res != nullptr) {
 #pragma unroll
@@ -748,6 +751,7 @@ int lora_gemm_pipe_launch_conv(const LoraGemmParams& p, hipStream_t stream) {
 int lora_gemm_pipe_launch_sgmv(const LoraGemmParams& p, int n_segments, hipStream_t stream) {
   // one 128x128 tile column covers all of a shrink's rank columns.  The shrink streams long rows: whole 128-byte
   // lines per stage and 8 waves per workgroup; the expand's K is the rank (a few 32-column tiles).
+  // (64-row tiles at two workgroups per CU were measured for the shrink: 15.7 against 12.2 us on 8 x 4096 x 640)
   if (p.sg_mode == 1 && p.K % 64 == 0) return launch_pcfg<PCfg<128, 128, 2, 4, 0, 3, 64>>(p, stream, n_segments);
   return launch_pcfg<PCfg<128, 128, 2, 2, 0, 4>>(p, stream, n_segments);
 }

@@ -20,7 +20,8 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
 constexpr int MG_BM = 128, MG_BN = 128, MG_THREADS = 256;
 constexpr int MG_RMAX = 128;                 // largest rank (one pass holds the whole rank axis in LDS)
-constexpr int MG_LDD = MG_BN + 2;            // sD row stride (elements): column reads of 2 bytes, rows 4 bytes apart in banks
+constexpr int MG_LDD = MG_BN + 4;            // sD row stride (elements): rows 8-byte aligned; the 8 rows a column read spans
+                                             // between the two wave halves fall 16 banks apart
 
 struct MergeRow {       // one layer; mirrors the six 64-bit words of the table in include/katz_hip.h
   uint64_t w, up, down; // device addresses: W [N,K] bf16, up [N,r], down [r,K]
@@ -69,13 +70,34 @@ __global__ __launch_bounds__(MG_THREADS) void lora_merge_kernel(const MergeRow* 
   bf16_t* W = reinterpret_cast<bf16_t*>(L.w);
   const int rp = (r + 15) & ~15;   // this layer's rank in whole MFMA steps, the excess zero-filled
 
-  for (int i = tid; i < MG_BM * rp; i += MG_THREADS) {         // coalesced along the rank axis
-    const int row = i / rp, k = i % rp;
-    sU[row * ldu + k] = (m0 + row < N && k < r) ? up[(size_t)(m0 + row) * L.r + k] : (uint16_t)0;
-  }
-  for (int i = tid; i < rp * MG_BN; i += MG_THREADS) {         // coalesced along W's columns
-    const int k = i / MG_BN, col = i % MG_BN;
-    sD[k * MG_LDD + col] = (k < r && n0 + col < K) ? down[(size_t)k * K + n0 + col] : (uint16_t)0;
+  // 16-byte pieces where the layer allows it (r % 8 == 0, K % 8 == 0, aligned bases: every linear of the UNet), else
+  // element by element
+  const bool fast = (L.r & 7) == 0 && (K & 7) == 0 && ((L.up | L.down) & 15) == 0;
+  if (fast) {
+    const int upr = rp / 8;                                     // pieces per up row
+    for (int i = tid; i < MG_BM * upr; i += MG_THREADS) {
+      const int row = i / upr, k = (i % upr) * 8;
+      u32x4 v = u32x4{0, 0, 0, 0};
+      if (m0 + row < N && k < r) v = *reinterpret_cast<const u32x4*>(up + (size_t)(m0 + row) * L.r + k);
+      *reinterpret_cast<u32x4*>(sU + row * ldu + k) = v;
+    }
+    for (int i = tid; i < rp * (MG_BN / 8); i += MG_THREADS) {
+      const int k = i / (MG_BN / 8), col = (i % (MG_BN / 8)) * 8;
+      u32x4 v = u32x4{0, 0, 0, 0};
+      if (k < r && n0 + col < K) v = *reinterpret_cast<const u32x4*>(down + (size_t)k * K + n0 + col);
+      u32x2* dst = reinterpret_cast<u32x2*>(sD + k * MG_LDD + col);
+      dst[0] = u32x2{v[0], v[1]};
+      dst[1] = u32x2{v[2], v[3]};
+    }
+  } else {
+    for (int i = tid; i < MG_BM * rp; i += MG_THREADS) {
+      const int row = i / rp, k = i % rp;
+      sU[row * ldu + k] = (m0 + row < N && k < r) ? up[(size_t)(m0 + row) * L.r + k] : (uint16_t)0;
+    }
+    for (int i = tid; i < rp * MG_BN; i += MG_THREADS) {
+      const int k = i / MG_BN, col = i % MG_BN;
+      sD[k * MG_LDD + col] = (k < r && n0 + col < K) ? down[(size_t)k * K + n0 + col] : (uint16_t)0;
+    }
   }
   __syncthreads();
 
