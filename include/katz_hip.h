@@ -41,7 +41,7 @@ const char* kh_error_string(int code);
  * kh_profile_begin and kh_profile_end every kernel of this library is launched with its own HIP
  * start/stop event pair on the launch stream.  kh_profile_end waits for them and writes, in launch
  * order, a kernel tag (1 lora_gemm, 2 lora_gemm_f32, 3 attention, 4 group_norm stats, 5 group_norm apply,
- * 6 layer_norm, 7 geglu, 8 residual_add, 9 concat_residual, 10 sgmv_shrink, 11 sgmv_expand, 12 lora_shrink, 13 conv3x3, 14 cfg_euler, 15 upsample, 16 lora_merge) and the
+ * 6 layer_norm, 7 geglu, 8 residual_add, 9 concat_residual, 10 sgmv_shrink, 11 sgmv_expand, 12 lora_shrink, 13 conv3x3, 14 cfg_euler, 15 upsample, 16 lora_merge, 17 conv_out + guidance + Euler) and the
  * duration in ms into HOST arrays; returns the number of launches (or -hipError_t).  Do not use under
  * graph capture. */
 int kh_profile_begin(void);
@@ -250,6 +250,19 @@ int kh_conv3x3_nhwc_bf16(const void* x, const void* w, const void* bias, const v
  * latents_out may equal latents (update in place); model_input_next must not overlap noise_pred. */
 int kh_cfg_euler_step_bf16(const void* noise_pred, const void* latents, void* latents_out, void* model_input_next,
                            int64_t n, float guidance_scale, const float* coef, int latents_f32, void* stream);
+
+/* The UNet's last convolution with the guidance + Euler step above as its epilogue: the whole tail of a denoising
+ * step, from the output of conv_norm_silu to the next step's model input, in one launch.
+ *   noise_pred = conv3x3(x, w) + bias          conv_out, unet_2d_condition.py:1327-1331 (4 output channels, padding 1)
+ *   then exactly kh_cfg_euler_step_bf16 on noise_pred rounded to bf16 (the model's output dtype).
+ * x: NHWC [2*Bl, H, W, Cin] bf16, rows 0..Bl-1 unconditional, Bl..2Bl-1 text-conditioned (the reference's
+ * torch.cat([latents] * 2) order, pipeline :1565); w [4,3,3,Cin] (the nn.Conv2d weight permuted to O,KH,KW,I);
+ * bias bf16 [4] or NULL; latents / latents_out [Bl,H,W,4] in NHWC memory, bf16 or fp32 (latents_f32), may be the same
+ * buffer; model_input_next [2*Bl,H,W,4] bf16 or NULL; noise_pred_out [2*Bl,H,W,4] bf16 or NULL (for callers that
+ * want the UNet's output as well); coef as for kh_cfg_euler_step_bf16.  Cin % 16 == 0. */
+int kh_conv_out_cfg_euler_bf16(const void* x, const void* w, const void* bias, const void* latents, void* latents_out,
+                               void* model_input_next, void* noise_pred_out, int64_t Bl, int64_t H, int64_t W,
+                               int64_t Cin, float guidance_scale, const float* coef, int latents_f32, void* stream);
 
 #ifdef __cplusplus
 }

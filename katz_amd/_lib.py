@@ -42,6 +42,7 @@ SIGNATURES = {
     "kh_concat_residual_bf16": (c_int, [_P, _P, _P, c_int, c_float, _P, _I, _I, _I, _P]),
     "kh_upsample_nearest2x_nhwc_bf16": (c_int, [_P, _P, _I, _I, _I, _I, _P]),
     "kh_cfg_euler_step_bf16": (c_int, [_P, _P, _P, _P, _I, c_float, _P, c_int, _P]),
+    "kh_conv_out_cfg_euler_bf16": (c_int, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, c_float, _P, c_int, _P]),
     "kh_conv3x3_nhwc_bf16": (c_int, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]),
 }
 

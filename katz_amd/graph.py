@@ -92,6 +92,10 @@ class GraphedDenoiseStep:
     graph) and one fp32 row {sigma_i, sigma_{i+1}, sqrt(sigma_{i+1}^2 + 1), sqrt(sigma_i^2 + 1), timestep_i} that
     `run` rewrites before every replay; so one graph serves all steps of a schedule.
 
+    The UNet's conv_out does not run as a convolution of its own: the graph ends with kh_conv_out_cfg_euler_bf16, which
+    computes it and applies guidance, the Euler update and the next input's scaling in its epilogue (fuse_tail=False
+    keeps conv_out and the scheduler kernel apart, as the eager denoise_loop runs them).
+
     hoist_cond_embedding: the ControlNet's conditioning embedding depends on the image only, which is the same in every
     step; it is computed once per `run` instead of inside the graph (the reference recomputes it every step,
     controlnet.py:780-783; same value, bit for bit).  Everything the notes on GraphedUNetStep say about rebuilding after
@@ -99,7 +103,7 @@ class GraphedDenoiseStep:
 
     def __init__(self, unet, controlnet, latents, encoder_hidden_states, added_cond_kwargs, controlnet_cond,
                  guidance_scale: float, conditioning_scale: float = 0.5, hoist_cond_embedding: bool = True,
-                 warmup: int = 2):
+                 warmup: int = 2, fuse_tail: bool = True):
         from . import ops
 
         self.unet, self.controlnet = unet, controlnet
@@ -117,6 +121,9 @@ class GraphedDenoiseStep:
         self.row[4] = 500.0
         self.hoist = hoist_cond_embedding
         self.cond_emb = None
+        co = unet.conv_out
+        self.fuse_tail = bool(fuse_tail and co.in_channels % 16 == 0 and co.out_channels == 4 and not co.adapters)
+        self._co_w = ops.pack_conv3x3_weight(co.weight) if self.fuse_tail else None   # [4,3,3,C], packed once
         unet.prepare()
         controlnet.prepare()
         keep = (self.latents.clone(), self.model_input.clone())
@@ -142,10 +149,18 @@ class GraphedDenoiseStep:
         t = self.row[4:5]
         down, mid = self.controlnet(self.model_input, t, self.ctx, self.cond, self.conditioning_scale,
                                     added_cond_kwargs=self.added, cond_embedding=self.cond_emb)
-        eps = self.unet(self.model_input, t, self.ctx, added_cond_kwargs=self.added,
-                        down_block_additional_residuals=down, mid_block_additional_residual=mid, return_dict=False)[0]
-        ops.cfg_euler_step(eps, self.latents, self.row, self.guidance_scale, latents_out=self.latents,
-                           model_input_next=self.model_input)
+        self.unet.defer_conv_out = self.fuse_tail
+        try:
+            eps = self.unet(self.model_input, t, self.ctx, added_cond_kwargs=self.added,
+                            down_block_additional_residuals=down, mid_block_additional_residual=mid, return_dict=False)[0]
+        finally:
+            self.unet.defer_conv_out = False
+        if self.fuse_tail:   # `eps` is the input of conv_out here
+            ops.conv_out_cfg_euler(eps, self._co_w, self.unet.conv_out.bias, self.latents, self.row, self.guidance_scale,
+                                   latents_out=self.latents, model_input_next=self.model_input)
+        else:
+            ops.cfg_euler_step(eps, self.latents, self.row, self.guidance_scale, latents_out=self.latents,
+                               model_input_next=self.model_input)
 
     def run(self, latents: torch.Tensor, scheduler, controlnet_cond: Optional[torch.Tensor] = None,
             check: bool = True) -> torch.Tensor:

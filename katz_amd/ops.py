@@ -631,10 +631,49 @@ def cfg_euler_step(noise_pred: torch.Tensor, latents: torch.Tensor, coef: torch.
     return latents_out
 
 
+def conv_out_cfg_euler(x: torch.Tensor, w_packed: torch.Tensor, bias: Optional[torch.Tensor], latents: torch.Tensor,
+                       coef: torch.Tensor, guidance_scale: float, latents_out: Optional[torch.Tensor] = None,
+                       model_input_next: Optional[torch.Tensor] = None, noise_pred_out: Optional[torch.Tensor] = None):
+    """The tail of a denoising step in one launch: conv_out (4 output channels) on x [2B,C,H,W] channels_last, then
+    guidance + Euler + the next step's scaled, duplicated input exactly as cfg_euler_step.  w_packed: [4,3,3,C]
+    (pack_conv3x3_weight of the conv's weight).  latents [B,4,H,W] channels_last, bf16 or fp32; latents_out may be
+    latents.  Returns latents_out."""
+    lib = _lib.load()
+    cl = torch.channels_last
+    if not x.is_cuda or x.dtype != BF16 or x.dim() != 4 or not x.is_contiguous(memory_format=cl):
+        raise ValueError("x must be a channels_last bfloat16 GPU tensor")
+    NB, C, H, W = x.shape
+    if NB % 2:
+        raise ValueError("x holds guidance pairs: an even number of rows, unconditional rows first")
+    Bl = NB // 2
+    _req(w_packed, BF16, "w_packed")
+    if tuple(w_packed.shape) != (4, 3, 3, C):
+        raise ValueError(f"w_packed must be [4,3,3,{C}], got {tuple(w_packed.shape)}")
+    if bias is not None:
+        _req(bias, BF16, "bias")
+    if (latents.dtype not in (BF16, torch.float32) or not latents.is_cuda or tuple(latents.shape) != (Bl, 4, H, W)
+            or not latents.is_contiguous(memory_format=cl)):
+        raise ValueError(f"latents must be a channels_last bfloat16 / float32 GPU tensor of shape {(Bl, 4, H, W)}")
+    if latents_out is None:
+        latents_out = torch.empty_like(latents)
+    if latents_out.dtype != latents.dtype or latents_out.shape != latents.shape or not latents_out.is_contiguous(memory_format=cl):
+        raise ValueError("latents_out must match latents")
+    for name, t in (("model_input_next", model_input_next), ("noise_pred_out", noise_pred_out)):
+        if t is not None and (t.dtype != BF16 or tuple(t.shape) != (NB, 4, H, W) or not t.is_contiguous(memory_format=cl)):
+            raise ValueError(f"{name} must be a channels_last bfloat16 tensor of shape {(NB, 4, H, W)}")
+    if coef.dtype != torch.float32 or not coef.is_cuda or coef.numel() < 3:
+        raise ValueError("coef must be a float32 GPU tensor of at least 3 elements")
+    rc = lib.kh_conv_out_cfg_euler_bf16(_ptr(x), _ptr(w_packed), _ptr(bias), _ptr(latents), _ptr(latents_out),
+                                        _ptr(model_input_next), _ptr(noise_pred_out), Bl, H, W, C, float(guidance_scale),
+                                        _ptr(coef), 1 if latents.dtype == torch.float32 else 0, _stream())
+    _lib.check(rc, "kh_conv_out_cfg_euler_bf16")
+    return latents_out
+
+
 # --------------------------------------------------------------------------------------- per-launch timing
 KERNEL_TAGS = {1: "lora_gemm", 2: "lora_gemm_f32", 3: "attention", 4: "group_norm_stats", 5: "group_norm_apply",
                6: "layer_norm", 7: "geglu", 8: "residual_add", 9: "concat_residual", 10: "sgmv_shrink",
-               11: "sgmv_expand", 12: "lora_shrink", 13: "conv3x3", 14: "cfg_euler", 15: "upsample", 16: "lora_merge"}
+               11: "sgmv_expand", 12: "lora_shrink", 13: "conv3x3", 14: "cfg_euler", 15: "upsample", 16: "lora_merge", 17: "conv_out_step"}
 
 
 def profile_begin() -> None:

@@ -549,7 +549,8 @@ class UNet2DConditionModel(nn.Module):
             ex, extra = extra[-n:], extra[:-n]
             sample = blk(sample, res, ex, temb_act, ctx)
         sample = self.conv_norm_silu(sample)
-        sample = self.conv_out(sample)
+        if not getattr(self, "defer_conv_out", False):   # the denoise-loop graph runs conv_out fused with the scheduler step
+            sample = self.conv_out(sample)
         if cross_attention_kwargs is not None:
             self.scale_lora_layers(1.0)  # unscale_lora_layers, unet_2d_condition.py:1334-1336
         if not return_dict:

@@ -9,7 +9,7 @@ import math
 import pytest
 import torch
 
-from helpers import assert_close_rel, bf16_round
+from helpers import cosine, assert_close_rel, bf16_round
 from oracle import ops as O
 
 pytestmark = pytest.mark.gpu
@@ -1109,3 +1109,57 @@ def test_unet_fuse_lora_through_the_batched_merge():
     for n, m in lin.items():
         assert_close_rel(fast[n], m.weight.float().cpu(), 8e-3, f"grouped vs per-layer fuse {n}")
         assert (m.weight.float() - w0[n].float()).abs().max() > 1e-3
+
+
+# ------------------------------------------------------------------------------------------- conv_out + guidance + Euler
+@pytest.mark.parametrize("Bl,H,W,C,f32", [(1, 128, 128, 320, False), (2, 16, 20, 64, False), (1, 9, 150, 48, True),
+                                          (1, 32, 32, 64, True)], ids=str)
+def test_conv_out_cfg_euler(Bl, H, W, C, f32):
+    """kh_conv_out_cfg_euler_bf16 (the UNet's conv_out with guidance + Euler step + next input scaling as its epilogue)
+    against the oracle: F.conv2d in fp32 rounded to the model dtype, then classifier_free_guidance and the scheduler's
+    step formula; and against the two separate kernels of the product (conv3x3 + cfg_euler_step)."""
+    from katz_amd import ops
+    from oracle import euler as OE
+
+    say("conv_out_cfg_euler", Bl, H, W, C, f32)
+    d = dev()
+    g = torch.Generator().manual_seed(Bl * 1000 + H + W + C)
+    x = randn(g, 2 * Bl, C, H, W).to(BF)
+    w = randn(g, 4, C, 3, 3, std=(9 * C) ** -0.5).to(BF)
+    b = randn(g, 4, std=0.1).to(BF)
+    lat = (randn(g, Bl, 4, H, W) * 3).to(BF)
+    sigma, sigma_next, gs = 4.2, 3.1, 7.5
+    coef = torch.tensor([sigma, sigma_next, (sigma_next ** 2 + 1) ** 0.5], dtype=torch.float32)
+    cl = lambda t: t.to(d).contiguous(memory_format=torch.channels_last)
+    lat_d = cl(lat.float() if f32 else lat)
+    nxt = torch.empty(2 * Bl, 4, H, W, dtype=BF, device=d).contiguous(memory_format=torch.channels_last)
+    noise = torch.empty_like(nxt)
+    out = ops.conv_out_cfg_euler(cl(x), ops.pack_conv3x3_weight(w.to(d)), b.to(d), lat_d, coef.to(d), gs,
+                                 model_input_next=nxt, noise_pred_out=noise)
+    torch.cuda.synchronize()
+    # oracle
+    ref_noise = bf16_round(torch.nn.functional.conv2d(x.float(), w.float(), b.float(), padding=1))
+    assert_close_rel(noise, ref_noise, REL_BF16, "conv_out noise")
+    u, t = noise.float().cpu()[:Bl], noise.float().cpu()[Bl:]          # the kernel's own rounded noise: exact arithmetic after it
+    eps = u + gs * (t - u)
+    xin = lat.float()
+    x0 = xin - sigma * eps
+    want = xin + ((xin - x0) / sigma) * (coef[1] - coef[0])
+    if not f32:
+        want = bf16_round(want)
+    assert out.dtype == (torch.float32 if f32 else BF)
+    assert (out.float().cpu() - want).abs().max().item() <= 1e-5 * want.abs().max().item() + (0 if f32 else 2 ** -8 * want.abs().max().item())
+    want_next = bf16_round(want / coef[2])
+    assert_close_rel(nxt[:Bl], want_next, 1e-2, "next input")
+    assert torch.equal(nxt[:Bl], nxt[Bl:])
+    # the product's two separate kernels on the same inputs
+    from katz_amd.layers import Conv3x3
+    conv = Conv3x3(C, 4)
+    with torch.no_grad():
+        conv.weight.copy_(w.float()); conv.bias.copy_(b.float())
+    conv = conv.to(d, BF)
+    with torch.no_grad():
+        e2 = conv(cl(x))
+    out2 = ops.cfg_euler_step(e2, lat_d, coef.to(d), gs)
+    assert_close_rel(noise, e2.float().cpu(), 1e-2, "fused conv vs conv kernel")
+    assert cosine(out, out2) >= 0.99999
