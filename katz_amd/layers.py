@@ -19,7 +19,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from . import ops
-from .lora import Adapter, PackedAdapters, interleave_geglu_rows, pack_adapters, rescale_
+from .lora import MAX_PACKED_RANK, Adapter, PackedAdapters, interleave_geglu_rows, pack_adapters, rescale_
 
 CL = torch.channels_last
 
@@ -116,8 +116,11 @@ class LoRALinear(nn.Module):
         if key == self._packed_key and self._packed is not None:
             rescale_(self._packed, self.adapters, self.global_scale)
             return
+        # more than 128 rank columns: the extra packs are applied one by one after the fused launch (forward), which for
+        # a GEGLU projection means before the activation, so everything is packed in the plain row order then
+        wide = sum(self.adapters[n].rank for n in names) > MAX_PACKED_RANK
         self._packed = pack_adapters(self.adapters, names, self.in_features, self.out_features, self.weight.dtype,
-                                     self.weight.device, self.global_scale, geglu_interleave=self.geglu)
+                                     self.weight.device, self.global_scale, geglu_interleave=self.geglu and not wide)
         self._packed_key = key
         _pack_epoch += 1
 
@@ -189,10 +192,28 @@ class LoRALinear(nn.Module):
         p = self._packed
         if p is None:
             return ops.lora_linear(x, w, b, residual=residual, geglu=self.geglu)
+        if p.overflow:
+            return self._forward_wide(x, residual, p)
         if LORA_MODE == "split" and x.dtype == torch.bfloat16 and self.in_features % 64 == 0:
             return ops.lora_linear_split(x, w, b, p.a_cat, p.col_scale, p.b_cat, residual=residual, geglu=self.geglu,
                                          two_launches=LORA_SHRINK == "separate", r_used=p.r_used)
         return ops.lora_linear(x, w, b, p.a_cat, p.b_cat, p.col_scale, residual=residual, geglu=self.geglu)
+
+    def _forward_wide(self, x, residual, p: PackedAdapters) -> torch.Tensor:
+        """More rank columns than one launch takes (sum of the active ranks > 128; peft has no such limit): the first
+        128 go with the base GEMM, every further pack adds ((x A^T) * scale) B^T with y as the residual of a GEMM over
+        its rank columns.  A GEGLU projection is computed in the reference's row order without the fused epilogue and
+        activated afterwards (all packs belong under the activation)."""
+        w = self.weight.detach() if self.geglu else self._rt[1]
+        b = (None if self.bias is None else self.bias.detach()) if self.geglu else self._rt[2]
+        y = ops.lora_linear(x, w, b, p.a_cat, p.b_cat, p.col_scale, residual=None if self.geglu else residual)
+        for c in p.overflow:
+            t = ops.lora_linear(x, c.a_cat, None)                       # [.., R] = x A^T
+            t.mul_(c.col_scale.to(t.dtype))
+            y = ops.lora_linear(t, c.b_cat, None, residual=y)
+        if self.geglu:
+            return ops.geglu(y)
+        return y
 
     def extra_repr(self) -> str:
         return f"in_features={self.in_features}, out_features={self.out_features}, bias={self.bias is not None}, geglu={self.geglu}"
@@ -479,6 +500,10 @@ class Conv1x1(_ConvLoRAFuse, nn.Conv2d):
             y = ops.lora_linear(x2, w2, self.bias)
         else:
             y = ops.lora_linear(x2, w2, self.bias, p.a_cat, p.b_cat, p.col_scale)
+            for c in p.overflow:      # rank columns beyond the 128 one launch takes (see LoRALinear._forward_wide)
+                t = ops.lora_linear(x2, c.a_cat, None)
+                t.mul_(c.col_scale.to(t.dtype))
+                y = ops.lora_linear(t, c.b_cat, None, residual=y)
         return y.view(nb, hh, ww, self.out_channels).permute(0, 3, 1, 2)
 
 
@@ -638,7 +663,7 @@ class Attention(nn.Module):
         st = self._qkv
         if st is None or st["sig"] != sig:
             packs = [l._packed for l in layers]
-            same = all(p is None for p in packs) or (all(p is not None for p in packs) and len({p.R for p in packs}) == 1)
+            same = all(p is None for p in packs) or (all(p is not None and not p.overflow for p in packs) and len({p.R for p in packs}) == 1)
             ok = same and (packs[0] is None or LORA_MODE == "split") and all(l.bias is None for l in layers)
             st = dict(sig=sig, ok=ok)
             if ok:
@@ -794,7 +819,7 @@ class ContextKVProjector:
             l.prepare()
         K = layers[0].in_features
         packs = [l._packed for l in layers]
-        uniform = all(p is None for p in packs) or (all(p is not None for p in packs) and len({p.R for p in packs}) == 1)
+        uniform = all(p is None for p in packs) or (all(p is not None and not p.overflow for p in packs) and len({p.R for p in packs}) == 1)
         ok = uniform and LORA_MODE == "split" and all(l.weight.dtype == torch.bfloat16 and not l.geglu for l in layers)
         st = dict(epoch=_pack_epoch, M=M, ok=ok, wptr=[l.weight.data_ptr() for l in layers])
         if ok:

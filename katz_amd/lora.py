@@ -49,6 +49,10 @@ class PackedAdapters:
     b_cat: torch.Tensor
     col_scale: torch.Tensor
     spans: List[tuple] = field(default_factory=list)  # (name, first column, rank)
+    # Rank columns beyond the kernels' 128: further packs of at most 128 columns each (A rows / B columns of the same
+    # adapters, continued).  Only LoRALinear's own forward applies them; the fused launches that stack several
+    # layers' packs take the per-layer path when a layer has any.
+    overflow: List["PackedAdapters"] = field(default_factory=list)
 
     @property
     def R(self) -> int:
@@ -83,34 +87,56 @@ def pack_adapters(adapters: Dict[str, Adapter], active: Sequence[str], in_featur
     names = [n for n in active if n in adapters]
     if not names:
         return None
-    total = sum(adapters[n].rank for n in names)
-    R = (total + RANK_PAD - 1) // RANK_PAD * RANK_PAD
-    if R > MAX_PACKED_RANK:
-        raise ValueError(f"sum of active ranks {total} exceeds the fused kernel's maximum {MAX_PACKED_RANK}")
-    a_cat = torch.zeros((R, in_features), dtype=dtype, device=device)
-    b_cat = torch.zeros((out_features, R), dtype=dtype, device=device)
-    col_scale = torch.zeros((R,), dtype=torch.float32, device=device)
-    spans, c = [], 0
     for n in names:
         ad = adapters[n]
-        r = ad.rank
-        if ad.down.shape != (r, in_features) or ad.up.shape != (out_features, r):
+        if ad.down.shape != (ad.rank, in_features) or ad.up.shape != (out_features, ad.rank):
             raise ValueError(f"adapter {n!r}: down {tuple(ad.down.shape)} / up {tuple(ad.up.shape)} do not fit "
                              f"a [{out_features},{in_features}] layer")
-        a_cat[c:c + r] = ad.down.to(device=device, dtype=dtype)
-        b_cat[:, c:c + r] = ad.up.to(device=device, dtype=dtype)
-        col_scale[c:c + r] = ad.multiplier(global_scale)
-        spans.append((n, c, r))
-        c += r
-    if geglu_interleave:
-        b_cat = interleave_geglu_rows(b_cat)
-    return PackedAdapters(a_cat, b_cat, col_scale, spans)
+    total = sum(adapters[n].rank for n in names)
+    if total > MAX_PACKED_RANK and geglu_interleave:
+        raise ValueError("more than 128 rank columns on a GEGLU projection need the plain row order: pack with "
+                         "geglu_interleave=False (LoRALinear does)")
+    # cut the adapters' rank rows, in order, into packs of at most MAX_PACKED_RANK columns
+    packs, pieces, width = [], [], 0
+    for n in names:
+        r, r0 = adapters[n].rank, 0
+        while r0 < r:
+            take = min(r - r0, MAX_PACKED_RANK - width)
+            pieces.append((n, r0, take))
+            width += take
+            r0 += take
+            if width == MAX_PACKED_RANK:
+                packs.append(pieces)
+                pieces, width = [], 0
+    if pieces:
+        packs.append(pieces)
+    built = []
+    for pcs in packs:
+        used = sum(t for _, _, t in pcs)
+        R = (used + RANK_PAD - 1) // RANK_PAD * RANK_PAD
+        a_cat = torch.zeros((R, in_features), dtype=dtype, device=device)
+        b_cat = torch.zeros((out_features, R), dtype=dtype, device=device)
+        col_scale = torch.zeros((R,), dtype=torch.float32, device=device)
+        spans, c = [], 0
+        for n, r0, take in pcs:
+            ad = adapters[n]
+            a_cat[c:c + take] = ad.down[r0:r0 + take].to(device=device, dtype=dtype)
+            b_cat[:, c:c + take] = ad.up[:, r0:r0 + take].to(device=device, dtype=dtype)
+            col_scale[c:c + take] = ad.multiplier(global_scale)
+            spans.append((n, c, take))
+            c += take
+        if geglu_interleave:
+            b_cat = interleave_geglu_rows(b_cat)
+        built.append(PackedAdapters(a_cat, b_cat, col_scale, spans))
+    built[0].overflow = built[1:]
+    return built[0]
 
 
 def rescale_(packed: PackedAdapters, adapters: Dict[str, Adapter], global_scale: float = 1.0) -> None:
     """Rewrite col_scale only (scale_lora_layers / set_adapters weight change); A_cat/B_cat stay put."""
-    for n, c, r in packed.spans:
-        packed.col_scale[c:c + r] = adapters[n].multiplier(global_scale)
+    for pk in [packed, *packed.overflow]:
+        for n, c, r in pk.spans:
+            pk.col_scale[c:c + r] = adapters[n].multiplier(global_scale)
 
 
 # ---- per-block adapter scales -------------------------------------------------------------------------------------

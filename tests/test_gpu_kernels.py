@@ -1163,3 +1163,41 @@ def test_conv_out_cfg_euler(Bl, H, W, C, f32):
     out2 = ops.cfg_euler_step(e2, lat_d, coef.to(d), gs)
     assert_close_rel(noise, e2.float().cpu(), 1e-2, "fused conv vs conv kernel")
     assert cosine(out, out2) >= 0.99999
+
+
+# ------------------------------------------------------------------------------------------- more than 128 rank columns
+@pytest.mark.parametrize("geglu", [False, True], ids=["linear", "geglu"])
+def test_lora_linear_with_more_than_128_rank_columns(geglu):
+    """Three rank-64 adapters and one rank-160 adapter active at once (peft has no limit on the sum of ranks): the
+    layer applies the first 128 rank columns in the fused launch and the rest pack by pack; against the oracle."""
+    from katz_amd.layers import LoRALinear
+
+    say("lora_linear wide rank", geglu)
+    d = dev()
+    g = torch.Generator().manual_seed(31)
+    K, N, M = 640, 1280, 300
+    lin = LoRALinear(K, N, geglu=geglu)
+    with torch.no_grad():
+        lin.weight.copy_(randn(g, N, K, std=0.03).to(BF).float()); lin.bias.copy_(randn(g, N, std=0.1).to(BF).float())
+    w, b = lin.weight.detach().clone(), lin.bias.detach().clone()
+    lin = lin.to(d, BF)
+    specs = [("a", 64, 0.8), ("b", 64, 0.6), ("c", 64, 1.1), ("d", 160, 0.4)]
+    ads = []
+    for name, r, wt in specs:
+        A, B = randn(g, r, K, std=0.05).to(BF).float(), randn(g, N, r, std=0.05).to(BF).float()
+        lin.add_adapter(name, A, B, alpha=float(r))
+        ads.append((A, B, wt))
+    lin.set_active([s[0] for s in specs], [s[2] for s in specs])
+    assert len(lin._packed.overflow) == 2      # 352 rank columns: 128 + 128 + 96
+    x = randn(g, M, K).to(BF)
+    res = None if geglu else randn(g, M, N).to(BF)
+    with torch.no_grad():
+        y = lin(x.to(d), residual=None if res is None else res.to(d))
+        torch.cuda.synchronize()
+    ref = O.lora_linear(x.float(), w, b, ads, residual=None if res is None else res.float())
+    if geglu:
+        ref = O.geglu(ref)
+    # every extra pack rounds y to bf16 once more (three roundings here, then the activation): 3e-2 instead of 2e-2
+    assert_close_rel(y, ref, 3e-2 if geglu else REL_BF16, "wide-rank lora linear")
+    lin.set_active(["a"], [1.0])
+    assert not lin._packed.overflow

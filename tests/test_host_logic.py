@@ -399,3 +399,29 @@ def test_fuse_that_fails_leaves_everything_as_it_was():
     assert all(m._fused for m in lin.values())
     unet.unfuse_lora()
     assert max((lin[n].weight - before[n]).abs().max().item() for n in names) < 1e-5
+
+
+def test_pack_adapters_cuts_wide_rank_sums_into_packs_of_128():
+    """Sum of active ranks above 128 (three rank-64 adapters; one rank-200 adapter): the rank rows are cut, in order,
+    into packs of at most 128 columns; every pack reproduces its slice of sum_i s_i B_i A_i; rescaling reaches all."""
+    import torch
+    from katz_amd.lora import Adapter, pack_adapters, rescale_
+
+    g = torch.Generator().manual_seed(0)
+    K, N = 48, 40
+    for ranks in ([64, 64, 64], [200], [100, 30, 7]):
+        ads = {f"a{i}": Adapter(torch.randn(r, K, generator=g), torch.randn(N, r, generator=g), alpha=2.0 * r, weight=0.5 + i)
+               for i, r in enumerate(ranks)}
+        p = pack_adapters(ads, list(ads), K, N, torch.float32, "cpu", 1.0)
+        packs = [p, *p.overflow]
+        assert all(q.R <= 128 and q.R % 64 == 0 for q in packs)
+        assert sum(r for q in packs for _, _, r in q.spans) == sum(ranks)
+        delta = sum((q.b_cat * q.col_scale) @ q.a_cat for q in packs)
+        want = sum(a.multiplier() * (a.up @ a.down) for a in ads.values())
+        assert torch.allclose(delta, want, atol=1e-3)
+        for a in ads.values():
+            a.weight *= 2
+        rescale_(p, ads, 0.5)
+        delta = sum((q.b_cat * q.col_scale) @ q.a_cat for q in packs)
+        assert torch.allclose(delta, want, atol=1e-3)       # weights doubled, global scale halved
+    assert len(pack_adapters({"a": Adapter(torch.zeros(96, K), torch.zeros(N, 96))}, ["a"], K, N, torch.float32, "cpu").overflow) == 0
