@@ -49,7 +49,11 @@ __global__ __launch_bounds__(CO_THREADS) void conv_out_step_kernel(const ConvOut
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, lh = lane >> 5;
   const int wb = wave >> 1, ws = wave & 1;                 // batch row of the pair, 32-pixel segment
-  const int x0 = blockIdx.x * CO_SEG, y = blockIdx.y, z = blockIdx.z;
+  // Workgroups go round-robin to the 8 XCDs; remapped so that every XCD owns a band of consecutive image rows and
+  // the halo rows two neighbouring workgroups share are found in that XCD's L2.
+  const uint32_t gx = gridDim.x;
+  const uint32_t logical = xcd_remap(blockIdx.y * gx + blockIdx.x, gx * gridDim.y);
+  const int x0 = (int)(logical % gx) * CO_SEG, y = (int)(logical / gx), z = blockIdx.z;
   const int brow[2] = {z, p.Bl + z};                       // uncond row, text row
   const int H = p.H, W = p.W, Cin = p.Cin;
 

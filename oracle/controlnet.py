@@ -7,8 +7,9 @@ conditioning_scale = 0.5, :693).  The encoder blocks are the ones pinned by the 
 (oracle/blocks.py).  Pinned here (tests/test_oracle_controlnet.py): freshly constructed (zero-initialised zero
 convs, :58-61 zero_module) every residual is exactly zero; with identity zero convs and a zero conditioning
 embedding the residuals equal conditioning_scale x the UNet encoder's skips (from_unet semantics, :432-506);
-residual shapes equal unet_2d_condition.py:539-563.  End-to-end numerical parity on real ControlNet weights:
-parity unpinned (the reference's only goldens need hub checkpoints).
+residual shapes equal unet_2d_condition.py:539-563; and numerically against outputs of the reference's own
+ControlNetModel (from_unet, random non-zero zero convolutions and conditioning embedding, conditioning_scale 0.5 and
+1.0) on a tiny SDXL-topology configuration, <= 1e-4 relative (tests/golden/unet_tiny_reference.safetensors).
 """
 from __future__ import annotations
 

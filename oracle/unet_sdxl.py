@@ -3,11 +3,12 @@
 Follows diffusers-hf/src/diffusers/models/unets/unet_2d_condition.py: constructor :279-507 (SDXL
 arguments), time / text_time embeddings :997-1021, :1055-1075, down + mid :1127-1252, ControlNet
 residual injection + up + post-process :1254-1341.  The blocks it wires are pinned by the reference's
-known-answer tests (oracle/blocks.py); the wiring itself is pinned structurally: the LoRA-able linear
-names must equal the 722 keys of the reference's lora_info_shm/*_key_match_unet.json fixture and the
-skip tensors must have the shapes of unet_2d_condition.py:539-563 (tests/test_oracle_unet.py).
-End-to-end numerical parity of the wiring against the reference on real weights: parity unpinned (the
-reference's only goldens for it need hub checkpoints).
+known-answer tests (oracle/blocks.py); the wiring itself is pinned numerically by outputs of the
+reference's own UNet2DConditionModel on a tiny SDXL-topology configuration (depths 1 / 2 / 3, text_time
+conditioning, with and without the 9 + 1 residuals; tests/golden/unet_tiny_reference.safetensors, <= 1e-4) and
+structurally: the LoRA-able linear names equal the 722 keys of the reference's
+lora_info_shm/*_key_match_unet.json fixture and the skip tensors have the shapes of
+unet_2d_condition.py:539-563 (tests/test_oracle_unet.py).
 """
 from __future__ import annotations
 
