@@ -425,3 +425,14 @@ def test_pack_adapters_cuts_wide_rank_sums_into_packs_of_128():
         delta = sum((q.b_cat * q.col_scale) @ q.a_cat for q in packs)
         assert torch.allclose(delta, want, atol=1e-3)       # weights doubled, global scale halved
     assert len(pack_adapters({"a": Adapter(torch.zeros(96, K), torch.zeros(N, 96))}, ["a"], K, N, torch.float32, "cpu").overflow) == 0
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py --gpus N with N > 1 exits with a message: this build runs on one GPU (no collectives, no sharding)."""
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    root = Path(__file__).resolve().parent.parent
+    r = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 2 and "ONE GPU" in r.stderr
