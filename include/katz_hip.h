@@ -103,6 +103,30 @@ int kh_lora_linear_pre_bf16(const void* x, const void* w, const void* bias, cons
 int kh_lora_linear_split_bf16(const void* x, const void* w, const void* bias, const void* a_cat, const float* col_scale,
                               const void* b_cat, void* t_scratch, int32_t* counters, const void* residual, void* y,
                               int64_t M, int64_t N, int64_t K, int64_t R, int64_t n_split, int flags, void* stream);
+/* The LoRA linear of kh_lora_linear_split_bf16 with the LayerNorm in front of it folded into the GEMM, and / or with the
+ * row statistics a folded LayerNorm BEHIND it needs written by its epilogue.  The reference's transformer block runs
+ * norm -> projection three times (diffusers-hf/src/diffusers/models/attention.py:338-403: norm1 -> attn1.to_q/k/v,
+ * norm2 -> attn2.to_q, norm3 -> ff.net.0.proj), each norm a pass over the hidden states of its own; here the producer
+ * of the hidden states (attn.to_out.0 / ff.net.2 / proj_in with their residual) leaves per-row partial sums, and the
+ * consumer GEMM reads the UN-normalised rows and finishes the normalisation per output element:
+ *   LN(x) W^T + b  =  rstd_m * (x W'^T - mean_m * c1) + c2,   W' = W * gamma (per K column),
+ *                     c1[n] = sum_k W'[n,k],  c2[n] = b[n] + sum_k beta[k] W[n,k].
+ * stats_out (may be NULL): float [16][M][2]; column tile j of the GEMM writes (sum, sum of squares) of its columns of
+ *   every output row (after bias and residual, over the bf16-rounded values) to pair [j][row], the pairs past the
+ *   last tile are zeroed.  N <= 2048, no GEGLU.
+ * ln_part (may be NULL): such an array for the rows of x.  Then w must be W' (and a_cat must be A_cat * gamma), bias
+ *   must be NULL (it is part of ln_c2), ln_c1 / ln_c2 are float [N] as above and, with R > 0, ln_ca1[r] = sum_k
+ *   a_cat'[r,k], ln_ca2[r] = sum_k beta[k] A_cat[r,k] (float [rows of a_cat]) let the shrink store
+ *   ((x A'^T) - mean * ca1 + ca2 / rstd) * col_scale, the adapters' share before the common factor rstd.
+ *   mean = sum / K, rstd = rsqrt(sumsq / K - mean^2 + ln_eps): the formula of kh_layer_norm_bf16.
+ * R == 0: plain linear (a_cat, col_scale, b_cat, t_scratch, counters NULL).  Everything else (counters, n_split, flags,
+ * shape limits) as for kh_lora_linear_split_bf16.  Results differ from LayerNorm followed by the linear by rounding
+ * only: the normalised row is never rounded to bf16, W' is. */
+int kh_lora_linear_norm_bf16(const void* x, const void* w, const void* bias, const void* a_cat, const float* col_scale,
+                             const void* b_cat, void* t_scratch, int32_t* counters, const void* residual, void* y,
+                             const float* ln_part, const float* ln_c1, const float* ln_c2, const float* ln_ca1,
+                             const float* ln_ca2, float ln_eps, float* stats_out, int64_t M, int64_t N, int64_t K,
+                             int64_t R, int64_t n_split, int flags, void* stream);
 /* Bounded waits of kh_lora_linear_split_bf16's in-launch shrink that have run out on the current device since the
  * process started (or since the last call with clear != 0): writes the number to *count (HOST pointer).  A GEMM workgroup
  * of that launch waits for the shrink workgroups of the same launch, which have lower workgroup ids and are therefore

@@ -1,6 +1,7 @@
 // Parameters shared by the LoRA GEMM kernels (host fills, kernels read by value).
 #pragma once
 #include "kh_common.h"
+#include <type_traits>
 
 struct LoraGemmParams {
   const bf16_t* x;
@@ -41,7 +42,100 @@ struct LoraGemmParams {
   // two-launch / in-launch forms: rank columns >= r_used of t_ext and b_cat are all zero (0: unknown, use R); the
   // 128x128 / 256x128 and 256x320 kernels then skip the MFMA steps that would only add zeros
   int r_used = 0;
+  // LayerNorm folded into the GEMM (ln_part != nullptr): x is the input of a LayerNorm over its K columns whose affine
+  // weight is already multiplied into w (and a_cat); the epilogue finishes the normalisation per output row,
+  //   y[m,n] = rstd_m * (acc[m,n] - mean_m * ln_c1[n]) + ln_c2[n]   (ln_c1 = row sums of w, ln_c2 = bias + w . beta),
+  // with mean / rstd from the row's 16 partial (sum, sum of squares) pairs in ln_part.  The shrink of such a layer
+  // stores t = ((x . a^T) - mean * ln_ca1 + ln_ca2 / rstd) * col_scale, i.e. the adapter's share divided by rstd.
+  const float* ln_part = nullptr;   // [16][M][2]
+  const float* ln_c1 = nullptr;     // [N]
+  const float* ln_c2 = nullptr;     // [N]
+  const float* ln_ca1 = nullptr;    // [ldt] (shrink)
+  const float* ln_ca2 = nullptr;    // [ldt]
+  float ln_eps = 0.f;
+  int ln_lds = 0;                   // byte offset of the workgroup's mean / rstd arrays in dynamic LDS (set by the launcher)
+  // Row statistics of the output for a following folded LayerNorm (st_part != nullptr): column tile j writes the
+  // (sum, sum of squares) of its columns of every row to st_part[j][row]; tile 0 also zeroes the slots past the last tile.
+  float* st_part = nullptr;         // [16][M][2]
 };
+
+constexpr int KH_LN_LDS = 4096;    // bytes of dynamic LDS a launch with a folded LayerNorm adds: mean, 1/std of up to 256 rows, c1, c2 of up to 256 columns
+constexpr int KH_LN_SLOTS = 16;     // partial pairs per row: at most 16 column tiles (N <= 2048 with 128-column tiles)
+
+// a column tile's pair for one output row, and (from tile 0) zeros in the slots no tile writes
+__device__ __forceinline__ void kh_ln_store_stats(float* part, int row, int M, int tile, int n_tiles, float s, float q) {
+  u32x2* dst = reinterpret_cast<u32x2*>(part) + row;
+  dst[(size_t)tile * M] = u32x2{__float_as_uint(s), __float_as_uint(q)};
+  if (tile == 0)
+    for (int t = n_tiles; t < KH_LN_SLOTS; ++t) dst[(size_t)t * M] = u32x2{0u, 0u};
+}
+
+// sum over the 16 lanes of a DPP row (lanes 16k .. 16k+15), the result in every lane: four cross-lane adds in the VALU
+__device__ __forceinline__ float kh_row16_sum(float v) {
+  auto dpp = [](float x, auto ctrl) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), decltype(ctrl)::value, 0xf, 0xf, true));
+  };
+  v += dpp(v, std::integral_constant<int, 0xb1>{});    // quad_perm [1,0,3,2]
+  v += dpp(v, std::integral_constant<int, 0x4e>{});    // quad_perm [2,3,0,1]
+  v += dpp(v, std::integral_constant<int, 0x141>{});   // row_half_mirror
+  v += dpp(v, std::integral_constant<int, 0x140>{});   // row_mirror
+  return v;
+}
+
+// mean and 1/std (or std, `want_sigma`) of ROWS consecutive rows from m0 into out_mean / out_2 (LDS), by all NT threads
+// of the workgroup, in two steps so that the loads fly while the kernel sets up its operands.  A wave takes sixteen rows
+// at a time: lane = (slot group g = lane / 16, row = lane % 16) loads the pairs of slots g, 4 + g, 8 + g, 12 + g (every
+// load instruction reads four whole 128-byte lines of the slot-major buffer [slot][row][2]), adds them up, and the four
+// groups meet by two cross-lane adds: a fixed order, deterministic.  M = rows of the buffer, D = the row's length.
+// Same formula as the stand-alone LayerNorm kernel: biased variance, rstd = rsqrt(var + eps).
+template <int ROWS, int NT>
+struct KhLnTileStats {
+  static constexpr int PASSES = (ROWS + (NT / 64) * 16 - 1) / ((NT / 64) * 16);
+  static_assert(KH_LN_SLOTS == 16 && ROWS % 16 == 0 && NT % 64 == 0, "four slot groups of four, sixteen rows per wave and pass");
+  u32x2 v[PASSES][4];
+
+  __device__ __forceinline__ void load(const float* part, int m0, int M, int tid) {
+    const int lane = tid & 63, r16 = lane & 15, g = lane >> 4;
+    const u32x2* src = reinterpret_cast<const u32x2*>(part) + (size_t)g * M;
+#pragma unroll
+    for (int ps = 0; ps < PASSES; ++ps) {
+      const int r = ((tid >> 6) + ps * (NT / 64)) * 16 + r16;          // beyond ROWS: a valid address, never stored
+      const int row = m0 + r < M ? m0 + r : M - 1;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) v[ps][j] = src[(size_t)(4 * j) * M + row];
+    }
+  }
+  __device__ __forceinline__ void finish(int D, float eps, int tid, float* out_mean, float* out_2, bool want_sigma) const {
+    const int lane = tid & 63, r16 = lane & 15, g = lane >> 4;
+#pragma unroll
+    for (int ps = 0; ps < PASSES; ++ps) {
+      const int r = ((tid >> 6) + ps * (NT / 64)) * 16 + r16;
+      float s = 0.f, q = 0.f;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) { s += __uint_as_float(v[ps][j][0]); q += __uint_as_float(v[ps][j][1]); }
+      s += __shfl_xor(s, 16, 64); q += __shfl_xor(q, 16, 64);
+      s += __shfl_xor(s, 32, 64); q += __shfl_xor(q, 32, 64);
+      if (g == 0 && r < ROWS) {
+        const float mean = s / (float)D;
+        float var = q / (float)D - mean * mean;
+        var = var > 0.f ? var : 0.f;
+        out_mean[r] = mean;
+        out_2[r] = want_sigma ? sqrtf(var + eps) : rsqrtf(var + eps);
+      }
+    }
+  }
+};
+
+// one thread's share of a row's statistics: the (sum, sum of squares) of the eight bf16 values of a 16-byte piece
+__device__ __forceinline__ void kh_piece_sums(const u32x4 o, float& s, float& q) {
+  s = 0.f; q = 0.f;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const float a = bf16_lo(o[e]), b = bf16_hi(o[e]);
+    s += a; q += a * a;
+    s += b; q += b * b;
+  }
+}
 
 // Software-pipelined kernel (lora_gemm_pipe.hip); needs K % 32 == 0.  tile_sel: 0 automatic, >= 16 forces a tile.
 int lora_gemm_pipe_launch(const LoraGemmParams& p, int tile_sel, hipStream_t stream);
@@ -65,6 +159,10 @@ int lora_gemm_ksplit_launch_conv(const LoraGemmParams& p, int row_groups, hipStr
 // GEGLU; M % 256 == 0, N % 320 == 0, K % 64 == 0.
 bool lora_gemm_wide_ok(const LoraGemmParams& p);
 int lora_gemm_wide_launch(LoraGemmParams p, hipStream_t stream);
+
+// The shrink of a layer, optionally with a folded LayerNorm in front (ln_part != nullptr; lora_shrink.hip).
+int lora_shrink_ln_launch(const void* x, const void* a_cat, const float* col_scale, void* t, int64_t M, int64_t K, int64_t R,
+                          const float* ln_part, const float* ln_ca1, const float* ln_ca2, float ln_eps, hipStream_t stream);
 
 extern "C" int kh_lora_shrink_bf16(const void* x, const void* a_cat, const float* col_scale, void* t, int64_t M, int64_t K,
                                    int64_t R, void* stream);

@@ -585,6 +585,47 @@ KH_EXPORT int kh_lora_linear_split_bf16(const void* x, const void* w, const void
   return kh_lora_linear_pre_bf16(x, w, bias, t_scratch, RT, n_split, b_cat, residual, y, M, N, K, R, flags & 0xff00ff, stream);
 }
 
+// LoRA linear behind a LayerNorm that is folded into the GEMM, and / or in front of one (row statistics out); see
+// include/katz_hip.h.
+KH_EXPORT int kh_lora_linear_norm_bf16(const void* x, const void* w, const void* bias, const void* a_cat,
+                                       const float* col_scale, const void* b_cat, void* t_scratch, int32_t* counters,
+                                       const void* residual, void* y, const float* ln_part, const float* ln_c1,
+                                       const float* ln_c2, const float* ln_ca1, const float* ln_ca2, float ln_eps,
+                                       float* stats_out, int64_t M, int64_t N, int64_t K, int64_t R, int64_t n_split,
+                                       int flags, void* stream) {
+  if (!x || !w || !y || M <= 0 || N <= 0 || K <= 0 || R < 0) return KH_ERR_INVALID_ARG;
+  if (R > 0 && (!a_cat || !col_scale || !b_cat || !t_scratch)) return KH_ERR_INVALID_ARG;
+  if (ln_part != nullptr && (!ln_c1 || !ln_c2 || bias != nullptr || (R > 0 && (!ln_ca1 || !ln_ca2)))) return KH_ERR_INVALID_ARG;
+  if (n_split < 0 || (n_split > 0 && (n_split % 128 != 0 || N % n_split != 0))) return KH_ERR_INVALID_ARG;
+  const int64_t RT = n_split > 0 ? (N / n_split) * R : R;   // columns of t_scratch / rows of a_cat
+  if (K % 64 != 0 || N % 8 != 0 || R % 32 != 0) return KH_ERR_UNSUPPORTED;
+  if (R > 128) return KH_ERR_TOO_LARGE;
+  if (M > (1 << 24) || N > (1 << 24) || K > (1 << 24)) return KH_ERR_TOO_LARGE;
+  const bool geglu = (flags & 1) != 0;
+  if (geglu && (N % 64 != 0 || residual != nullptr || stats_out != nullptr)) return KH_ERR_UNSUPPORTED;
+  if (stats_out != nullptr && N > 128 * KH_LN_SLOTS) return KH_ERR_TOO_LARGE;
+  if (((flags >> 16) & 0xff) * 16 > R) return KH_ERR_INVALID_ARG;
+  if (!kh_aligned16(x) || !kh_aligned16(w) || !kh_aligned16(y) || (R > 0 && (!kh_aligned16(a_cat) || !kh_aligned16(b_cat) ||
+      !kh_aligned16(t_scratch))) || (residual && !kh_aligned16(residual)) || (ln_part && !kh_aligned16(ln_part)) ||
+      (stats_out && !kh_aligned16(stats_out)))
+    return KH_ERR_ALIGNMENT;
+  LoraGemmParams p = split_params(x, w, bias, a_cat, col_scale, b_cat, R > 0 ? t_scratch : nullptr, counters, residual, y, M, N, K,
+                                  R, n_split, geglu);
+  p.r_used = ((flags >> 16) & 0xff) * 16;
+  p.ln_part = ln_part; p.ln_c1 = ln_c1; p.ln_c2 = ln_c2; p.ln_ca1 = ln_ca1; p.ln_ca2 = ln_ca2; p.ln_eps = ln_eps;
+  p.st_part = stats_out;
+  const int tile_sel = (flags >> 8) & 0xff;
+  if (R == 0) {
+    p.ldt = 0; p.t_nsplit = 0; p.il_cnt = nullptr;
+    return lora_gemm_pipe_launch(p, tile_sel, (hipStream_t)stream);
+  }
+  if (counters != nullptr && tile_sel == 0 && lora_gemm_pipe_il_ok(p)) return lora_gemm_pipe_launch_il(p, (hipStream_t)stream);
+  const int rc = lora_shrink_ln_launch(x, a_cat, col_scale, t_scratch, M, K, RT, ln_part, ln_ca1, ln_ca2, ln_eps, (hipStream_t)stream);
+  if (rc != KH_OK) return rc;
+  p.a_cat = nullptr; p.col_scale = nullptr; p.il_cnt = nullptr;
+  return lora_gemm_pipe_launch(p, tile_sel == 1 ? 0 : tile_sel, (hipStream_t)stream);
+}
+
 // 3x3 convolution, padding 1, NHWC, as an implicit GEMM on the pipelined kernel; see include/katz_hip.h.
 KH_EXPORT int kh_conv3x3_nhwc_bf16(const void* x, const void* w, const void* bias, const void* residual, void* y,
                                    int64_t Nb, int64_t H, int64_t W, int64_t Cin, int64_t Cout, int64_t stride,

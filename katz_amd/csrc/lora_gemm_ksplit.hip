@@ -76,6 +76,22 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_ksplit_kernel(const LoraGemm
   const int KT1 = K / 64;
   const int KT = KT1 + (p.t_ext != nullptr ? p.R / 64 : 0);
   const bool has_hi = wave < N_HI;
+  // folded LayerNorm: mean and 1/std of this tile's x rows, read in the epilogue (the barriers of the K loop lie between)
+  // and the two per-column terms of this column tile; requested here, finished once the bias loads are under way
+  float* sMu = reinterpret_cast<float*>(smem + p.ln_lds);
+  float* sRs = sMu + 256;
+  float* sc1 = sRs + 256;
+  float* sc2 = sc1 + 256;
+  KhLnTileStats<BM, 512> ln_stats;
+  float ln_c1v = 0.f, ln_c2v = 0.f;
+  if (p.ln_part != nullptr) {
+    ln_stats.load(p.ln_part, m0, M, tid);
+    if (tid < BN) {
+      ln_c1v = n0 + tid < N ? p.ln_c1[n0 + tid] : 0.f;
+      ln_c2v = n0 + tid < N ? p.ln_c2[n0 + tid] : 0.f;
+    }
+  }
+
 
   // DMA sources of this lane: unit u = wave + 8*q covers stage rows u*8 .. u*8+7 (x rows first, then W rows);
   // LDS slot = lane: row lane/8, physical piece lane%8, which holds logical piece (lane%8) ^ ((row/2)%8)
@@ -169,6 +185,10 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_ksplit_kernel(const LoraGemm
     const int col = n0 + j * 32 + l32;
     bv[j] = (p.bias != nullptr && col < N) ? (float)p.bias[col] : 0.f;
   }
+  if (p.ln_part != nullptr) {
+    ln_stats.finish(K, p.ln_eps, tid, sMu, sRs, false);
+    if (tid < BN) { sc1[tid] = ln_c1v; sc2[tid] = ln_c2v; }
+  }
   wait_cnt<0, 15>();
 
   // K loop.  Iteration t: tile t is in registers (f_cur); tile t+1 becomes visible at the barrier, after which
@@ -236,17 +256,63 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_ksplit_kernel(const LoraGemm
           acc[j][4 * g] += v[0]; acc[j][4 * g + 1] += v[1]; acc[j][4 * g + 2] += v[2]; acc[j][4 * g + 3] += v[3];
         }
     }
+    if (p.ln_part != nullptr) {
+      // y = rstd_row * (acc - mean_row * c1_col) + c2_col: four consecutive rows per accumulator group
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int col = j * 32 + l32;
+      for (int g = 0; g < 4; ++g) {
+        const int trow = wm * 32 + 8 * g + 4 * lh;
+        const f32x4 mu = *reinterpret_cast<const f32x4*>(sMu + trow), rs = *reinterpret_cast<const f32x4*>(sRs + trow);
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int row = wm * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
-        sC[row * C::LDC + col] = (bf16_t)(acc[j][v] + bv[j]);
+        for (int j = 0; j < TN; ++j) {
+          const float c1 = sc1[j * 32 + l32], c2 = sc2[j * 32 + l32];
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            sC[(trow + e) * C::LDC + j * 32 + l32] = (bf16_t)(rs[e] * (acc[j][4 * g + e] - mu[e] * c1) + c2);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int col = j * 32 + l32;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int row = wm * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+          sC[row * C::LDC + col] = (bf16_t)(acc[j][v] + bv[j]);
+        }
       }
     }
   }
   __syncthreads();
+  if (p.st_part != nullptr) {
+    // as below, and every row's (sum, sum of squares) over this tile's columns for a following folded LayerNorm: the 20
+    // pieces of a row meet in LDS (the partial strips are dead) and are added in a fixed order
+    float* sp = reinterpret_cast<float*>(smem);          // [BM][20][2]
+    static_assert(BM * 20 * 8 <= C::PART, "row statistics fit the dead partial strips");
+#pragma unroll
+    for (int q = 0; q < C::OPT; ++q) {
+      const int c = tid + q * 512, srow = c / (BN / 8), ch = c % (BN / 8);
+      const int grow = m0 + srow, gcol = n0 + ch * 8;
+      const bool ok = c < C::OPC && grow < M && gcol < N;
+      u32x4 o = ok ? *reinterpret_cast<const u32x4*>(sC + srow * C::LDC + ch * 8) : u32x4{0, 0, 0, 0};
+      if (p.res != nullptr) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          o[e] = pack_bf16x2(bf16_lo(o[e]) + bf16_lo(rr[q][e]), bf16_hi(o[e]) + bf16_hi(rr[q][e]));
+      }
+      if (ok) *reinterpret_cast<u32x4*>(p.y + (size_t)grow * N + gcol) = o;
+      float ps, pq;
+      kh_piece_sums(o, ps, pq);
+      if (c < C::OPC) *reinterpret_cast<u32x2*>(sp + 2 * c) = u32x2{__float_as_uint(ps), __float_as_uint(pq)};
+    }
+    __syncthreads();
+    if (tid < BM && m0 + tid < M) {
+      float s = 0.f, q2 = 0.f;
+#pragma unroll
+      for (int ch = 0; ch < BN / 8; ++ch) { s += sp[2 * (tid * (BN / 8) + ch)]; q2 += sp[2 * (tid * (BN / 8) + ch) + 1]; }
+      kh_ln_store_stats(p.st_part, m0 + tid, M, n_blk, p.n_tiles, s, q2);
+    }
+    return;
+  }
 #pragma unroll
   for (int q = 0; q < C::OPT; ++q) {
     const int c = tid + q * 512, srow = c / (BN / 8), ch = c % (BN / 8);
@@ -267,7 +333,12 @@ template <class C, bool CONV = false>
 int launch_ksplit(LoraGemmParams p, hipStream_t stream) {
   p.m_tiles = (p.M + C::BM - 1) / C::BM;
   p.n_tiles = (p.N + C::BN - 1) / C::BN;
-  if (hipError_t e = kh_allow_lds<lora_gemm_ksplit_kernel<C, CONV>>(C::LDS); e != hipSuccess) return (int)e;
+  static_assert(C::LDS + KH_LN_LDS <= 160 * 1024, "LDS budget with the row statistics");
+  if (hipError_t e = kh_allow_lds<lora_gemm_ksplit_kernel<C, CONV>>(C::LDS + KH_LN_LDS); e != hipSuccess) return (int)e;
+  if ((p.ln_part != nullptr || p.st_part != nullptr) && CONV) return KH_ERR_UNSUPPORTED;
+  if (p.st_part != nullptr && p.n_tiles > KH_LN_SLOTS) return KH_ERR_UNSUPPORTED;
+  p.ln_lds = C::LDS;
+  const size_t lds = (size_t)C::LDS + (p.ln_part != nullptr ? KH_LN_LDS : 0);
   // the XCD grid whose per-XCD block touches the fewest operand rows, padding counted as cost
   double best = 0;
   p.xg_n = 0;
@@ -278,7 +349,7 @@ int launch_ksplit(LoraGemmParams p, hipStream_t stream) {
     if (p.xg_n == 0 || cost < best) { best = cost; p.xg_n = gn; p.xr_m = rm; p.xr_n = rn; }
   }
   const unsigned grid = 8u * (unsigned)p.xr_m * (unsigned)p.xr_n;
-  kh_launch(CONV ? KH_TAG_CONV : KH_TAG_LORA_GEMM, lora_gemm_ksplit_kernel<C, CONV>, dim3(grid), dim3(512), C::LDS, stream, p);
+  kh_launch(CONV ? KH_TAG_CONV : KH_TAG_LORA_GEMM, lora_gemm_ksplit_kernel<C, CONV>, dim3(grid), dim3(512), lds, stream, p);
   KH_RETURN_LAST_ERROR();
 }
 

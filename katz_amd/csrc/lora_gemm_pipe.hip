@@ -282,7 +282,9 @@ __device__ __forceinline__ void k_loop(char* smem, const Dma<C, SHRINK>& dma, co
   }
 }
 
-template <class C, bool CONV = false, bool IL = false>
+// LNF bit 0: the instantiation can fold a LayerNorm in front of the layer into its epilogue (ln_part); bit 1: it can write
+// the row statistics for one behind it (st_part).  The plain one (0) carries none of that code.
+template <class C, bool CONV = false, bool IL = false, int LNF = 0>
 __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const LoraGemmParams pin) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   LoraGemmParams p = pin;
@@ -297,7 +299,8 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
       ShrinkParams sp;
       sp.x = pin.x; sp.a_cat = pin.a_cat; sp.col_scale = pin.col_scale; sp.t = const_cast<bf16_t*>(pin.t_ext);
       sp.M = pin.M; sp.K = pin.K; sp.R = pin.ldt;
-      lora_shrink_tile<SCfg<4, 2, 2>, true>(sp, bx, by, smem);
+      if (LNF & 1) { sp.ln_part = pin.ln_part; sp.ln_ca1 = pin.ln_ca1; sp.ln_ca2 = pin.ln_ca2; sp.ln_eps = pin.ln_eps; }
+      lora_shrink_tile<SCfg<4, 2, 2>, true, C::NT>(sp, bx, by, smem);
       __builtin_amdgcn_s_waitcnt(0);                          // this thread's write-through stores have completed
       __syncthreads();
       if (threadIdx.x == 0)
@@ -363,6 +366,25 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
   if (m0 >= p.M) return;   // segmented launches size the grid for the longest segment
   const int K = p.K, M = p.M, N = p.N;
   constexpr int BKP = C::BKP, ROWB = C::ROWB;
+  // folded LayerNorm: mean and 1/std of this tile's x rows, read in the epilogue (the barriers of the K loop lie between)
+  // and the two per-column terms of this (single) column tile
+  float* sMu = reinterpret_cast<float*>(smem + p.ln_lds);
+  float* sRs = sMu + 256;
+  float* sc1 = sRs + 256;
+  float* sc2 = sc1 + 256;
+  static_assert(C::BM <= 256 && C::BN <= 256 && C::BN <= C::NT, "LayerNorm terms: room in LDS, one column per thread");
+  // requested first, finished once the DMA descriptors and the bias loads below are under way
+  KhLnTileStats<C::BM, C::NT> ln_stats;
+  float ln_c1v = 0.f, ln_c2v = 0.f;
+  if ((LNF & 1) && p.ln_part != nullptr) {
+    ln_stats.load(p.ln_part, m0, M, tid);
+    if (tid < C::BN) {
+      const int col = chunk * p.n_chunk * C::BN + tid;
+      ln_c1v = col < N ? p.ln_c1[col] : 0.f;
+      ln_c2v = col < N ? p.ln_c2[col] : 0.f;
+    }
+  }
+
   const int KT1 = k_cols / BKP;                                        // K tiles of x / W
   // + rank tiles of T / B_cat (two-launch form).  Only the first r_used rank columns can be non-zero: tiles beyond
   // them are not visited, and of a last tile that they fill at most half only that half is multiplied.
@@ -385,7 +407,9 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
   auto stamp = [](int) {};
 #endif
   stamp(0);
-  for (int jt = 0; jt < p.n_chunk; ++jt) {
+  // (only the instantiations that keep T in LDS walk several column tiles; the others have exactly one per workgroup: no
+  // loop, so nothing of the epilogue's address arithmetic is hoisted above the K loop, where registers are scarcest)
+  for (int jt = 0; jt < (NRT == 0 ? 1 : p.n_chunk); ++jt) {
     const int n_tile = chunk * p.n_chunk + jt;
     if (n_tile >= p.n_tiles) break;  // uniform over the workgroup
     const int n0 = n_tile * BN;
@@ -462,6 +486,11 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
     float csv[NRTT];
 #pragma unroll
     for (int r = 0; r < NRTT; ++r) csv[r] = (shrink && NRT > 0) ? p.col_scale[r * 32 + l32] : 0.f;
+    if ((LNF & 1) && p.ln_part != nullptr && jt == 0) {
+      ln_stats.finish(K, p.ln_eps, tid, sMu, sRs, false);
+      if (tid < C::BN) { sc1[tid] = ln_c1v; sc2[tid] = ln_c2v; }
+    }
+
     constexpr int RCH = R > 0 ? R / 8 : 1;                       // 16-byte pieces per T / B_cat row
     constexpr int BCH = NRT > 0 ? BN * RCH / C::NT : 0;          // pieces of the B_cat tile per thread
     static_assert(NRT == 0 || (BN * RCH) % C::NT == 0, "expand tile split");
@@ -558,17 +587,60 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
           rr[q] = (grow < M && gcol < N) ? ld16(p.res + (size_t)grow * N + gcol) : u32x4{0, 0, 0, 0};
         }
       }
+      if ((LNF & 1) && p.ln_part != nullptr) {
+        // y = rstd_row * (acc - mean_row * c1_col) + c2_col: four consecutive rows per accumulator group
 #pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        const int col = wn * C::WTN + j * 32 + l32;
+        for (int g = 0; g < 4; ++g) {
+          const int trow = wm * C::WTM + i * 32 + 8 * g + 4 * lh;
+          const f32x4 mu = *reinterpret_cast<const f32x4*>(sMu + trow), rs = *reinterpret_cast<const f32x4*>(sRs + trow);
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const int row = wm * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
-          sC[row * C::LDC + col] = (bf16_t)(acc[i][j][v] * oscale + bv[j]);
+          for (int j = 0; j < TN; ++j) {
+            const int col = wn * C::WTN + j * 32 + l32;
+            const float c1 = sc1[col], c2 = sc2[col];
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              sC[(wm * 32 + 8 * g + 4 * lh + e) * C::LDC + col] = (bf16_t)(rs[e] * (acc[i][j][4 * g + e] - mu[e] * c1) + c2);
+          }
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          const int col = wn * C::WTN + j * 32 + l32;
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            const int row = wm * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+            sC[row * C::LDC + col] = (bf16_t)(acc[i][j][v] * oscale + bv[j]);
+          }
         }
       }
       __syncthreads();
-      if (!p.geglu) {
+      if ((LNF & 2) && !p.geglu && p.st_part != nullptr) {
+        // as below, and every row's (sum, sum of squares) over this tile's columns for a following folded LayerNorm:
+        // the CPR pieces of a row sit in CPR neighbouring lanes
+#pragma unroll
+        for (int q = 0; q < ECH; ++q) {
+          const int c = tid + q * C::NT, srow = c / CPR, ch = c % CPR;
+          const int grow = m0 + (srow >> 5) * C::WTM + i * 32 + (srow & 31), gcol = n0 + ch * 8;
+          const bool ok = grow < M && gcol < N;
+          u32x4 o = ok ? *reinterpret_cast<const u32x4*>(sC + srow * C::LDC + ch * 8) : u32x4{0, 0, 0, 0};
+          if (p.res != nullptr) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              o[e] = pack_bf16x2(bf16_lo(o[e]) + bf16_lo(rr[q][e]), bf16_hi(o[e]) + bf16_hi(rr[q][e]));
+          }
+          if (ok) *reinterpret_cast<u32x4*>(p.y + (size_t)grow * N + gcol) = o;
+          float ps, pq;
+          kh_piece_sums(o, ps, pq);
+          static_assert(CPR == 16 || CPR == 32, "a row's pieces fill one or two DPP rows");
+          ps = kh_row16_sum(ps);
+          pq = kh_row16_sum(pq);
+          if constexpr (CPR == 32) {
+            ps += __shfl_xor(ps, 16, 64);
+            pq += __shfl_xor(pq, 16, 64);
+          }
+          if (ch == 0 && grow < M) kh_ln_store_stats(p.st_part, grow, M, n_tile, p.n_tiles, ps, pq);
+        }
+      } else if (!p.geglu) {
 #pragma unroll
         for (int q = 0; q < ECH; ++q) {
           const int c = tid + q * C::NT, srow = c / CPR, ch = c % CPR;
@@ -624,7 +696,10 @@ int launch_pcfg(LoraGemmParams p, hipStream_t stream, int n_groups = 1) {
   }
   p.n_chunk = nc;
   p.n_chunks = (p.n_tiles + nc - 1) / nc;
-  if (hipError_t e = kh_allow_lds<lora_gemm_pipe_kernel<C, CONV>>((int)C::LDS_BYTES); e != hipSuccess) return (int)e;
+  constexpr bool ln_fits = C::LDS_BYTES + KH_LN_LDS <= 160 * 1024 && C::NRT == 0 && !CONV;
+  if ((p.ln_part != nullptr || p.st_part != nullptr) && (!ln_fits || p.sg_mode != 0 || p.grp != nullptr)) return KH_ERR_UNSUPPORTED;
+  if (p.st_part != nullptr && (p.geglu || p.n_tiles > KH_LN_SLOTS)) return KH_ERR_UNSUPPORTED;
+  p.ln_lds = (int)C::LDS_BYTES;
   unsigned grid = (unsigned)(p.m_tiles * p.n_chunks);
   p.xg_n = p.xr_m = p.xr_n = 0;
   if (C::NRT == 0 && !KH_DBG(p, 8)) {
@@ -638,6 +713,19 @@ int launch_pcfg(LoraGemmParams p, hipStream_t stream, int n_groups = 1) {
     }
     grid = 8u * (unsigned)p.xr_m * (unsigned)p.xr_n;
   }
+  if constexpr (ln_fits) {
+    auto go = [&](auto lnf) {
+      constexpr int L = decltype(lnf)::value;
+      if (hipError_t e = kh_allow_lds<lora_gemm_pipe_kernel<C, false, false, L>>((int)C::LDS_BYTES + KH_LN_LDS); e != hipSuccess) return (int)e;
+      kh_launch(KH_TAG_LORA_GEMM, lora_gemm_pipe_kernel<C, false, false, L>, dim3(grid, (unsigned)n_groups), dim3(C::NT),
+                C::LDS_BYTES + KH_LN_LDS, stream, p);
+      KH_RETURN_LAST_ERROR();
+    };
+    if (p.ln_part != nullptr && p.st_part != nullptr) return go(std::integral_constant<int, 3>{});
+    if (p.ln_part != nullptr) return go(std::integral_constant<int, 1>{});
+    if (p.st_part != nullptr) return go(std::integral_constant<int, 2>{});
+  }
+  if (hipError_t e = kh_allow_lds<lora_gemm_pipe_kernel<C, CONV>>((int)C::LDS_BYTES); e != hipSuccess) return (int)e;
   kh_launch(CONV ? KH_TAG_CONV : KH_TAG_LORA_GEMM, lora_gemm_pipe_kernel<C, CONV>, dim3(grid, (unsigned)n_groups), dim3(C::NT), C::LDS_BYTES, stream, p);
   KH_RETURN_LAST_ERROR();
 }
@@ -712,7 +800,7 @@ static int launch_il(const LoraGemmParams& pin, hipStream_t stream) {
   p.n_chunk = 1;
   p.n_chunks = p.n_tiles;
   constexpr int LDS = (int)C::LDS_BYTES > S::LDS ? (int)C::LDS_BYTES : S::LDS;
-  if (hipError_t e = kh_allow_lds<lora_gemm_pipe_kernel<C, false, true>>(LDS); e != hipSuccess) return (int)e;
+  p.ln_lds = LDS;
   double best = 0;
   p.xg_n = 0;
   for (int gm = 1; gm <= 8; gm *= 2) {
@@ -724,6 +812,19 @@ static int launch_il(const LoraGemmParams& pin, hipStream_t stream) {
   const int shr = ((p.M + 63) / 64) * (p.ldt / 64);
   p.il_blocks = (shr + 7) / 8 * 8;
   const unsigned grid = (unsigned)p.il_blocks + 8u * (unsigned)p.xr_m * (unsigned)p.xr_n;
+  if (p.ln_part != nullptr || p.st_part != nullptr) {
+    if (p.st_part != nullptr && p.n_tiles > KH_LN_SLOTS) return KH_ERR_UNSUPPORTED;
+    auto go = [&](auto lnf) {
+      constexpr int L = decltype(lnf)::value;
+      if (hipError_t e = kh_allow_lds<lora_gemm_pipe_kernel<C, false, true, L>>(LDS + KH_LN_LDS); e != hipSuccess) return (int)e;
+      kh_launch(KH_TAG_LORA_GEMM, lora_gemm_pipe_kernel<C, false, true, L>, dim3(grid), dim3(C::NT), (size_t)LDS + KH_LN_LDS, stream, p);
+      KH_RETURN_LAST_ERROR();
+    };
+    if (p.ln_part != nullptr && p.st_part != nullptr) return go(std::integral_constant<int, 3>{});
+    if (p.ln_part != nullptr) return go(std::integral_constant<int, 1>{});
+    return go(std::integral_constant<int, 2>{});
+  }
+  if (hipError_t e = kh_allow_lds<lora_gemm_pipe_kernel<C, false, true>>(LDS); e != hipSuccess) return (int)e;
   kh_launch(KH_TAG_LORA_GEMM, lora_gemm_pipe_kernel<C, false, true>, dim3(grid), dim3(C::NT), (size_t)LDS, stream, p);
   KH_RETURN_LAST_ERROR();
 }

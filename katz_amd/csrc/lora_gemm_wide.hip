@@ -47,6 +47,8 @@ struct WCfg {
   static constexpr int TAB_OFF = 2 * STAGE;
   static constexpr int BIAS_OFF = TAB_OFF + 2 * WTAB_N * 2;   // the tile's bias values (bf16)
   static constexpr int LDS = BIAS_OFF + BN * 2;
+  static constexpr int LN_LDS = 2 * BM * 4 + 2 * BN * 4;      // folded LayerNorm: mean, 1/std per row; c1, c2 per column (fp32)
+  static_assert(LDS % 16 == 0 && LDS + LN_LDS <= 160 * 1024, "LDS budget with the LayerNorm terms");
   static constexpr int XU = 2 * TM, WU = TN, LPS = XU + WU;   // DMA instructions per wave per stage (x rows, W rows)
   // staged row of the epilogue: (BN + pad) / 2 dwords = 4 mod 64 banks
   static constexpr int LDC = BN + ((8 + 128 - BN % 128) % 128);
@@ -142,6 +144,14 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_wide_kernel(const LoraGemmPa
       for (int j = 0; j < WTN; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.b[j], f.a[i], acc[i][j], 0, 0, 0);   // D = W . x^T: lane = row of x
   };
 
+  // folded LayerNorm: the rows' statistics and the columns' terms are requested before the first stage (older than its
+  // loads: they have arrived when it has) and put into LDS after the table below is built
+  KhLnTileStats<WBM, 512> ln_stats;
+  float ln_c1v = 0.f, ln_c2v = 0.f;
+  if (p.ln_part != nullptr) {
+    ln_stats.load(p.ln_part, m0, p.M, tid);
+    if (tid < WBN) { ln_c1v = p.ln_c1[n0 + tid]; ln_c2v = p.ln_c2[n0 + tid]; }
+  }
   // K loop over stages t (stage t & 1).  Steps 0..3 of a stage alternate between the fragment buffers fa / fb.
   WFr fa, fb;
   issue(0, 0);
@@ -149,6 +159,10 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_wide_kernel(const LoraGemmPa
   uint16_t* gtab = reinterpret_cast<uint16_t*>(smem + WTAB_OFF);
   uint16_t* sbias = reinterpret_cast<uint16_t*>(smem + WBIAS_OFF);   // like the table: written now, read in the epilogue
   if (tid < WBN) sbias[tid] = p.bias != nullptr ? reinterpret_cast<const uint16_t*>(p.bias)[n0 + tid] : (uint16_t)0;
+  float* sMu = reinterpret_cast<float*>(smem + C::LDS);   // folded LayerNorm (launched with LN_LDS more bytes)
+  float* sRs = sMu + WBM;
+  float* sc1 = sRs + WBM;
+  float* sc2 = sc1 + WBN;
   if (p.geglu) {   // published by the barriers of the K loop, read in the epilogue
 #pragma unroll
     for (int k = 0; k < 2 * WTAB_N / 512; ++k) {
@@ -156,6 +170,10 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_wide_kernel(const LoraGemmPa
       const uint32_t bits = (uint32_t)(i >= WTAB_N ? 0x8000 + (i - WTAB_N) : i) + WTAB_LO;
       gtab[i] = (uint16_t)pack_bf16x2(kh_gelu_erf(bf16_lo(bits)), 0.f);
     }
+  }
+  if (p.ln_part != nullptr) {
+    ln_stats.finish(K, p.ln_eps, tid, sMu, sRs, false);
+    if (tid < WBN) { sc1[tid] = ln_c1v; sc2[tid] = ln_c2v; }
   }
   if (KT > 1) wait_cnt<WLPS, 15>(); else wait_cnt<0, 15>();
   __builtin_amdgcn_s_barrier();
@@ -200,16 +218,33 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_wide_kernel(const LoraGemmPa
     // the MFMA operands are swapped (W rows first), so a lane holds one output row (l32) and, per group of four
     // accumulator registers, four consecutive columns: 8-byte LDS writes.  With 196-dword rows the 16 rows x 2 halves
     // of one write phase cover all 64 banks.
+    if (p.ln_part != nullptr) {
+      // y = rstd_row * (acc - mean_row * c1_col) + c2_col; this lane's row is one
+      const float mu = sMu[wm * WR + i * 32 + l32], rs = sRs[wm * WR + i * 32 + l32];
 #pragma unroll
-    for (int j = 0; j < WTN; ++j) {
+      for (int j = 0; j < WTN; ++j) {
 #pragma unroll
-      for (int g4 = 0; g4 < 4; ++g4) {
-        const int col = wn * WC + j * 32 + 8 * g4 + 4 * lh;
-        const u32x2 bb = *reinterpret_cast<const u32x2*>(sbias + col);
-        u32x2 o;
-        o[0] = pack_bf16x2(acc[i][j][4 * g4] + bf16_lo(bb[0]), acc[i][j][4 * g4 + 1] + bf16_hi(bb[0]));
-        o[1] = pack_bf16x2(acc[i][j][4 * g4 + 2] + bf16_lo(bb[1]), acc[i][j][4 * g4 + 3] + bf16_hi(bb[1]));
-        *reinterpret_cast<u32x2*>(sC + (wm * 32 + l32) * WLDC + col) = o;
+        for (int g4 = 0; g4 < 4; ++g4) {
+          const int col = wn * WC + j * 32 + 8 * g4 + 4 * lh;
+          const f32x4 c1 = *reinterpret_cast<const f32x4*>(sc1 + col), c2 = *reinterpret_cast<const f32x4*>(sc2 + col);
+          u32x2 o;
+          o[0] = pack_bf16x2(rs * (acc[i][j][4 * g4] - mu * c1[0]) + c2[0], rs * (acc[i][j][4 * g4 + 1] - mu * c1[1]) + c2[1]);
+          o[1] = pack_bf16x2(rs * (acc[i][j][4 * g4 + 2] - mu * c1[2]) + c2[2], rs * (acc[i][j][4 * g4 + 3] - mu * c1[3]) + c2[3]);
+          *reinterpret_cast<u32x2*>(sC + (wm * 32 + l32) * WLDC + col) = o;
+        }
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < WTN; ++j) {
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+          const int col = wn * WC + j * 32 + 8 * g4 + 4 * lh;
+          const u32x2 bb = *reinterpret_cast<const u32x2*>(sbias + col);
+          u32x2 o;
+          o[0] = pack_bf16x2(acc[i][j][4 * g4] + bf16_lo(bb[0]), acc[i][j][4 * g4 + 1] + bf16_hi(bb[0]));
+          o[1] = pack_bf16x2(acc[i][j][4 * g4 + 2] + bf16_lo(bb[1]), acc[i][j][4 * g4 + 3] + bf16_hi(bb[1]));
+          *reinterpret_cast<u32x2*>(sC + (wm * 32 + l32) * WLDC + col) = o;
+        }
       }
     }
     __syncthreads();
@@ -263,7 +298,7 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_wide_kernel(const LoraGemmPa
 template <class C>
 bool wide_ok(const LoraGemmParams& p) {
   const bool plain = p.R == 0 || p.t_ext != nullptr;
-  return plain && p.grp == nullptr && p.sg_mode == 0 && p.conv_cin == 0 && p.M % C::BM == 0 && p.N % C::BN == 0 &&
+  return plain && p.grp == nullptr && p.sg_mode == 0 && p.conv_cin == 0 && p.st_part == nullptr && p.M % C::BM == 0 && p.N % C::BN == 0 &&
          p.K % 64 == 0 && p.K >= 64 && (p.t_ext == nullptr || (p.R % 64 == 0 && p.ldt % 8 == 0)) &&
          (p.t_nsplit == 0 || p.t_nsplit % C::BN == 0) && (long)C::BM * (p.K > p.ldt ? p.K : p.ldt) < (1L << 31) &&
          (long)C::BN * p.K < (1L << 31);
@@ -274,7 +309,8 @@ int wide_launch(LoraGemmParams p, hipStream_t stream) {
   if (!wide_ok<C>(p)) return KH_ERR_UNSUPPORTED;
   p.m_tiles = p.M / C::BM;
   p.n_tiles = p.N / C::BN;
-  if (hipError_t e = kh_allow_lds<lora_gemm_wide_kernel<C>>(C::LDS); e != hipSuccess) return (int)e;
+  if (hipError_t e = kh_allow_lds<lora_gemm_wide_kernel<C>>(C::LDS + C::LN_LDS); e != hipSuccess) return (int)e;
+  const size_t lds = (size_t)C::LDS + (p.ln_part != nullptr ? C::LN_LDS : 0);
   // the XCD grid whose per-XCD block touches the fewest operand rows, padding counted as cost
   double best = 0;
   p.xg_n = 0;
@@ -285,7 +321,7 @@ int wide_launch(LoraGemmParams p, hipStream_t stream) {
     if (p.xg_n == 0 || cost < best) { best = cost; p.xg_n = gn; p.xr_m = rm; p.xr_n = rn; }
   }
   const unsigned grid = 8u * (unsigned)p.xr_m * (unsigned)p.xr_n;
-  kh_launch(KH_TAG_LORA_GEMM, lora_gemm_wide_kernel<C>, dim3(grid), dim3(512), C::LDS, stream, p);
+  kh_launch(KH_TAG_LORA_GEMM, lora_gemm_wide_kernel<C>, dim3(grid), dim3(512), lds, stream, p);
   KH_RETURN_LAST_ERROR();
 }
 

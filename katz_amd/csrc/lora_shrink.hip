@@ -27,7 +27,7 @@ namespace {
 template <class C>
 __global__ __launch_bounds__(C::NW * 64) void lora_shrink_kernel(const ShrinkParams p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  lora_shrink_tile<C, false>(p, blockIdx.x, blockIdx.y, smem);
+  lora_shrink_tile<C, false, C::NW * 64>(p, blockIdx.x, blockIdx.y, smem);
 }
 
 template <class C>
@@ -50,14 +50,21 @@ int launch_shrink_k(const ShrinkParams& p, hipStream_t stream) {
 
 KH_EXPORT int kh_lora_shrink_bf16(const void* x, const void* a_cat, const float* col_scale, void* t, int64_t M,
                                   int64_t K, int64_t R, void* stream) {
+  return lora_shrink_ln_launch(x, a_cat, col_scale, t, M, K, R, nullptr, nullptr, nullptr, 0.f, (hipStream_t)stream);
+}
+
+// The shrink, optionally of a layer with a folded LayerNorm (ln_part != nullptr; see ShrinkParams).
+int lora_shrink_ln_launch(const void* x, const void* a_cat, const float* col_scale, void* t, int64_t M, int64_t K, int64_t R,
+                          const float* ln_part, const float* ln_ca1, const float* ln_ca2, float ln_eps, hipStream_t s) {
   if (!x || !a_cat || !col_scale || !t || M <= 0 || K <= 0 || R <= 0) return KH_ERR_INVALID_ARG;
+  if (ln_part != nullptr && (!ln_ca1 || !ln_ca2)) return KH_ERR_INVALID_ARG;
   if (K % 64 != 0 || R % 32 != 0) return KH_ERR_UNSUPPORTED;
   if (R > 65535 * 32 || M > (1 << 24)) return KH_ERR_TOO_LARGE;
-  if (!kh_aligned16(x) || !kh_aligned16(a_cat) || !kh_aligned16(t)) return KH_ERR_ALIGNMENT;
+  if (!kh_aligned16(x) || !kh_aligned16(a_cat) || !kh_aligned16(t) || (ln_part && !kh_aligned16(ln_part))) return KH_ERR_ALIGNMENT;
   ShrinkParams p;
   p.x = (const bf16_t*)x; p.a_cat = (const bf16_t*)a_cat; p.col_scale = col_scale; p.t = (bf16_t*)t;
   p.M = (int)M; p.K = (int)K; p.R = (int)R;
-  hipStream_t s = (hipStream_t)stream;
+  p.ln_part = ln_part; p.ln_ca1 = ln_ca1; p.ln_ca2 = ln_ca2; p.ln_eps = ln_eps;
   // the largest output tile that still gives most CUs a workgroup (a 64x64 tile reads half the bytes per output of a 32x64 one)
   if (R % 64 == 0 && ((M + 63) / 64) * (R / 64) >= 160) return launch_shrink_k<2, 2, 4, 5>(p, s);
   if (R % 64 == 0 && ((M + 31) / 32) * (R / 64) >= 256) return launch_shrink_k<1, 2, 4, 5>(p, s);

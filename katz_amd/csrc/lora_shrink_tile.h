@@ -2,12 +2,17 @@
 // runs its shrink on otherwise idle CUs (lora_gemm_pipe.hip).  See lora_shrink.hip for the design.
 #pragma once
 #include "kh_common.h"
+#include "lora_gemm.h"
 
 namespace {
 
 struct ShrinkParams {
   const bf16_t* x; const bf16_t* a_cat; const float* col_scale; bf16_t* t;
   int M, K, R;
+  // x is the input of a LayerNorm folded into the layer (see LoraGemmParams): a_cat already carries the norm's weight, and
+  // the tile stores ((x . a^T) - mean * ln_ca1 + std * ln_ca2) * col_scale, the adapter's share divided by 1/std
+  const float* ln_part = nullptr; const float* ln_ca1 = nullptr; const float* ln_ca2 = nullptr;
+  float ln_eps = 0.f;
 };
 
 typedef const __attribute__((address_space(1))) void* gptr_t;
@@ -35,7 +40,7 @@ struct SCfg {
 // One output tile (bx, by) of t = bf16((x . A_cat^T) * col_scale).  The block may have more waves than C::NW: the extra
 // ones only join the barriers and the final fold.  WT: the results are stored write-through at agent scope (for
 // readers on other XCDs inside the same launch).
-template <class C, bool WT>
+template <class C, bool WT, int NTB>   // NTB: threads of the block
 __device__ __forceinline__ void lora_shrink_tile(const ShrinkParams& p, int bx, int by, char* smem) {
   constexpr int NW = C::NW, TR = C::TR, TC = C::TC, NS = C::NS, UNITS = C::UNITS, STAGE = C::STAGE, LD = C::LD;
   const int tid = threadIdx.x, lane = tid & 63;
@@ -77,8 +82,13 @@ __device__ __forceinline__ void lora_shrink_tile(const ShrinkParams& p, int bx, 
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
   const int sw = (l32 >> 1) & 7;
 
+  // folded LayerNorm: the rows' statistics are requested before the first chunk (older than every DMA load, so they have
+  // arrived when the first chunk has) and reduced after the loop
+  KhLnTileStats<TR * 32, NTB> ln_stats;
+  if (p.ln_part != nullptr) ln_stats.load(p.ln_part, m0, p.M, tid);
   if (n > 0) issue(0);
   if (n > 1) issue(1);
+
   for (int i = 0; i < n; ++i) {
     if (i + 1 < n) wait_vm<UNITS>(); else wait_vm<0>();   // chunk i has landed; chunk i+1 may be in flight
     const char* st = ring + (i % NS) * STAGE;
@@ -103,6 +113,10 @@ __device__ __forceinline__ void lora_shrink_tile(const ShrinkParams& p, int bx, 
   }
   __syncthreads();                  // every ring is dead: the partial sums reuse the memory
   float* part = reinterpret_cast<float*>(smem);   // [NW][TR*32][LD]
+  float* sMu = reinterpret_cast<float*>(smem + C::PART);   // behind the partial sums
+  float* sSg = sMu + TR * 32;
+  static_assert(C::PART + 2 * TR * 32 * 4 <= C::LDS, "room for the row statistics");
+  if (p.ln_part != nullptr) ln_stats.finish(K, p.ln_eps, tid, sMu, sSg, true);   // mean and std of this tile's rows
   if (active) {
 #pragma unroll
     for (int i = 0; i < TR; ++i)
@@ -123,6 +137,11 @@ __device__ __forceinline__ void lora_shrink_tile(const ShrinkParams& p, int bx, 
       s1 += part[(w * ROWS + rr) * LD + c + 1];
     }
     if (m0 + rr < p.M && r0 + c < p.R) {
+      if (p.ln_part != nullptr) {
+        const float mu = sMu[rr], sg = sSg[rr];
+        s0 = s0 - mu * p.ln_ca1[r0 + c] + sg * p.ln_ca2[r0 + c];
+        s1 = s1 - mu * p.ln_ca1[r0 + c + 1] + sg * p.ln_ca2[r0 + c + 1];
+      }
       const uint32_t v = pack_bf16x2(s0 * p.col_scale[r0 + c], s1 * p.col_scale[r0 + c + 1]);
       uint32_t* dst = reinterpret_cast<uint32_t*>(p.t + (size_t)(m0 + rr) * p.R + r0 + c);
       if (WT) __hip_atomic_store(dst, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

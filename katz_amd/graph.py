@@ -18,7 +18,8 @@ class GraphedUNetStep:
     """One captured step with static input / output tensors.
 
     The graph holds device addresses: of the weights, of the kernel-side weight copies (stacked q/k/v, interleaved
-    GEGLU rows, packed convolution weights, stacked time_emb_proj), of the packed adapters and of the scratch buffers.
+    GEGLU rows, the copies scaled by a folded LayerNorm's weight, packed convolution weights, stacked time_emb_proj), of
+    the packed adapters and of the scratch buffers.
     It stays valid across everything that is written IN PLACE -- new inputs, adapter weights and the global LoRA scale
     (`set_adapters` with the same adapter set, `cross_attention_kwargs["scale"]`: only `col_scale` of the linear layers is
     rewritten; adapters on 3x3 convolutions repack on any change).

@@ -19,7 +19,8 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from . import ops
-from .lora import MAX_PACKED_RANK, Adapter, PackedAdapters, interleave_geglu_rows, pack_adapters, rescale_
+from .lora import (MAX_PACKED_RANK, Adapter, PackedAdapters, fold_layer_norm, interleave_geglu_rows, pack_adapters,
+                   rescale_)
 
 CL = torch.channels_last
 
@@ -34,6 +35,22 @@ LORA_MODE = os.getenv("KATZ_LORA_MODE", "split")
 # split mode: "in_launch" lets kh_lora_linear_split_bf16 run the shrink inside the GEMM launch where the GEMM leaves
 # CUs idle; "separate" always makes two launches (for measurements)
 LORA_SHRINK = os.getenv("KATZ_LORA_SHRINK", "in_launch")
+
+# The three LayerNorms of a transformer block (attention.py:338-403) are folded into the projections behind them: the
+# linear that produces the hidden states leaves per-row sums, the linear that consumes the norm's output reads the
+# un-normalised rows and finishes the normalisation in its epilogue (kh_lora_linear_norm_bf16).  "0": run every
+# LayerNorm as a kernel of its own (for measurements).
+LN_FOLD = os.getenv("KATZ_LN_FOLD", "1") != "0"
+
+
+class RowStats:
+    """Per-row (sum, sum of squares) partials of the current hidden states of a transformer, written by the linear
+    that produced them (`valid`), read by the linear behind the next LayerNorm."""
+
+    def __init__(self, M: int, device):
+        self.buf = ops.row_stats_buffer(M, device)
+        self.valid = False
+
 
 # bumped whenever any layer rebuilds its packed adapter buffers (not on pure scale changes): consumers
 # that cache pointers into those buffers (grouped launches) rebuild when it moves
@@ -63,6 +80,7 @@ class LoRALinear(nn.Module):
         self._packed: Optional[PackedAdapters] = None
         self._packed_key = None
         self._rt = None          # (weight version, weight ptr, runtime weight, runtime bias)
+        self._ln_rt = None       # (key, folded operands) for the LayerNorm in front of this layer
         self._fused: Dict[str, float] = {}   # adapter name -> multiplier merged into weight
         self.reset_parameters()
 
@@ -186,10 +204,55 @@ class LoRALinear(nn.Module):
         self._packed_key = None  # weights moved or changed: repack on their device / dtype
         self.refresh_adapters()
 
-    def forward(self, x: torch.Tensor, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+    def norm_path_ok(self, x: torch.Tensor, stats: bool = False) -> bool:
+        """Can this call go through kh_lora_linear_norm_bf16 (a folded LayerNorm in front, row statistics out)?"""
+        p = self._packed
+        return (LN_FOLD and x.dtype == torch.bfloat16 and self.weight.dtype == torch.bfloat16 and self.in_features % 64 == 0
+                and self.out_features % 8 == 0 and (p is None or (not p.overflow and LORA_MODE == "split"))
+                and (not stats or (self.out_features <= 128 * ops.LN_SLOTS and not self.geglu)))
+
+    def _ln_terms(self, norm: "LayerNorm"):
+        """(W', c1, c2, A', ca1, ca2) of this layer behind `norm` (lora.fold_layer_norm), rebuilt when the weights, the
+        norm's parameters or the packed adapters change."""
+        _, w, b = self._rt
+        p = self._packed
+        key = (self._rt[0], id(norm), norm.weight._version, norm.bias._version, norm.weight.data_ptr(),
+               None if p is None else (p.a_cat.data_ptr(), p.a_cat._version))
+        if self._ln_rt is None or self._ln_rt[0] != key:
+            self._ln_rt = (key, fold_layer_norm(w, b, norm.weight, norm.bias, None if p is None else p.a_cat))
+        return self._ln_rt[1]
+
+    def forward(self, x: torch.Tensor, residual: Optional[torch.Tensor] = None, ln=None,
+                stats_out: Optional[RowStats] = None) -> torch.Tensor:
+        """ln = (LayerNorm module, RowStats of x): the layer computes on norm(x); with valid statistics the norm is folded
+        into the GEMM, otherwise it runs as a kernel of its own.  stats_out: left describing the result (valid) when the
+        layer can write them, marked invalid otherwise."""
         self.prepare()
         _, w, b = self._rt
         p = self._packed
+        fold = ln is not None and ln[1] is not None and ln[1].valid and self.norm_path_ok(x)
+        emit = stats_out is not None and self.norm_path_ok(x, stats=True) and not (fold and ln[1] is stats_out)
+        if ln is not None and not fold:
+            x = ln[0](x)
+        if fold or emit:
+            a = s = bc = lnarg = None
+            r_used = 0
+            if p is not None:
+                a, s, bc, r_used = p.a_cat, p.col_scale, p.b_cat, p.r_used
+            if fold:
+                norm, st = ln
+                w, c1, c2, ap, ca1, ca2 = self._ln_terms(norm)
+                b = None
+                a = ap if p is not None else None
+                lnarg = (st.buf, c1, c2, ca1, ca2, norm.eps)
+            y = ops.lora_linear_norm(x, w, b, a, s, bc, residual=residual, geglu=self.geglu,
+                                     two_launches=LORA_SHRINK == "separate", r_used=r_used, ln=lnarg,
+                                     stats_out=stats_out.buf if emit else None)
+            if stats_out is not None:
+                stats_out.valid = emit
+            return y
+        if stats_out is not None:
+            stats_out.valid = False
         if p is None:
             return ops.lora_linear(x, w, b, residual=residual, geglu=self.geglu)
         if p.overflow:
@@ -609,15 +672,19 @@ class KatzAttnProcessor:
     the to_out projection's epilogue."""
 
     def __call__(self, attn, hidden_states, encoder_hidden_states=None, attention_mask=None, temb=None,
-                 residual=None, **kwargs):
+                 residual=None, ln=None, stats_out=None, **kwargs):
+        """ln = (LayerNorm module, RowStats): hidden_states are the input of that norm, which is folded into the query
+        (self-attention: q/k/v) projection; stats_out: a RowStats the output projection fills (see LoRALinear.forward)."""
         if attention_mask is not None:
             raise NotImplementedError("attention masks are not used on the SDXL path and not implemented")
+        qkv = attn.fused_qkv(hidden_states, ln=ln) if encoder_hidden_states is None else None
+        if qkv is None and ln is not None and encoder_hidden_states is None:
+            hidden_states, ln = ln[0](hidden_states), None   # three separate projections: normalise once
         ctx = hidden_states if encoder_hidden_states is None else encoder_hidden_states
-        qkv = attn.fused_qkv(hidden_states) if encoder_hidden_states is None else None
         if qkv is not None:
             q, k, v = qkv  # self-attention: one shrink + one GEMM for the three projections
         else:
-            q = attn.to_q(hidden_states)
+            q = attn.to_q(hidden_states, ln=ln)
         if qkv is not None:
             pass
         elif encoder_hidden_states is not None and attn.ctx_kv is not None and attn.ctx_kv[0] is encoder_hidden_states:
@@ -626,7 +693,7 @@ class KatzAttnProcessor:
             k = attn.to_k(ctx)
             v = attn.to_v(ctx)
         o = ops.attention(q, k, v, attn.heads, attn.scale)
-        o = attn.to_out[0](o, residual=residual)
+        o = attn.to_out[0](o, residual=residual, stats_out=stats_out)
         return attn.to_out[1](o)
 
 
@@ -648,7 +715,7 @@ class Attention(nn.Module):
         self.ctx_kv = None  # (context tensor, k, v) filled by ContextKVProjector for the current step
         self._qkv = None    # fused to_q/to_k/to_v state (self-attention only)
 
-    def fused_qkv(self, x: torch.Tensor):
+    def fused_qkv(self, x: torch.Tensor, ln=None):
         """to_q / to_k / to_v of a self-attention as ONE GEMM over the stacked weights ([3N,K]: three
         times the workgroups of a single projection, which alone covers 160 of 256 CUs) and, with
         adapters, ONE shrink over the stacked A matrices.  Returns (q, k, v) as column views of the
@@ -680,6 +747,20 @@ class Attention(nn.Module):
             self._qkv = st
         if not st["ok"]:
             return None
+        if ln is not None and ln[1] is not None and ln[1].valid and LN_FOLD:
+            # the norm in front is folded into the stacked GEMM (ln = (LayerNorm, RowStats of x))
+            norm, stats = ln
+            key = (id(norm), norm.weight._version, norm.bias._version, norm.weight.data_ptr())
+            if st.get("ln_key") != key:
+                st["ln"] = fold_layer_norm(st["w"], None, norm.weight, norm.bias, st["a"] if st["R"] else None)
+                st["ln_key"] = key
+            wp, c1, c2, ap, ca1, ca2 = st["ln"]
+            y = ops.lora_linear_norm(x, wp, None, ap, st["s"] if st["R"] else None, st["b"] if st["R"] else None,
+                                     two_launches=LORA_SHRINK == "separate", n_split=N if st["R"] else 0,
+                                     r_used=st["r_used"] if st["R"] else 0, ln=(stats.buf, c1, c2, ca1, ca2, norm.eps))
+            return y.split(N, dim=-1)
+        if ln is not None:
+            x = ln[0](x)
         if st["R"]:
             y = ops.lora_linear_split(x, st["w"], None, st["a"], st["s"], st["b"], n_split=N,
                                       two_launches=LORA_SHRINK == "separate", r_used=st["r_used"])
@@ -721,10 +802,10 @@ class GEGLU(nn.Module):
         self.enable_fused_geglu = env_flag("ENABLE_FUSED_GEGLU")
         self.proj = LoRALinear(dim_in, dim_out * 2, geglu=not self.enable_fused_geglu)
 
-    def forward(self, x):
+    def forward(self, x, ln=None):
         if self.enable_fused_geglu:
-            return ops.geglu(self.proj(x), approximate="tanh")
-        return self.proj(x)
+            return ops.geglu(self.proj(x, ln=ln), approximate="tanh")
+        return self.proj(x, ln=ln)
 
 
 class FeedForward(nn.Module):
@@ -733,8 +814,8 @@ class FeedForward(nn.Module):
         inner = dim * mult
         self.net = nn.ModuleList([GEGLU(dim, inner), nn.Dropout(0.0), LoRALinear(inner, dim)])
 
-    def forward(self, x, residual=None):
-        return self.net[2](self.net[0](x), residual=residual)
+    def forward(self, x, residual=None, ln=None, stats_out=None):
+        return self.net[2](self.net[0](x, ln=ln), residual=residual, stats_out=stats_out)
 
 
 class BasicTransformerBlock(nn.Module):
@@ -753,11 +834,18 @@ class BasicTransformerBlock(nn.Module):
         self.norm3 = LayerNorm(dim, 1e-5)
         self.ff = FeedForward(dim)
 
-    def forward(self, h, encoder_hidden_states=None):
-        h = self.attn1(self.norm1(h), residual=h)
+    def forward(self, h, encoder_hidden_states=None, stats: Optional[RowStats] = None, last: bool = False):
+        """stats: the row statistics of h as its producer left them (or invalid); on return they describe the result,
+        unless `last` (nobody reads them).  Without it every norm runs as a kernel of its own."""
+        if stats is None:
+            h = self.attn1(self.norm1(h), residual=h)
+            if self.attn2 is not None:
+                h = self.attn2(self.norm2(h), encoder_hidden_states=encoder_hidden_states, residual=h)
+            return self.ff(self.norm3(h), residual=h)
+        h = self.attn1(h, ln=(self.norm1, stats), residual=h, stats_out=stats)
         if self.attn2 is not None:
-            h = self.attn2(self.norm2(h), encoder_hidden_states=encoder_hidden_states, residual=h)
-        return self.ff(self.norm3(h), residual=h)
+            h = self.attn2(h, encoder_hidden_states=encoder_hidden_states, ln=(self.norm2, stats), residual=h, stats_out=stats)
+        return self.ff(h, ln=(self.norm3, stats), residual=h, stats_out=None if last else stats)
 
 
 class Transformer2DModel(nn.Module):
@@ -782,9 +870,10 @@ class Transformer2DModel(nn.Module):
         tokens = lambda t: t.permute(0, 2, 3, 1).reshape(N, H * W, C)  # a view of channels_last memory
         residual = tokens(hidden_states)
         h = tokens(self.norm(hidden_states))
-        h = self.proj_in(h)
-        for blk in self.transformer_blocks:
-            h = blk(h, encoder_hidden_states)
+        stats = RowStats(N * H * W, h.device) if LN_FOLD and h.dtype == torch.bfloat16 else None
+        h = self.proj_in(h, stats_out=stats)
+        for i, blk in enumerate(self.transformer_blocks):
+            h = blk(h, encoder_hidden_states, stats=stats, last=i + 1 == len(self.transformer_blocks))
         h = self.proj_out(h, residual=residual)
         return h.view(N, H, W, C).permute(0, 3, 1, 2)
 

@@ -197,3 +197,30 @@ def module_weight(weight_for_adapter, module_name: str) -> float:
         if layer_name in module_name:
             return float(w)
     raise RuntimeError(f"No LoRA weight found for module {module_name}.")
+
+
+def fold_layer_norm(weight: torch.Tensor, bias, gamma: torch.Tensor, beta, a_cat=None):
+    """The operands of a linear whose LayerNorm (weight gamma, bias beta over the input features) is folded into the GEMM
+    (kh_lora_linear_norm_bf16):  LN(x) W^T + b = rstd * (x W'^T - mean * c1) + c2.
+    Returns (W', c1, c2, A', ca1, ca2): W' = W * gamma per input column (rounded to the weight's dtype), c1 the row sums
+    of the rounded W', c2 = b + W beta; A' / ca1 / ca2 the same for the stacked adapter A matrices (None without)."""
+    g = gamma.detach().double()
+    b = None if beta is None else beta.detach().double()
+
+    def terms(m):
+        md = m.detach().double()
+        mp = (md * g).to(m.dtype)
+        s1 = mp.double().sum(dim=1)
+        s2 = md @ b if b is not None else torch.zeros_like(s1)
+        return mp.contiguous(), s1, s2
+
+    wp, c1, c2 = terms(weight)
+    if bias is not None:
+        c2 = c2 + bias.detach().double()
+    out = [wp, c1.float().contiguous(), c2.float().contiguous()]
+    if a_cat is not None:
+        ap, ca1, ca2 = terms(a_cat)
+        out += [ap, ca1.float().contiguous(), ca2.float().contiguous()]
+    else:
+        out += [None, None, None]
+    return tuple(out)

@@ -280,6 +280,84 @@ def lora_linear_split(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torc
     return out
 
 
+LN_SLOTS = 16   # KH_LN_SLOTS: (sum, sum of squares) pairs per row in a row-statistics buffer
+
+
+def row_stats_buffer(M: int, device) -> torch.Tensor:
+    """float32 [16, M, 2]: what a linear with stats_out= writes and a linear with ln= reads (kh_lora_linear_norm_bf16)."""
+    return torch.empty((LN_SLOTS, M, 2), dtype=torch.float32, device=device)
+
+
+def lora_linear_norm(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                     a_cat: Optional[torch.Tensor] = None, col_scale: Optional[torch.Tensor] = None,
+                     b_cat: Optional[torch.Tensor] = None, residual: Optional[torch.Tensor] = None, geglu: bool = False,
+                     two_launches: bool = False, n_split: int = 0, r_used: int = 0, ln=None,
+                     stats_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The LoRA linear with a LayerNorm folded in front of it and / or the row statistics for one behind it
+    (kh_lora_linear_norm_bf16).
+
+    ln = (part, c1, c2, ca1, ca2, eps): x is then the UN-normalised input, `part` the statistics of its rows (written by
+    the linear that produced x), weight / a_cat already carry the norm's weight, c1 / c2 (float [N]) and ca1 / ca2 (float
+    [rows of a_cat], None without adapters) are the folded terms; bias must be None (it is part of c2).
+    stats_out: a row_stats_buffer for the rows of the result (after bias and residual)."""
+    lib = _lib.load()
+    _req(x, BF16, "x"); _req(weight, BF16, "weight")
+    K = x.shape[-1]
+    N = weight.shape[0]
+    M = x.numel() // K
+    R = RT = 0
+    if a_cat is not None:
+        _req(a_cat, BF16, "a_cat"); _req(b_cat, BF16, "b_cat"); _req(col_scale, torch.float32, "col_scale")
+        RT, R = a_cat.shape[0], b_cat.shape[1]
+        if n_split and (N % n_split or RT != (N // n_split) * R):
+            raise ValueError("stacked layers: a_cat must have N / n_split * R rows")
+        if not n_split and RT != R:
+            raise ValueError("a_cat and b_cat disagree on the rank")
+        if a_cat.shape != (RT, K) or b_cat.shape != (N, R) or col_scale.shape != (RT,):
+            raise ValueError("a_cat / b_cat / col_scale do not match x and weight")
+    if weight.shape[1] != K:
+        raise ValueError("weight does not match x")
+    if bias is not None:
+        _req(bias, BF16, "bias")
+    if residual is not None:
+        _req(residual, BF16, "residual")
+        if residual.numel() != M * N:
+            raise ValueError("residual must have the shape of the output")
+    part = c1 = c2 = ca1 = ca2 = None
+    eps = 0.0
+    if ln is not None:
+        part, c1, c2, ca1, ca2, eps = ln
+        if bias is not None:
+            raise ValueError("with a folded LayerNorm the bias belongs into c2")
+        for t_, n_, name in ((c1, N, "c1"), (c2, N, "c2")) + (((ca1, RT, "ca1"), (ca2, RT, "ca2")) if R else ()):
+            _req(t_, torch.float32, name)
+            if t_.numel() != n_:
+                raise ValueError(f"{name} must have {n_} elements")
+        _req(part, torch.float32, "ln part")
+        if part.numel() != M * LN_SLOTS * 2:
+            raise ValueError("ln part must be a row_stats_buffer for the rows of x")
+    if stats_out is not None:
+        _req(stats_out, torch.float32, "stats_out")
+        if stats_out.numel() != M * LN_SLOTS * 2:
+            raise ValueError("stats_out must be a row_stats_buffer for the rows of the output")
+    n_out = N // 2 if geglu else N
+    out = torch.empty(tuple(x.shape[:-1]) + (n_out,), dtype=BF16, device=x.device)
+    t = cnt = None
+    if R:
+        t = torch.empty((M, RT), dtype=BF16, device=x.device)
+        cnt = _split_counters(x.device, M)
+    flags = (1 if geglu else 0) | ((1 if two_launches else 0) << 8) | (_r_used_bits(r_used, R) << 16 if R else 0)
+    if CALL_LOG is not None:   # one entry per kernel launch
+        if R and lib.kh_lora_linear_split_launches(M, N, K, R, n_split, flags) == 2:
+            CALL_LOG.append(("lora_shrink", M, K, RT))
+        CALL_LOG.append(("lora_linear", M, N, K, R, bool(geglu), residual is not None))
+    rc = lib.kh_lora_linear_norm_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(a_cat), _ptr(col_scale), _ptr(b_cat), _ptr(t),
+                                      _ptr(cnt), _ptr(residual), _ptr(out), _ptr(part), _ptr(c1), _ptr(c2), _ptr(ca1), _ptr(ca2),
+                                      float(eps), _ptr(stats_out), M, N, K, R, n_split, flags, _stream())
+    _lib.check(rc, "kh_lora_linear_norm_bf16")
+    return out
+
+
 def lora_merge_grouped(weights: Sequence[torch.Tensor], ups: Sequence[torch.Tensor], downs: Sequence[torch.Tensor],
                        scale: float = 1.0, layer_scales: Optional[Sequence[float]] = None) -> None:
     """W_l += scale * layer_scales[l] * up_l @ down_l for all layers in ONE launch, in place (kh_lora_merge_grouped_bf16).
