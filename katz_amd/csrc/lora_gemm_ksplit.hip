@@ -24,6 +24,7 @@ namespace {
 
 typedef const __attribute__((address_space(1))) void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
 
 template <int VM, int LGKM>
 __device__ __forceinline__ void wait_cnt() {  // gfx9 encoding: vmcnt = [15:14|3:0], expcnt = [6:4], lgkmcnt = [11:8]
@@ -58,6 +59,7 @@ __device__ __attribute__((aligned(256))) const uint32_t ks_zero_page[64] = {0};
 // whose tap falls outside the image read zeros.
 template <class C, bool CONV>
 __global__ __launch_bounds__(512, 2) void lora_gemm_ksplit_kernel(const LoraGemmParams p) {
+#if __HIP_DEVICE_COMPILE__   // the host pass only needs the kernel's symbol (it cannot lower the buffer-resource type)
   extern __shared__ __attribute__((aligned(16))) char smem[];
   constexpr int BM = C::BM, BN = C::BN, TN = C::TN, KSW = C::KSW, NST = C::NST, STAGE = C::STAGE;
   constexpr int LPS_LO = C::LPS_LO, LPS_HI = C::LPS_HI, N_HI = C::N_HI;
@@ -93,18 +95,22 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_ksplit_kernel(const LoraGemm
   }
 
 
-  // DMA sources of this lane: unit u = wave + 8*q covers stage rows u*8 .. u*8+7 (x rows first, then W rows);
-  // LDS slot = lane: row lane/8, physical piece lane%8, which holds logical piece (lane%8) ^ ((row/2)%8)
-  const bf16_t* src[LPS_HI];
-  const bf16_t* src2[LPS_HI];
+  // DMA of this lane: unit u = wave + 8*q covers stage rows u*8 .. u*8+7 (x rows first, then W rows); LDS slot = lane:
+  // row lane/8, physical piece lane%8, which holds logical piece (lane%8) ^ ((row/2)%8).  The loads are buffer loads:
+  // a byte offset per lane that never changes (voff: row and piece) plus a scalar byte offset per K tile, so that the
+  // loop carries no vector address arithmetic (with per-lane 64-bit pointers the adds and selects of every stage sat in
+  // the same issue stream as the MFMAs and the loop ran at the sum of both).  An offset at or beyond the buffer's size
+  // reads zeros without touching memory: that is what a 3x3 convolution's taps in the padding do.
+  constexpr uint32_t OOB = 0x80000000u;                // every buffer here is shorter than 2 GiB
+  uint32_t voff[LPS_HI], voff2[LPS_HI];
   int tapmask[LPS_HI];                                 // CONV, x units: bit t = tap t of this lane's row is inside the image
   constexpr int XQ = BM / 64;                          // units q < XQ are x rows for every wave, the others W rows
 #pragma unroll
   for (int q = 0; q < LPS_HI; ++q) {
     int u = wave + 8 * q;
-    u = u < C::UNITS ? u : C::UNITS - 1;               // never issued (has_hi), keep the address valid
+    u = u < C::UNITS ? u : C::UNITS - 1;               // never issued (has_hi), keep the offset valid
     const int r = u * 8 + (lane >> 3);
-    const int pc = ((lane & 7) ^ ((r >> 1) & 7)) * 8;
+    const uint32_t pcb = (uint32_t)(((lane & 7) ^ ((r >> 1) & 7)) * 16);
     tapmask[q] = 0;
     if (CONV && r < BM) {
       int row = m0 + r; row = row < M ? row : M - 1;
@@ -115,55 +121,91 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_ksplit_kernel(const LoraGemm
         const int hi = hi0 + tap / 3, wi = wi0 + tap % 3;
         tapmask[q] |= (hi >= 0 && hi < p.conv_h && wi >= 0 && wi < p.conv_w) ? (1 << tap) : 0;
       }
-      src[q] = p.x + ((long)(nb * p.conv_h + hi0) * p.conv_w + wi0) * p.conv_cin + pc;
-      src2[q] = src[q];
+      // relative to one row and one pixel in front of the image (the buffer's base), so that it is never negative
+      voff[q] = (uint32_t)(((nb * p.conv_h + hi0 + 1) * p.conv_w + wi0 + 1) * p.conv_cin) * 2u + pcb;
+      voff2[q] = voff[q];
     } else if (r < BM) {
       int row = m0 + r; row = row < M ? row : M - 1;
-      src[q] = p.x + (size_t)row * K + pc;
-      src2[q] = p.t_ext == nullptr ? src[q] : p.t_ext + (size_t)row * p.ldt + pc + (p.t_nsplit > 0 ? (n0 / p.t_nsplit) * p.R : 0);
+      voff[q] = (uint32_t)row * (uint32_t)K * 2u + pcb;
+      voff2[q] = ((uint32_t)row * (uint32_t)p.ldt + (uint32_t)(p.t_nsplit > 0 ? (n0 / p.t_nsplit) * p.R : 0)) * 2u + pcb;
     } else {
       int row = n0 + r - BM; row = row < N ? row : N - 1;
-      src[q] = p.w + (size_t)row * K + pc;
-      src2[q] = p.t_ext == nullptr ? src[q] : p.b_cat + (size_t)row * p.R + pc;
+      voff[q] = (uint32_t)row * (uint32_t)K * 2u + pcb;
+      voff2[q] = (uint32_t)row * (uint32_t)p.R * 2u + pcb;
     }
   }
-  // CONV: K tiles are requested in order, so the tap and the channel offset of the next request are running scalars
+  const size_t x_bytes = CONV ? (size_t)(M / (p.conv_ho * p.conv_wo)) * p.conv_h * p.conv_w * p.conv_cin * 2 : (size_t)M * K * 2;
+  const size_t x_lead = CONV ? (size_t)(p.conv_w + 1) * p.conv_cin * 2 : 0;
+  const rsrc_t rs_x = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(reinterpret_cast<const char*>(p.x) - x_lead), 0,
+                                                         (int)(x_bytes + x_lead), 0x00020000);
+  const rsrc_t rs_w = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(p.w), 0, (int)((size_t)N * K * 2), 0x00020000);
+  const rsrc_t rs_t = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(p.t_ext != nullptr ? p.t_ext : p.x), 0,
+                                                         p.t_ext != nullptr ? (int)((size_t)M * p.ldt * 2) : 0, 0x00020000);
+  const rsrc_t rs_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(p.t_ext != nullptr ? p.b_cat : p.w), 0,
+                                                         p.t_ext != nullptr ? (int)((size_t)N * p.R * 2) : 0, 0x00020000);
+  // CONV: K tiles are requested in order, so the tap and the channel offset of the next request are running scalars, and
+  // the x offsets with the current tap's padding applied change only when the tap does
   int cv_tap = 0, cv_kw = 0, cv_c0 = 0, cv_shift = 0, cv_row = 0;
-  auto issue = [&](int t, int st) {                    // K tile t into ring stage st
-    char* stage = smem + st * STAGE;
+  uint32_t xvo[XQ];
 #pragma unroll
-    for (int q = 0; q < LPS_HI; ++q) {
-      if (q < LPS_LO || has_hi) {
-        const bf16_t* g;
-        if (CONV && q < XQ)
-          g = ((tapmask[q] >> cv_tap) & 1) ? src[q] + (cv_shift + cv_c0) : reinterpret_cast<const bf16_t*>(ks_zero_page);
-        else
-          g = t < KT1 ? src[q] + (size_t)t * 64 : src2[q] + (size_t)(t - KT1) * 64;
-        __builtin_amdgcn_global_load_lds((gptr_t)g, (lptr_t)(stage + (wave + 8 * q) * 1024), 16, 0, 0);
+  for (int q = 0; q < XQ; ++q) xvo[q] = (tapmask[q] & 1) ? voff[q] : OOB;
+  auto issue = [&](int t, auto stc) {                  // K tile t into ring stage stc
+    char* stage = smem + decltype(stc)::value * STAGE;
+    if (CONV || t < KT1) {
+      const int so = t * 128;
+#pragma unroll
+      for (int q = 0; q < LPS_HI; ++q) {
+        if (q < LPS_LO || has_hi) {
+          if (CONV && q < XQ)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_x, (lptr_t)(stage + (wave + 8 * q) * 1024), 16, xvo[q], (cv_shift + cv_c0) * 2, 0, 0);
+          else
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(q < XQ ? rs_x : rs_w, (lptr_t)(stage + (wave + 8 * q) * 1024), 16, voff[q], so, 0, 0);
+        }
       }
+    } else {
+      const int so = (t - KT1) * 128;
+#pragma unroll
+      for (int q = 0; q < LPS_HI; ++q)
+        if (q < LPS_LO || has_hi)
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(q < XQ ? rs_t : rs_b, (lptr_t)(stage + (wave + 8 * q) * 1024), 16, voff2[q], so, 0, 0);
     }
     if (CONV) {
       cv_c0 += 64;
       if (cv_c0 == p.conv_cin) {
         cv_c0 = 0; ++cv_tap; ++cv_kw; cv_shift += p.conv_cin;
         if (cv_kw == 3) { cv_kw = 0; cv_row += p.conv_w * p.conv_cin; cv_shift = cv_row; }
+#pragma unroll
+        for (int q = 0; q < XQ; ++q) xvo[q] = ((tapmask[q] >> cv_tap) & 1) ? voff[q] : OOB;
       }
     }
   };
-  // wait until at most `tiles` of this wave's younger K tiles are outstanding (and its LDS reads are done)
+  // wait until at most one of this wave's younger K tiles is outstanding (and its LDS reads are done)
   auto wait_tiles1 = [&]() { if (has_hi) wait_cnt<LPS_HI, 0>(); else wait_cnt<LPS_LO, 0>(); };
   auto wait_tiles0 = [&]() { wait_cnt<0, 0>(); };
 
+  // fragment addresses: byte offsets into a stage that never change (the stage is a compile-time constant of every
+  // unrolled step and lands in the instruction's offset field; stage 2 lies beyond that field's 64 KB and gets a
+  // second set)
   struct Fr { bf16x8 a[KSW]; bf16x8 b[KSW][TN]; };
   const int sw = (l32 >> 1) & 7;
-  auto read_frags = [&](int st, Fr& f) {
-    const char* s = smem + st * STAGE;
+  int fa[KSW], fb[KSW], fa2[KSW], fb2[KSW];
+#pragma unroll
+  for (int k = 0; k < KSW; ++k) {
+    const int po = ((2 * (wk * KSW + k) + lh) ^ sw) * 16;
+    fa[k] = (wm * 32 + l32) * 128 + po;
+    fb[k] = (BM + l32) * 128 + po;
+    fa2[k] = fa[k] + 2 * STAGE;
+    fb2[k] = fb[k] + 2 * STAGE;
+  }
+  auto read_frags = [&](auto stc, Fr& f) {
+    constexpr int ST = decltype(stc)::value;
 #pragma unroll
     for (int k = 0; k < KSW; ++k) {
-      const int po = ((2 * (wk * KSW + k) + lh) ^ sw) * 16;
-      f.a[k] = *reinterpret_cast<const bf16x8*>(s + (wm * 32 + l32) * 128 + po);
+      const char* pa = ST == 2 ? smem + fa2[k] : smem + fa[k] + ST * STAGE;
+      const char* pb = ST == 2 ? smem + fb2[k] : smem + fb[k] + ST * STAGE;
+      f.a[k] = *reinterpret_cast<const bf16x8*>(pa);
 #pragma unroll
-      for (int j = 0; j < TN; ++j) f.b[k][j] = *reinterpret_cast<const bf16x8*>(s + (BM + j * 32 + l32) * 128 + po);
+      for (int j = 0; j < TN; ++j) f.b[k][j] = *reinterpret_cast<const bf16x8*>(pb + j * 32 * 128);
     }
   };
   f32x16 acc[TN];
@@ -191,17 +233,19 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_ksplit_kernel(const LoraGemm
   }
   wait_cnt<0, 15>();
 
-  // K loop.  Iteration t: tile t is in registers (f_cur); tile t+1 becomes visible at the barrier, after which
-  // every wave has read tile t out of its stage, so that stage takes tile t+3.
+  // K loop.  Step t: tile t is in registers (cur); tile t+1 becomes visible at the barrier, after which every wave has
+  // read tile t out of its stage, so that stage takes tile t+3.  Six steps (three ring stages x two register buffers)
+  // are written out, so the stage of every access is a constant.
+  using S0 = std::integral_constant<int, 0>; using S1 = std::integral_constant<int, 1>; using S2 = std::integral_constant<int, 2>;
   Fr f0, f1;
-  issue(0, 0);
-  if (KT > 1) issue(1, 1);
+  issue(0, S0{});
+  if (KT > 1) issue(1, S1{});
   if (KT > 1) wait_tiles1(); else wait_tiles0();
   __builtin_amdgcn_s_barrier();
-  if (KT > 2) issue(2, 2);
-  read_frags(0, f0);
-  int st_next = 1, st_fill = 0;                        // stage of tile t+1, stage that tile t+3 refills (= stage of tile t)
-  auto step = [&](int t, const Fr& cur, Fr& nxt) {
+  if (KT > 2) issue(2, S2{});
+  read_frags(S0{}, f0);
+  // st_next: stage of tile t+1; st_fill: stage that tile t+3 refills (= stage of tile t)
+  auto step = [&](int t, const Fr& cur, Fr& nxt, auto st_next, auto st_fill) {
     if (t + 1 < KT) {
       if (t + 2 < KT) wait_tiles1(); else wait_tiles0();
       __builtin_amdgcn_s_barrier();
@@ -209,15 +253,21 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_ksplit_kernel(const LoraGemm
       read_frags(st_next, nxt);
     }
     mma(cur);
-    st_fill = st_next;
-    st_next = st_next + 1 == NST ? 0 : st_next + 1;
   };
   int t = 0;
-  for (; t + 1 < KT; t += 2) {
-    step(t, f0, f1);
-    step(t + 1, f1, f0);
+  for (; t + 6 <= KT; t += 6) {
+    step(t, f0, f1, S1{}, S0{});
+    step(t + 1, f1, f0, S2{}, S1{});
+    step(t + 2, f0, f1, S0{}, S2{});
+    step(t + 3, f1, f0, S1{}, S0{});
+    step(t + 4, f0, f1, S2{}, S1{});
+    step(t + 5, f1, f0, S0{}, S2{});
   }
-  if (t < KT) step(t, f0, f1);
+  if (t < KT) step(t, f0, f1, S1{}, S0{});
+  if (t + 1 < KT) step(t + 1, f1, f0, S2{}, S1{});
+  if (t + 2 < KT) step(t + 2, f0, f1, S0{}, S2{});
+  if (t + 3 < KT) step(t + 3, f1, f0, S1{}, S0{});
+  if (t + 4 < KT) step(t + 4, f0, f1, S2{}, S1{});
   __syncthreads();   // the ring is dead: partial strips and the staging tile reuse it
 
   // residual pieces of this thread, requested before the reduction
@@ -327,6 +377,7 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_ksplit_kernel(const LoraGemm
       *reinterpret_cast<u32x4*>(p.y + (size_t)grow * N + gcol) = o;
     }
   }
+#endif
 }
 
 template <class C, bool CONV = false>
@@ -355,9 +406,17 @@ int launch_ksplit(LoraGemmParams p, hipStream_t stream) {
 
 }  // namespace
 
+// every operand is addressed as a buffer with 32-bit byte offsets: shorter than 2 GiB each
+static bool ks_fits_buffers(const LoraGemmParams& p) {
+  const size_t lim = (size_t)1 << 31;
+  const size_t xb = p.conv_cin > 0 ? ((size_t)(p.M / (p.conv_ho * p.conv_wo)) * p.conv_h + 1) * p.conv_w * p.conv_cin * 2 + 2 * (size_t)p.conv_cin
+                                   : (size_t)p.M * p.K * 2;
+  return xb < lim && (size_t)p.N * p.K * 2 < lim && (size_t)p.M * (p.ldt > 0 ? p.ldt : 1) * 2 < lim && (size_t)p.N * (p.R > 0 ? p.R : 1) * 2 < lim;
+}
+
 bool lora_gemm_ksplit_ok(const LoraGemmParams& p) {
   const bool plain = p.R == 0 || p.t_ext != nullptr;
-  return plain && p.grp == nullptr && p.sg_mode == 0 && p.conv_cin == 0 && !p.geglu && p.K % 64 == 0 && p.K >= 64 &&
+  return plain && ks_fits_buffers(p) && p.grp == nullptr && p.sg_mode == 0 && p.conv_cin == 0 && !p.geglu && p.K % 64 == 0 && p.K >= 64 &&
          (p.t_ext == nullptr || (p.R % 64 == 0 && p.ldt % 8 == 0)) && (p.t_nsplit == 0 || p.t_nsplit % 160 == 0) &&
          p.N % 8 == 0;
 }
@@ -369,7 +428,7 @@ int lora_gemm_ksplit_launch(const LoraGemmParams& p, int row_groups, hipStream_t
 
 // 3x3 convolution on the same tiles (conv_* fields set, R == 0, K == 9 * conv_cin, conv_cin % 64 == 0).
 bool lora_gemm_ksplit_conv_ok(const LoraGemmParams& p) {
-  return p.conv_cin > 0 && p.conv_cin % 64 == 0 && p.K == 9 * p.conv_cin && p.R == 0 && p.t_ext == nullptr && p.grp == nullptr &&
+  return p.conv_cin > 0 && p.conv_cin % 64 == 0 && p.K == 9 * p.conv_cin && ks_fits_buffers(p) && p.R == 0 && p.t_ext == nullptr && p.grp == nullptr &&
          p.sg_mode == 0 && !p.geglu && p.N % 8 == 0;
 }
 

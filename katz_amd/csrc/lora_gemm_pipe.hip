@@ -867,6 +867,7 @@ int lora_gemm_pipe_launch(const LoraGemmParams& p, int tile_sel, hipStream_t str
     case 20: return deep_stage_ok(p) ? launch_pcfg<PCfg<128, 128, 2, 2, 0, 3, 64>>(p, stream) : KH_ERR_UNSUPPORTED;
     case 27: return plain_ok(p) ? launch_pcfg<PCfg<256, 128, 4, 2, 0, 4>>(p, stream) : KH_ERR_UNSUPPORTED;
     case 28: return plain_ok(p) ? launch_pcfg<PCfg<128, 256, 2, 4, 0, 4>>(p, stream) : KH_ERR_UNSUPPORTED;
+    case 29: return deep_stage_ok(p) ? launch_pcfg<PCfg<256, 128, 4, 2, 0, 3, 64>>(p, stream) : KH_ERR_UNSUPPORTED;
     case 32: return deep_stage_ok(p) ? launch_pcfg<PCfg<128, 128, 2, 4, 0, 3, 64>>(p, stream) : KH_ERR_UNSUPPORTED;
     case 40: return lora_gemm_ksplit_launch(p, 2, stream);
     case 41: return lora_gemm_ksplit_launch(p, 4, stream);
