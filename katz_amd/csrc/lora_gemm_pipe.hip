@@ -282,6 +282,184 @@ __device__ __forceinline__ void k_loop(char* smem, const Dma<C, SHRINK>& dma, co
   }
 }
 
+// The K loop of every instantiation that does not accumulate the shrink itself.  What differs from k_loop above is
+// how addresses are formed.  Loads are buffer loads: a byte offset per lane that never changes (row and swizzled piece
+// inside the tile) plus a scalar byte offset per K tile; fragment reads use per-lane offsets that never change plus the
+// stage as an instruction offset, because the ring's stages are written out as constants (lcm(NST, 2) steps per group:
+// ring position x register buffer).  The loop then carries no vector address arithmetic: with per-lane 64-bit pointers
+// the adds and selects of every stage shared the issue stream with the MFMAs, and a stage cost the sum of both.
+// An offset at or beyond the buffer's size reads zeros without touching memory: the convolution's taps in the padding.
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+template <int I> using IC = std::integral_constant<int, I>;
+
+template <class C>
+struct Dma2 {
+  static constexpr int XI = C::UX / C::NW, WI = C::UW / C::NW, LPS = XI + WI;
+  uint32_t voff[LPS];    // x units first, then W units: byte offset of this lane's 16 bytes at K column 0
+  uint32_t voff2[LPS];   // the same in the K-extension operands (T for the x rows, B_cat for the W rows)
+  int tapmask[XI];       // CONV: bit t = tap t of this lane's pixel is inside the image
+};
+
+struct Rsrc4 { rsrc_t x, w, t, b; };
+
+template <class C, bool CONV, bool IL>
+__device__ __forceinline__ void k_loop2(char* smem, const Dma2<C>& dma, const Rsrc4& rs, int KT, int KT1, int lane, int wave,
+                                        int wm, int wn, int l32, int lh, int sw, f32x16 (&acc)[C::TM][C::TN], ConvGeom cg,
+                                        const int* il_cnt, int il_target, int* il_err, bool half_last) {
+#if __HIP_DEVICE_COMPILE__
+  constexpr int TM = C::TM, TN = C::TN, NST = C::NST, BKP = C::BKP, ROWB = C::ROWB, KS = C::KS, STAGE = C::STAGE;
+  constexpr int PD = NST - 1;                           // prefetch distance in K tiles
+  constexpr int U = (NST % 2 == 0) ? NST : 2 * NST;     // steps per written-out group
+  static_assert(NST == 3 || NST == 4, "groups of 6 or 4 steps");
+  using D = Dma2<C>;
+  using F = Frags<C, false>;
+  constexpr uint32_t OOB = 0x80000000u;                 // a convolution's image is shorter than 2 GiB
+  int cv_tap = 0, cv_kw = 0, cv_c0 = 0, cv_shift = 0, cv_row = 0;
+  uint32_t xvo[D::XI];                                  // CONV: the x offsets with the current tap's padding applied
+#pragma unroll
+  for (int q = 0; q < D::XI; ++q) xvo[q] = (!CONV || (dma.tapmask[q] & 1)) ? dma.voff[q] : OOB;
+
+  auto issue = [&](int t, auto stc) {
+    char* stage = smem + decltype(stc)::value * STAGE;
+    if (CONV || t < KT1) {
+      const int so = t * (BKP * 2);
+#pragma unroll
+      for (int q = 0; q < D::XI; ++q)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs.x, (lptr_t)(stage + (wave * D::XI + q) * 1024), 16, CONV ? xvo[q] : dma.voff[q],
+                                                 CONV ? (cv_shift + cv_c0) * 2 : so, 0, 0);
+#pragma unroll
+      for (int q = 0; q < D::WI; ++q)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs.w, (lptr_t)(stage + C::SW_OFF + (wave * D::WI + q) * 1024), 16, dma.voff[D::XI + q], so, 0, 0);
+      if (CONV) {
+        cv_c0 += BKP;
+        if (cv_c0 == cg.cin) {
+          cv_c0 = 0; ++cv_tap; ++cv_kw; cv_shift += cg.cin;
+          if (cv_kw == 3) { cv_kw = 0; cv_row += cg.w * cg.cin; cv_shift = cv_row; }
+#pragma unroll
+          for (int q = 0; q < D::XI; ++q) xvo[q] = ((dma.tapmask[q] >> cv_tap) & 1) ? dma.voff[q] : OOB;
+        }
+      }
+    } else {
+      // K tiles >= KT1 come from the extension operands: y = [x | T] . [W | B_cat]^T
+      if (IL && t == KT1) {
+        // first request for T: wait (bounded) until the shrink workgroups of this row block have all arrived
+        if (lane == 0) {
+          int it = 0;
+          while (__hip_atomic_load(il_cnt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < il_target && ++it < (1 << 20))
+            __builtin_amdgcn_s_sleep(8);
+          if (it >= (1 << 20)) {
+            __hip_atomic_store(il_err, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_fetch_add(&kh_split_timeout_count, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
+        }
+      }
+      const int so = (t - KT1) * (BKP * 2);
+#pragma unroll
+      for (int q = 0; q < D::XI; ++q) {
+        // (IL) T was written inside this launch, maybe on another XCD: read past the (non-coherent) L2
+        if (IL) __builtin_amdgcn_raw_ptr_buffer_load_lds(rs.t, (lptr_t)(stage + (wave * D::XI + q) * 1024), 16, dma.voff2[q], so, 0, 17 /* sc0 sc1 */);
+        else __builtin_amdgcn_raw_ptr_buffer_load_lds(rs.t, (lptr_t)(stage + (wave * D::XI + q) * 1024), 16, dma.voff2[q], so, 0, 0);
+      }
+#pragma unroll
+      for (int q = 0; q < D::WI; ++q)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs.b, (lptr_t)(stage + C::SW_OFF + (wave * D::WI + q) * 1024), 16, dma.voff2[D::XI + q], so, 0, 0);
+    }
+  };
+  // fragment offsets inside a stage; stages 2 and 3 lie beyond the 64 KB an instruction offset reaches: second set
+  int fa[KS], fb[KS], fa2[KS], fb2[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    const int po = ((2 * ks + lh) ^ sw) * 16;
+    fa[ks] = (wm * C::WTM + l32) * ROWB + po;
+    fb[ks] = C::SW_OFF + (wn * C::WTN + l32) * ROWB + po;
+    fa2[ks] = fa[ks] + 2 * STAGE;
+    fb2[ks] = fb[ks] + 2 * STAGE;
+  }
+  auto read_frags = [&](auto stc, F& f) {
+    constexpr int ST = decltype(stc)::value;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const char* pa = ST >= 2 ? smem + fa2[ks] + (ST - 2) * STAGE : smem + fa[ks] + ST * STAGE;
+      const char* pb = ST >= 2 ? smem + fb2[ks] + (ST - 2) * STAGE : smem + fb[ks] + ST * STAGE;
+#pragma unroll
+      for (int i = 0; i < TM; ++i) f.a[ks][i] = lds_frag(pa + i * 32 * ROWB);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) f.b[ks][j] = lds_frag(pb + j * 32 * ROWB);
+    }
+  };
+  auto mma = [&](const F& f, int half) {  // half 0 / 1 of the tile's k-steps
+#pragma unroll
+    for (int k2 = 0; k2 < KS / 2; ++k2) {
+      const int ks = half * (KS / 2) + k2;
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a[ks][i], f.b[ks][j], acc[i][j], 0, 0, 0);
+    }
+  };
+  // wait until at most n of this wave's younger K tiles are outstanding, and its LDS reads are done
+  auto wait_younger = [&](int n) {
+    if (n >= PD - 1) wait_cnt<D::LPS * (PD - 1), 0>();
+    else if (n == 1) wait_cnt<D::LPS, 0>();
+    else wait_cnt<0, 0>();
+  };
+  // Step t: tile t is in `cur`.  Half its MFMAs, then tile t+1 becomes visible (this wave's loads of it are complete,
+  // its LDS reads of tile t are complete, bare s_barrier: a fence would drain the prefetches), the stage of tile t takes
+  // tile t+1+PD, the fragments of tile t+1 are read, the other half of the MFMAs runs under those reads.
+  auto step = [&](int t, const F& cur, F& nxt, auto st_next, auto st_fill, auto steady) {
+    mma(cur, 0);
+    if constexpr (decltype(steady)::value) {
+      wait_cnt<D::LPS * (PD - 1), 0>();
+      __builtin_amdgcn_s_barrier();
+      issue(t + 1 + PD, st_fill);
+      read_frags(st_next, nxt);
+      mma(cur, 1);
+    } else {
+      if (t + 1 < KT) {
+        wait_younger(KT - 2 - t);
+        __builtin_amdgcn_s_barrier();
+        if (t + 1 + PD < KT) issue(t + 1 + PD, st_fill);
+        read_frags(st_next, nxt);
+      }
+      if (!(half_last && t == KT - 1)) mma(cur, 1);
+    }
+  };
+
+  wait_cnt<0, 15>();  // stores of an earlier phase are out of the way of the counting below
+  F f0, f1;
+  issue(0, IC<0>{});
+  if (KT > 1) issue(1, IC<1>{});
+  if (PD > 2 && KT > 2) issue(2, IC<2>{});
+  wait_younger(KT - 1);
+  __builtin_amdgcn_s_barrier();
+  if (KT > PD) issue(PD, IC<PD>{});
+  read_frags(IC<0>{}, f0);
+  using T1 = std::true_type; using T0 = std::false_type;
+  int t = 0;
+  for (; t + U + PD < KT; t += U) {
+    step(t, f0, f1, IC<1 % NST>{}, IC<0>{}, T1{});
+    step(t + 1, f1, f0, IC<2 % NST>{}, IC<1 % NST>{}, T1{});
+    step(t + 2, f0, f1, IC<3 % NST>{}, IC<2 % NST>{}, T1{});
+    step(t + 3, f1, f0, IC<4 % NST>{}, IC<3 % NST>{}, T1{});
+    if constexpr (U == 6) {
+      step(t + 4, f0, f1, IC<5 % NST>{}, IC<4 % NST>{}, T1{});
+      step(t + 5, f1, f0, IC<6 % NST>{}, IC<5 % NST>{}, T1{});
+    }
+  }
+  for (; t < KT; t += U) {
+    step(t, f0, f1, IC<1 % NST>{}, IC<0>{}, T0{});
+    if (t + 1 < KT) step(t + 1, f1, f0, IC<2 % NST>{}, IC<1 % NST>{}, T0{});
+    if (t + 2 < KT) step(t + 2, f0, f1, IC<3 % NST>{}, IC<2 % NST>{}, T0{});
+    if (t + 3 < KT) step(t + 3, f1, f0, IC<4 % NST>{}, IC<3 % NST>{}, T0{});
+    if constexpr (U == 6) {
+      if (t + 4 < KT) step(t + 4, f0, f1, IC<5 % NST>{}, IC<4 % NST>{}, T0{});
+      if (t + 5 < KT) step(t + 5, f1, f0, IC<6 % NST>{}, IC<5 % NST>{}, T0{});
+    }
+  }
+#endif
+}
+
 // LNF bit 0: the instantiation can fold a LayerNorm in front of the layer into its epilogue (ln_part); bit 1: it can write
 // the row statistics for one behind it (st_part).  The plain one (0) carries none of that code.
 template <class C, bool CONV = false, bool IL = false, int LNF = 0>
@@ -511,18 +689,77 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
         dma_setup(d);
         k_loop<C, true, BCH, false>(smem, d, p.x, p.w, p.a_cat, p.t_ext, p.b_cat, KT, KT1, lane, wm, wn, l32, lh, sw, acc, tacc, tail_loads, ConvGeom{0, 0});
       }
-    } else {
+    } else if constexpr (NRT > 0) {
+      // later column tiles of an instantiation that keeps T in LDS: the B_cat tile rides in the old loop's tail
       Dma<C, false> d;
       dma_setup(d);
+      k_loop<C, false, BCH, CONV>(smem, d, p.x, p.w, p.a_cat, p.t_ext, p.b_cat, KT, KT1, lane, wm, wn, l32, lh, sw, acc, tacc, tail_loads,
+                                  ConvGeom{p.conv_w, p.conv_cin}, false, false, nullptr, 0, nullptr, half_last);
+    } else {
+#if __HIP_DEVICE_COMPILE__
+      // buffer form of the operands: every buffer starts at this tile's first row, so the per-lane offsets stay small
+      // whatever the size of the matrix (a convolution's image as a whole: shorter than 2 GiB, checked by the launcher)
+      Dma2<C> d;
+      using D2 = Dma2<C>;
+#pragma unroll
+      for (int i = 0; i < D2::XI; ++i) {
+        const int r = (wave * D2::XI + i) * C::UROWS + u_row;  // row inside the x tile
+        const uint32_t pcb = (uint32_t)(((lane % C::PPR) ^ ((r / C::SWR) % C::PPR)) * 16);
+        int row = m0 + r; row = row < M ? row : M - 1;
+        if constexpr (CONV) {
+          // output pixel -> the input pixel above-left of its 3x3 window, and which taps are inside the image; the
+          // offset is relative to one row and one pixel in front of the image (the buffer's base): never negative
+          const int wo = row % p.conv_wo, t2 = row / p.conv_wo, ho = t2 % p.conv_ho, nb = t2 / p.conv_ho;
+          const int hi0 = ho * p.conv_stride - 1, wi0 = wo * p.conv_stride - 1;
+          int mask = 0;
+#pragma unroll
+          for (int tap = 0; tap < 9; ++tap) {
+            const int hi = hi0 + tap / 3, wi = wi0 + tap % 3;
+            mask |= (hi >= 0 && hi < p.conv_h && wi >= 0 && wi < p.conv_w) ? (1 << tap) : 0;
+          }
+          d.voff[i] = (uint32_t)(((nb * p.conv_h + hi0 + 1) * p.conv_w + wi0 + 1) * p.conv_cin) * 2u + pcb;
+          d.voff2[i] = d.voff[i];
+          d.tapmask[i] = mask;
+        } else {
+          d.voff[i] = (uint32_t)(row - m0) * (uint32_t)K * 2u + pcb;
+          d.voff2[i] = (uint32_t)(row - m0) * (uint32_t)p.ldt * 2u + pcb;
+          d.tapmask[i] = 0;
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < D2::WI; ++i) {
+        const int r = (wave * D2::WI + i) * C::UROWS + u_row;
+        const uint32_t pcb = (uint32_t)(((lane % C::PPR) ^ ((r / C::SWR) % C::PPR)) * 16);
+        int row = n0 + r; row = row < N ? row : N - 1;
+        d.voff[D2::XI + i] = (uint32_t)(row - n0) * (uint32_t)K * 2u + pcb;
+        d.voff2[D2::XI + i] = (uint32_t)(row - n0) * (uint32_t)p.R * 2u + pcb;
+      }
+      auto clamp32 = [](size_t bytes) { return (int)(uint32_t)(bytes < 0xFFFFFFFFull ? bytes : 0xFFFFFFFFull); };
+      auto mk = [&](const bf16_t* base, size_t bytes) {
+        return __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(base), 0, clamp32(bytes), 0x00020000);
+      };
+      Rsrc4 rs;
+      if constexpr (CONV) {
+        const size_t lead = (size_t)(p.conv_w + 1) * p.conv_cin;
+        rs.x = mk(p.x - lead, ((size_t)(M / (p.conv_ho * p.conv_wo)) * p.conv_h * p.conv_w * p.conv_cin + lead) * 2);
+      } else {
+        rs.x = mk(p.x + (size_t)m0 * K, (size_t)(M - m0) * K * 2);
+      }
+      rs.w = mk(p.w + (size_t)n0 * K, (size_t)(N - n0) * K * 2);
+      const bool ext = p.t_ext != nullptr;
+      const size_t tcol = p.t_nsplit > 0 ? (size_t)(n0 / p.t_nsplit) * p.R : 0;
+      rs.t = mk(ext ? p.t_ext + (size_t)m0 * p.ldt + tcol : p.x, ext ? ((size_t)(M - m0) * p.ldt - tcol) * 2 : 0);
+      rs.b = mk(ext ? p.b_cat + (size_t)n0 * p.R : p.w, ext ? (size_t)(N - n0) * p.R * 2 : 0);
       if constexpr (IL) {
         constexpr int TPB = BM / 64;                                                   // 64-row shrink tiles per row block
         const int gx = (M + 63) / 64, rt = gx - TPB * m_blk < TPB ? gx - TPB * m_blk : TPB;
-        k_loop<C, false, BCH, CONV, decltype(tail_loads), true>(smem, d, p.x, p.w, p.a_cat, p.t_ext, p.b_cat, KT, KT1, lane, wm, wn, l32, lh, sw, acc, tacc, tail_loads, ConvGeom{0, 0}, false, false,
-                                                                p.il_cnt + m_blk, rt * (p.ldt / 64), p.il_cnt + (p.M + 127) / 128, half_last);
+        k_loop2<C, CONV, true>(smem, d, rs, KT, KT1, lane, wave, wm, wn, l32, lh, sw, acc, ConvGeom{0, 0},
+                               p.il_cnt + m_blk, rt * (p.ldt / 64), p.il_cnt + (p.M + 127) / 128, half_last);
       } else {
-        k_loop<C, false, BCH, CONV>(smem, d, p.x, p.w, p.a_cat, p.t_ext, p.b_cat, KT, KT1, lane, wm, wn, l32, lh, sw, acc, tacc, tail_loads, ConvGeom{p.conv_w, p.conv_cin}, KH_DBG(p, 64), KH_DBG(p, 128),
-                                    nullptr, 0, nullptr, half_last);
+        k_loop2<C, CONV, false>(smem, d, rs, KT, KT1, lane, wave, wm, wn, l32, lh, sw, acc, ConvGeom{p.conv_w, p.conv_cin},
+                                nullptr, 0, nullptr, half_last);
       }
+#endif
     }
     stamp(2);
     __syncthreads();  // every wave is done reading the ring before sB / sC reuse it
