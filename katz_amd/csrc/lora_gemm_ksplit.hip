@@ -25,16 +25,17 @@ namespace {
 typedef const __attribute__((address_space(1))) void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
 typedef __amdgpu_buffer_rsrc_t rsrc_t;
+template <int I> using IC = std::integral_constant<int, I>;
 
 template <int VM, int LGKM>
 __device__ __forceinline__ void wait_cnt() {  // gfx9 encoding: vmcnt = [15:14|3:0], expcnt = [6:4], lgkmcnt = [11:8]
   __builtin_amdgcn_s_waitcnt((VM & 15) | (7 << 4) | ((LGKM & 15) << 8) | ((VM >> 4) << 14));
 }
 
-template <int WM_>
+template <int WM_, int NST_ = 4>
 struct KCfg {
   static constexpr int WM = WM_, WK = 8 / WM_;       // row groups x k-slices = 8 waves
-  static constexpr int BM = 32 * WM, BN = 160, BK = 64, NST = 3, TN = 5;
+  static constexpr int BM = 32 * WM, BN = 160, BK = 64, NST = NST_, TN = 5;   // NST ring stages: loads run NST - 1 K tiles ahead
   static constexpr int KSW = 4 / WK;                 // 16-column MFMA steps of a stage per wave
   static constexpr int UNITS = (BM + BN) / 8;        // DMA instructions per stage (8 rows x 128 B each)
   static constexpr int LPS_LO = UNITS / 8, N_HI = UNITS % 8, LPS_HI = LPS_LO + (N_HI ? 1 : 0);
@@ -179,9 +180,14 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_ksplit_kernel(const LoraGemm
       }
     }
   };
-  // wait until at most one of this wave's younger K tiles is outstanding (and its LDS reads are done)
-  auto wait_tiles1 = [&]() { if (has_hi) wait_cnt<LPS_HI, 0>(); else wait_cnt<LPS_LO, 0>(); };
-  auto wait_tiles0 = [&]() { wait_cnt<0, 0>(); };
+  // wait until at most n of this wave's younger K tiles are outstanding (and its LDS reads are done)
+  constexpr int PD = NST - 1;                            // prefetch distance in K tiles
+  static_assert(NST == 3 || NST == 4, "groups of 6 or 4 written-out steps");
+  auto wait_younger = [&](int n) {
+    if (n >= PD - 1) { if (has_hi) wait_cnt<LPS_HI * (PD - 1), 0>(); else wait_cnt<LPS_LO * (PD - 1), 0>(); }
+    else if (n == 1) { if (has_hi) wait_cnt<LPS_HI, 0>(); else wait_cnt<LPS_LO, 0>(); }
+    else wait_cnt<0, 0>();
+  };
 
   // fragment addresses: byte offsets into a stage that never change (the stage is a compile-time constant of every
   // unrolled step and lands in the instruction's offset field; stage 2 lies beyond that field's 64 KB and gets a
@@ -201,8 +207,8 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_ksplit_kernel(const LoraGemm
     constexpr int ST = decltype(stc)::value;
 #pragma unroll
     for (int k = 0; k < KSW; ++k) {
-      const char* pa = ST == 2 ? smem + fa2[k] : smem + fa[k] + ST * STAGE;
-      const char* pb = ST == 2 ? smem + fb2[k] : smem + fb[k] + ST * STAGE;
+      const char* pa = ST >= 2 ? smem + fa2[k] + (ST - 2) * STAGE : smem + fa[k] + ST * STAGE;
+      const char* pb = ST >= 2 ? smem + fb2[k] + (ST - 2) * STAGE : smem + fb[k] + ST * STAGE;
       f.a[k] = *reinterpret_cast<const bf16x8*>(pa);
 #pragma unroll
       for (int j = 0; j < TN; ++j) f.b[k][j] = *reinterpret_cast<const bf16x8*>(pb + j * 32 * 128);
@@ -234,40 +240,54 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_ksplit_kernel(const LoraGemm
   wait_cnt<0, 15>();
 
   // K loop.  Step t: tile t is in registers (cur); tile t+1 becomes visible at the barrier, after which every wave has
-  // read tile t out of its stage, so that stage takes tile t+3.  Six steps (three ring stages x two register buffers)
-  // are written out, so the stage of every access is a constant.
-  using S0 = std::integral_constant<int, 0>; using S1 = std::integral_constant<int, 1>; using S2 = std::integral_constant<int, 2>;
+  // read tile t out of its stage, so that stage takes tile t+1+PD.  lcm(NST, 2) steps (ring stages x two register
+  // buffers) are written out, so the stage of every access is a constant; the steady group carries no conditions.
   Fr f0, f1;
-  issue(0, S0{});
-  if (KT > 1) issue(1, S1{});
-  if (KT > 1) wait_tiles1(); else wait_tiles0();
+  issue(0, IC<0>{});
+  if (KT > 1) issue(1, IC<1>{});
+  if (PD > 2 && KT > 2) issue(2, IC<2>{});
+  wait_younger(KT - 1);
   __builtin_amdgcn_s_barrier();
-  if (KT > 2) issue(2, S2{});
-  read_frags(S0{}, f0);
-  // st_next: stage of tile t+1; st_fill: stage that tile t+3 refills (= stage of tile t)
-  auto step = [&](int t, const Fr& cur, Fr& nxt, auto st_next, auto st_fill) {
-    if (t + 1 < KT) {
-      if (t + 2 < KT) wait_tiles1(); else wait_tiles0();
+  if (KT > PD) issue(PD, IC<PD>{});
+  read_frags(IC<0>{}, f0);
+  // st_next: stage of tile t+1; st_fill: stage that tile t+1+PD refills (= stage of tile t)
+  auto step = [&](int t, const Fr& cur, Fr& nxt, auto st_next, auto st_fill, auto steady) {
+    if constexpr (decltype(steady)::value) {
+      wait_younger(PD - 1);
       __builtin_amdgcn_s_barrier();
-      if (t + 3 < KT) issue(t + 3, st_fill);
+      issue(t + 1 + PD, st_fill);
+      read_frags(st_next, nxt);
+    } else if (t + 1 < KT) {
+      wait_younger(KT - 2 - t);
+      __builtin_amdgcn_s_barrier();
+      if (t + 1 + PD < KT) issue(t + 1 + PD, st_fill);
       read_frags(st_next, nxt);
     }
     mma(cur);
   };
+  constexpr int U = (NST % 2 == 0) ? NST : 2 * NST;
+  using T1 = std::true_type; using T0 = std::false_type;
   int t = 0;
-  for (; t + 6 <= KT; t += 6) {
-    step(t, f0, f1, S1{}, S0{});
-    step(t + 1, f1, f0, S2{}, S1{});
-    step(t + 2, f0, f1, S0{}, S2{});
-    step(t + 3, f1, f0, S1{}, S0{});
-    step(t + 4, f0, f1, S2{}, S1{});
-    step(t + 5, f1, f0, S0{}, S2{});
+  for (; t + U + PD < KT; t += U) {
+    step(t, f0, f1, IC<1 % NST>{}, IC<0>{}, T1{});
+    step(t + 1, f1, f0, IC<2 % NST>{}, IC<1 % NST>{}, T1{});
+    step(t + 2, f0, f1, IC<3 % NST>{}, IC<2 % NST>{}, T1{});
+    step(t + 3, f1, f0, IC<4 % NST>{}, IC<3 % NST>{}, T1{});
+    if constexpr (U == 6) {
+      step(t + 4, f0, f1, IC<5 % NST>{}, IC<4 % NST>{}, T1{});
+      step(t + 5, f1, f0, IC<6 % NST>{}, IC<5 % NST>{}, T1{});
+    }
   }
-  if (t < KT) step(t, f0, f1, S1{}, S0{});
-  if (t + 1 < KT) step(t + 1, f1, f0, S2{}, S1{});
-  if (t + 2 < KT) step(t + 2, f0, f1, S0{}, S2{});
-  if (t + 3 < KT) step(t + 3, f1, f0, S1{}, S0{});
-  if (t + 4 < KT) step(t + 4, f0, f1, S2{}, S1{});
+  for (; t < KT; t += U) {
+    step(t, f0, f1, IC<1 % NST>{}, IC<0>{}, T0{});
+    if (t + 1 < KT) step(t + 1, f1, f0, IC<2 % NST>{}, IC<1 % NST>{}, T0{});
+    if (t + 2 < KT) step(t + 2, f0, f1, IC<3 % NST>{}, IC<2 % NST>{}, T0{});
+    if (t + 3 < KT) step(t + 3, f1, f0, IC<4 % NST>{}, IC<3 % NST>{}, T0{});
+    if constexpr (U == 6) {
+      if (t + 4 < KT) step(t + 4, f0, f1, IC<5 % NST>{}, IC<4 % NST>{}, T0{});
+      if (t + 5 < KT) step(t + 5, f1, f0, IC<6 % NST>{}, IC<5 % NST>{}, T0{});
+    }
+  }
   __syncthreads();   // the ring is dead: partial strips and the staging tile reuse it
 
   // residual pieces of this thread, requested before the reduction

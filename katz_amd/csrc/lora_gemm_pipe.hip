@@ -689,10 +689,19 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
         dma_setup(d);
         k_loop<C, true, BCH, false>(smem, d, p.x, p.w, p.a_cat, p.t_ext, p.b_cat, KT, KT1, lane, wm, wn, l32, lh, sw, acc, tacc, tail_loads, ConvGeom{0, 0});
       }
-    } else if constexpr (NRT > 0) {
-      // later column tiles of an instantiation that keeps T in LDS: the B_cat tile rides in the old loop's tail
+    } else if constexpr (NRT > 0 || (IL && C::BM == 128)) {
+      // k_loop: later column tiles of an instantiation that keeps T in LDS (the B_cat tile rides in that loop's tail),
+      // and the 128x128 tiles that run beside their layer's shrink workgroups.  The latter by measurement: on operands
+      // that come from HBM, as the weights do in a UNet step, the pointer-form loop is the faster one there (K = 5120:
+      // 52.6 against 55.7 us inside the step) although it loses on cache-resident operands (52.7 against 44.2 us).
       Dma<C, false> d;
       dma_setup(d);
+      if constexpr (IL) {
+        constexpr int TPB = BM / 64;
+        const int gx = (M + 63) / 64, rt = gx - TPB * m_blk < TPB ? gx - TPB * m_blk : TPB;
+        k_loop<C, false, BCH, CONV, decltype(tail_loads), true>(smem, d, p.x, p.w, p.a_cat, p.t_ext, p.b_cat, KT, KT1, lane, wm, wn, l32, lh, sw, acc, tacc, tail_loads, ConvGeom{0, 0}, false, false,
+                                                                p.il_cnt + m_blk, rt * (p.ldt / 64), p.il_cnt + (p.M + 127) / 128, half_last);
+      } else
       k_loop<C, false, BCH, CONV>(smem, d, p.x, p.w, p.a_cat, p.t_ext, p.b_cat, KT, KT1, lane, wm, wn, l32, lh, sw, acc, tacc, tail_loads,
                                   ConvGeom{p.conv_w, p.conv_cin}, false, false, nullptr, 0, nullptr, half_last);
     } else {
@@ -1068,8 +1077,8 @@ static int launch_il(const LoraGemmParams& pin, hipStream_t stream) {
 
 int lora_gemm_pipe_launch_il(const LoraGemmParams& p, hipStream_t stream) {
   switch (il_form(p)) {
-    case 1: return launch_il<PCfg<128, 128, 2, 4, 0, 3, 64>>(p, stream);
-    case 2: return launch_il<PCfg<256, 128, 4, 2, 0, 4>>(p, stream);
+    case 1: return launch_il<PCfg<128, 128, 2, 4, 0, 4, 64>>(p, stream);
+    case 2: return launch_il<PCfg<256, 128, 4, 2, 0, 3, 64>>(p, stream);
     default: return KH_ERR_UNSUPPORTED;
   }
 }
@@ -1082,7 +1091,7 @@ int lora_gemm_pipe_launch_conv(const LoraGemmParams& p, hipStream_t stream) {
     if ((tiles > 256 && tiles <= 384 && m128 * n160 <= 256) || (p.N % 128 != 0 && (m128 * n160) % 256 == 0)) return lora_gemm_ksplit_launch_conv(p, 4, stream);
     if (tiles <= 192 && m64 * n160 <= 256 && m64 * n160 > tiles && p.K >= 2560) return lora_gemm_ksplit_launch_conv(p, 2, stream);
   }
-  if (tiles <= 256 && p.conv_cin % 64 == 0) return launch_pcfg<PCfg<128, 128, 2, 4, 0, 3, 64>, true>(p, stream);
+  if (tiles <= 256 && p.conv_cin % 64 == 0) return launch_pcfg<PCfg<128, 128, 2, 4, 0, 4, 64>, true>(p, stream);
   return launch_pcfg<PCfg<128, 128, 2, 2, 0, 4>, true>(p, stream);
 }
 
@@ -1090,7 +1099,7 @@ int lora_gemm_pipe_launch_sgmv(const LoraGemmParams& p, int n_segments, hipStrea
   // one 128x128 tile column covers all of a shrink's rank columns.  The shrink streams long rows: whole 128-byte
   // lines per stage and 8 waves per workgroup; the expand's K is the rank (a few 32-column tiles).
   // (64-row tiles at two workgroups per CU were measured for the shrink: 15.7 against 12.2 us on 8 x 4096 x 640)
-  if (p.sg_mode == 1 && p.K % 64 == 0) return launch_pcfg<PCfg<128, 128, 2, 4, 0, 3, 64>>(p, stream, n_segments);
+  if (p.sg_mode == 1 && p.K % 64 == 0) return launch_pcfg<PCfg<128, 128, 2, 4, 0, 4, 64>>(p, stream, n_segments);
   return launch_pcfg<PCfg<128, 128, 2, 2, 0, 4>>(p, stream, n_segments);
 }
 
@@ -1105,7 +1114,8 @@ int lora_gemm_pipe_launch(const LoraGemmParams& p, int tile_sel, hipStream_t str
     case 27: return plain_ok(p) ? launch_pcfg<PCfg<256, 128, 4, 2, 0, 4>>(p, stream) : KH_ERR_UNSUPPORTED;
     case 28: return plain_ok(p) ? launch_pcfg<PCfg<128, 256, 2, 4, 0, 4>>(p, stream) : KH_ERR_UNSUPPORTED;
     case 29: return deep_stage_ok(p) ? launch_pcfg<PCfg<256, 128, 4, 2, 0, 3, 64>>(p, stream) : KH_ERR_UNSUPPORTED;
-    case 32: return deep_stage_ok(p) ? launch_pcfg<PCfg<128, 128, 2, 4, 0, 3, 64>>(p, stream) : KH_ERR_UNSUPPORTED;
+    case 32: return deep_stage_ok(p) ? launch_pcfg<PCfg<128, 128, 2, 4, 0, 4, 64>>(p, stream) : KH_ERR_UNSUPPORTED;
+    case 33: return deep_stage_ok(p) ? launch_pcfg<PCfg<128, 128, 2, 4, 0, 3, 64>>(p, stream) : KH_ERR_UNSUPPORTED;
     case 40: return lora_gemm_ksplit_launch(p, 2, stream);
     case 41: return lora_gemm_ksplit_launch(p, 4, stream);
     case 42: return lora_gemm_wide_launch(p, stream);
@@ -1133,8 +1143,8 @@ int lora_gemm_pipe_launch(const LoraGemmParams& p, int tile_sel, hipStream_t str
       if (tiles <= 192 && (long)((p.M + 63) / 64) * n160 <= 256 && (long)((p.M + 63) / 64) * n160 > tiles && p.K >= 2560)
         return lora_gemm_ksplit_launch(p, 2, stream);
     }
-    if (tiles >= 480 && p.K >= 1024 && !p.geglu) return launch_pcfg<PCfg<256, 128, 4, 2, 0, 4>>(p, stream);
-    if (tiles <= 256 && p.M >= 1024 && deep_stage_ok(p)) return launch_pcfg<PCfg<128, 128, 2, 4, 0, 3, 64>>(p, stream);
+    if (tiles >= 480 && p.K >= 1024 && !p.geglu) return deep_stage_ok(p) ? launch_pcfg<PCfg<256, 128, 4, 2, 0, 3, 64>>(p, stream) : launch_pcfg<PCfg<256, 128, 4, 2, 0, 4>>(p, stream);
+    if (tiles <= 256 && p.M >= 1024 && deep_stage_ok(p)) return launch_pcfg<PCfg<128, 128, 2, 4, 0, 4, 64>>(p, stream);
   }
   return launch_prank<128, 128, 2, 2, 4>(p, stream);
 }
