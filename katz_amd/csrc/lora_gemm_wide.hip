@@ -24,6 +24,7 @@ namespace {
 
 typedef const __attribute__((address_space(1))) void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
 
 template <int VM, int LGKM>
 __device__ __forceinline__ void wait_cnt() {  // gfx9 encoding: vmcnt = [15:14|3:0], expcnt = [6:4], lgkmcnt = [11:8]
@@ -63,6 +64,7 @@ struct WFrT { bf16x8 a[C::TM]; bf16x8 b[C::TN]; };
 
 template <class C>
 __global__ __launch_bounds__(512, 2) void lora_gemm_wide_kernel(const LoraGemmParams p) {
+#if __HIP_DEVICE_COMPILE__   // the host pass only needs the kernel's symbol (it cannot lower the buffer-resource type)
   extern __shared__ __attribute__((aligned(16))) char smem[];
   constexpr int WBM = C::BM, WBN = C::BN, WTM = C::TM, WTN = C::TN, WSTAGE = C::STAGE, WLDC = C::LDC;
   constexpr int WXU = C::XU, WWU = C::WU, WLPS = C::LPS, WTAB_OFF = C::TAB_OFF, WBIAS_OFF = C::BIAS_OFF;
@@ -92,43 +94,63 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_wide_kernel(const LoraGemmPa
   // (stage row / 2) % 8 of instruction q is that of instruction 0 plus 4q mod 8: the piece flips bit 2 for odd q,
   // so two element offsets (even / odd q) per operand describe all of a lane's sources; M and N are multiples of
   // the tile (no clamping).
+  // The loads are buffer loads: per lane two byte offsets per operand that never change (row of instruction 0 with the
+  // piece of the even / of the odd instructions), everything that moves (K tile, row group of instruction q) is a scalar
+  // offset; fragment reads add the stage as a constant (the two stages are written out).  The loop carries next to no
+  // vector address arithmetic: with per-lane 64-bit pointers those adds shared the issue stream with the MFMAs.
   const int r8 = lane >> 3;
   const int rx0 = wave * (WBM / 8) + r8, rx1 = rx0 + 8;               // stage rows of x instructions 0 / 1
-  const int pcx0 = ((lane & 7) ^ ((rx0 >> 1) & 7)) * 8, pcx1 = ((lane & 7) ^ ((rx1 >> 1) & 7)) * 8;
+  const int pcx0 = ((lane & 7) ^ ((rx0 >> 1) & 7)) * 16, pcx1 = ((lane & 7) ^ ((rx1 >> 1) & 7)) * 16;
   const int rw0 = WBM + wave * (WBN / 8) + r8, rw1 = rw0 + 8;          // stage rows of W instructions 0 / 1
-  const int pcw0 = ((lane & 7) ^ ((rw0 >> 1) & 7)) * 8, pcw1 = ((lane & 7) ^ ((rw1 >> 1) & 7)) * 8;
+  const int pcw0 = ((lane & 7) ^ ((rw0 >> 1) & 7)) * 16, pcw1 = ((lane & 7) ^ ((rw1 >> 1) & 7)) * 16;
   const int wrow = wave * (WBN / 8) + r8;                              // W row of instruction 0 inside the tile
-  const bf16_t* px = p.x + (size_t)m0 * K;
-  const bf16_t* pw = p.w + (size_t)n0 * K;
-  const bf16_t* px2 = p.t_ext != nullptr ? p.t_ext + (size_t)m0 * p.ldt + (p.t_nsplit > 0 ? (n0 / p.t_nsplit) * p.R : 0) : px;
-  const bf16_t* pw2 = p.t_ext != nullptr ? p.b_cat + (size_t)n0 * p.R : pw;
   const int ldt = p.ldt, R = p.R;
-  // one stage from operands with row strides sx / sw_ (elements); bx / bw already point at the stage's first column
-  auto issue_from = [&](const bf16_t* bx, const bf16_t* bw, int sx, int sw_, char* stage) {
-    const bf16_t* gx0 = bx + rx0 * sx + pcx0;                   // row of instruction 0, piece of the even ones
-    const bf16_t* gx1 = bx + rx0 * sx + pcx1;                   // same row, piece of the odd ones
-    const bf16_t* gw0 = bw + wrow * sw_ + pcw0;
-    const bf16_t* gw1 = bw + wrow * sw_ + pcw1;
+  const uint32_t vx0 = (uint32_t)rx0 * (uint32_t)K * 2u + pcx0, vx1 = (uint32_t)rx0 * (uint32_t)K * 2u + pcx1;
+  const uint32_t vw0 = (uint32_t)wrow * (uint32_t)K * 2u + pcw0, vw1 = (uint32_t)wrow * (uint32_t)K * 2u + pcw1;
+  auto clamp32 = [](size_t bytes) { return (int)(uint32_t)(bytes < 0xFFFFFFFFull ? bytes : 0xFFFFFFFFull); };
+  auto mk = [&](const bf16_t* base, size_t bytes) { return __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(base), 0, clamp32(bytes), 0x00020000); };
+  const bool ext = p.t_ext != nullptr;
+  const size_t tcol = ext && p.t_nsplit > 0 ? (size_t)(n0 / p.t_nsplit) * p.R : 0;
+  const rsrc_t rs_x = mk(p.x + (size_t)m0 * K, (size_t)(p.M - m0) * K * 2);
+  const rsrc_t rs_w = mk(p.w + (size_t)n0 * K, (size_t)(N - n0) * K * 2);
+  const rsrc_t rs_t = mk(ext ? p.t_ext + (size_t)m0 * ldt + tcol : p.x, ext ? ((size_t)(p.M - m0) * ldt - tcol) * 2 : 0);
+  const rsrc_t rs_b = mk(ext ? p.b_cat + (size_t)n0 * R : p.w, ext ? (size_t)(N - n0) * R * 2 : 0);
+  auto issue = [&](int t, auto stc) {                           // K tile t into stage stc
+    char* stage = smem + decltype(stc)::value * WSTAGE;
+    if (t < KT1) {
+      const int so = t * 128, rstep = 8 * K * 2;                // bytes: K tile, 8 rows further
 #pragma unroll
-    for (int q = 0; q < WXU; ++q)
-      __builtin_amdgcn_global_load_lds((gptr_t)(((q & 1) ? gx1 : gx0) + q * 8 * sx), (lptr_t)(stage + (wave * (WBM / 8) + q * 8) * 128), 16, 0, 0);
+      for (int q = 0; q < WXU; ++q)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_x, (lptr_t)(stage + (wave * (WBM / 8) + q * 8) * 128), 16, (q & 1) ? vx1 : vx0, so + q * rstep, 0, 0);
 #pragma unroll
-    for (int q = 0; q < WWU; ++q)
-      __builtin_amdgcn_global_load_lds((gptr_t)(((q & 1) ? gw1 : gw0) + q * 8 * sw_), (lptr_t)(stage + (WBM + wave * (WBN / 8) + q * 8) * 128), 16, 0, 0);
-  };
-  auto issue = [&](int t, int st) {                             // K tile t into stage st
-    char* stage = smem + st * WSTAGE;
-    if (t < KT1) issue_from(px + t * 64, pw + t * 64, K, K, stage);
-    else issue_from(px2 + (t - KT1) * 64, pw2 + (t - KT1) * 64, ldt, R, stage);
+      for (int q = 0; q < WWU; ++q)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_w, (lptr_t)(stage + (WBM + wave * (WBN / 8) + q * 8) * 128), 16, (q & 1) ? vw1 : vw0, so + q * rstep, 0, 0);
+    } else {
+      // the rank columns: y = [x | T] . [W | B_cat]^T (one or two stages per tile: their offsets are formed here)
+      const int so = (t - KT1) * 128;
+      const uint32_t tx0 = (uint32_t)rx0 * (uint32_t)ldt * 2u + pcx0, tx1 = (uint32_t)rx0 * (uint32_t)ldt * 2u + pcx1;
+      const uint32_t tw0 = (uint32_t)wrow * (uint32_t)R * 2u + pcw0, tw1 = (uint32_t)wrow * (uint32_t)R * 2u + pcw1;
+#pragma unroll
+      for (int q = 0; q < WXU; ++q)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_t, (lptr_t)(stage + (wave * (WBM / 8) + q * 8) * 128), 16, (q & 1) ? tx1 : tx0, so + q * 8 * ldt * 2, 0, 0);
+#pragma unroll
+      for (int q = 0; q < WWU; ++q)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, (lptr_t)(stage + (WBM + wave * (WBN / 8) + q * 8) * 128), 16, (q & 1) ? tw1 : tw0, so + q * 8 * R * 2, 0, 0);
+    }
   };
   const int sw = (l32 >> 1) & 7;
-  auto read_frags = [&](int st, int ks, WFr& f) {               // MFMA step ks (16 columns) of the stage
-    const char* s = smem + st * WSTAGE;
-    const int po = ((2 * ks + lh) ^ sw) * 16;
+  const int abase = (wm * WR + l32) * 128, bbase = (WBM + wn * WC + l32) * 128;
+  int po4[4];
 #pragma unroll
-    for (int i = 0; i < WTM; ++i) f.a[i] = *reinterpret_cast<const bf16x8*>(s + (wm * WR + i * 32 + l32) * 128 + po);
+  for (int ks = 0; ks < 4; ++ks) po4[ks] = ((2 * ks + lh) ^ sw) * 16;
+  auto read_frags = [&](auto stc, int ks, WFr& f) {             // MFMA step ks (16 columns) of stage stc
+    const char* s = smem + decltype(stc)::value * WSTAGE;
+    const char* pa = s + (abase + po4[ks]);
+    const char* pb = s + (bbase + po4[ks]);
 #pragma unroll
-    for (int j = 0; j < WTN; ++j) f.b[j] = *reinterpret_cast<const bf16x8*>(s + (WBM + wn * WC + j * 32 + l32) * 128 + po);
+    for (int i = 0; i < WTM; ++i) f.a[i] = *reinterpret_cast<const bf16x8*>(pa + i * 32 * 128);
+#pragma unroll
+    for (int j = 0; j < WTN; ++j) f.b[j] = *reinterpret_cast<const bf16x8*>(pb + j * 32 * 128);
   };
   f32x16 acc[WTM][WTN];
 #pragma unroll
@@ -154,8 +176,9 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_wide_kernel(const LoraGemmPa
   }
   // K loop over stages t (stage t & 1).  Steps 0..3 of a stage alternate between the fragment buffers fa / fb.
   WFr fa, fb;
-  issue(0, 0);
-  if (KT > 1) issue(1, 1);
+  using S0 = std::integral_constant<int, 0>; using S1 = std::integral_constant<int, 1>;
+  issue(0, S0{});
+  if (KT > 1) issue(1, S1{});
   uint16_t* gtab = reinterpret_cast<uint16_t*>(smem + WTAB_OFF);
   uint16_t* sbias = reinterpret_cast<uint16_t*>(smem + WBIAS_OFF);   // like the table: written now, read in the epilogue
   if (tid < WBN) sbias[tid] = p.bias != nullptr ? reinterpret_cast<const uint16_t*>(p.bias)[n0 + tid] : (uint16_t)0;
@@ -177,30 +200,43 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_wide_kernel(const LoraGemmPa
   }
   if (KT > 1) wait_cnt<WLPS, 15>(); else wait_cnt<0, 15>();
   __builtin_amdgcn_s_barrier();
-  read_frags(0, 0, fa);
-  read_frags(0, 1, fb);
-  for (int t = 0; t + 1 < KT; ++t) {   // every stage but the last
-    const int st = t & 1;
+  read_frags(S0{}, 0, fa);
+  read_frags(S0{}, 1, fb);
+  auto stage_body = [&](int t, auto stc, auto nxc) {   // every stage but the last: stage stc, the next one nxc
     mma(fa);                         // step 0
-    read_frags(st, 2, fa);
+    read_frags(stc, 2, fa);
     mma(fb);                         // step 1
-    read_frags(st, 3, fb);
+    read_frags(stc, 3, fb);
     mma(fa);                         // step 2
     // stage t+1 has landed (this wave's share; the barrier collects everyone's); every read of stage t is done
     wait_cnt<0, 0>();
     __builtin_amdgcn_s_barrier();
-    if (t + 2 < KT) issue(t + 2, st);
-    read_frags(st ^ 1, 0, fa);
+    if (t + 2 < KT) issue(t + 2, stc);
+    read_frags(nxc, 0, fa);
     mma(fb);                         // step 3
-    read_frags(st ^ 1, 1, fb);
+    read_frags(nxc, 1, fb);
+  };
+  auto read_frags_rt = [&](int st, int ks, WFr& f) {    // the same with the stage as a value
+    const char* pa = smem + (st * WSTAGE + abase + po4[ks]);
+    const char* pb = smem + (st * WSTAGE + bbase + po4[ks]);
+#pragma unroll
+    for (int i = 0; i < WTM; ++i) f.a[i] = *reinterpret_cast<const bf16x8*>(pa + i * 32 * 128);
+#pragma unroll
+    for (int j = 0; j < WTN; ++j) f.b[j] = *reinterpret_cast<const bf16x8*>(pb + j * 32 * 128);
+  };
+  int t = 0;
+  for (; t + 2 < KT; t += 2) {
+    stage_body(t, S0{}, S1{});
+    stage_body(t + 1, S1{}, S0{});
   }
+  if (t + 1 < KT) stage_body(t, S0{}, S1{});
   {                                  // the last stage: all four steps, or two when its upper half is zero padding
     const int st = (KT - 1) & 1;
     mma(fa);
-    if (!half_last) read_frags(st, 2, fa);
+    if (!half_last) read_frags_rt(st, 2, fa);
     mma(fb);
     if (!half_last) {
-      read_frags(st, 3, fb);
+      read_frags_rt(st, 3, fb);
       mma(fa);
       mma(fb);
     }
@@ -293,6 +329,7 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_wide_kernel(const LoraGemmPa
     }
     __syncthreads();
   }
+#endif
 }
 
 template <class C>
