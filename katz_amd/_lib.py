@@ -36,6 +36,7 @@ SIGNATURES = {
     "kh_lora_linear_norm_bf16": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, c_float, _P,
                                          _I, _I, _I, _I, _I, c_int, _P]),
     "kh_lora_split_timeouts": (c_int, [_P, c_int]),
+    "kh_set_weight_prefetch": (c_int, [_P, _I]),
     "kh_lora_linear_split_launches": (c_int, [_I, _I, _I, _I, _I, c_int]),
     "kh_layer_norm_bf16": (c_int, [_P, _P, _P, _P, _I, _I, c_float, _P]),
     "kh_geglu_bf16": (c_int, [_P, _P, _I, _I, c_int, _P]),

@@ -57,10 +57,38 @@ struct LoraGemmParams {
   // Row statistics of the output for a following folded LayerNorm (st_part != nullptr): column tile j writes the
   // (sum, sum of squares) of its columns of every row to st_part[j][row]; tile 0 also zeroes the slots past the last tile.
   float* st_part = nullptr;         // [16][M][2]
+  // Weight prefetch (pf != nullptr): the launch also touches every 128-byte line of pf[0 .. 128 * pf_lines), the weights
+  // of the NEXT launch of this family, so that they wait in the memory-side cache when that launch asks for them (a
+  // step reads 2.5 GB of weights once each: every launch would otherwise meet its weights in HBM, where the XCDs that
+  // share a weight block each fetch it again).  Set from kh_set_weight_prefetch by the entry points.
+  const void* pf = nullptr;
+  uint32_t pf_lines = 0;
 };
+
+// The pending weight prefetch of this host thread (kh_set_weight_prefetch), handed to the next launch.
+void kh_take_weight_prefetch(LoraGemmParams& p);
 
 constexpr int KH_LN_LDS = 4096;    // bytes of dynamic LDS a launch with a folded LayerNorm adds: mean, 1/std of up to 256 rows, c1, c2 of up to 256 columns
 constexpr int KH_LN_SLOTS = 16;     // partial pairs per row: at most 16 column tiles (N <= 2048 with 128-column tiles)
+
+// Touch lines first, first + n_wg * NT, ... of the prefetch range: one dword per line and lane, loaded into 256 bytes of
+// LDS that belong to this wave alone and that its own later DMA overwrites (a wave's loads land in order), so no
+// register and no wait is spent on data nobody reads.  wg / n_wg: this workgroup's index among those that take part.
+__device__ __forceinline__ void kh_prefetch_lines(const void* pf, uint32_t lines, char* wave_lds, int wg, int n_wg, int tid, int nt) {
+#if __HIP_DEVICE_COMPILE__
+  if (pf == nullptr) return;
+  const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(pf), 0, (int)(lines << 7), 0x00020000);
+  const uint32_t stride = (uint32_t)n_wg * (uint32_t)nt;
+  // four rounds (64 MB with 256 workgroups of 512 threads), no loop; the per-lane offset carries the round, because only
+  // it is checked against the range: an offset beyond the range reads nothing
+  const uint32_t first = ((uint32_t)wg * (uint32_t)nt + (uint32_t)tid) << 7, step = stride << 7;
+#pragma unroll
+  for (uint32_t r = 0; r < 4; ++r) {
+    const uint32_t off = first + r * step;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)wave_lds, 4, off >= first ? off : 0xFFFFFFFFu, 0, 0, 0);
+  }
+#endif
+}
 
 // a column tile's pair for one output row, and (from tile 0) zeros in the slots no tile writes
 __device__ __forceinline__ void kh_ln_store_stats(float* part, int row, int M, int tile, int n_tiles, float s, float q) {

@@ -455,6 +455,23 @@ __global__ __launch_bounds__(256) void lora_gemm_f32_kernel(const float* __restr
 
 }  // namespace
 
+// See include/katz_hip.h: the weights of the launch after the next one of this family, per host thread.
+static thread_local const void* g_pf_ptr = nullptr;
+static thread_local uint32_t g_pf_lines = 0;
+
+KH_EXPORT int kh_set_weight_prefetch(const void* weights, int64_t bytes) {
+  if (bytes < 0 || (weights == nullptr && bytes != 0)) return KH_ERR_INVALID_ARG;
+  const int64_t lines = bytes >> 7;
+  g_pf_ptr = lines > 0 ? weights : nullptr;
+  g_pf_lines = (uint32_t)(lines < (1 << 24) ? lines : (1 << 24));   // at most 2 GiB
+  return KH_OK;
+}
+
+void kh_take_weight_prefetch(LoraGemmParams& p) {
+  p.pf = g_pf_ptr; p.pf_lines = g_pf_lines;
+  g_pf_ptr = nullptr; g_pf_lines = 0;
+}
+
 // See include/katz_hip.h for the contract.
 KH_EXPORT int kh_lora_linear_bf16(const void* x, const void* w, const void* bias, const void* a_cat,
                                   const void* b_cat, const float* col_scale, const void* residual, void* y,
@@ -488,6 +505,7 @@ KH_EXPORT int kh_lora_linear_bf16(const void* x, const void* w, const void* bias
   hipStream_t s = (hipStream_t)stream;
   const int tile_sel = (flags >> 8) & 0xff;  // 0 = automatic
   // K % 32 == 0 (every SDXL layer): the software-pipelined kernel; tile_sel 1/2 force the simple kernel
+  kh_take_weight_prefetch(p);
   if (K % 32 == 0 && (tile_sel == 0 || tile_sel >= 16)) return lora_gemm_pipe_launch(p, tile_sel, s);
   if (tile_sel == 2) return R > 96 ? KH_ERR_UNSUPPORTED : launch_rank<256, 128, 2, 2>(p, s);
   if (tile_sel == 1) return launch_rank<128, 128, 2, 2>(p, s);
@@ -522,6 +540,7 @@ KH_EXPORT int kh_lora_linear_pre_bf16(const void* x, const void* w, const void* 
   p.conv_cin = p.conv_h = p.conv_w = p.conv_ho = p.conv_wo = p.conv_stride = 0;
   p.r_used = ((flags >> 16) & 0xff) * 16;
   if (p.r_used > p.R) return KH_ERR_INVALID_ARG;
+  kh_take_weight_prefetch(p);
   return lora_gemm_pipe_launch(p, (flags >> 8) & 0xff, (hipStream_t)stream);
 }
 
@@ -578,6 +597,7 @@ KH_EXPORT int kh_lora_linear_split_bf16(const void* x, const void* w, const void
   if (counters != nullptr && kh_lora_linear_split_launches(M, N, K, R, n_split, flags) == 1) {
     LoraGemmParams p = split_params(x, w, bias, a_cat, col_scale, b_cat, t_scratch, counters, residual, y, M, N, K, R, n_split, geglu);
     p.r_used = ((flags >> 16) & 0xff) * 16;
+    kh_take_weight_prefetch(p);
     return lora_gemm_pipe_launch_il(p, (hipStream_t)stream);
   }
   const int rc = kh_lora_shrink_bf16(x, a_cat, col_scale, t_scratch, M, K, RT, stream);
@@ -614,6 +634,7 @@ KH_EXPORT int kh_lora_linear_norm_bf16(const void* x, const void* w, const void*
   p.r_used = ((flags >> 16) & 0xff) * 16;
   p.ln_part = ln_part; p.ln_c1 = ln_c1; p.ln_c2 = ln_c2; p.ln_ca1 = ln_ca1; p.ln_ca2 = ln_ca2; p.ln_eps = ln_eps;
   p.st_part = stats_out;
+  kh_take_weight_prefetch(p);
   const int tile_sel = (flags >> 8) & 0xff;
   if (R == 0) {
     p.ldt = 0; p.t_nsplit = 0; p.il_cnt = nullptr;
@@ -650,6 +671,7 @@ KH_EXPORT int kh_conv3x3_nhwc_bf16(const void* x, const void* w, const void* bia
   p.sg_start = p.sg_adapter = p.sg_rank = nullptr; p.sg_scale = nullptr; p.sg_mode = 0; p.sg_wstride = 0;
   p.conv_cin = (int)Cin; p.conv_h = (int)H; p.conv_w = (int)W; p.conv_ho = (int)Ho; p.conv_wo = (int)Wo;
   p.conv_stride = (int)stride;
+  kh_take_weight_prefetch(p);
   return lora_gemm_pipe_launch_conv(p, (hipStream_t)stream);
 }
 

@@ -69,6 +69,7 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_ksplit_kernel(const LoraGemm
   const int wm = wave / C::WK, wk = wave % C::WK;
   const int l32 = lane & 31, lh = lane >> 5;
 
+  kh_prefetch_lines(p.pf, p.pf_lines, smem + wave * 1024, blockIdx.x, gridDim.x, tid, 512);   // the next launch's weights
   // tile of this workgroup: XCD b % 8 owns a block of xr_m x xr_n tiles (its W rows stay in its L2)
   const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
   const int m_blk = (xcd / p.xg_n) * p.xr_m + local / p.xr_n;

@@ -487,6 +487,11 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
     }
   }
   const int bid = IL ? (int)blockIdx.x - pin.il_blocks : (int)blockIdx.x;
+  // the next launch's weights, towards the memory-side cache (see LoraGemmParams::pf); not from the 256x128 tiles that run
+  // beside their shrink: with a folded LayerNorm they have no register to spare, and a kernel with scratch loses more
+  if (!(IL && C::BM == 256) && blockIdx.y == 0)
+    kh_prefetch_lines(pin.pf, pin.pf_lines, smem + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) * (C::UX / C::NW) * 1024, bid,
+                      (int)gridDim.x - (IL ? pin.il_blocks : 0), threadIdx.x, C::NT);
   if (pin.grp != nullptr) {  // grouped launch: this workgroup's layer
     const uint64_t* g = pin.grp + (size_t)blockIdx.y * 5;
     p.w = reinterpret_cast<const bf16_t*>(g[0]);

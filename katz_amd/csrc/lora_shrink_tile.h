@@ -42,7 +42,6 @@ struct SCfg {
 // readers on other XCDs inside the same launch).
 template <class C, bool WT, int NTB>   // NTB: threads of the block
 __device__ __forceinline__ void lora_shrink_tile(const ShrinkParams& p, int bx, int by, char* smem) {
-#if __HIP_DEVICE_COMPILE__   // (the host pass cannot lower the buffer-resource type)
   constexpr int NW = C::NW, TR = C::TR, TC = C::TC, NS = C::NS, UNITS = C::UNITS, STAGE = C::STAGE, LD = C::LD;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -54,33 +53,25 @@ __device__ __forceinline__ void lora_shrink_tile(const ShrinkParams& p, int bx, 
   char* ring = smem + (active ? wave : 0) * (NS * STAGE);
 
   // DMA: lane i of a unit lands in LDS slot i = row i/8, physical piece i%8, which holds logical piece
-  // (i%8) ^ ((row/2)%8); the swizzle is applied to the address the lane fetches.  Buffer loads: a byte offset per lane
-  // and unit that never changes (relative to the tile's first x / A_cat row) plus a scalar offset per chunk, so the
-  // loop carries no vector address arithmetic.
-  uint32_t voff[UNITS];
+  // (i%8) ^ ((row/2)%8); the swizzle is applied to the address the lane fetches
+  const bf16_t* src[UNITS];
 #pragma unroll
   for (int u = 0; u < UNITS; ++u) {
     const int ru = u * 8 + (lane >> 3);                // row inside the stacked [x rows | A_cat rows] stage
-    const uint32_t pcb = (uint32_t)(((lane & 7) ^ ((ru >> 1) & 7)) * 16);
+    const int pc = ((lane & 7) ^ ((ru >> 1) & 7)) * 8;
     if (u < TR * 4) {
       int row = m0 + ru; row = row < p.M ? row : p.M - 1;
-      voff[u] = (uint32_t)(row - m0) * (uint32_t)K * 2u + pcb;
+      src[u] = p.x + (size_t)row * K + wave * 64 + pc;
     } else {
       int row = r0 + ru - TR * 32; row = row < p.R ? row : p.R - 1;
-      voff[u] = (uint32_t)(row - r0) * (uint32_t)K * 2u + pcb;
+      src[u] = p.a_cat + (size_t)row * K + wave * 64 + pc;
     }
   }
-  auto clamp32 = [](size_t bytes) { return (int)(uint32_t)(bytes < 0xFFFFFFFFull ? bytes : 0xFFFFFFFFull); };
-  const __amdgpu_buffer_rsrc_t rs_x = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(p.x + (size_t)m0 * K), 0,
-                                                                        clamp32((size_t)(p.M - m0) * K * 2), 0x00020000);
-  const __amdgpu_buffer_rsrc_t rs_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(p.a_cat + (size_t)r0 * K), 0,
-                                                                        clamp32((size_t)(p.R - r0) * K * 2), 0x00020000);
-  auto issue = [&](int i, auto stc) {                  // this wave's i-th chunk into its ring stage stc
-    char* st = ring + decltype(stc)::value * STAGE;
-    const int so = (wave + i * NW) * 128;              // bytes: chunk wave + i * NW of 64 columns
+  auto issue = [&](int i) {                            // this wave's i-th chunk
+    char* st = ring + (i % NS) * STAGE;
 #pragma unroll
     for (int u = 0; u < UNITS; ++u)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(u < TR * 4 ? rs_x : rs_a, (lptr_t)(st + u * 1024), 16, voff[u], so, 0, 0);
+      __builtin_amdgcn_global_load_lds((gptr_t)(src[u] + (size_t)i * (NW * 64)), (lptr_t)(st + u * 1024), 16, 0, 0);
   };
   f32x16 acc[TR][TC];
 #pragma unroll
@@ -95,28 +86,23 @@ __device__ __forceinline__ void lora_shrink_tile(const ShrinkParams& p, int bx, 
   // arrived when the first chunk has) and reduced after the loop
   KhLnTileStats<TR * 32, NTB> ln_stats;
   if (p.ln_part != nullptr) ln_stats.load(p.ln_part, m0, p.M, tid);
-  using S0 = std::integral_constant<int, 0>; using S1 = std::integral_constant<int, 1>;
-  static_assert(NS == 2, "the two ring stages are written out");
-  if (n > 0) issue(0, S0{});
-  if (n > 1) issue(1, S1{});
+  if (n > 0) issue(0);
+  if (n > 1) issue(1);
 
-  // fragment offsets inside a stage: constant per lane; the stage is a constant of each written-out step
-  int fo[4];
-#pragma unroll
-  for (int ks = 0; ks < 4; ++ks) fo[ks] = (active ? wave : 0) * (NS * STAGE) + l32 * 128 + ((2 * ks + lh) ^ sw) * 16;
-  auto chunk = [&](int i, auto stc) {
+  for (int i = 0; i < n; ++i) {
     if (i + 1 < n) wait_vm<UNITS>(); else wait_vm<0>();   // chunk i has landed; chunk i+1 may be in flight
-    const char* st = smem + decltype(stc)::value * STAGE;   // (the wave's ring is part of fo)
+    const char* st = ring + (i % NS) * STAGE;
     bf16x8 a[4][TR], b[4][TC];
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
+      const int po = ((2 * ks + lh) ^ sw) * 16;
 #pragma unroll
-      for (int r = 0; r < TR; ++r) a[ks][r] = *reinterpret_cast<const bf16x8*>(st + fo[ks] + r * 32 * 128);
+      for (int r = 0; r < TR; ++r) a[ks][r] = *reinterpret_cast<const bf16x8*>(st + (r * 32 + l32) * 128 + po);
 #pragma unroll
-      for (int c = 0; c < TC; ++c) b[ks][c] = *reinterpret_cast<const bf16x8*>(st + fo[ks] + (TR + c) * 32 * 128);
+      for (int c = 0; c < TC; ++c) b[ks][c] = *reinterpret_cast<const bf16x8*>(st + ((TR + c) * 32 + l32) * 128 + po);
     }
     wait_lgkm0();                   // fragments are in registers: the stage may be refilled
-    if (i + NS < n) issue(i + NS, stc);
+    if (i + NS < n) issue(i + NS);
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
@@ -124,13 +110,7 @@ __device__ __forceinline__ void lora_shrink_tile(const ShrinkParams& p, int bx, 
 #pragma unroll
         for (int c = 0; c < TC; ++c)
           acc[r][c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[ks][r], b[ks][c], acc[r][c], 0, 0, 0);
-  };
-  int i = 0;
-  for (; i + 2 <= n; i += 2) {
-    chunk(i, S0{});
-    chunk(i + 1, S1{});
   }
-  if (i < n) chunk(i, S0{});
   __syncthreads();                  // every ring is dead: the partial sums reuse the memory
   float* part = reinterpret_cast<float*>(smem);   // [NW][TR*32][LD]
   float* sMu = reinterpret_cast<float*>(smem + C::PART);   // behind the partial sums
@@ -168,7 +148,6 @@ __device__ __forceinline__ void lora_shrink_tile(const ShrinkParams& p, int bx, 
       else *dst = v;
     }
   }
-#endif
 }
 
 }  // namespace

@@ -9,6 +9,7 @@ from __future__ import annotations
 
 import ctypes
 import math
+import os
 from typing import Optional, Sequence
 
 import torch
@@ -39,6 +40,27 @@ def _req(t: torch.Tensor, dtype, name: str) -> None:
 
 
 # --------------------------------------------------------------------------------------- K1
+# Weight prefetch: a linear / convolution launch can touch the weights of the launch that follows it, so that those wait in
+# the memory-side cache (kh_set_weight_prefetch).  Which weights follow which is learned from the previous pass over
+# the model: a launch with weights W hints at what followed W last time.  The table keeps the tensors alive.
+WEIGHT_PREFETCH = os.getenv("KATZ_WEIGHT_PREFETCH", "1") != "0"
+_pf_next: dict = {}     # data_ptr of a launch's weights -> the weights tensor of the launch that followed it
+_pf_last: list = [None]
+
+
+def _weight_prefetch_hint(weight: torch.Tensor) -> None:
+    if not WEIGHT_PREFETCH:
+        return
+    key = weight.data_ptr()
+    last = _pf_last[0]
+    if last is not None and last != key:
+        _pf_next[last] = weight
+    _pf_last[0] = key
+    nxt = _pf_next.get(key)
+    if nxt is not None:
+        _lib.load().kh_set_weight_prefetch(nxt.data_ptr(), nxt.numel() * nxt.element_size())
+
+
 def lora_linear(
     x: torch.Tensor,
     weight: torch.Tensor,
@@ -89,6 +111,7 @@ def lora_linear(
         CALL_LOG.append(("lora_linear", M, N, K, R, bool(geglu), residual is not None))
     if dt == BF16:
         flags = (1 if geglu else 0) | ((tile & 0xFF) << 8)
+        _weight_prefetch_hint(weight)
         rc = lib.kh_lora_linear_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(a_cat), _ptr(b_cat), _ptr(col_scale),
                                      _ptr(residual), _ptr(out), M, N, K, R, flags, _stream())
     elif dt == torch.float32:
@@ -155,6 +178,7 @@ def lora_linear_pre(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.
     if CALL_LOG is not None:
         CALL_LOG.append(("lora_linear", M, N, K, R, bool(geglu), residual is not None))
     flags = (1 if geglu else 0) | ((tile & 0xFF) << 8) | (_r_used_bits(r_used, R) << 16)
+    _weight_prefetch_hint(weight)
     rc = lib.kh_lora_linear_pre_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(t), t.stride(0), n_split, _ptr(b_cat),
                                      _ptr(residual), _ptr(out), M, N, K, R, flags, _stream())
     _lib.check(rc, "kh_lora_linear_pre_bf16")
@@ -274,6 +298,7 @@ def lora_linear_split(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torc
         if lib.kh_lora_linear_split_launches(M, N, K, R, n_split, flags) == 2:
             CALL_LOG.append(("lora_shrink", M, K, RT))
         CALL_LOG.append(("lora_linear", M, N, K, R, bool(geglu), residual is not None))
+    _weight_prefetch_hint(weight)
     rc = lib.kh_lora_linear_split_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(a_cat), _ptr(col_scale), _ptr(b_cat), _ptr(t),
                                        _ptr(cnt), _ptr(residual), _ptr(out), M, N, K, R, n_split, flags, _stream())
     _lib.check(rc, "kh_lora_linear_split_bf16")
@@ -351,6 +376,7 @@ def lora_linear_norm(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch
         if R and lib.kh_lora_linear_split_launches(M, N, K, R, n_split, flags) == 2:
             CALL_LOG.append(("lora_shrink", M, K, RT))
         CALL_LOG.append(("lora_linear", M, N, K, R, bool(geglu), residual is not None))
+    _weight_prefetch_hint(weight)
     rc = lib.kh_lora_linear_norm_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(a_cat), _ptr(col_scale), _ptr(b_cat), _ptr(t),
                                       _ptr(cnt), _ptr(residual), _ptr(out), _ptr(part), _ptr(c1), _ptr(c2), _ptr(ca1), _ptr(ca2),
                                       float(eps), _ptr(stats_out), M, N, K, R, n_split, flags, _stream())
@@ -665,6 +691,7 @@ def conv3x3(x: torch.Tensor, w_packed: torch.Tensor, bias: Optional[torch.Tensor
         raise ValueError("residual must be a channels_last bfloat16 tensor of the output's shape")
     if CALL_LOG is not None:
         CALL_LOG.append(("conv3x3", Nb * Ho * Wo, Cout, 9 * Cin, stride))
+    _weight_prefetch_hint(w_packed)
     rc = lib.kh_conv3x3_nhwc_bf16(_ptr(x), _ptr(w_packed), _ptr(bias), _ptr(residual), _ptr(out), Nb, H, W, Cin, Cout,
                                   stride, _stream())
     _lib.check(rc, "kh_conv3x3_nhwc_bf16")
