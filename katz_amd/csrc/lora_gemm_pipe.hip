@@ -694,19 +694,10 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
         dma_setup(d);
         k_loop<C, true, BCH, false>(smem, d, p.x, p.w, p.a_cat, p.t_ext, p.b_cat, KT, KT1, lane, wm, wn, l32, lh, sw, acc, tacc, tail_loads, ConvGeom{0, 0});
       }
-    } else if constexpr (NRT > 0 || (IL && C::BM == 128)) {
-      // k_loop: later column tiles of an instantiation that keeps T in LDS (the B_cat tile rides in that loop's tail),
-      // and the 128x128 tiles that run beside their layer's shrink workgroups.  The latter by measurement: on operands
-      // that come from HBM, as the weights do in a UNet step, the pointer-form loop is the faster one there (K = 5120:
-      // 52.6 against 55.7 us inside the step) although it loses on cache-resident operands (52.7 against 44.2 us).
+    } else if constexpr (NRT > 0) {
+      // later column tiles of an instantiation that keeps T in LDS: the B_cat tile rides in that loop's tail
       Dma<C, false> d;
       dma_setup(d);
-      if constexpr (IL) {
-        constexpr int TPB = BM / 64;
-        const int gx = (M + 63) / 64, rt = gx - TPB * m_blk < TPB ? gx - TPB * m_blk : TPB;
-        k_loop<C, false, BCH, CONV, decltype(tail_loads), true>(smem, d, p.x, p.w, p.a_cat, p.t_ext, p.b_cat, KT, KT1, lane, wm, wn, l32, lh, sw, acc, tacc, tail_loads, ConvGeom{0, 0}, false, false,
-                                                                p.il_cnt + m_blk, rt * (p.ldt / 64), p.il_cnt + (p.M + 127) / 128, half_last);
-      } else
       k_loop<C, false, BCH, CONV>(smem, d, p.x, p.w, p.a_cat, p.t_ext, p.b_cat, KT, KT1, lane, wm, wn, l32, lh, sw, acc, tacc, tail_loads,
                                   ConvGeom{p.conv_w, p.conv_cin}, false, false, nullptr, 0, nullptr, half_last);
     } else {
