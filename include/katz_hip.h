@@ -137,13 +137,15 @@ int kh_lora_linear_norm_bf16(const void* x, const void* w, const void* bias, con
 int kh_lora_split_timeouts(int32_t* count, int clear);
 /* Weight prefetch hint; no counterpart in the reference (its cuBLAS / cuDNN calls take no such hint).  The next launch of
  * the linear / convolution family made by this host thread (kh_lora_linear_bf16, _pre, _split, _norm, kh_conv3x3_nhwc_bf16)
- * also touches every 128-byte line of weights[0 .. bytes): the weights of the launch that FOLLOWS it, so that they are
- * in the memory-side cache when that launch asks for them.  A UNet step reads its 2.5 GB of weights once each, so every
- * launch would otherwise meet its weights in HBM, and each XCD that shares a weight block would fetch it again; measured
- * on the SDXL feed-forward output projection (M 2048, N 1280, K 5120): 53 us with the weights in HBM, 45 us prefetched,
- * 42 us cache-resident.  The hint is consumed by that one launch (also under graph capture, where the pointer is
- * recorded: the range must stay allocated while the graph is replayed).  weights == NULL or bytes < 128 clears a pending
- * hint.  At most 2 GiB are touched.  Wrong hints cost bandwidth, never correctness; the range must be readable. */
+ * also touches every 128-byte line of weights[0 .. bytes): an operand of the launch that FOLLOWS it, so that it is in
+ * the memory-side cache when that launch asks for it.  Up to three ranges may be queued by consecutive calls (weights,
+ * A_cat, B_cat; of the second and third at most the first 16 MB are touched); a fourth returns KH_ERR_TOO_LARGE.
+ * A UNet step reads its 2.5 GB of weights once each, so every launch would otherwise meet its weights in HBM, and each
+ * XCD that shares a weight block would fetch it again; measured on the SDXL feed-forward output projection (M 2048,
+ * N 1280, K 5120): 53 us with the weights in HBM, 45 us prefetched, 42 us cache-resident.  The hints are consumed by
+ * that one launch (also under graph capture, where the pointers are recorded: the ranges must stay allocated while the
+ * graph is replayed).  weights == NULL or bytes < 128 clears what is pending.  At most 2 GiB per range.  Wrong hints
+ * cost bandwidth, never correctness; the ranges must be readable. */
 int kh_set_weight_prefetch(const void* weights, int64_t bytes);
 /* How many kernel launches kh_lora_linear_split_bf16 makes for this shape when counters are given (1 or 2; negative:
  * KH_ERR_*).  No counterpart in the reference; for callers that account per launch (benchmarks). */

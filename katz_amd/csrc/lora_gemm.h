@@ -61,8 +61,8 @@ struct LoraGemmParams {
   // of the NEXT launch of this family, so that they wait in the memory-side cache when that launch asks for them (a
   // step reads 2.5 GB of weights once each: every launch would otherwise meet its weights in HBM, where the XCDs that
   // share a weight block each fetch it again).  Set from kh_set_weight_prefetch by the entry points.
-  const void* pf = nullptr;
-  uint32_t pf_lines = 0;
+  const void* pf[3] = {nullptr, nullptr, nullptr};   // up to three ranges: weights, A_cat, B_cat of that launch
+  uint32_t pf_lines[3] = {0, 0, 0};
 };
 
 // The pending weight prefetch of this host thread (kh_set_weight_prefetch), handed to the next launch.
@@ -74,18 +74,23 @@ constexpr int KH_LN_SLOTS = 16;     // partial pairs per row: at most 16 column 
 // Touch lines first, first + n_wg * NT, ... of the prefetch range: one dword per line and lane, loaded into 256 bytes of
 // LDS that belong to this wave alone and that its own later DMA overwrites (a wave's loads land in order), so no
 // register and no wait is spent on data nobody reads.  wg / n_wg: this workgroup's index among those that take part.
-__device__ __forceinline__ void kh_prefetch_lines(const void* pf, uint32_t lines, char* wave_lds, int wg, int n_wg, int tid, int nt) {
+__device__ __forceinline__ void kh_prefetch_lines(const void* const (&pf)[3], const uint32_t (&lines)[3], char* wave_lds, int wg, int n_wg,
+                                                  int tid, int nt) {
 #if __HIP_DEVICE_COMPILE__
-  if (pf == nullptr) return;
-  const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(pf), 0, (int)(lines << 7), 0x00020000);
-  const uint32_t stride = (uint32_t)n_wg * (uint32_t)nt;
-  // four rounds (64 MB with 256 workgroups of 512 threads), no loop; the per-lane offset carries the round, because only
-  // it is checked against the range: an offset beyond the range reads nothing
-  const uint32_t first = ((uint32_t)wg * (uint32_t)nt + (uint32_t)tid) << 7, step = stride << 7;
+  if (pf[0] == nullptr) return;
+  // four rounds over the first range (64 MB with 256 workgroups of 512 threads), one over the others (adapter matrices),
+  // no loop; the per-lane offset carries the round, because only it is checked against the range: an offset beyond the
+  // range reads nothing
+  const uint32_t first = ((uint32_t)wg * (uint32_t)nt + (uint32_t)tid) << 7, step = ((uint32_t)n_wg * (uint32_t)nt) << 7;
 #pragma unroll
-  for (uint32_t r = 0; r < 4; ++r) {
-    const uint32_t off = first + r * step;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)wave_lds, 4, off >= first ? off : 0xFFFFFFFFu, 0, 0, 0);
+  for (int k = 0; k < 3; ++k) {
+    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(pf[k] != nullptr ? pf[k] : pf[0]), 0,
+                                                                        pf[k] != nullptr ? (int)(lines[k] << 7) : 0, 0x00020000);
+#pragma unroll
+    for (uint32_t r = 0; r < (k == 0 ? 4u : 1u); ++r) {
+      const uint32_t off = first + r * step;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)wave_lds, 4, off >= first ? off : 0xFFFFFFFFu, 0, 0, 0);
+    }
   }
 #endif
 }

@@ -455,21 +455,28 @@ __global__ __launch_bounds__(256) void lora_gemm_f32_kernel(const float* __restr
 
 }  // namespace
 
-// See include/katz_hip.h: the weights of the launch after the next one of this family, per host thread.
-static thread_local const void* g_pf_ptr = nullptr;
-static thread_local uint32_t g_pf_lines = 0;
+// See include/katz_hip.h: operands of the launch after the next one of this family, per host thread.
+static thread_local const void* g_pf_ptr[3] = {nullptr, nullptr, nullptr};
+static thread_local uint32_t g_pf_lines[3] = {0, 0, 0};
+static thread_local int g_pf_n = 0;
 
 KH_EXPORT int kh_set_weight_prefetch(const void* weights, int64_t bytes) {
   if (bytes < 0 || (weights == nullptr && bytes != 0)) return KH_ERR_INVALID_ARG;
   const int64_t lines = bytes >> 7;
-  g_pf_ptr = lines > 0 ? weights : nullptr;
-  g_pf_lines = (uint32_t)(lines < (1 << 24) ? lines : (1 << 24));   // at most 2 GiB
+  if (weights == nullptr || lines == 0) { g_pf_n = 0; return KH_OK; }   // clears what is pending
+  if (g_pf_n == 3) return KH_ERR_TOO_LARGE;
+  g_pf_ptr[g_pf_n] = weights;
+  g_pf_lines[g_pf_n] = (uint32_t)(lines < (1 << 24) ? lines : (1 << 24));   // at most 2 GiB
+  ++g_pf_n;
   return KH_OK;
 }
 
 void kh_take_weight_prefetch(LoraGemmParams& p) {
-  p.pf = g_pf_ptr; p.pf_lines = g_pf_lines;
-  g_pf_ptr = nullptr; g_pf_lines = 0;
+  for (int k = 0; k < 3; ++k) {
+    p.pf[k] = k < g_pf_n ? g_pf_ptr[k] : nullptr;
+    p.pf_lines[k] = k < g_pf_n ? g_pf_lines[k] : 0;
+  }
+  g_pf_n = 0;
 }
 
 // See include/katz_hip.h for the contract.

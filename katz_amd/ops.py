@@ -40,25 +40,35 @@ def _req(t: torch.Tensor, dtype, name: str) -> None:
 
 
 # --------------------------------------------------------------------------------------- K1
-# Weight prefetch: a linear / convolution launch can touch the weights of the launch that follows it, so that those wait in
-# the memory-side cache (kh_set_weight_prefetch).  Which weights follow which is learned from the previous pass over
-# the model: a launch with weights W hints at what followed W last time.  The table keeps the tensors alive.
+# Weight prefetch: a linear / convolution launch can touch the operands of the launch that follows it (weights, and the
+# packed adapter matrices), so that those wait in the memory-side cache (kh_set_weight_prefetch).  Which operands follow
+# which is learned from the previous pass over the model: a launch with weights W hints at what followed W last time.
+# The table keeps the tensors alive.
 WEIGHT_PREFETCH = os.getenv("KATZ_WEIGHT_PREFETCH", "1") != "0"
-_pf_next: dict = {}     # data_ptr of a launch's weights -> the weights tensor of the launch that followed it
+_pf_next: dict = {}     # data_ptr of a launch's weights -> (weights, a_cat, b_cat) of the launch that followed it
 _pf_last: list = [None]
+_pf_shrink_a: list = [None]   # A_cat of a separate shrink launch, for the hint of the GEMM it belongs to
 
 
-def _weight_prefetch_hint(weight: torch.Tensor) -> None:
+def _weight_prefetch_hint(weight: torch.Tensor, a_cat: Optional[torch.Tensor] = None,
+                          b_cat: Optional[torch.Tensor] = None) -> None:
     if not WEIGHT_PREFETCH:
         return
+    if a_cat is None:
+        a_cat = _pf_shrink_a[0]
+    _pf_shrink_a[0] = None
     key = weight.data_ptr()
     last = _pf_last[0]
     if last is not None and last != key:
-        _pf_next[last] = weight
+        _pf_next[last] = (weight, a_cat, b_cat)
     _pf_last[0] = key
     nxt = _pf_next.get(key)
     if nxt is not None:
-        _lib.load().kh_set_weight_prefetch(nxt.data_ptr(), nxt.numel() * nxt.element_size())
+        lib = _lib.load()
+        lib.kh_set_weight_prefetch(None, 0)
+        for t in nxt:
+            if t is not None:
+                lib.kh_set_weight_prefetch(t.data_ptr(), t.numel() * t.element_size())
 
 
 def lora_linear(
@@ -111,7 +121,7 @@ def lora_linear(
         CALL_LOG.append(("lora_linear", M, N, K, R, bool(geglu), residual is not None))
     if dt == BF16:
         flags = (1 if geglu else 0) | ((tile & 0xFF) << 8)
-        _weight_prefetch_hint(weight)
+        _weight_prefetch_hint(weight, a_cat, b_cat)
         rc = lib.kh_lora_linear_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(a_cat), _ptr(b_cat), _ptr(col_scale),
                                      _ptr(residual), _ptr(out), M, N, K, R, flags, _stream())
     elif dt == torch.float32:
@@ -138,6 +148,7 @@ def lora_shrink(x: torch.Tensor, a_cat: torch.Tensor, col_scale: torch.Tensor, o
         out = torch.empty((M, R), dtype=BF16, device=x.device)
     if CALL_LOG is not None:
         CALL_LOG.append(("lora_shrink", M, K, R))
+    _pf_shrink_a[0] = a_cat
     rc = lib.kh_lora_shrink_bf16(_ptr(x), _ptr(a_cat), _ptr(col_scale), _ptr(out), M, K, R, _stream())
     _lib.check(rc, "kh_lora_shrink_bf16")
     return out
@@ -178,7 +189,7 @@ def lora_linear_pre(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.
     if CALL_LOG is not None:
         CALL_LOG.append(("lora_linear", M, N, K, R, bool(geglu), residual is not None))
     flags = (1 if geglu else 0) | ((tile & 0xFF) << 8) | (_r_used_bits(r_used, R) << 16)
-    _weight_prefetch_hint(weight)
+    _weight_prefetch_hint(weight, None, b_cat)
     rc = lib.kh_lora_linear_pre_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(t), t.stride(0), n_split, _ptr(b_cat),
                                      _ptr(residual), _ptr(out), M, N, K, R, flags, _stream())
     _lib.check(rc, "kh_lora_linear_pre_bf16")
@@ -298,7 +309,7 @@ def lora_linear_split(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torc
         if lib.kh_lora_linear_split_launches(M, N, K, R, n_split, flags) == 2:
             CALL_LOG.append(("lora_shrink", M, K, RT))
         CALL_LOG.append(("lora_linear", M, N, K, R, bool(geglu), residual is not None))
-    _weight_prefetch_hint(weight)
+    _weight_prefetch_hint(weight, a_cat, b_cat)
     rc = lib.kh_lora_linear_split_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(a_cat), _ptr(col_scale), _ptr(b_cat), _ptr(t),
                                        _ptr(cnt), _ptr(residual), _ptr(out), M, N, K, R, n_split, flags, _stream())
     _lib.check(rc, "kh_lora_linear_split_bf16")
@@ -376,7 +387,7 @@ def lora_linear_norm(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch
         if R and lib.kh_lora_linear_split_launches(M, N, K, R, n_split, flags) == 2:
             CALL_LOG.append(("lora_shrink", M, K, RT))
         CALL_LOG.append(("lora_linear", M, N, K, R, bool(geglu), residual is not None))
-    _weight_prefetch_hint(weight)
+    _weight_prefetch_hint(weight, a_cat, b_cat)
     rc = lib.kh_lora_linear_norm_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(a_cat), _ptr(col_scale), _ptr(b_cat), _ptr(t),
                                       _ptr(cnt), _ptr(residual), _ptr(out), _ptr(part), _ptr(c1), _ptr(c2), _ptr(ca1), _ptr(ca2),
                                       float(eps), _ptr(stats_out), M, N, K, R, n_split, flags, _stream())
