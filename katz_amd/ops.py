@@ -45,6 +45,7 @@ def _req(t: torch.Tensor, dtype, name: str) -> None:
 # which is learned from the previous pass over the model: a launch with weights W hints at what followed W last time.
 # The table keeps the tensors alive.
 WEIGHT_PREFETCH = os.getenv("KATZ_WEIGHT_PREFETCH", "1") != "0"
+PREFETCH_MIN_K = int(os.getenv("KATZ_PREFETCH_MIN_K", "2560"))
 _pf_next: dict = {}     # data_ptr of a launch's weights -> (weights, a_cat, b_cat) of the launch that followed it
 _pf_last: list = [None]
 _pf_shrink_a: list = [None]   # A_cat of a separate shrink launch, for the hint of the GEMM it belongs to
@@ -66,7 +67,13 @@ def _weight_prefetch_hint(weight: torch.Tensor, a_cat: Optional[torch.Tensor] = 
     if nxt is not None:
         lib = _lib.load()
         lib.kh_set_weight_prefetch(None, 0)
-        for t in nxt:
+        w_next = nxt[0]
+        # The prefetch is not free for the launch that carries it (its own first operands queue behind it: up to 3.5 us
+        # for 26 MB), so weights are only hinted where meeting them in HBM costs more than that: long rows (K >= 2560,
+        # the feed-forward output projections and the 3x3 convolutions), whose launches are latency-bound on their
+        # operand stream.  The adapter matrices are small and always hinted.
+        k_next = w_next.shape[-1] * (9 if w_next.dim() == 4 else 1)
+        for t in ((w_next if k_next >= PREFETCH_MIN_K else None),) + tuple(nxt[1:]):
             if t is not None:
                 lib.kh_set_weight_prefetch(t.data_ptr(), t.numel() * t.element_size())
 
