@@ -154,7 +154,7 @@ def sgmv_rooflines(dev):
     g = torch.Generator(device=dev).manual_seed(2)
     rn = lambda *s, std=1.0: (torch.randn(*s, device=dev, generator=g) * std).to(bf)
     ranks = [64, 8, 128, 32, 16, 64, 128, 32]
-    rows = {"shrink": [], "expand": []}
+    rows = {"shrink": [], "expand": [], "fused": []}
     for T, K, N in ((4096, 640, 640), (1024, 1280, 1280), (77, 2048, 1280)):
         RP = 128
         # several input sets, used in turn, together larger than the 256 MB memory-side cache: a launch does not find
@@ -187,16 +187,28 @@ def sgmv_rooflines(dev):
             one(i)
         ls = ops.profile_end()
         assert len(ls) == 2 * reps, len(ls)    # one launch per call
-        for kind, nbytes in (("shrink", 2.0 * (8 * T * K + sr * K + T * sr)), ("expand", 2.0 * (T * sr + sr * N + 2 * 8 * T * N))):
-            ds = sorted(d for i, (_, d) in enumerate(ls) if (i % 2 == 0) == (kind == "shrink"))   # launches alternate
+        # the same in one launch (t stays in the workgroup): x read, y read and written, the adapter matrices
+        ops.profile_begin()
+        for i in range(reps):
+            j = i % nbuf
+            ops.sgmv_fused_(ys[j], xs[j], a_all, b_all, ss, sa, rp, sc, T)
+        lf = ops.profile_end()
+        assert len(lf) == reps, len(lf)
+        for kind, nbytes in (("shrink", 2.0 * (8 * T * K + sr * K + T * sr)), ("expand", 2.0 * (T * sr + sr * N + 2 * 8 * T * N)),
+                             ("fused", 2.0 * (8 * T * K + sr * K + sr * N + 2 * 8 * T * N))):
+            if kind == "fused":
+                ds = sorted(d for _, d in lf)
+            else:
+                ds = sorted(d for i, (_, d) in enumerate(ls) if (i % 2 == 0) == (kind == "shrink"))   # launches alternate
             med = ds[len(ds) // 2]
             rows[kind].append({"shape": f"8 requests x {T} rows, K{K} N{N}, ranks {ranks}", "avg_us": round(med * 1e3, 2),
                                "achieved": round(nbytes / (med * 1e-3) / 1e9, 1),
                                "frac": round(nbytes / (med * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)})
     out = []
-    for kind in ("shrink", "expand"):
+    for kind in ("shrink", "expand", "fused"):
         best = rows[kind][0]
-        out.append({"kernel": f"segmented multi-adapter {kind} (kh_sgmv_{kind}_bf16), median over launches that rotate through input sets larger than the memory-side cache",
+        what = "shrink + expand in one launch" if kind == "fused" else kind
+        out.append({"kernel": f"segmented multi-adapter {what} (kh_sgmv_{kind}_bf16), median over launches that rotate through input sets larger than the memory-side cache",
                     "bound": "hbm", "achieved": best["achieved"], "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": best["frac"],
                     "by_shape": rows[kind]})
     return out

@@ -193,6 +193,13 @@ int kh_sgmv_shrink_bf16(const void* x, const void* a_all, void* t, const int32_t
 int kh_sgmv_expand_bf16(const void* t, const void* b_all, void* y, const int32_t* seg_start,
                         const int32_t* seg_adapter, const int32_t* adapter_rank, const float* adapter_scale,
                         int64_t n_segments, int64_t max_seg_rows, int64_t N, int64_t RP, void* stream);
+/* Both in one launch: y[rows,:] += scale_a * bf16(x[rows,:] A_a^T) B_a^T per segment, t kept inside the workgroup (no
+ * counterpart in the reference, as above; the arithmetic and roundings of kh_sgmv_shrink_bf16 followed by
+ * kh_sgmv_expand_bf16).  K % 64 == 0, N % 128 == 0, RP % 32 == 0, RP <= 128; other shapes: KH_ERR_UNSUPPORTED (use the
+ * two launches). */
+int kh_sgmv_fused_bf16(const void* x, const void* a_all, const void* b_all, void* y, const int32_t* seg_start,
+                       const int32_t* seg_adapter, const int32_t* adapter_rank, const float* adapter_scale,
+                       int64_t n_segments, int64_t max_seg_rows, int64_t N, int64_t K, int64_t RP, void* stream);
 
 /* ---- K3: attention ----------------------------------------------------------------------------
  * o = softmax(q k^T * scale) v per (batch, head); replaces F.scaled_dot_product_attention in

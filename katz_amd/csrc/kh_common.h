@@ -43,7 +43,7 @@ enum KhKernelTag {
   KH_TAG_LORA_GEMM = 1, KH_TAG_LORA_GEMM_F32 = 2, KH_TAG_ATTENTION = 3, KH_TAG_GN_STATS = 4, KH_TAG_GN_APPLY = 5,
   KH_TAG_LAYER_NORM = 6, KH_TAG_GEGLU = 7, KH_TAG_RESIDUAL_ADD = 8, KH_TAG_CONCAT_RESIDUAL = 9,
   KH_TAG_SGMV_SHRINK = 10, KH_TAG_SGMV_EXPAND = 11, KH_TAG_LORA_SHRINK = 12, KH_TAG_CONV = 13, KH_TAG_CFG_EULER = 14,
-  KH_TAG_UPSAMPLE = 15, KH_TAG_LORA_MERGE = 16, KH_TAG_CONV_OUT_STEP = 17
+  KH_TAG_UPSAMPLE = 15, KH_TAG_LORA_MERGE = 16, KH_TAG_CONV_OUT_STEP = 17, KH_TAG_SGMV_FUSED = 18
 };
 bool kh_prof_enabled();
 void kh_prof_events(int tag, hipEvent_t* start, hipEvent_t* stop);

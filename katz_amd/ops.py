@@ -497,6 +497,26 @@ def sgmv_expand_(y, t, b_all, seg_start, seg_adapter, adapter_rank, adapter_scal
     return y
 
 
+def sgmv_fused_(y, x, a_all, b_all, seg_start, seg_adapter, adapter_rank, adapter_scale, max_seg_rows: int):
+    """y[rows] += scale_a * bf16(x[rows] A_a^T) B_a^T per segment, in place, in ONE launch (kh_sgmv_fused_bf16): the
+    arithmetic of sgmv_shrink followed by sgmv_expand_ without the round trip of t.  K % 64 == 0, N % 128 == 0."""
+    lib = _lib.load()
+    _req(y, BF16, "y"); _req(x, BF16, "x"); _req(a_all, BF16, "a_all"); _req(b_all, BF16, "b_all")
+    _req(adapter_scale, torch.float32, "adapter_scale")
+    for n, t in (("seg_start", seg_start), ("seg_adapter", seg_adapter), ("adapter_rank", adapter_rank)):
+        _req(t, torch.int32, n)
+    rows, K = x.shape
+    N = y.shape[1]
+    RP = a_all.shape[1]
+    if y.shape[0] != rows or a_all.shape[2] != K or b_all.shape[1:] != (N, RP) or b_all.shape[0] != a_all.shape[0]:
+        raise ValueError("x [rows, K], y [rows, N], a_all [n_adapters, RP, K], b_all [n_adapters, N, RP]")
+    nseg = seg_adapter.numel()
+    rc = lib.kh_sgmv_fused_bf16(_ptr(x), _ptr(a_all), _ptr(b_all), _ptr(y), _ptr(seg_start), _ptr(seg_adapter),
+                                _ptr(adapter_rank), _ptr(adapter_scale), nseg, max_seg_rows, N, K, RP, _stream())
+    _lib.check(rc, "kh_sgmv_fused_bf16")
+    return y
+
+
 # --------------------------------------------------------------------------------------- K3
 def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, heads: int, scale: Optional[float] = None,
               out: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -796,7 +816,7 @@ def conv_out_cfg_euler(x: torch.Tensor, w_packed: torch.Tensor, bias: Optional[t
 # --------------------------------------------------------------------------------------- per-launch timing
 KERNEL_TAGS = {1: "lora_gemm", 2: "lora_gemm_f32", 3: "attention", 4: "group_norm_stats", 5: "group_norm_apply",
                6: "layer_norm", 7: "geglu", 8: "residual_add", 9: "concat_residual", 10: "sgmv_shrink",
-               11: "sgmv_expand", 12: "lora_shrink", 13: "conv3x3", 14: "cfg_euler", 15: "upsample", 16: "lora_merge", 17: "conv_out_step"}
+               11: "sgmv_expand", 12: "lora_shrink", 13: "conv3x3", 14: "cfg_euler", 15: "upsample", 16: "lora_merge", 17: "conv_out_step", 18: "sgmv_fused"}
 
 
 def profile_begin() -> None:

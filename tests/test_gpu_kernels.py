@@ -491,6 +491,49 @@ def test_sgmv_heterogeneous_batch(T, K, N):
     a0 = seg_adapter[0]
     t_ref = torch.nn.functional.linear(x[:T], adapters[a0][0])
     assert_close_rel(t[:T, : ranks[a0]], t_ref, REL_BF16, "sgmv shrink")
+    # both in one launch (t stays in the workgroup): same oracle, the adapter-free request untouched, and the two-launch
+    # result to within the last bf16 place (the K order of the two products is the same; tiles differ)
+    y2 = y_base.clone()
+    ops.sgmv_fused_(y2, xd, a_all.to(d, BF), b_all.to(d, BF), ss, sa, rank_pad, scales, T)
+    torch.cuda.synchronize()
+    assert_close_rel(y2, ref, REL_BF16, "sgmv fused")
+    assert torch.equal(y2[3 * T:4 * T], y_base[3 * T:4 * T])
+    assert_close_rel(y2, y.float().cpu(), 1e-2, "sgmv fused vs two launches")
+
+
+def test_sgmv_fused_ragged_segments_and_small_rank_pad():
+    """Segments of unequal length (one empty, one shorter than a tile, one not a multiple of 128) and RP = 64."""
+    from katz_amd import ops
+
+    say("sgmv fused ragged")
+    g = torch.Generator().manual_seed(11)
+    lens = [300, 0, 77, 128, 513]
+    K, N, RP = 640, 1280, 64
+    ranks = [8, 64, 32, 16, 64]
+    seg_adapter = [2, 0, -1, 4, 1]
+    seg_start = [0]
+    for n in lens:
+        seg_start.append(seg_start[-1] + n)
+    rows = seg_start[-1]
+    x = randn(g, rows, K)
+    base = randn(g, rows, N)
+    adapters = [(randn(g, r, K, std=0.02), randn(g, N, r, std=0.02), 0.3 + 0.2 * i) for i, r in enumerate(ranks)]
+    a_all = torch.zeros(len(ranks), RP, K); b_all = torch.zeros(len(ranks), N, RP)
+    for i, (A, B, _) in enumerate(adapters):
+        a_all[i, : A.shape[0]] = A
+        b_all[i, :, : B.shape[1]] = B
+    d = dev()
+    rank_pad = torch.tensor([(r + 31) // 32 * 32 for r in ranks], dtype=torch.int32, device=d)
+    scales = torch.tensor([a[2] for a in adapters], dtype=torch.float32, device=d)
+    ss = torch.tensor(seg_start, dtype=torch.int32, device=d)
+    sa = torch.tensor(seg_adapter, dtype=torch.int32, device=d)
+    y = base.to(d, BF).clone()
+    guard = y.clone()
+    ops.sgmv_fused_(y, x.to(d, BF), a_all.to(d, BF), b_all.to(d, BF), ss, sa, rank_pad, scales, max(lens))
+    torch.cuda.synchronize()
+    ref = O.sgmv(x.to(BF).float(), seg_start, seg_adapter, adapters, base.to(BF).float())
+    assert_close_rel(y, ref, REL_BF16, "sgmv fused ragged")
+    assert torch.equal(y[seg_start[2]:seg_start[3]], guard[seg_start[2]:seg_start[3]])   # the request without an adapter
 
 
 def test_fused_qkv_matches_separate_projections():
