@@ -10,6 +10,7 @@ from __future__ import annotations
 import ctypes
 import math
 import os
+import weakref
 from typing import Optional, Sequence
 
 import torch
@@ -43,10 +44,10 @@ def _req(t: torch.Tensor, dtype, name: str) -> None:
 # Weight prefetch: a linear / convolution launch can touch the operands of the launch that follows it (weights, and the
 # packed adapter matrices), so that those wait in the memory-side cache (kh_set_weight_prefetch).  Which operands follow
 # which is learned from the previous pass over the model: a launch with weights W hints at what followed W last time.
-# The table keeps the tensors alive.
+# The table holds weak references only: a hint never keeps a tensor alive, and a dead one is dropped instead of hinted.
 WEIGHT_PREFETCH = os.getenv("KATZ_WEIGHT_PREFETCH", "1") != "0"
 PREFETCH_MIN_K = int(os.getenv("KATZ_PREFETCH_MIN_K", "2560"))
-_pf_next: dict = {}     # data_ptr of a launch's weights -> (weights, a_cat, b_cat) of the launch that followed it
+_pf_next: dict = {}     # data_ptr of a launch's weights -> weak references to (weights, a_cat, b_cat) of the launch after it
 _pf_last: list = [None]
 _pf_shrink_a: list = [None]   # A_cat of a separate shrink launch, for the hint of the GEMM it belongs to
 
@@ -55,27 +56,34 @@ def _weight_prefetch_hint(weight: torch.Tensor, a_cat: Optional[torch.Tensor] = 
                           b_cat: Optional[torch.Tensor] = None) -> None:
     if not WEIGHT_PREFETCH:
         return
-    if a_cat is None:
-        a_cat = _pf_shrink_a[0]
+    if a_cat is None and _pf_shrink_a[0] is not None:
+        a_cat = _pf_shrink_a[0]()
     _pf_shrink_a[0] = None
     key = weight.data_ptr()
     last = _pf_last[0]
     if last is not None and last != key:
-        _pf_next[last] = (weight, a_cat, b_cat)
+        _pf_next[last] = tuple(None if t is None else weakref.ref(t) for t in (weight, a_cat, b_cat))
+        if len(_pf_next) > 65536:     # models come and go: forget everything rather than grow without bound
+            _pf_next.clear()
     _pf_last[0] = key
     nxt = _pf_next.get(key)
-    if nxt is not None:
-        lib = _lib.load()
-        lib.kh_set_weight_prefetch(None, 0)
-        w_next = nxt[0]
-        # The prefetch is not free for the launch that carries it (its own first operands queue behind it: up to 3.5 us
-        # for 26 MB), so weights are only hinted where meeting them in HBM costs more than that: long rows (K >= 2560,
-        # the feed-forward output projections and the 3x3 convolutions), whose launches are latency-bound on their
-        # operand stream.  The adapter matrices are small and always hinted.
-        k_next = w_next.shape[-1] * (9 if w_next.dim() == 4 else 1)
-        for t in ((w_next if k_next >= PREFETCH_MIN_K else None),) + tuple(nxt[1:]):
-            if t is not None:
-                lib.kh_set_weight_prefetch(t.data_ptr(), t.numel() * t.element_size())
+    if nxt is None:
+        return
+    live = [None if r is None else r() for r in nxt]
+    w_next = live[0]
+    if w_next is None:                # the tensor that followed last time is gone
+        del _pf_next[key]
+        return
+    lib = _lib.load()
+    lib.kh_set_weight_prefetch(None, 0)
+    # The prefetch is not free for the launch that carries it (its own first operands queue behind it: up to 3.5 us
+    # for 26 MB), so weights are only hinted where meeting them in HBM costs more than that: long rows (K >= 2560,
+    # the feed-forward output projections and the 3x3 convolutions), whose launches are latency-bound on their
+    # operand stream.  The adapter matrices are small and always hinted.
+    k_next = w_next.shape[-1] * (9 if w_next.dim() == 4 else 1)
+    for t in ((w_next if k_next >= PREFETCH_MIN_K else None),) + tuple(live[1:]):
+        if t is not None:
+            lib.kh_set_weight_prefetch(t.data_ptr(), t.numel() * t.element_size())
 
 
 def lora_linear(
@@ -155,7 +163,7 @@ def lora_shrink(x: torch.Tensor, a_cat: torch.Tensor, col_scale: torch.Tensor, o
         out = torch.empty((M, R), dtype=BF16, device=x.device)
     if CALL_LOG is not None:
         CALL_LOG.append(("lora_shrink", M, K, R))
-    _pf_shrink_a[0] = a_cat
+    _pf_shrink_a[0] = weakref.ref(a_cat)
     rc = lib.kh_lora_shrink_bf16(_ptr(x), _ptr(a_cat), _ptr(col_scale), _ptr(out), M, K, R, _stream())
     _lib.check(rc, "kh_lora_shrink_bf16")
     return out

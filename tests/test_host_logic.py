@@ -436,3 +436,48 @@ def test_bench_refuses_more_than_one_gpu():
     root = Path(__file__).resolve().parent.parent
     r = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
     assert r.returncode == 2 and "ONE GPU" in r.stderr
+
+
+def test_weight_prefetch_hints_are_learned_from_the_previous_pass(monkeypatch):
+    """ops._weight_prefetch_hint: the first pass over a sequence of launches gives no hints; the second hints, at launch
+    i, the operands of launch i + 1 - weights only for long rows (K >= 2560 or a 3x3 kernel), adapter matrices always;
+    a tensor that has been freed is dropped instead of hinted."""
+    import gc
+
+    from katz_amd import ops
+
+    calls = []
+
+    class FakeLib:
+        def kh_set_weight_prefetch(self, ptr, nbytes):
+            calls.append((ptr, nbytes))
+            return 0
+
+    monkeypatch.setattr(ops._lib, "load", lambda: FakeLib())
+    monkeypatch.setattr(ops, "WEIGHT_PREFETCH", True)
+    ops._pf_next.clear()
+    ops._pf_last[0] = None
+    w_small = torch.zeros(8, 1280)             # K 1280: not hinted
+    w_long = torch.zeros(8, 5120)              # K 5120: hinted
+    w_conv = torch.zeros(4, 3, 3, 320)         # 9 * 320 = 2880: hinted
+    a_cat, b_cat = torch.zeros(128, 5120), torch.zeros(8, 128)
+    seq = [(w_small, None, None), (w_long, a_cat, b_cat), (w_conv, None, None)]
+    for w, a, b in seq:
+        ops._weight_prefetch_hint(w, a, b)
+    assert calls == []                          # nothing known on the first pass
+    for w, a, b in seq:
+        ops._weight_prefetch_hint(w, a, b)
+    hinted = [c for c in calls if c[0] is not None]
+    assert hinted == [(w_long.data_ptr(), w_long.numel() * 4), (a_cat.data_ptr(), a_cat.numel() * 4),
+                      (b_cat.data_ptr(), b_cat.numel() * 4), (w_conv.data_ptr(), w_conv.numel() * 4)]
+    # what followed w_conv last time is w_small (the wrap-around), K 1280: its entry exists but hints nothing
+    assert ops._pf_next[w_conv.data_ptr()][0]() is w_small
+    # a freed successor: dropped
+    key = w_small.data_ptr()
+    del w_long, seq, w, a, b
+    gc.collect()
+    calls.clear()
+    ops._weight_prefetch_hint(w_small)
+    assert [c for c in calls if c[0] is not None] == [] and key not in ops._pf_next
+    ops._pf_next.clear()
+    ops._pf_last[0] = None
