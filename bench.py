@@ -580,7 +580,8 @@ def main():
         e = by_kernel.setdefault(name, [0, 0.0])
         e[0] += 1
         e[1] += dur
-    gemm_calls = [c for c in log if c[0] in ("lora_linear", "lora_linear_grouped")]
+    # (a cross-attention's query projection that runs the attention in its epilogue is one launch of the GEMM family)
+    gemm_calls = [c for c in log if c[0] in ("lora_linear", "lora_linear_grouped", "lora_linear_xattn")]
     gemm_ms = [d for n, d in launches if n == "lora_gemm"]
     assert len(gemm_calls) == len(gemm_ms), (len(gemm_calls), len(gemm_ms))
     # two-launch layers: the shrink launch belongs to the layer whose GEMM follows it
@@ -597,23 +598,27 @@ def main():
                    for (M, K, R), (cnt, tot) in sorted(shrink_shapes.items(), key=lambda kv: -kv[1][1])]
     n_layers = lambda c: c[5] if c[0] == "lora_linear_grouped" else 1
     rank_of = lambda c: true_rank if c[4] > 0 else 0
-    gemm_flops = sum(n_layers(c) * lora_linear_flops(c[1], c[2], c[3], rank_of(c)) for c in gemm_calls)
+    keys_of = lambda c: c[7] if c[0] == "lora_linear_xattn" else 0      # attention inside the launch: 4 M N S more FLOPs
+    call_flops = lambda c: n_layers(c) * lora_linear_flops(c[1], c[2], c[3], rank_of(c)) + 4.0 * c[1] * c[2] * keys_of(c)
+    gemm_flops = sum(call_flops(c) for c in gemm_calls)
     gemm_total_ms = sum(gemm_ms) + shrink_ms
     attn_flops = sum(4.0 * c[1] * c[2] * c[3] * c[4] * c[5] for c in log if c[0] == "attention")
     step_flops = gemm_flops + attn_flops + conv_flops
     achieved_tf = gemm_flops / (gemm_total_ms * 1e-3) / 1e12
     by_shape = {}
     for c, d in zip(gemm_calls, gemm_ms):
-        e = by_shape.setdefault(tuple(c[1:4]) + (rank_of(c), n_layers(c)), [0, 0.0])
+        e = by_shape.setdefault(tuple(c[1:4]) + (rank_of(c), n_layers(c), keys_of(c)), [0, 0.0])
         e[0] += 1
         e[1] += d
     shape_rows = []
-    for (M, N, K, R, G), (cnt, tot) in sorted(by_shape.items(), key=lambda kv: -kv[1][1]):
-        fl = G * lora_linear_flops(M, N, K, R)
+    for (M, N, K, R, G, S), (cnt, tot) in sorted(by_shape.items(), key=lambda kv: -kv[1][1]):
+        fl = G * lora_linear_flops(M, N, K, R) + 4.0 * M * N * S
         tf = fl / (tot / cnt * 1e-3) / 1e12
         shape_rows.append({"M": M, "N": N, "K": K, "rank": R, "layers_per_launch": G, "launches": cnt,
                            "avg_us": round(tot / cnt * 1e3, 2), "ms_per_step": round(tot, 3), "tflops": round(tf, 1),
                            "frac": round(tf / PEAK_BF16_TFLOPS, 3)})
+        if S:
+            shape_rows[-1]["attention_keys_in_epilogue"] = S
     traffic, traffic_src = traffic_from_profiles("lora_gemm M2048 K1280 N10240")
 
     # ---- the other kernels of the path against their own rooflines ----------------------------------------------

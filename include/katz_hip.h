@@ -127,6 +127,26 @@ int kh_lora_linear_norm_bf16(const void* x, const void* w, const void* bias, con
                              const float* ln_part, const float* ln_c1, const float* ln_c2, const float* ln_ca1,
                              const float* ln_ca2, float ln_eps, float* stats_out, int64_t M, int64_t N, int64_t K,
                              int64_t R, int64_t n_split, int flags, void* stream);
+/* A cross-attention's query projection and the attention itself in ONE launch: o = softmax(q k^T * scale) v with
+ * q = kh_lora_linear_norm_bf16(x, ...) never written to memory.  The reference runs to_q, then the attention processor
+ * on its result (diffusers-hf/src/diffusers/models/attention_processor.py:1231-1296: attn.to_q :1256, head split
+ * :1269-1272, F.scaled_dot_product_attention :1276); on the SDXL text context (S = 77 keys) the attention alone is a
+ * launch of a few microseconds whose 128 queries x 2 heads are exactly one 128 x 128 output tile of the projection, so
+ * the GEMM's epilogue keeps the tile in LDS, loads the S keys / values of its two heads and runs the attention there.
+ * x [M,K] with M = B * T (rows of sample b: b*T .. b*T + T - 1), w [N,K], N = heads * 64; k, v: [B,S,N] views (row
+ * strides ldk / ldv, sample strides bsk / bsv, in elements); o [M,N] with row stride ldo, head h at columns 64 h.
+ * The projection's arguments (bias, adapters, t_scratch, counters, folded LayerNorm, flags bits 8..23) are
+ * kh_lora_linear_norm_bf16's, without residual, statistics, GEGLU and n_split.  M % 128 == 0, T % 128 == 0, N % 128 == 0,
+ * K % 64 == 0, R % 64 == 0, R <= 128, S <= 96, at most 256 tiles of 128 x 128: kh_lora_linear_xattn_ok says whether a
+ * shape is taken (1) or not (0: run the projection and kh_attention_bf16).  Against those two calls the result differs
+ * by rounding only (one softmax pass over all keys instead of a running maximum over 64-key tiles). */
+int kh_lora_linear_xattn_bf16(const void* x, const void* w, const void* bias, const void* a_cat, const float* col_scale,
+                              const void* b_cat, void* t_scratch, int32_t* counters, const float* ln_part,
+                              const float* ln_c1, const float* ln_c2, const float* ln_ca1, const float* ln_ca2, float ln_eps,
+                              const void* k, const void* v, void* o, int64_t M, int64_t N, int64_t K, int64_t R, int64_t T,
+                              int64_t S, int64_t ldk, int64_t ldv, int64_t ldo, int64_t bsk, int64_t bsv, float scale,
+                              int flags, void* stream);
+int kh_lora_linear_xattn_ok(int64_t M, int64_t N, int64_t K, int64_t R, int64_t T, int64_t S);
 /* Bounded waits of kh_lora_linear_split_bf16's in-launch shrink that have run out on the current device since the
  * process started (or since the last call with clear != 0): writes the number to *count (HOST pointer).  A GEMM workgroup
  * of that launch waits for the shrink workgroups of the same launch, which have lower workgroup ids and are therefore

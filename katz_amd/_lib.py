@@ -36,6 +36,8 @@ SIGNATURES = {
     "kh_lora_linear_split_bf16": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, c_int, _P]),
     "kh_lora_linear_norm_bf16": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, c_float, _P,
                                          _I, _I, _I, _I, _I, c_int, _P]),
+    "kh_lora_linear_xattn_bf16": (c_int, [_P] * 8 + [_P] * 5 + [c_float] + [_P] * 3 + [_I] * 11 + [c_float, c_int, _P]),
+    "kh_lora_linear_xattn_ok": (c_int, [_I] * 6),
     "kh_lora_split_timeouts": (c_int, [_P, c_int]),
     "kh_set_weight_prefetch": (c_int, [_P, _I]),
     "kh_lora_linear_split_launches": (c_int, [_I, _I, _I, _I, _I, c_int]),

@@ -61,6 +61,14 @@ struct LoraGemmParams {
   // of the NEXT launch of this family, so that they wait in the memory-side cache when that launch asks for them (a
   // step reads 2.5 GB of weights once each: every launch would otherwise meet its weights in HBM, where the XCDs that
   // share a weight block each fetch it again).  Set from kh_set_weight_prefetch by the entry points.
+  // Cross-attention in the epilogue (xa_k != nullptr; the 128x128 / 8-wave tiles only): the layer is an attention's to_q
+  // and a 128 x 128 output tile holds 128 queries of two 64-wide heads; instead of storing them the workgroup runs
+  // softmax(q k^T * scale) v for them against the xa_S <= 96 keys of those heads and stores that to xa_o (rows like y's,
+  // head h at columns 64 h).  Rows m belong to batch sample m / xa_T (xa_T % 128 == 0); k / v: [B, S, heads * 64] views.
+  const bf16_t* xa_k = nullptr; const bf16_t* xa_v = nullptr; bf16_t* xa_o = nullptr;
+  int xa_S = 0, xa_T = 0;
+  long xa_ldk = 0, xa_ldv = 0, xa_ldo = 0, xa_bsk = 0, xa_bsv = 0;
+  float xa_scale_log2e = 0.f;
   const void* pf[3] = {nullptr, nullptr, nullptr};   // up to three ranges: weights, A_cat, B_cat of that launch
   uint32_t pf_lines[3] = {0, 0, 0};
 };
@@ -182,6 +190,9 @@ int lora_gemm_pipe_launch_grouped(const LoraGemmParams& p, int n_groups, hipStre
 // scratch for the shrink result, p.il_cnt = counters); KH_ERR_UNSUPPORTED when the shape does not qualify.
 bool lora_gemm_pipe_il_ok(const LoraGemmParams& p);
 int lora_gemm_pipe_launch_il(const LoraGemmParams& p, hipStream_t stream);
+// query projection + cross-attention in its epilogue (xa_k set)
+bool lora_gemm_pipe_xattn_ok(const LoraGemmParams& p);
+int lora_gemm_pipe_launch_xattn(const LoraGemmParams& p, hipStream_t stream);
 // Narrow-output variant (lora_gemm_ksplit.hip): (32 * row_groups) x 160 tiles, 8 waves as row_groups x k-slices;
 // plain or K-extended GEMM with bias / residual, K % 64 == 0.  row_groups 2 or 4.
 bool lora_gemm_ksplit_ok(const LoraGemmParams& p);

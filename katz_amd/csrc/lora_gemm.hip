@@ -614,13 +614,21 @@ KH_EXPORT int kh_lora_linear_split_bf16(const void* x, const void* w, const void
 
 // LoRA linear behind a LayerNorm that is folded into the GEMM, and / or in front of one (row statistics out); see
 // include/katz_hip.h.
-KH_EXPORT int kh_lora_linear_norm_bf16(const void* x, const void* w, const void* bias, const void* a_cat,
-                                       const float* col_scale, const void* b_cat, void* t_scratch, int32_t* counters,
-                                       const void* residual, void* y, const float* ln_part, const float* ln_c1,
-                                       const float* ln_c2, const float* ln_ca1, const float* ln_ca2, float ln_eps,
-                                       float* stats_out, int64_t M, int64_t N, int64_t K, int64_t R, int64_t n_split,
-                                       int flags, void* stream) {
-  if (!x || !w || !y || M <= 0 || N <= 0 || K <= 0 || R < 0) return KH_ERR_INVALID_ARG;
+namespace {
+struct XAttnArgs {   // the attention behind a query projection (kh_lora_linear_xattn_bf16)
+  const void* k; const void* v; void* o;
+  int64_t T, S, ldk, ldv, ldo, bsk, bsv;
+  float scale;
+};
+}  // namespace
+
+static int lora_linear_norm_impl(const void* x, const void* w, const void* bias, const void* a_cat,
+                                 const float* col_scale, const void* b_cat, void* t_scratch, int32_t* counters,
+                                 const void* residual, void* y, const float* ln_part, const float* ln_c1,
+                                 const float* ln_c2, const float* ln_ca1, const float* ln_ca2, float ln_eps,
+                                 float* stats_out, int64_t M, int64_t N, int64_t K, int64_t R, int64_t n_split,
+                                 int flags, void* stream, const XAttnArgs* xa) {
+  if (!x || !w || (!y && !xa) || M <= 0 || N <= 0 || K <= 0 || R < 0) return KH_ERR_INVALID_ARG;
   if (R > 0 && (!a_cat || !col_scale || !b_cat || !t_scratch)) return KH_ERR_INVALID_ARG;
   if (ln_part != nullptr && (!ln_c1 || !ln_c2 || bias != nullptr || (R > 0 && (!ln_ca1 || !ln_ca2)))) return KH_ERR_INVALID_ARG;
   if (n_split < 0 || (n_split > 0 && (n_split % 128 != 0 || N % n_split != 0))) return KH_ERR_INVALID_ARG;
@@ -632,7 +640,7 @@ KH_EXPORT int kh_lora_linear_norm_bf16(const void* x, const void* w, const void*
   if (geglu && (N % 64 != 0 || residual != nullptr || stats_out != nullptr)) return KH_ERR_UNSUPPORTED;
   if (stats_out != nullptr && N > 128 * KH_LN_SLOTS) return KH_ERR_TOO_LARGE;
   if (((flags >> 16) & 0xff) * 16 > R) return KH_ERR_INVALID_ARG;
-  if (!kh_aligned16(x) || !kh_aligned16(w) || !kh_aligned16(y) || (R > 0 && (!kh_aligned16(a_cat) || !kh_aligned16(b_cat) ||
+  if (!kh_aligned16(x) || !kh_aligned16(w) || (y && !kh_aligned16(y)) || (R > 0 && (!kh_aligned16(a_cat) || !kh_aligned16(b_cat) ||
       !kh_aligned16(t_scratch))) || (residual && !kh_aligned16(residual)) || (ln_part && !kh_aligned16(ln_part)) ||
       (stats_out && !kh_aligned16(stats_out)))
     return KH_ERR_ALIGNMENT;
@@ -641,8 +649,30 @@ KH_EXPORT int kh_lora_linear_norm_bf16(const void* x, const void* w, const void*
   p.r_used = ((flags >> 16) & 0xff) * 16;
   p.ln_part = ln_part; p.ln_c1 = ln_c1; p.ln_c2 = ln_c2; p.ln_ca1 = ln_ca1; p.ln_ca2 = ln_ca2; p.ln_eps = ln_eps;
   p.st_part = stats_out;
-  kh_take_weight_prefetch(p);
   const int tile_sel = (flags >> 8) & 0xff;
+  if (xa != nullptr) {
+    // the projection's result never reaches memory: its 128 x 128 tiles are 128 queries of two heads each
+    if (!xa->k || !xa->v || !xa->o || xa->T <= 0 || xa->S <= 0 || M % xa->T != 0) return KH_ERR_INVALID_ARG;
+    if (residual != nullptr || stats_out != nullptr || geglu || n_split != 0 || (tile_sel != 0 && tile_sel != 1)) return KH_ERR_INVALID_ARG;
+    if (xa->S > 96 || xa->T % 128 != 0 || N % 128 != 0 || (R % 64) != 0) return KH_ERR_UNSUPPORTED;
+    if ((xa->ldk | xa->ldv | xa->ldo | xa->bsk | xa->bsv) % 8 != 0) return KH_ERR_ALIGNMENT;
+    if (xa->ldk < N || xa->ldv < N || xa->ldo < N) return KH_ERR_INVALID_ARG;
+    if (!kh_aligned16(xa->k) || !kh_aligned16(xa->v) || !kh_aligned16(xa->o)) return KH_ERR_ALIGNMENT;
+    p.xa_k = (const bf16_t*)xa->k; p.xa_v = (const bf16_t*)xa->v; p.xa_o = (bf16_t*)xa->o;
+    p.xa_S = (int)xa->S; p.xa_T = (int)xa->T;
+    p.xa_ldk = xa->ldk; p.xa_ldv = xa->ldv; p.xa_ldo = xa->ldo; p.xa_bsk = xa->bsk; p.xa_bsv = xa->bsv;
+    p.xa_scale_log2e = xa->scale * 1.4426950408889634f;
+    if (R == 0) { p.ldt = 0; p.t_nsplit = 0; p.il_cnt = nullptr; }
+    if (!lora_gemm_pipe_xattn_ok(p)) return KH_ERR_UNSUPPORTED;
+    kh_take_weight_prefetch(p);
+    if (R == 0) return lora_gemm_pipe_launch_xattn(p, (hipStream_t)stream);
+    if (counters != nullptr && tile_sel == 0 && lora_gemm_pipe_il_ok(p)) return lora_gemm_pipe_launch_xattn(p, (hipStream_t)stream);
+    const int rc = lora_shrink_ln_launch(x, a_cat, col_scale, t_scratch, M, K, RT, ln_part, ln_ca1, ln_ca2, ln_eps, (hipStream_t)stream);
+    if (rc != KH_OK) return rc;
+    p.a_cat = nullptr; p.col_scale = nullptr; p.il_cnt = nullptr;
+    return lora_gemm_pipe_launch_xattn(p, (hipStream_t)stream);
+  }
+  kh_take_weight_prefetch(p);
   if (R == 0) {
     p.ldt = 0; p.t_nsplit = 0; p.il_cnt = nullptr;
     return lora_gemm_pipe_launch(p, tile_sel, (hipStream_t)stream);
@@ -652,6 +682,36 @@ KH_EXPORT int kh_lora_linear_norm_bf16(const void* x, const void* w, const void*
   if (rc != KH_OK) return rc;
   p.a_cat = nullptr; p.col_scale = nullptr; p.il_cnt = nullptr;
   return lora_gemm_pipe_launch(p, tile_sel == 1 ? 0 : tile_sel, (hipStream_t)stream);
+}
+
+KH_EXPORT int kh_lora_linear_norm_bf16(const void* x, const void* w, const void* bias, const void* a_cat,
+                                       const float* col_scale, const void* b_cat, void* t_scratch, int32_t* counters,
+                                       const void* residual, void* y, const float* ln_part, const float* ln_c1,
+                                       const float* ln_c2, const float* ln_ca1, const float* ln_ca2, float ln_eps,
+                                       float* stats_out, int64_t M, int64_t N, int64_t K, int64_t R, int64_t n_split,
+                                       int flags, void* stream) {
+  return lora_linear_norm_impl(x, w, bias, a_cat, col_scale, b_cat, t_scratch, counters, residual, y, ln_part, ln_c1, ln_c2, ln_ca1,
+                               ln_ca2, ln_eps, stats_out, M, N, K, R, n_split, flags, stream, nullptr);
+}
+
+// Query projection (kh_lora_linear_norm_bf16 without residual / statistics) with the cross-attention on its result inside
+// the same launch; see include/katz_hip.h.
+KH_EXPORT int kh_lora_linear_xattn_bf16(const void* x, const void* w, const void* bias, const void* a_cat,
+                                        const float* col_scale, const void* b_cat, void* t_scratch, int32_t* counters,
+                                        const float* ln_part, const float* ln_c1, const float* ln_c2, const float* ln_ca1,
+                                        const float* ln_ca2, float ln_eps, const void* k, const void* v, void* o, int64_t M,
+                                        int64_t N, int64_t K, int64_t R, int64_t T, int64_t S, int64_t ldk, int64_t ldv,
+                                        int64_t ldo, int64_t bsk, int64_t bsv, float scale, int flags, void* stream) {
+  const XAttnArgs xa = {k, v, o, T, S, ldk, ldv, ldo, bsk, bsv, scale};
+  return lora_linear_norm_impl(x, w, bias, a_cat, col_scale, b_cat, t_scratch, counters, nullptr, nullptr, ln_part, ln_c1, ln_c2,
+                               ln_ca1, ln_ca2, ln_eps, nullptr, M, N, K, R, 0, flags, stream, &xa);
+}
+
+// 1 if kh_lora_linear_xattn_bf16 takes these shapes, else 0 (then: the projection and kh_attention_bf16).
+KH_EXPORT int kh_lora_linear_xattn_ok(int64_t M, int64_t N, int64_t K, int64_t R, int64_t T, int64_t S) {
+  if (M <= 0 || N <= 0 || K <= 0 || R < 0 || T <= 0 || S <= 0 || M > (1 << 24) || N > (1 << 24) || K > (1 << 24)) return 0;
+  if (M % 128 != 0 || N % 128 != 0 || K % 64 != 0 || R % 64 != 0 || R > 128 || T % 128 != 0 || M % T != 0 || S > 96) return 0;
+  return (M / 128) * (N / 128) <= 256 ? 1 : 0;
 }
 
 // 3x3 convolution, padding 1, NHWC, as an implicit GEMM on the pipelined kernel; see include/katz_hip.h.

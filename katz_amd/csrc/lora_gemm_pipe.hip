@@ -460,9 +460,141 @@ __device__ __forceinline__ void k_loop2(char* smem, const Dma2<C>& dma, const Rs
 #endif
 }
 
+// Cross-attention of a staged query tile (see LoraGemmParams::xa_k): sQ holds the 128 x 128 bf16 tile (row stride LDQ), i.e.
+// 128 queries of heads h0 = n0 / 64 and h0 + 1; wave w takes head w / 4 and queries 32 (w % 4) .. + 31.  The arithmetic is
+// kh_attention_bf16's (attention.hip) in one pass over at most 96 keys: S^T = K . Q^T on the MFMA with one query per lane,
+// exp2 of the scaled scores against the row maximum, O^T += V^T . P^T with P straight from the score registers, the row
+// sums as one more MFMA against ones.  K and V^T (keys in pairs per 32-bit word) sit in LDS behind the tile.
+template <int LDQ>
+struct XAttnTile {
+  static constexpr int XS = 96, LDH = 64 + 8, LDV = XS + 8, NT = 512;
+  static constexpr int Q_BYTES = 128 * LDQ * 2, K_BYTES = 2 * XS * LDH * 2, V_BYTES = 2 * 64 * LDV * 2;
+  static constexpr int LDS_BYTES = Q_BYTES + K_BYTES + V_BYTES;
+  static constexpr int VCHUNKS = 2 * (XS / 2) * 8;   // (head, key pair, 8-column piece)
+  u32x4 rk[3], rv[2][2];
+
+  // K: 2 heads x 96 keys x 8 pieces of 16 bytes; V: 2 heads x 48 key pairs x 8 pieces (transposed on the way into LDS).
+  // Requested before the query tile is staged; keys beyond S read as zeros and are masked in the scores.
+  __device__ __forceinline__ void load(const LoraGemmParams& p, int m0, int n0, int tid) {
+    const int S = p.xa_S, b = m0 / p.xa_T;
+    const bf16_t* kp = p.xa_k + (size_t)b * p.xa_bsk + n0;
+    const bf16_t* vp = p.xa_v + (size_t)b * p.xa_bsv + n0;
+    const u32x4 z4 = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int i = 0; i < 3; ++i) {
+      const int c = tid + i * NT, hh = c / (XS * 8), key = (c % (XS * 8)) >> 3, pc = c & 7;
+      rk[i] = key < S ? *reinterpret_cast<const u32x4*>(kp + (size_t)key * p.xa_ldk + hh * 64 + pc * 8) : z4;
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int c = tid + j * NT, hh = c / (VCHUNKS / 2), rest = c % (VCHUNKS / 2), v_kp = rest % (XS / 2), v_dch = rest / (XS / 2);
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int key = 2 * v_kp + i;
+        rv[j][i] = (c < VCHUNKS && key < S) ? *reinterpret_cast<const u32x4*>(vp + (size_t)key * p.xa_ldv + hh * 64 + v_dch * 8) : z4;
+      }
+    }
+  }
+
+  // after every wave has written its part of sQ (no barrier needed before: K / V^T go to their own LDS ranges)
+  __device__ __forceinline__ void run(char* smem, const LoraGemmParams& p, int m0, int n0, int tid) {
+    bf16_t* sQ = reinterpret_cast<bf16_t*>(smem);
+    bf16_t* sK = reinterpret_cast<bf16_t*>(smem + Q_BYTES);
+    uint32_t* sVt = reinterpret_cast<uint32_t*>(smem + Q_BYTES + K_BYTES);     // [2][64][LDV / 2] words of two keys
+    const int lane = tid & 63, wave = tid >> 6, l32 = lane & 31, lh = lane >> 5;
+    const int S = p.xa_S;
+#pragma unroll
+    for (int i = 0; i < 3; ++i) {
+      const int c = tid + i * NT, hh = c / (XS * 8), key = (c % (XS * 8)) >> 3, pc = c & 7;
+      *reinterpret_cast<u32x4*>(sK + (hh * XS + key) * LDH + pc * 8) = rk[i];
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int c = tid + j * NT;
+      if (c < VCHUNKS) {
+        const int hh = c / (VCHUNKS / 2), rest = c % (VCHUNKS / 2), v_kp = rest % (XS / 2), v_dch = rest / (XS / 2);
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          const uint32_t a = rv[j][0][w], c2 = rv[j][1][w];
+          sVt[(hh * 64 + v_dch * 8 + 2 * w) * (LDV / 2) + v_kp] = (a & 0xffffu) | (c2 << 16);
+          sVt[(hh * 64 + v_dch * 8 + 2 * w + 1) * (LDV / 2) + v_kp] = (a >> 16) | (c2 & 0xffff0000u);
+        }
+      }
+    }
+    __syncthreads();   // the query tile, K and V^T are in LDS
+
+    const int hh = wave >> 2, qg = wave & 3;
+    bf16x8 qf[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) qf[ks] = *reinterpret_cast<const bf16x8*>(sQ + (qg * 32 + l32) * LDQ + hh * 64 + ks * 16 + lh * 8);
+    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    // S^T tiles: st[kt][v]: key = kt*32 + 8*(v/4) + 4*lh + v%4, query = l32
+    f32x16 st[3];
+#pragma unroll
+    for (int kt = 0; kt < 3; ++kt)
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(sK + (hh * XS + kt * 32 + l32) * LDH + ks * 16 + lh * 8);
+        st[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], ks == 0 ? zero : st[kt], 0, 0, 0);
+      }
+    float mx = -1.0e30f;
+#pragma unroll
+    for (int kt = 0; kt < 3; ++kt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int key = kt * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+        if (key >= S) st[kt][v] = -1.0e30f;
+        mx = fmaxf(mx, st[kt][v]);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float mb = mx * p.xa_scale_log2e;
+    bf16x8 pf[3][2];
+#pragma unroll
+    for (int kt = 0; kt < 3; ++kt)
+#pragma unroll
+      for (int v = 0; v < 16; v += 2) {
+        pf[kt][v >> 3][v & 7] = (bf16_t)__builtin_amdgcn_exp2f(st[kt][v] * p.xa_scale_log2e - mb);
+        pf[kt][v >> 3][(v & 7) + 1] = (bf16_t)__builtin_amdgcn_exp2f(st[kt][v + 1] * p.xa_scale_log2e - mb);
+      }
+    // O^T += V^T . P^T: A fragment row d = dt*32 + l32, element e <-> key kt*32 + 8*(2s + e/4) + 4*lh + e%4
+    const bf16_t one = (bf16_t)1.0f;
+    const bf16x8 ones = {one, one, one, one, one, one, one, one};
+    f32x16 oacc[2] = {zero, zero}, rsum = zero;
+    const bf16_t* sV = reinterpret_cast<const bf16_t*>(sVt);
+#pragma unroll
+    for (int kt = 0; kt < 3; ++kt)
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {
+#pragma unroll
+        for (int dt = 0; dt < 2; ++dt) {
+          const bf16_t* base = sV + (hh * 64 + dt * 32 + l32) * LDV + kt * 32 + 16 * s2 + 4 * lh;
+          const bf16x4 v0 = *reinterpret_cast<const bf16x4*>(base);
+          const bf16x4 v1 = *reinterpret_cast<const bf16x4*>(base + 8);
+          bf16x8 vf;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) { vf[e] = v0[e]; vf[4 + e] = v1[e]; }
+          oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[kt][s2], oacc[dt], 0, 0, 0);
+        }
+        rsum = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pf[kt][s2], rsum, 0, 0, 0);
+      }
+    const float inv = 1.0f / rsum[0];
+    bf16_t* op = p.xa_o + (size_t)(m0 + qg * 32 + l32) * p.xa_ldo + n0 + hh * 64;
+#pragma unroll
+    for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        u32x2 o2;
+        o2[0] = pack_bf16x2(oacc[dt][4 * g + 0] * inv, oacc[dt][4 * g + 1] * inv);
+        o2[1] = pack_bf16x2(oacc[dt][4 * g + 2] * inv, oacc[dt][4 * g + 3] * inv);
+        *reinterpret_cast<u32x2*>(op + dt * 32 + 8 * g + 4 * lh) = o2;
+      }
+  }
+};
+
 // LNF bit 0: the instantiation can fold a LayerNorm in front of the layer into its epilogue (ln_part); bit 1: it can write
 // the row statistics for one behind it (st_part).  The plain one (0) carries none of that code.
-template <class C, bool CONV = false, bool IL = false, int LNF = 0>
+// XA: the output tile is an attention's queries and the epilogue runs the cross-attention on it (XAttnTile).
+template <class C, bool CONV = false, bool IL = false, int LNF = 0, bool XA = false>
 __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const LoraGemmParams pin) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   LoraGemmParams p = pin;
@@ -818,10 +950,20 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
     constexpr int OPR = BN / 16;                                  // GEGLU: output pieces per staged row
     constexpr int GCH = C::WAVES_M * 32 * OPR / C::NT;
     static_assert((C::WAVES_M * 32 * CPR) % C::NT == 0 && (C::WAVES_M * 32 * OPR) % C::NT == 0, "epilogue split");
+    // cross-attention epilogue: this tile's keys and values are requested first and arrive while the tile is staged
+    // (requesting them before the K loop was measured: no faster, and one instantiation then needs scratch memory)
+    XAttnTile<C::LDC> xat;
+    if constexpr (XA) {
+      static_assert(!XA || (BM == 128 && BN == 128 && C::NT == 512 && NRT == 0 && !CONV), "cross-attention epilogue: 128 x 128 tiles");
+      static_assert(!XA || XAttnTile<C::LDC>::LDS_BYTES <= (int)C::LDS_BYTES, "cross-attention epilogue: LDS");
+      xat.load(p, m0, n0, tid);
+    }
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
+      // rows of the staging tile: one 32-row pass per i, or (XA) the whole tile side by side
+      const int srb = XA ? wm * C::WTM + i * 32 : wm * 32;
       u32x4 rr[ECH];
-      if (p.res != nullptr) {
+      if (!XA && p.res != nullptr) {
 #pragma unroll
         for (int q = 0; q < ECH; ++q) {
           const int c = tid + q * C::NT, srow = c / CPR, ch = c % CPR;
@@ -841,7 +983,7 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
             const float c1 = sc1[col], c2 = sc2[col];
 #pragma unroll
             for (int e = 0; e < 4; ++e)
-              sC[(wm * 32 + 8 * g + 4 * lh + e) * C::LDC + col] = (bf16_t)(rs[e] * (acc[i][j][4 * g + e] - mu[e] * c1) + c2);
+              sC[(srb + 8 * g + 4 * lh + e) * C::LDC + col] = (bf16_t)(rs[e] * (acc[i][j][4 * g + e] - mu[e] * c1) + c2);
           }
         }
       } else {
@@ -850,11 +992,12 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
           const int col = wn * C::WTN + j * 32 + l32;
 #pragma unroll
           for (int v = 0; v < 16; ++v) {
-            const int row = wm * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+            const int row = srb + 8 * (v >> 2) + 4 * lh + (v & 3);
             sC[row * C::LDC + col] = (bf16_t)(acc[i][j][v] * oscale + bv[j]);
           }
         }
       }
+      if constexpr (XA) continue;
       __syncthreads();
       if ((LNF & 2) && !p.geglu && p.st_part != nullptr) {
         // as below, and every row's (sum, sum of squares) over this tile's columns for a following folded LayerNorm:
@@ -923,6 +1066,7 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
       }
       __syncthreads();
     }
+    if constexpr (XA) xat.run(smem, p, m0, n0, tid);
     stamp(5);
   }
 }
@@ -954,6 +1098,21 @@ int launch_pcfg(LoraGemmParams p, hipStream_t stream, int n_groups = 1) {
       if (p.xg_n == 0 || cost < best) { best = cost; p.xg_n = gn; p.xr_m = rm; p.xr_n = rn; }
     }
     grid = 8u * (unsigned)p.xr_m * (unsigned)p.xr_n;
+  }
+  if (p.xa_k != nullptr) {   // cross-attention in the epilogue: the 128x128 / 8-wave tiles only
+    if constexpr (std::is_same<C, PCfg<128, 128, 2, 4, 0, 4, 64>>::value && !CONV) {
+      if (n_groups != 1 || p.sg_mode != 0 || p.geglu || p.res != nullptr || p.st_part != nullptr || p.M % 128 != 0 || p.N % 128 != 0)
+        return KH_ERR_UNSUPPORTED;
+      auto go = [&](auto lnf) {
+        constexpr int L = decltype(lnf)::value;
+        if (hipError_t e = kh_allow_lds<lora_gemm_pipe_kernel<C, false, false, L, true>>((int)C::LDS_BYTES + KH_LN_LDS); e != hipSuccess) return (int)e;
+        kh_launch(KH_TAG_LORA_GEMM, lora_gemm_pipe_kernel<C, false, false, L, true>, dim3(grid), dim3(C::NT), C::LDS_BYTES + KH_LN_LDS, stream, p);
+        KH_RETURN_LAST_ERROR();
+      };
+      return p.ln_part != nullptr ? go(std::integral_constant<int, 1>{}) : go(std::integral_constant<int, 0>{});
+    } else {
+      return KH_ERR_UNSUPPORTED;
+    }
   }
   if constexpr (ln_fits) {
     auto go = [&](auto lnf) {
@@ -1054,6 +1213,20 @@ static int launch_il(const LoraGemmParams& pin, hipStream_t stream) {
   const int shr = ((p.M + 63) / 64) * (p.ldt / 64);
   p.il_blocks = (shr + 7) / 8 * 8;
   const unsigned grid = (unsigned)p.il_blocks + 8u * (unsigned)p.xr_m * (unsigned)p.xr_n;
+  if (p.xa_k != nullptr) {
+    if constexpr (std::is_same<C, PCfg<128, 128, 2, 4, 0, 4, 64>>::value) {
+      if (p.res != nullptr || p.st_part != nullptr || p.M % 128 != 0 || p.N % 128 != 0) return KH_ERR_UNSUPPORTED;
+      auto go = [&](auto lnf) {
+        constexpr int L = decltype(lnf)::value;
+        if (hipError_t e = kh_allow_lds<lora_gemm_pipe_kernel<C, false, true, L, true>>(LDS + KH_LN_LDS); e != hipSuccess) return (int)e;
+        kh_launch(KH_TAG_LORA_GEMM, lora_gemm_pipe_kernel<C, false, true, L, true>, dim3(grid), dim3(C::NT), (size_t)LDS + KH_LN_LDS, stream, p);
+        KH_RETURN_LAST_ERROR();
+      };
+      return p.ln_part != nullptr ? go(std::integral_constant<int, 1>{}) : go(std::integral_constant<int, 0>{});
+    } else {
+      return KH_ERR_UNSUPPORTED;
+    }
+  }
   if (p.ln_part != nullptr || p.st_part != nullptr) {
     if (p.st_part != nullptr && p.n_tiles > KH_LN_SLOTS) return KH_ERR_UNSUPPORTED;
     auto go = [&](auto lnf) {
@@ -1077,6 +1250,20 @@ int lora_gemm_pipe_launch_il(const LoraGemmParams& p, hipStream_t stream) {
     case 2: return launch_il<PCfg<256, 128, 4, 2, 0, 3, 64>>(p, stream);
     default: return KH_ERR_UNSUPPORTED;
   }
+}
+
+// A query projection with its cross-attention in the epilogue (LoraGemmParams::xa_k): one round of 128x128 tiles, T either
+// made inside the launch (il_cnt given and the shape suits that form) or given (t_ext with a_cat == NULL), or R == 0.
+bool lora_gemm_pipe_xattn_ok(const LoraGemmParams& p) {
+  const long tiles = (long)(p.M / 128) * (p.N / 128);
+  return p.M % 128 == 0 && p.N % 128 == 0 && tiles <= 256 && deep_stage_ok(p) && p.xa_T > 0 && p.xa_T % 128 == 0 &&
+         p.M % p.xa_T == 0 && p.xa_S >= 1 && p.xa_S <= 96 && !p.geglu && p.res == nullptr && p.st_part == nullptr;
+}
+
+int lora_gemm_pipe_launch_xattn(const LoraGemmParams& p, hipStream_t stream) {
+  if (p.xa_k == nullptr || !lora_gemm_pipe_xattn_ok(p)) return KH_ERR_UNSUPPORTED;
+  if (p.a_cat != nullptr && p.il_cnt != nullptr && il_form(p) == 1) return launch_il<PCfg<128, 128, 2, 4, 0, 4, 64>>(p, stream);
+  return launch_pcfg<PCfg<128, 128, 2, 4, 0, 4, 64>>(p, stream);
 }
 
 int lora_gemm_pipe_launch_conv(const LoraGemmParams& p, hipStream_t stream) {

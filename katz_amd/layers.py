@@ -42,6 +42,11 @@ LORA_SHRINK = os.getenv("KATZ_LORA_SHRINK", "in_launch")
 # LayerNorm as a kernel of its own (for measurements).
 LN_FOLD = os.getenv("KATZ_LN_FOLD", "1") != "0"
 
+# A cross-attention over a short context (the 77 text tokens) runs inside the epilogue of its query projection where the
+# projection's 128 x 128 tiles fill at most one round of CUs (kh_lora_linear_xattn_bf16).  "0": projection, then the
+# attention kernel (for measurements).
+XATTN_FUSE = os.getenv("KATZ_XATTN_FUSE", "1") != "0"
+
 
 class RowStats:
     """Per-row (sum, sum of squares) partials of the current hidden states of a transformer, written by the linear
@@ -261,6 +266,39 @@ class LoRALinear(nn.Module):
             return ops.lora_linear_split(x, w, b, p.a_cat, p.col_scale, p.b_cat, residual=residual, geglu=self.geglu,
                                          two_launches=LORA_SHRINK == "separate", r_used=p.r_used)
         return ops.lora_linear(x, w, b, p.a_cat, p.b_cat, p.col_scale, residual=residual, geglu=self.geglu)
+
+    def forward_attention(self, x: torch.Tensor, k: torch.Tensor, v: torch.Tensor, heads: int, scale: float, ln=None):
+        """This layer as the query projection of an attention over k / v [B,S,heads*64]: softmax(q k^T * scale) v with
+        q = forward(x, ln=ln), in one launch where the kernel takes the shapes (ops.lora_linear_xattn); None otherwise
+        (the caller then runs forward and the attention kernel)."""
+        if not XATTN_FUSE or x.dim() != 3 or not x.is_cuda or x.dtype != torch.bfloat16 or self.geglu:
+            return None
+        self.prepare()
+        _, w, b = self._rt
+        p = self._packed
+        B, T, K = x.shape
+        R = 0 if p is None else p.R
+        if w.dtype != torch.bfloat16 or (p is not None and (p.overflow or LORA_MODE != "split")):
+            return None
+        if k.shape != (B, k.shape[1], self.out_features) or v.shape != k.shape or k.stride(-1) != 1 or v.stride(-1) != 1:
+            return None
+        if not ops.lora_linear_xattn_ok(B * T, self.out_features, K, R, T, k.shape[1], heads):
+            return None
+        a = sc = bc = lnarg = None
+        r_used = 0
+        if p is not None:
+            a, sc, bc, r_used = p.a_cat, p.col_scale, p.b_cat, p.r_used
+        if ln is not None:
+            if ln[1] is not None and ln[1].valid and self.norm_path_ok(x):
+                norm, st = ln
+                w, c1, c2, ap, ca1, ca2 = self._ln_terms(norm)
+                b = None
+                a = ap if p is not None else None
+                lnarg = (st.buf, c1, c2, ca1, ca2, norm.eps)
+            else:
+                x = ln[0](x)
+        return ops.lora_linear_xattn(x, w, k, v, heads, scale, bias=b, a_cat=a, col_scale=sc, b_cat=bc,
+                                     two_launches=LORA_SHRINK == "separate", r_used=r_used, ln=lnarg)
 
     def _forward_wide(self, x, residual, p: PackedAdapters) -> torch.Tensor:
         """More rank columns than one launch takes (sum of the active ranks > 128; peft has no such limit): the first
@@ -683,16 +721,20 @@ class KatzAttnProcessor:
         ctx = hidden_states if encoder_hidden_states is None else encoder_hidden_states
         if qkv is not None:
             q, k, v = qkv  # self-attention: one shrink + one GEMM for the three projections
-        else:
-            q = attn.to_q(hidden_states, ln=ln)
-        if qkv is not None:
-            pass
         elif encoder_hidden_states is not None and attn.ctx_kv is not None and attn.ctx_kv[0] is encoder_hidden_states:
             _, k, v = attn.ctx_kv  # projected for every cross-attention at once at the start of the step
         else:
             k = attn.to_k(ctx)
             v = attn.to_v(ctx)
-        o = ops.attention(q, k, v, attn.heads, attn.scale)
+        o = None
+        if qkv is None:
+            # a short context: the attention runs inside the query projection's launch where the kernel takes the shapes
+            if encoder_hidden_states is not None:
+                o = attn.to_q.forward_attention(hidden_states, k, v, attn.heads, attn.scale, ln=ln)
+            if o is None:
+                q = attn.to_q(hidden_states, ln=ln)
+        if o is None:
+            o = ops.attention(q, k, v, attn.heads, attn.scale)
         o = attn.to_out[0](o, residual=residual, stats_out=stats_out)
         return attn.to_out[1](o)
 

@@ -410,6 +410,76 @@ def lora_linear_norm(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch
     return out
 
 
+def lora_linear_xattn_ok(M: int, N: int, K: int, R: int, T: int, S: int, heads: int) -> bool:
+    """Does lora_linear_xattn take this query projection ([M,K] -> [M,N], adapters' padded rank R) and attention (T queries
+    and S keys per sample, 64-wide heads)?"""
+    return N == heads * 64 and bool(_lib.load().kh_lora_linear_xattn_ok(M, N, K, R, T, S))
+
+
+def lora_linear_xattn(x: torch.Tensor, weight: torch.Tensor, k: torch.Tensor, v: torch.Tensor, heads: int,
+                      scale: Optional[float] = None, bias: Optional[torch.Tensor] = None,
+                      a_cat: Optional[torch.Tensor] = None, col_scale: Optional[torch.Tensor] = None,
+                      b_cat: Optional[torch.Tensor] = None, two_launches: bool = False, r_used: int = 0,
+                      ln=None) -> torch.Tensor:
+    """attention(lora_linear_norm(x, weight, ...), k, v) in one launch (kh_lora_linear_xattn_bf16): the query projection of a
+    cross-attention over a short context (S <= 96) whose 128 x 128 output tiles (128 queries of two heads) go through the
+    attention inside the GEMM's epilogue instead of to memory.  x [B,T,K]; k / v [B,S,heads*64] (last-dim-contiguous
+    views); the other arguments as for lora_linear_norm.  Returns [B,T,heads*64]."""
+    lib = _lib.load()
+    _req(x, BF16, "x"); _req(weight, BF16, "weight")
+    if x.dim() != 3:
+        raise ValueError("x must be [B,T,K]")
+    B, T, K = x.shape
+    N = weight.shape[0]
+    M = B * T
+    S = k.shape[1]
+    if weight.shape[1] != K or N != heads * 64:
+        raise ValueError("weight must be [heads*64, K]")
+    for n, t in (("k", k), ("v", v)):
+        if not t.is_cuda or t.dtype != BF16 or t.stride(-1) != 1 or t.shape != (B, S, N):
+            raise ValueError(f"{n} must be a bfloat16 [B,S,heads*64] GPU tensor with a contiguous last axis")
+    R = 0
+    if a_cat is not None:
+        _req(a_cat, BF16, "a_cat"); _req(b_cat, BF16, "b_cat"); _req(col_scale, torch.float32, "col_scale")
+        R = b_cat.shape[1]
+        if a_cat.shape != (R, K) or b_cat.shape != (N, R) or col_scale.shape != (R,):
+            raise ValueError("a_cat / b_cat / col_scale do not match x and weight")
+    if bias is not None:
+        _req(bias, BF16, "bias")
+    part = c1 = c2 = ca1 = ca2 = None
+    eps = 0.0
+    if ln is not None:
+        part, c1, c2, ca1, ca2, eps = ln
+        if bias is not None:
+            raise ValueError("with a folded LayerNorm the bias belongs into c2")
+        for t_, n_, name in ((c1, N, "c1"), (c2, N, "c2")) + (((ca1, R, "ca1"), (ca2, R, "ca2")) if R else ()):
+            _req(t_, torch.float32, name)
+            if t_.numel() != n_:
+                raise ValueError(f"{name} must have {n_} elements")
+        _req(part, torch.float32, "ln part")
+        if part.numel() != M * LN_SLOTS * 2:
+            raise ValueError("ln part must be a row_stats_buffer for the rows of x")
+    if scale is None:
+        scale = 1.0 / 8.0
+    out = torch.empty((B, T, N), dtype=BF16, device=x.device)
+    t = cnt = None
+    if R:
+        t = torch.empty((M, R), dtype=BF16, device=x.device)
+        cnt = _split_counters(x.device, M)
+    flags = ((1 if two_launches else 0) << 8) | (_r_used_bits(r_used, R) << 16 if R else 0)
+    if CALL_LOG is not None:   # one entry per kernel launch
+        if R and lib.kh_lora_linear_split_launches(M, N, K, R, 0, flags) == 2:
+            CALL_LOG.append(("lora_shrink", M, K, R))
+        CALL_LOG.append(("lora_linear_xattn", M, N, K, R, heads, T, S))
+    _weight_prefetch_hint(weight, a_cat, b_cat)
+    rc = lib.kh_lora_linear_xattn_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(a_cat), _ptr(col_scale), _ptr(b_cat), _ptr(t),
+                                       _ptr(cnt), _ptr(part), _ptr(c1), _ptr(c2), _ptr(ca1), _ptr(ca2), float(eps),
+                                       _ptr(k), _ptr(v), _ptr(out), M, N, K, R, T, S, k.stride(1), v.stride(1), out.stride(1),
+                                       k.stride(0), v.stride(0), float(scale), flags, _stream())
+    _lib.check(rc, "kh_lora_linear_xattn_bf16")
+    return out
+
+
 def lora_merge_grouped(weights: Sequence[torch.Tensor], ups: Sequence[torch.Tensor], downs: Sequence[torch.Tensor],
                        scale: float = 1.0, layer_scales: Optional[Sequence[float]] = None) -> None:
     """W_l += scale * layer_scales[l] * up_l @ down_l for all layers in ONE launch, in place (kh_lora_merge_grouped_bf16).
