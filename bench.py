@@ -321,6 +321,14 @@ def kernel_probe():
         q, k, v = rn(B, T, H * 64), rn(B, S, H * 64), rn(B, S, H * 64)
         add(f"attention B{B} H{H} T{T} S{S}", lambda q=q, k=k, v=v, H=H: ops.attention(q, k, v, H),
             4.0 * B * H * T * S * 64, 2.0 * 64 * B * H * (2 * T + 2 * S))
+    # K3b: the text cross-attention of the 32x32 level inside its query projection's launch (adapters: shrink in launch)
+    B, H, T, S, K, R = 2, 20, 1024, 77, 1280, 128
+    xq, wq, kx, vx = rn(B, T, K), rn(H * 64, K, std=0.02), rn(B, S, H * 64), rn(B, S, H * 64)
+    aq, bq, sq = rn(R, K, std=0.02), rn(H * 64, R, std=0.02), torch.full((R,), 0.8, device=dev)
+    add(f"lora_linear_xattn M{B * T} K{K} N{H * 64} R{R} S{S} (to_q + attention)",
+        lambda: ops.lora_linear_xattn(xq, wq, kx, vx, H, a_cat=aq, col_scale=sq, b_cat=bq),
+        2.0 * B * T * H * 64 * (K + R) + 2.0 * B * T * K * R + 4.0 * B * H * T * S * 64,
+        2.0 * (B * T * K + K * H * 64 + B * T * H * 64 + R * H * 64 + R * K + 2 * B * S * H * 64))
     # K2: segmented shrink / expand, 8 requests x 4096 tokens, d = 640, one adapter each (ranks 8 .. 128)
     T, dm, RP = 4096, 640, 128
     ranks = [64, 8, 128, 32, 16, 64, 128, 32]
@@ -340,6 +348,9 @@ def kernel_probe():
         2.0 * (8 * T * dm + sr * dm + T * sr))
     add("sgmv_expand 8x4096x640", lambda: ops.sgmv_expand_(y, tb, b_all, ss, sa, rp, sc, T), 2.0 * T * dm * sr,
         2.0 * (T * sr + sr * dm + 2 * 8 * T * dm))
+    y2 = rn(8 * T, dm)
+    add("sgmv_fused 8x4096x640", lambda: ops.sgmv_fused_(y2, x, a_all, b_all, ss, sa, rp, sc, T), 4.0 * T * dm * sr,
+        2.0 * (8 * T * dm + sr * dm + sr * dm + 2 * 8 * T * dm))
     # K4 / K5: norms and the ControlNet residual injection
     xg, gam, bet = cl(rn(2, 320, 128, 128)), rn(320), rn(320)
     add("group_norm+silu 2x320x128x128 nhwc", lambda: ops.group_norm(xg, 32, gam, bet, 1e-5, "silu"), 0.0, 4.0 * xg.numel())
