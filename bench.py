@@ -641,6 +641,20 @@ def main():
         assert len(durs) == per_call * len(calls), (call_name, len(durs), len(calls))
         return [(sum(durs[i * per_call:(i + 1) * per_call]), work_of(c), c) for i, c in enumerate(calls)]
 
+    def gn_rows():
+        """GroupNorm calls in call order: a full call owns the next statistics and the next apply launch, a call whose
+        statistics came out of a convolution's epilogue owns the next apply launch only."""
+        st = iter([d for n, d in launches if n == "group_norm_stats"])
+        ap = iter([d for n, d in launches if n == "group_norm_apply"])
+        rows = []
+        for c in log:
+            if c[0] == "group_norm":
+                rows.append((next(st) + next(ap), 4.0 * c[1] * c[2] * c[3], c))
+            elif c[0] == "group_norm_apply":
+                rows.append((next(ap), 4.0 * c[1] * c[2] * c[3], c))
+        assert next(st, None) is None and next(ap, None) is None
+        return rows
+
     def roofline_rows(name, bound, rows, key_of):
         peak, unit, scale = (PEAK_BF16_TFLOPS, "TFLOP/s", 1e12) if bound == "mfma" else (PEAK_HBM_GBS, "GB/s", 1e9)
         tot_ms = sum(r[0] for r in rows)
@@ -663,9 +677,9 @@ def main():
         roofline_rows("conv3x3 implicit GEMM (kh_conv3x3_nhwc_bf16)", "mfma",
                       pair(("conv3x3",), "conv3x3", lambda c: 2.0 * c[1] * c[2] * c[3]),
                       lambda c: f"M{c[1]} Cout{c[2]} K{c[3]} stride{c[4]}"),
-        roofline_rows("GroupNorm(+SiLU), statistics + apply launches (kh_group_norm_bf16); bytes = one read + one write",
-                      "hbm", pair(("group_norm_stats", "group_norm_apply"), "group_norm", lambda c: 4.0 * c[1] * c[2] * c[3]),
-                      lambda c: f"N{c[1]} C{c[2]} HW{c[3]}"),
+        roofline_rows("GroupNorm(+SiLU): statistics + apply launches (kh_group_norm_bf16), or the apply launch alone where the "
+                      "convolution in front left the statistics (kh_group_norm_apply_bf16); bytes = one read + one write",
+                      "hbm", gn_rows(), lambda c: f"N{c[1]} C{c[2]} HW{c[3]}" + (" (apply only)" if c[0] == "group_norm_apply" else "")),
         roofline_rows("LayerNorm (kh_layer_norm_bf16)", "hbm",
                       pair(("layer_norm",), "layer_norm", lambda c: 4.0 * c[1] * c[2]), lambda c: f"M{c[1]} D{c[2]}"),
         roofline_rows("ControlNet residual injection folded into the up-block concat (kh_concat_residual_bf16)", "hbm",

@@ -69,6 +69,12 @@ struct LoraGemmParams {
   int xa_S = 0, xa_T = 0;
   long xa_ldk = 0, xa_ldv = 0, xa_ldo = 0, xa_bsk = 0, xa_bsv = 0;
   float xa_scale_log2e = 0.f;
+  // GroupNorm statistics of a convolution's result as a by-product of its epilogue (gn_part != nullptr; 3x3 convolutions on
+  // the 160-column tiles): a tile holds whole groups of gn_cg channels of BM pixels of one image (gn_hw pixels each), and
+  // its workgroup writes their (sum, sum of squares) over conv + gn_add[image][c] to gn_part[image][group][row tile of
+  // the image][2] -- the layout kh_group_norm_bf16's second pass folds.
+  float* gn_part = nullptr; const bf16_t* gn_add = nullptr;
+  int gn_cg = 0, gn_hw = 0;
   const void* pf[3] = {nullptr, nullptr, nullptr};   // up to three ranges: weights, A_cat, B_cat of that launch
   uint32_t pf_lines[3] = {0, 0, 0};
 };
@@ -199,6 +205,9 @@ bool lora_gemm_ksplit_ok(const LoraGemmParams& p);
 int lora_gemm_ksplit_launch(const LoraGemmParams& p, int row_groups, hipStream_t stream);
 bool lora_gemm_ksplit_conv_ok(const LoraGemmParams& p);
 int lora_gemm_ksplit_launch_conv(const LoraGemmParams& p, int row_groups, hipStream_t stream);
+// the convolution that also leaves GroupNorm statistics (gn_cg / gn_hw set): row groups of the 160-column tiles it would run
+// on, 0 when the rules give it other tiles or the groups do not fit them
+int lora_gemm_conv_gn_row_groups(const LoraGemmParams& p);
 // Wide-tile variant (lora_gemm_wide.hip): 256 x 320 tiles, 8 waves; plain or K-extended GEMM with bias / residual /
 // GEGLU; M % 256 == 0, N % 320 == 0, K % 64 == 0.
 bool lora_gemm_wide_ok(const LoraGemmParams& p);

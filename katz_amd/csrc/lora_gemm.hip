@@ -715,9 +715,9 @@ KH_EXPORT int kh_lora_linear_xattn_ok(int64_t M, int64_t N, int64_t K, int64_t R
 }
 
 // 3x3 convolution, padding 1, NHWC, as an implicit GEMM on the pipelined kernel; see include/katz_hip.h.
-KH_EXPORT int kh_conv3x3_nhwc_bf16(const void* x, const void* w, const void* bias, const void* residual, void* y,
-                                   int64_t Nb, int64_t H, int64_t W, int64_t Cin, int64_t Cout, int64_t stride,
-                                   void* stream) {
+namespace {
+int conv3x3_params(LoraGemmParams& p, const void* x, const void* w, const void* bias, const void* residual, void* y, int64_t Nb,
+                   int64_t H, int64_t W, int64_t Cin, int64_t Cout, int64_t stride) {
   if (!x || !w || !y || Nb <= 0 || H <= 0 || W <= 0 || Cin <= 0 || Cout <= 0) return KH_ERR_INVALID_ARG;
   if (stride != 1 && stride != 2) return KH_ERR_UNSUPPORTED;
   if (Cin % 32 != 0 || Cout % 8 != 0) return KH_ERR_UNSUPPORTED;
@@ -726,7 +726,6 @@ KH_EXPORT int kh_conv3x3_nhwc_bf16(const void* x, const void* w, const void* bia
   if (M > (1 << 24) || Cout > (1 << 24) || 9 * Cin > (1 << 24) || Nb * H * W * Cin >= ((int64_t)1 << 40)) return KH_ERR_TOO_LARGE;
   if (!kh_aligned16(x) || !kh_aligned16(w) || !kh_aligned16(y) || (residual && !kh_aligned16(residual)))
     return KH_ERR_ALIGNMENT;
-  LoraGemmParams p;
   p.x = (const bf16_t*)x; p.w = (const bf16_t*)w; p.bias = (const bf16_t*)bias;
   p.a_cat = nullptr; p.b_cat = nullptr; p.col_scale = nullptr;
   p.t_ext = nullptr; p.ldt = 0; p.grp = nullptr; p.dbg = 0; p.t_nsplit = 0;
@@ -738,6 +737,39 @@ KH_EXPORT int kh_conv3x3_nhwc_bf16(const void* x, const void* w, const void* bia
   p.sg_start = p.sg_adapter = p.sg_rank = nullptr; p.sg_scale = nullptr; p.sg_mode = 0; p.sg_wstride = 0;
   p.conv_cin = (int)Cin; p.conv_h = (int)H; p.conv_w = (int)W; p.conv_ho = (int)Ho; p.conv_wo = (int)Wo;
   p.conv_stride = (int)stride;
+  return KH_OK;
+}
+}  // namespace
+
+KH_EXPORT int kh_conv3x3_nhwc_bf16(const void* x, const void* w, const void* bias, const void* residual, void* y,
+                                   int64_t Nb, int64_t H, int64_t W, int64_t Cin, int64_t Cout, int64_t stride,
+                                   void* stream) {
+  LoraGemmParams p;
+  if (const int rc = conv3x3_params(p, x, w, bias, residual, y, Nb, H, W, Cin, Cout, stride); rc != KH_OK) return rc;
+  kh_take_weight_prefetch(p);
+  return lora_gemm_pipe_launch_conv(p, (hipStream_t)stream);
+}
+
+// See include/katz_hip.h: row tiles per image of the statistics the convolution leaves, 0 when the shape is not taken.
+KH_EXPORT int64_t kh_conv3x3_gn_splits(int64_t Nb, int64_t H, int64_t W, int64_t Cin, int64_t Cout, int64_t stride, int64_t G) {
+  static const char dummy[16] __attribute__((aligned(16))) = {0};
+  LoraGemmParams p;
+  if (G <= 0 || Cout % G != 0) return 0;
+  if (conv3x3_params(p, dummy, dummy, nullptr, nullptr, const_cast<char*>(dummy), Nb, H, W, Cin, Cout, stride) != KH_OK) return 0;
+  p.gn_cg = (int)(Cout / G); p.gn_hw = p.conv_ho * p.conv_wo;
+  const int rg = lora_gemm_conv_gn_row_groups(p);
+  return rg == 0 ? 0 : p.gn_hw / (32 * rg);
+}
+
+KH_EXPORT int kh_conv3x3_gn_stats_nhwc_bf16(const void* x, const void* w, const void* bias, const void* add_nc, void* y,
+                                            float* partials, int64_t Nb, int64_t H, int64_t W, int64_t Cin, int64_t Cout,
+                                            int64_t stride, int64_t G, void* stream) {
+  if (!partials || G <= 0 || Cout % G != 0) return KH_ERR_INVALID_ARG;
+  LoraGemmParams p;
+  if (const int rc = conv3x3_params(p, x, w, bias, nullptr, y, Nb, H, W, Cin, Cout, stride); rc != KH_OK) return rc;
+  p.gn_cg = (int)(Cout / G); p.gn_hw = p.conv_ho * p.conv_wo;
+  if (lora_gemm_conv_gn_row_groups(p) == 0) return KH_ERR_UNSUPPORTED;
+  p.gn_part = partials; p.gn_add = (const bf16_t*)add_nc;
   kh_take_weight_prefetch(p);
   return lora_gemm_pipe_launch_conv(p, (hipStream_t)stream);
 }

@@ -58,7 +58,8 @@ __device__ __attribute__((aligned(256))) const uint32_t ks_zero_page[64] = {0};
 // ordered (kh, kw, ci), see lora_gemm_pipe.hip): a stage of 64 K columns is 64 channels of one tap, the x rows of tap
 // (kh, kw) sit (kh * W + kw) * Cin elements after the row's base (the pixel above-left of its window), and rows
 // whose tap falls outside the image read zeros.
-template <class C, bool CONV>
+// GNF: the epilogue also leaves the GroupNorm statistics of the result (LoraGemmParams::gn_part).
+template <class C, bool CONV, bool GNF = false>
 __global__ __launch_bounds__(512, 2) void lora_gemm_ksplit_kernel(const LoraGemmParams p) {
 #if __HIP_DEVICE_COMPILE__   // the host pass only needs the kernel's symbol (it cannot lower the buffer-resource type)
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -354,6 +355,55 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_ksplit_kernel(const LoraGemm
     }
   }
   __syncthreads();
+  if constexpr (GNF) {
+    // GroupNorm statistics as a by-product: the staged tile is BM pixels of one image times BN / gn_cg whole groups; their
+    // (sum, sum of squares) over the bf16-rounded values plus the per-(image, channel) term -- what a GroupNorm kernel
+    // reading the stored result would take -- go to gn_part[image][group][row tile of the image].  Three short passes,
+    // sums in fixed orders (deterministic); the tile itself is stored below as usual.
+    constexpr int PCS = BN / 8, RP = 512 / PCS;               // 16-byte pieces per row, row parts (25 of 20 threads)
+    float* colp = reinterpret_cast<float*>(smem);             // [RP][BN][2]: the partial strips are dead
+    float* cols = colp + RP * BN * 2;                         // [BN][2] column sums
+    static_assert((RP * BN * 2 + BN * 2) * 4 <= C::PART, "column sums fit the dead partial strips");
+    const int cg = p.gn_cg, ng = BN / cg, G = N / cg;
+    const int n_img = m0 / p.gn_hw, split = (m0 % p.gn_hw) / BM, splits = p.gn_hw / BM;
+    // the per-(image, channel) term enters through sum(a + t) = sum(a) + n t and sum((a + t)^2) = sum(a^2) + 2 t sum(a) + n t^2:
+    // requested now, used after the first pass
+    const float ad = (tid < BN && p.gn_add != nullptr) ? (float)p.gn_add[(size_t)n_img * N + n0 + tid] : 0.f;
+    if (tid < RP * PCS) {
+      const int ch = tid % PCS, part = tid / PCS;
+      float cs[8], cq[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) cs[e] = cq[e] = 0.f;
+#pragma unroll
+      for (int i = 0; i < (BM + RP - 1) / RP; ++i) {
+        const int r = part + i * RP;
+        if (r < BM) {
+          const u32x4 v = *reinterpret_cast<const u32x4*>(sC + r * C::LDC + ch * 8);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float a = bf16_lo(v[e]), b2 = bf16_hi(v[e]);
+            cs[2 * e] += a; cq[2 * e] = fmaf(a, a, cq[2 * e]);
+            cs[2 * e + 1] += b2; cq[2 * e + 1] = fmaf(b2, b2, cq[2 * e + 1]);
+          }
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) *reinterpret_cast<f32x2*>(colp + ((part * BN) + ch * 8 + e) * 2) = f32x2{cs[e], cq[e]};
+    }
+    __syncthreads();
+    if (tid < BN) {
+      float s = 0.f, q = 0.f;
+#pragma unroll
+      for (int part = 0; part < RP; ++part) { const f32x2 v = *reinterpret_cast<const f32x2*>(colp + (part * BN + tid) * 2); s += v[0]; q += v[1]; }
+      *reinterpret_cast<f32x2*>(cols + tid * 2) = f32x2{s + (float)BM * ad, q + 2.f * ad * s + (float)BM * ad * ad};
+    }
+    __syncthreads();
+    if (tid < ng) {
+      float s = 0.f, q = 0.f;
+      for (int c = tid * cg; c < (tid + 1) * cg; ++c) { s += cols[2 * c]; q += cols[2 * c + 1]; }
+      *reinterpret_cast<f32x2*>(p.gn_part + (((size_t)n_img * G + n0 / cg + tid) * splits + split) * 2) = f32x2{s, q};
+    }
+  }
   if (p.st_part != nullptr) {
     // as below, and every row's (sum, sum of squares) over this tile's columns for a following folded LayerNorm: the 20
     // pieces of a row meet in LDS (the partial strips are dead) and are added in a fixed order
@@ -401,12 +451,12 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_ksplit_kernel(const LoraGemm
 #endif
 }
 
-template <class C, bool CONV = false>
+template <class C, bool CONV = false, bool GNF = false>
 int launch_ksplit(LoraGemmParams p, hipStream_t stream) {
   p.m_tiles = (p.M + C::BM - 1) / C::BM;
   p.n_tiles = (p.N + C::BN - 1) / C::BN;
   static_assert(C::LDS + KH_LN_LDS <= 160 * 1024, "LDS budget with the row statistics");
-  if (hipError_t e = kh_allow_lds<lora_gemm_ksplit_kernel<C, CONV>>(C::LDS + KH_LN_LDS); e != hipSuccess) return (int)e;
+  if (hipError_t e = kh_allow_lds<lora_gemm_ksplit_kernel<C, CONV, GNF>>(C::LDS + KH_LN_LDS); e != hipSuccess) return (int)e;
   if ((p.ln_part != nullptr || p.st_part != nullptr) && CONV) return KH_ERR_UNSUPPORTED;
   if (p.st_part != nullptr && p.n_tiles > KH_LN_SLOTS) return KH_ERR_UNSUPPORTED;
   p.ln_lds = C::LDS;
@@ -421,7 +471,13 @@ int launch_ksplit(LoraGemmParams p, hipStream_t stream) {
     if (p.xg_n == 0 || cost < best) { best = cost; p.xg_n = gn; p.xr_m = rm; p.xr_n = rn; }
   }
   const unsigned grid = 8u * (unsigned)p.xr_m * (unsigned)p.xr_n;
-  kh_launch(CONV ? KH_TAG_CONV : KH_TAG_LORA_GEMM, lora_gemm_ksplit_kernel<C, CONV>, dim3(grid), dim3(512), lds, stream, p);
+  if constexpr (GNF) {
+    // whole groups per tile, whole tiles per image, no residual (the statistics are taken before it would be added)
+    if (p.res != nullptr || p.st_part != nullptr || p.gn_cg <= 0 || C::BN % p.gn_cg != 0 || p.N % C::BN != 0 || p.gn_hw % C::BM != 0 ||
+        p.M % p.gn_hw != 0)
+      return KH_ERR_UNSUPPORTED;
+  }
+  kh_launch(CONV ? KH_TAG_CONV : KH_TAG_LORA_GEMM, lora_gemm_ksplit_kernel<C, CONV, GNF>, dim3(grid), dim3(512), lds, stream, p);
   KH_RETURN_LAST_ERROR();
 }
 
@@ -455,5 +511,6 @@ bool lora_gemm_ksplit_conv_ok(const LoraGemmParams& p) {
 
 int lora_gemm_ksplit_launch_conv(const LoraGemmParams& p, int row_groups, hipStream_t stream) {
   if (!lora_gemm_ksplit_conv_ok(p)) return KH_ERR_UNSUPPORTED;
+  if (p.gn_part != nullptr) return row_groups == 4 ? launch_ksplit<KCfg<4>, true, true>(p, stream) : launch_ksplit<KCfg<2>, true, true>(p, stream);
   return row_groups == 4 ? launch_ksplit<KCfg<4>, true>(p, stream) : launch_ksplit<KCfg<2>, true>(p, stream);
 }

@@ -1266,7 +1266,24 @@ int lora_gemm_pipe_launch_xattn(const LoraGemmParams& p, hipStream_t stream) {
   return launch_pcfg<PCfg<128, 128, 2, 4, 0, 4, 64>>(p, stream);
 }
 
+// The 160-column tiles the rules below give this convolution, when the GroupNorm statistics of its result can be a
+// by-product of its epilogue: whole tiles per image, whole groups per tile, no residual.
+int lora_gemm_conv_gn_row_groups(const LoraGemmParams& p) {
+  if (p.N % 160 != 0 || !lora_gemm_ksplit_conv_ok(p) || p.res != nullptr || p.gn_cg <= 0 || 160 % p.gn_cg != 0 || p.gn_hw <= 0 || p.M % p.gn_hw != 0)
+    return 0;
+  const long tiles = (long)((p.M + 127) / 128) * ((p.N + 127) / 128);
+  const long n160 = p.N / 160, m128 = (p.M + 127) / 128, m64 = (p.M + 63) / 64;
+  int rg = 0;
+  if ((tiles > 256 && tiles <= 384 && m128 * n160 <= 256) || (p.N % 128 != 0 && (m128 * n160) % 256 == 0)) rg = 4;
+  else if (tiles <= 192 && m64 * n160 <= 256 && m64 * n160 > tiles && p.K >= 2560) rg = 2;
+  return (rg == 0 || p.gn_hw % (32 * rg) != 0) ? 0 : rg;
+}
+
 int lora_gemm_pipe_launch_conv(const LoraGemmParams& p, hipStream_t stream) {
+  if (p.gn_part != nullptr) {   // the caller has asked lora_gemm_conv_gn_row_groups
+    const int rg = lora_gemm_conv_gn_row_groups(p);
+    return rg == 0 ? KH_ERR_UNSUPPORTED : lora_gemm_ksplit_launch_conv(p, rg, stream);
+  }
   const long tiles = (long)((p.M + 127) / 128) * ((p.N + 127) / 128);
   // 160-column tiles (lora_gemm_ksplit.hip) by the rules of the linear layers
   if (p.N % 160 == 0 && lora_gemm_ksplit_conv_ok(p)) {

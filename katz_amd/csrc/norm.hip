@@ -429,6 +429,38 @@ KH_EXPORT int kh_group_norm_bf16(const void* x, void* y, const void* gamma, cons
   KH_RETURN_LAST_ERROR();
 }
 
+// Second pass alone, on statistics some other kernel has left (kh_conv3x3_gn_stats_nhwc_bf16); see include/katz_hip.h.
+KH_EXPORT int kh_group_norm_apply_bf16(const void* x, void* y, const void* gamma, const void* beta, const void* add_nc,
+                                       const float* partials, int64_t splits, int64_t N, int64_t C, int64_t HW, int64_t G,
+                                       float eps, int activation, void* stream) {
+  if (!x || !y || !partials || splits <= 0 || N <= 0 || C <= 0 || HW <= 0 || G <= 0 || C % G != 0) return KH_ERR_INVALID_ARG;
+  if (activation != 0 && activation != 1) return KH_ERR_INVALID_ARG;
+  if (!kh_aligned16(x) || !kh_aligned16(y) || (gamma && !kh_aligned16(gamma)) || (beta && !kh_aligned16(beta)) ||
+      (add_nc && !kh_aligned16(add_nc)) || ((uintptr_t)partials & 7) != 0)
+    return KH_ERR_ALIGNMENT;
+  if (N > 65535 || splits > (1 << 20)) return KH_ERR_TOO_LARGE;
+  if (C % 8 != 0 || C > GN_MAX_C || G > 512) return KH_ERR_UNSUPPORTED;
+  GnGeom g;
+  g.N = (int)N; g.C = (int)C; g.HW = (int)HW; g.G = (int)G; g.Cg = (int)(C / G);
+  g.splits = (int)splits;
+  g.CP = (int)(C / 8);
+  int ntx = g.CP < GN_THREADS ? g.CP : GN_THREADS;
+  while (g.CP % ntx != 0) --ntx;
+  g.NTX = ntx; g.CPT = g.CP / ntx; g.PL = GN_THREADS / ntx;
+  if (g.CPT > GN_MAX_CPT) return KH_ERR_UNSUPPORTED;
+  g.asplits = gn_apply_splits_nhwc(N, HW);
+  const dim3 agrid((unsigned)g.asplits, (unsigned)N);
+  hipStream_t s = (hipStream_t)stream;
+  const bf16_t* xp = (const bf16_t*)x; bf16_t* yp = (bf16_t*)y;
+  const bf16_t* gp = (const bf16_t*)gamma; const bf16_t* bp = (const bf16_t*)beta; const bf16_t* ap = (const bf16_t*)add_nc;
+  if (activation == 1)
+    kh_launch(KH_TAG_GN_APPLY, gn_apply_nhwc<true>, agrid, dim3(GN_THREADS), 0, s, xp, yp, gp, bp, ap, partials, g, eps);
+  else
+    kh_launch(KH_TAG_GN_APPLY, gn_apply_nhwc<false>, agrid, dim3(GN_THREADS), 0, s, xp, yp, gp, bp, ap, partials, g, eps);
+  KH_RETURN_LAST_ERROR();
+}
+
+
 // Device address of `scratch` on the current device, resolved once per device.
 static int gn_static_workspace(float** out) {
   constexpr int MAX_DEV = 64;

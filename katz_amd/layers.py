@@ -47,6 +47,11 @@ LN_FOLD = os.getenv("KATZ_LN_FOLD", "1") != "0"
 # attention kernel (for measurements).
 XATTN_FUSE = os.getenv("KATZ_XATTN_FUSE", "1") != "0"
 
+# conv1 of a residual block leaves the statistics of the GroupNorm behind it as a by-product of its epilogue
+# (kh_conv3x3_gn_stats_nhwc_bf16), so that norm is one launch instead of two.  "0": convolution, then the norm's two
+# launches (for measurements).
+CONV_GN_FUSE = os.getenv("KATZ_CONV_GN_FUSE", "1") != "0"
+
 
 class RowStats:
     """Per-row (sum, sum of squares) partials of the current hidden states of a transformer, written by the linear
@@ -501,6 +506,28 @@ class Conv3x3(_ConvLoRAFuse, nn.Conv2d):
             self._packed = (w.data_ptr(), w._version, ops.pack_conv3x3_weight(wp), b)
         return self._packed[2], self._packed[3]
 
+    def forward_norm(self, x, norm: "GroupNorm", add_nc=None):
+        """norm(self(x), add_nc=add_nc) with the norm's statistics taken in the convolution's epilogue where the kernel takes
+        the shape (ops.conv3x3_group_norm); None otherwise (the caller then runs the two modules one after the other)."""
+        if not (CONV_GN_FUSE and x.is_cuda and x.dtype == torch.bfloat16 and self.weight.dtype == torch.bfloat16
+                and self.padding == (1, 1) and self.in_channels % 32 == 0 and self.out_channels % 8 == 0
+                and norm.activation in ("none", "silu") and norm.num_channels == self.out_channels):
+            return None
+        if self.adapters and self._lora_pack()[0] is not None:
+            return None   # the low-rank branch adds to the convolution's result before the norm
+        if add_nc is not None and (add_nc.dtype != torch.bfloat16 or add_nc.numel() != x.shape[0] * self.out_channels):
+            return None
+        if ops.conv3x3_gn_splits(x, self.out_channels, norm.num_groups, self.stride[0]) == 0:
+            return None
+        x = x.contiguous(memory_format=torch.channels_last)
+        w_packed, b_packed = self.packed_weight()
+        w, b = norm.weight, norm.bias
+        if w is not None and w.dtype != torch.bfloat16:
+            return None
+        return ops.conv3x3_group_norm(x, w_packed, b_packed, norm.num_groups, None if w is None else w.detach(),
+                                      None if b is None else b.detach(), norm.eps, norm.activation,
+                                      add_nc=None if add_nc is None else add_nc.contiguous(), stride=self.stride[0])
+
     def forward(self, x, residual=None):
         native = (x.is_cuda and x.dtype == torch.bfloat16 and self.weight.dtype == torch.bfloat16 and self.padding == (1, 1))
         a_cat, b_cat = self._lora_pack() if self.adapters else (None, None)
@@ -656,10 +683,12 @@ class ResnetBlock2D(nn.Module):
     def forward(self, input_tensor, temb_act):
         """temb_act = silu(temb), computed once per step by the caller."""
         h = self.norm_silu1(input_tensor)
-        h = self.conv1(h)
-        # hidden_states + temb[:, :, None, None] rides inside the second norm (no separate pass)
+        # hidden_states + temb[:, :, None, None] rides inside the second norm (no separate pass), and where the kernel takes
+        # the shape conv1's epilogue leaves that norm's statistics
         tp, self.temb_proj = self.temb_proj, None
-        h = self.norm_silu2[0](h, add_nc=self.time_emb_proj(temb_act) if tp is None else tp)
+        add = self.time_emb_proj(temb_act) if tp is None else tp
+        fused = self.conv1.forward_norm(h, self.norm_silu2[0], add)
+        h = fused if fused is not None else self.norm_silu2[0](self.conv1(h), add_nc=add)
         if self.conv_shortcut is not None:
             input_tensor = self.conv_shortcut(input_tensor)
         out = self.conv2(h, residual=input_tensor)   # input_tensor + conv2(h), the add in the conv's epilogue

@@ -273,7 +273,11 @@ def check_split_timeouts(device=None) -> None:
 
 
 def _split_counters(device, M: int) -> torch.Tensor:
-    n = (M + 127) // 128 + 1   # KH_SPLIT_COUNTER_INTS(M)
+    return _arena_ints(device, (M + 127) // 128 + 1)   # KH_SPLIT_COUNTER_INTS(M)
+
+
+def _arena_ints(device, n: int) -> torch.Tensor:
+    """n zeroed int32 of the device's counter arena (zero since the last split_counters_reset)."""
     st = _arena(device)
     if st[1] + n > SPLIT_ARENA_INTS:
         split_counters_reset(device)
@@ -811,6 +815,58 @@ def conv3x3(x: torch.Tensor, w_packed: torch.Tensor, bias: Optional[torch.Tensor
     rc = lib.kh_conv3x3_nhwc_bf16(_ptr(x), _ptr(w_packed), _ptr(bias), _ptr(residual), _ptr(out), Nb, H, W, Cin, Cout,
                                   stride, _stream())
     _lib.check(rc, "kh_conv3x3_nhwc_bf16")
+    return out
+
+
+def conv3x3_gn_splits(x: torch.Tensor, cout: int, num_groups: int, stride: int = 1) -> int:
+    """Row tiles per image of the GroupNorm statistics conv3x3_group_norm's convolution leaves for this input and output
+    width, 0 when the shape is not taken (then: conv3x3 followed by group_norm)."""
+    if not x.is_cuda or x.dtype != BF16 or x.dim() != 4:
+        return 0
+    Nb, Cin, H, W = x.shape
+    return int(_lib.load().kh_conv3x3_gn_splits(Nb, H, W, Cin, cout, stride, num_groups))
+
+
+def conv3x3_group_norm(x: torch.Tensor, w_packed: torch.Tensor, bias: Optional[torch.Tensor], num_groups: int,
+                       gamma: Optional[torch.Tensor], beta: Optional[torch.Tensor], eps: float = 1e-5,
+                       activation: str = "none", add_nc: Optional[torch.Tensor] = None, stride: int = 1) -> torch.Tensor:
+    """group_norm(conv3x3(x, w_packed, bias), num_groups, gamma, beta, eps, activation, add_nc=add_nc) in two launches
+    instead of three: the convolution leaves the norm's statistics as a by-product of its epilogue
+    (kh_conv3x3_gn_stats_nhwc_bf16), the norm's second pass alone follows (kh_group_norm_apply_bf16).  Only for shapes with
+    conv3x3_gn_splits(...) > 0."""
+    lib = _lib.load()
+    if not x.is_cuda or x.dtype != BF16 or x.dim() != 4 or not x.is_contiguous(memory_format=torch.channels_last):
+        raise ValueError("x must be a channels_last bfloat16 GPU tensor")
+    if activation not in ("none", "silu"):
+        raise ValueError(f"unknown activation {activation!r}")
+    Nb, Cin, H, W = x.shape
+    Cout = w_packed.shape[0]
+    if w_packed.shape != (Cout, 3, 3, Cin) or not w_packed.is_contiguous() or w_packed.dtype != BF16:
+        raise ValueError("w_packed must be a contiguous bfloat16 [Cout,3,3,Cin] tensor")
+    for t_, name in ((bias, "bias"), (gamma, "gamma"), (beta, "beta")):
+        if t_ is not None and (t_.shape != (Cout,) or t_.dtype != BF16 or not t_.is_contiguous()):
+            raise ValueError(f"{name} must be a contiguous bfloat16 [Cout] tensor")
+    if add_nc is not None:
+        add_nc = add_nc.reshape(Nb, Cout)
+        if add_nc.dtype != BF16 or not add_nc.is_contiguous():
+            raise ValueError("add_nc must be a contiguous bfloat16 [N,Cout] tensor")
+    splits = int(lib.kh_conv3x3_gn_splits(Nb, H, W, Cin, Cout, stride, num_groups))
+    if splits == 0:
+        raise _lib.KatzHipError("kh_conv3x3_gn_stats_nhwc_bf16 does not take this shape (see conv3x3_gn_splits)")
+    Ho, Wo = (H - 1) // stride + 1, (W - 1) // stride + 1
+    conv = torch.empty((Nb, Cout, Ho, Wo), dtype=BF16, device=x.device, memory_format=torch.channels_last)
+    out = torch.empty_like(conv)
+    ws = _workspace(Nb * num_groups * splits * 8, x.device)
+    if CALL_LOG is not None:
+        CALL_LOG.append(("conv3x3", Nb * Ho * Wo, Cout, 9 * Cin, stride))
+        CALL_LOG.append(("group_norm_apply", Nb, Cout, Ho * Wo))
+    _weight_prefetch_hint(w_packed)
+    rc = lib.kh_conv3x3_gn_stats_nhwc_bf16(_ptr(x), _ptr(w_packed), _ptr(bias), _ptr(add_nc), _ptr(conv), _ptr(ws), Nb, H, W,
+                                           Cin, Cout, stride, num_groups, _stream())
+    _lib.check(rc, "kh_conv3x3_gn_stats_nhwc_bf16")
+    rc = lib.kh_group_norm_apply_bf16(_ptr(conv), _ptr(out), _ptr(gamma), _ptr(beta), _ptr(add_nc), _ptr(ws), splits, Nb, Cout,
+                                      Ho * Wo, num_groups, float(eps), 1 if activation == "silu" else 0, _stream())
+    _lib.check(rc, "kh_group_norm_apply_bf16")
     return out
 
 
