@@ -306,24 +306,25 @@ int kh_upsample_nearest2x_nhwc_bf16(const void* x, void* y, int64_t N, int64_t H
  * K = 9*Cin) on the MFMA pipeline of kh_lora_linear_bf16.  Cin % 32 == 0, Cout % 8 == 0. */
 int kh_conv3x3_nhwc_bf16(const void* x, const void* w, const void* bias, const void* residual, void* y, int64_t Nb,
                          int64_t H, int64_t W, int64_t Cin, int64_t Cout, int64_t stride, void* stream);
-/* conv1 of a residual block that leaves the statistics of the GroupNorm behind it as a by-product of its epilogue:
- *   y = conv3x3(x) + bias (as kh_conv3x3_nhwc_bf16, no residual), and per (image, group, row tile of the image) the
+/* A convolution of a residual block that leaves the statistics of the GroupNorm behind it as a by-product of its epilogue:
+ *   y = conv3x3(x) + bias (+ residual), exactly as kh_conv3x3_nhwc_bf16, and per (image, group, row tile of the image) the
  *   (sum, sum of squares) of y + add_nc[n, c] over the tile's pixels and the group's channels
- * -- `hidden_states = conv1(...)`, `hidden_states + temb`, then norm2 of ResnetBlock2D.forward
- * (diffusers-hf/src/diffusers/models/resnet.py:378, :389, :390).  fast_kernel's group_norm_fp16 (normalization.py:91)
+ * -- conv1, `hidden_states + temb`, then norm2 of ResnetBlock2D.forward (diffusers-hf/src/diffusers/models/resnet.py:378,
+ * :389, :390), and conv2 with the block's skip (resnet.py:408-413) in front of the next module's GroupNorm (the
+ * transformer's, transformers/transformer_2d.py:481, or the next block's norm1).  fast_kernel's group_norm_fp16 (normalization.py:91)
  * reads the activation twice (statistics, then normalisation); here the first of the two reads never happens: the
  * convolution's output tiles hold whole groups, so their workgroups sum them while the tile is still in LDS, and
  * kh_group_norm_apply_bf16 folds the partial sums (fp64, fixed order) and normalises.  The statistics are taken over the
- * bf16-rounded result plus add_nc, as kh_group_norm_bf16 takes them from memory: against convolution + kh_group_norm_bf16
- * the result differs by the summation order of the statistics only.
+ * bf16-rounded stored result plus add_nc, as kh_group_norm_bf16 takes them from memory: against convolution +
+ * kh_group_norm_bf16 the result differs by the summation order of the statistics only.
  * kh_conv3x3_gn_splits(...) = row tiles per image when the shape is taken (the convolution runs on 160-column tiles,
  * Cout % 160 == 0, 160 % (Cout / G) == 0, whole tiles per image: every resnet convolution of SDXL), else 0 (run
  * kh_conv3x3_nhwc_bf16 and kh_group_norm_bf16).  partials: float [Nb * G * splits * 2], written completely.
  * add_nc bf16 [Nb, Cout] or NULL.  Everything else as for kh_conv3x3_nhwc_bf16. */
 int64_t kh_conv3x3_gn_splits(int64_t Nb, int64_t H, int64_t W, int64_t Cin, int64_t Cout, int64_t stride, int64_t G);
-int kh_conv3x3_gn_stats_nhwc_bf16(const void* x, const void* w, const void* bias, const void* add_nc, void* y,
-                                  float* partials, int64_t Nb, int64_t H, int64_t W, int64_t Cin, int64_t Cout, int64_t stride,
-                                  int64_t G, void* stream);
+int kh_conv3x3_gn_stats_nhwc_bf16(const void* x, const void* w, const void* bias, const void* residual, const void* add_nc,
+                                  void* y, float* partials, int64_t Nb, int64_t H, int64_t W, int64_t Cin, int64_t Cout,
+                                  int64_t stride, int64_t G, void* stream);
 
 /* ---- Classifier-free guidance + Euler step --------------------------------------------------------------
  * eps = u + g*(t - u) with noise_pred = [u; t] (uncond rows first)      pipeline_controlnet_sd_xl_katz.py:1649-1650

@@ -51,7 +51,7 @@ SIGNATURES = {
     "kh_conv_out_cfg_euler_bf16": (c_int, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, c_float, _P, c_int, _P]),
     "kh_conv3x3_nhwc_bf16": (c_int, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]),
     "kh_conv3x3_gn_splits": (_I, [_I] * 7),
-    "kh_conv3x3_gn_stats_nhwc_bf16": (c_int, [_P] * 6 + [_I] * 7 + [_P]),
+    "kh_conv3x3_gn_stats_nhwc_bf16": (c_int, [_P] * 7 + [_I] * 7 + [_P]),
     "kh_group_norm_apply_bf16": (c_int, [_P] * 6 + [_I] * 5 + [c_float, c_int, _P]),
 }
 

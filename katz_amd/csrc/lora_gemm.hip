@@ -761,12 +761,12 @@ KH_EXPORT int64_t kh_conv3x3_gn_splits(int64_t Nb, int64_t H, int64_t W, int64_t
   return rg == 0 ? 0 : p.gn_hw / (32 * rg);
 }
 
-KH_EXPORT int kh_conv3x3_gn_stats_nhwc_bf16(const void* x, const void* w, const void* bias, const void* add_nc, void* y,
-                                            float* partials, int64_t Nb, int64_t H, int64_t W, int64_t Cin, int64_t Cout,
-                                            int64_t stride, int64_t G, void* stream) {
+KH_EXPORT int kh_conv3x3_gn_stats_nhwc_bf16(const void* x, const void* w, const void* bias, const void* residual,
+                                            const void* add_nc, void* y, float* partials, int64_t Nb, int64_t H, int64_t W,
+                                            int64_t Cin, int64_t Cout, int64_t stride, int64_t G, void* stream) {
   if (!partials || G <= 0 || Cout % G != 0) return KH_ERR_INVALID_ARG;
   LoraGemmParams p;
-  if (const int rc = conv3x3_params(p, x, w, bias, nullptr, y, Nb, H, W, Cin, Cout, stride); rc != KH_OK) return rc;
+  if (const int rc = conv3x3_params(p, x, w, bias, residual, y, Nb, H, W, Cin, Cout, stride); rc != KH_OK) return rc;
   p.gn_cg = (int)(Cout / G); p.gn_hw = p.conv_ho * p.conv_wo;
   if (lora_gemm_conv_gn_row_groups(p) == 0) return KH_ERR_UNSUPPORTED;
   p.gn_part = partials; p.gn_add = (const bf16_t*)add_nc;

@@ -357,8 +357,8 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_ksplit_kernel(const LoraGemm
   __syncthreads();
   if constexpr (GNF) {
     // GroupNorm statistics as a by-product: the staged tile is BM pixels of one image times BN / gn_cg whole groups; their
-    // (sum, sum of squares) over the bf16-rounded values plus the per-(image, channel) term -- what a GroupNorm kernel
-    // reading the stored result would take -- go to gn_part[image][group][row tile of the image].  Three short passes,
+    // (sum, sum of squares) over the bf16-rounded values (residual included) plus the per-(image, channel) term -- what a GroupNorm
+    // kernel reading the stored result would take -- go to gn_part[image][group][row tile of the image].  Three short passes,
     // sums in fixed orders (deterministic); the tile itself is stored below as usual.
     constexpr int PCS = BN / 8, RP = 512 / PCS;               // 16-byte pieces per row, row parts (25 of 20 threads)
     float* colp = reinterpret_cast<float*>(smem);             // [RP][BN][2]: the partial strips are dead
@@ -366,6 +366,22 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_ksplit_kernel(const LoraGemm
     static_assert((RP * BN * 2 + BN * 2) * 4 <= C::PART, "column sums fit the dead partial strips");
     const int cg = p.gn_cg, ng = BN / cg, G = N / cg;
     const int n_img = m0 / p.gn_hw, split = (m0 % p.gn_hw) / BM, splits = p.gn_hw / BM;
+    if (p.res != nullptr) {
+      // the statistics are those of the stored result: the residual goes into the staged tile first (the same rounded adds
+      // the store loop would make), and the store loop below then writes the tile as it is
+#pragma unroll
+      for (int q = 0; q < C::OPT; ++q) {
+        const int c = tid + q * 512, srow = c / (BN / 8), ch = c % (BN / 8);
+        if (c < C::OPC) {
+          u32x4 o = *reinterpret_cast<const u32x4*>(sC + srow * C::LDC + ch * 8);
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            o[e] = pack_bf16x2(bf16_lo(o[e]) + bf16_lo(rr[q][e]), bf16_hi(o[e]) + bf16_hi(rr[q][e]));
+          *reinterpret_cast<u32x4*>(sC + srow * C::LDC + ch * 8) = o;
+        }
+      }
+      __syncthreads();
+    }
     // the per-(image, channel) term enters through sum(a + t) = sum(a) + n t and sum((a + t)^2) = sum(a^2) + 2 t sum(a) + n t^2:
     // requested now, used after the first pass
     const float ad = (tid < BN && p.gn_add != nullptr) ? (float)p.gn_add[(size_t)n_img * N + n0 + tid] : 0.f;
@@ -440,7 +456,7 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_ksplit_kernel(const LoraGemm
     const int grow = m0 + srow, gcol = n0 + ch * 8;
     if (c < C::OPC && grow < M && gcol < N) {
       u32x4 o = *reinterpret_cast<const u32x4*>(sC + srow * C::LDC + ch * 8);
-      if (p.res != nullptr) {
+      if (!GNF && p.res != nullptr) {   // (GNF: already added into the staged tile)
 #pragma unroll
         for (int e = 0; e < 4; ++e)
           o[e] = pack_bf16x2(bf16_lo(o[e]) + bf16_lo(rr[q][e]), bf16_hi(o[e]) + bf16_hi(rr[q][e]));
@@ -472,8 +488,8 @@ int launch_ksplit(LoraGemmParams p, hipStream_t stream) {
   }
   const unsigned grid = 8u * (unsigned)p.xr_m * (unsigned)p.xr_n;
   if constexpr (GNF) {
-    // whole groups per tile, whole tiles per image, no residual (the statistics are taken before it would be added)
-    if (p.res != nullptr || p.st_part != nullptr || p.gn_cg <= 0 || C::BN % p.gn_cg != 0 || p.N % C::BN != 0 || p.gn_hw % C::BM != 0 ||
+    // whole groups per tile, whole tiles per image
+    if (p.st_part != nullptr || p.gn_cg <= 0 || C::BN % p.gn_cg != 0 || p.N % C::BN != 0 || p.gn_hw % C::BM != 0 ||
         p.M % p.gn_hw != 0)
       return KH_ERR_UNSUPPORTED;
   }

@@ -1267,9 +1267,9 @@ int lora_gemm_pipe_launch_xattn(const LoraGemmParams& p, hipStream_t stream) {
 }
 
 // The 160-column tiles the rules below give this convolution, when the GroupNorm statistics of its result can be a
-// by-product of its epilogue: whole tiles per image, whole groups per tile, no residual.
+// by-product of its epilogue: whole tiles per image, whole groups per tile.
 int lora_gemm_conv_gn_row_groups(const LoraGemmParams& p) {
-  if (p.N % 160 != 0 || !lora_gemm_ksplit_conv_ok(p) || p.res != nullptr || p.gn_cg <= 0 || 160 % p.gn_cg != 0 || p.gn_hw <= 0 || p.M % p.gn_hw != 0)
+  if (p.N % 160 != 0 || !lora_gemm_ksplit_conv_ok(p) || p.gn_cg <= 0 || 160 % p.gn_cg != 0 || p.gn_hw <= 0 || p.M % p.gn_hw != 0)
     return 0;
   const long tiles = (long)((p.M + 127) / 128) * ((p.N + 127) / 128);
   const long n160 = p.N / 160, m128 = (p.M + 127) / 128, m64 = (p.M + 63) / 64;

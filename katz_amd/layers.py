@@ -47,9 +47,9 @@ LN_FOLD = os.getenv("KATZ_LN_FOLD", "1") != "0"
 # attention kernel (for measurements).
 XATTN_FUSE = os.getenv("KATZ_XATTN_FUSE", "1") != "0"
 
-# conv1 of a residual block leaves the statistics of the GroupNorm behind it as a by-product of its epilogue
-# (kh_conv3x3_gn_stats_nhwc_bf16), so that norm is one launch instead of two.  "0": convolution, then the norm's two
-# launches (for measurements).
+# The 3x3 convolutions of a residual block leave the statistics of the GroupNorm behind them as a by-product of their
+# epilogue (kh_conv3x3_gn_stats_nhwc_bf16), so that norm is one launch instead of two.  "0": convolution, then the norm's
+# two launches (for measurements).
 CONV_GN_FUSE = os.getenv("KATZ_CONV_GN_FUSE", "1") != "0"
 
 
@@ -340,7 +340,23 @@ class GroupNorm(nn.Module):
             self.weight = self.bias = None
 
     def forward(self, x: torch.Tensor, add_nc: Optional[torch.Tensor] = None) -> torch.Tensor:
+        st = getattr(x, "_katz_gn_stats", None)
+        if (st is not None and CONV_GN_FUSE and st.num_groups == self.num_groups and st.version == x._version
+                and st.add_nc is add_nc and (self.weight is None or self.weight.dtype == torch.bfloat16)):
+            # the convolution that produced x left this norm's statistics (Conv3x3.forward, stats_for): one launch
+            return ops.group_norm_from_stats(x, self.num_groups, self.weight, self.bias, self.eps, self.activation,
+                                             st.partials, st.splits, add_nc=add_nc)
         return ops.group_norm(x, self.num_groups, self.weight, self.bias, self.eps, self.activation, add_nc=add_nc)
+
+
+class GnStats:
+    """GroupNorm statistics that ride on a convolution's output tensor (attribute `_katz_gn_stats`) to the norm behind it:
+    partial (sum, sum of squares) per (image, group, row tile) of the tensor + add_nc, valid while the tensor's version
+    counter has not moved."""
+    __slots__ = ("partials", "splits", "num_groups", "add_nc", "version")
+
+    def __init__(self, partials, splits, num_groups, add_nc, version):
+        self.partials, self.splits, self.num_groups, self.add_nc, self.version = partials, splits, num_groups, add_nc, version
 
 
 def fused_norm_silu(num_channels: int, norm_num_groups: int, eps: float, affine: bool = True):
@@ -506,31 +522,26 @@ class Conv3x3(_ConvLoRAFuse, nn.Conv2d):
             self._packed = (w.data_ptr(), w._version, ops.pack_conv3x3_weight(wp), b)
         return self._packed[2], self._packed[3]
 
-    def forward_norm(self, x, norm: "GroupNorm", add_nc=None):
-        """norm(self(x), add_nc=add_nc) with the norm's statistics taken in the convolution's epilogue where the kernel takes
-        the shape (ops.conv3x3_group_norm); None otherwise (the caller then runs the two modules one after the other)."""
-        if not (CONV_GN_FUSE and x.is_cuda and x.dtype == torch.bfloat16 and self.weight.dtype == torch.bfloat16
-                and self.padding == (1, 1) and self.in_channels % 32 == 0 and self.out_channels % 8 == 0
-                and norm.activation in ("none", "silu") and norm.num_channels == self.out_channels):
-            return None
-        if self.adapters and self._lora_pack()[0] is not None:
-            return None   # the low-rank branch adds to the convolution's result before the norm
-        if add_nc is not None and (add_nc.dtype != torch.bfloat16 or add_nc.numel() != x.shape[0] * self.out_channels):
-            return None
-        if ops.conv3x3_gn_splits(x, self.out_channels, norm.num_groups, self.stride[0]) == 0:
-            return None
-        x = x.contiguous(memory_format=torch.channels_last)
-        w_packed, b_packed = self.packed_weight()
-        w, b = norm.weight, norm.bias
-        if w is not None and w.dtype != torch.bfloat16:
-            return None
-        return ops.conv3x3_group_norm(x, w_packed, b_packed, norm.num_groups, None if w is None else w.detach(),
-                                      None if b is None else b.detach(), norm.eps, norm.activation,
-                                      add_nc=None if add_nc is None else add_nc.contiguous(), stride=self.stride[0])
-
-    def forward(self, x, residual=None):
+    def forward(self, x, residual=None, stats_for=None):
+        """stats_for = (num_groups, add_nc or None): a GroupNorm of that many groups follows (on the result + add_nc per image
+        and channel); where the kernel takes the shape the convolution's epilogue leaves its statistics, which ride on
+        the returned tensor (GnStats) and make that norm one launch instead of two."""
         native = (x.is_cuda and x.dtype == torch.bfloat16 and self.weight.dtype == torch.bfloat16 and self.padding == (1, 1))
         a_cat, b_cat = self._lora_pack() if self.adapters else (None, None)
+        if (stats_for is not None and CONV_GN_FUSE and native and a_cat is None and self.in_channels % 32 == 0
+                and self.out_channels % 8 == 0):
+            groups, add_nc = stats_for
+            add_ok = add_nc is None or (add_nc.dtype == torch.bfloat16 and add_nc.numel() == x.shape[0] * self.out_channels
+                                        and add_nc.is_contiguous())
+            if add_ok and ops.conv3x3_gn_splits(x, self.out_channels, groups, self.stride[0]) > 0:
+                x = x.contiguous(memory_format=torch.channels_last)
+                if residual is not None:
+                    residual = residual.contiguous(memory_format=torch.channels_last)
+                w_packed, b_packed = self.packed_weight()
+                y, partials, splits = ops.conv3x3_stats(x, w_packed, b_packed, groups, add_nc=add_nc, residual=residual,
+                                                        stride=self.stride[0])
+                y._katz_gn_stats = GnStats(partials, splits, groups, add_nc, y._version)
+                return y
         if not native:
             if a_cat is not None:
                 raise NotImplementedError("LoRA on a convolution needs the katz_hip conv kernel (bf16 GPU tensors, padding 1)")
@@ -684,14 +695,16 @@ class ResnetBlock2D(nn.Module):
         """temb_act = silu(temb), computed once per step by the caller."""
         h = self.norm_silu1(input_tensor)
         # hidden_states + temb[:, :, None, None] rides inside the second norm (no separate pass), and where the kernel takes
-        # the shape conv1's epilogue leaves that norm's statistics
+        # the shape conv1's epilogue leaves that norm's statistics (they ride on conv1's output tensor)
         tp, self.temb_proj = self.temb_proj, None
         add = self.time_emb_proj(temb_act) if tp is None else tp
-        fused = self.conv1.forward_norm(h, self.norm_silu2[0], add)
-        h = fused if fused is not None else self.norm_silu2[0](self.conv1(h), add_nc=add)
+        norm2 = self.norm_silu2[0]
+        h = norm2(self.conv1(h, stats_for=(norm2.num_groups, add)), add_nc=add)
         if self.conv_shortcut is not None:
             input_tensor = self.conv_shortcut(input_tensor)
-        out = self.conv2(h, residual=input_tensor)   # input_tensor + conv2(h), the add in the conv's epilogue
+        # input_tensor + conv2(h), the add in the conv's epilogue; what follows a resnet is mostly another GroupNorm (the
+        # transformer's, the next resnet's, conv_norm_out) with this block's number of groups: its statistics ride along
+        out = self.conv2(h, residual=input_tensor, stats_for=(norm2.num_groups, None))
         if self.output_scale_factor != 1.0:
             out = out / self.output_scale_factor
         return out

@@ -748,6 +748,7 @@ def residual_add_(dst: torch.Tensor, residuals: Sequence[torch.Tensor]) -> torch
     rc = lib.kh_residual_add_bf16(_ptr(dst), _ptr_array(residuals), len(residuals), 1.0 / len(residuals),
                                   dst.numel(), _stream())
     _lib.check(rc, "kh_residual_add_bf16")
+    torch.autograd.graph.increment_version(dst)   # as an in-place torch op would: anything derived from dst is now stale
     return dst
 
 
@@ -827,25 +828,21 @@ def conv3x3_gn_splits(x: torch.Tensor, cout: int, num_groups: int, stride: int =
     return int(_lib.load().kh_conv3x3_gn_splits(Nb, H, W, Cin, cout, stride, num_groups))
 
 
-def conv3x3_group_norm(x: torch.Tensor, w_packed: torch.Tensor, bias: Optional[torch.Tensor], num_groups: int,
-                       gamma: Optional[torch.Tensor], beta: Optional[torch.Tensor], eps: float = 1e-5,
-                       activation: str = "none", add_nc: Optional[torch.Tensor] = None, stride: int = 1) -> torch.Tensor:
-    """group_norm(conv3x3(x, w_packed, bias), num_groups, gamma, beta, eps, activation, add_nc=add_nc) in two launches
-    instead of three: the convolution leaves the norm's statistics as a by-product of its epilogue
-    (kh_conv3x3_gn_stats_nhwc_bf16), the norm's second pass alone follows (kh_group_norm_apply_bf16).  Only for shapes with
-    conv3x3_gn_splits(...) > 0."""
+def conv3x3_stats(x: torch.Tensor, w_packed: torch.Tensor, bias: Optional[torch.Tensor], num_groups: int,
+                  add_nc: Optional[torch.Tensor] = None, residual: Optional[torch.Tensor] = None, stride: int = 1):
+    """conv3x3(x, w_packed, bias, stride, residual) that also leaves the statistics of a GroupNorm(num_groups) of its result
+    (+ add_nc per image and channel) as a by-product of its epilogue (kh_conv3x3_gn_stats_nhwc_bf16).  Returns
+    (y, partials, splits): partials is a float [N, num_groups, splits, 2] tensor for group_norm_from_stats.  Only for
+    shapes with conv3x3_gn_splits(...) > 0."""
     lib = _lib.load()
     if not x.is_cuda or x.dtype != BF16 or x.dim() != 4 or not x.is_contiguous(memory_format=torch.channels_last):
         raise ValueError("x must be a channels_last bfloat16 GPU tensor")
-    if activation not in ("none", "silu"):
-        raise ValueError(f"unknown activation {activation!r}")
     Nb, Cin, H, W = x.shape
     Cout = w_packed.shape[0]
     if w_packed.shape != (Cout, 3, 3, Cin) or not w_packed.is_contiguous() or w_packed.dtype != BF16:
         raise ValueError("w_packed must be a contiguous bfloat16 [Cout,3,3,Cin] tensor")
-    for t_, name in ((bias, "bias"), (gamma, "gamma"), (beta, "beta")):
-        if t_ is not None and (t_.shape != (Cout,) or t_.dtype != BF16 or not t_.is_contiguous()):
-            raise ValueError(f"{name} must be a contiguous bfloat16 [Cout] tensor")
+    if bias is not None and (bias.shape != (Cout,) or bias.dtype != BF16 or not bias.is_contiguous()):
+        raise ValueError("bias must be a contiguous bfloat16 [Cout] tensor")
     if add_nc is not None:
         add_nc = add_nc.reshape(Nb, Cout)
         if add_nc.dtype != BF16 or not add_nc.is_contiguous():
@@ -854,20 +851,56 @@ def conv3x3_group_norm(x: torch.Tensor, w_packed: torch.Tensor, bias: Optional[t
     if splits == 0:
         raise _lib.KatzHipError("kh_conv3x3_gn_stats_nhwc_bf16 does not take this shape (see conv3x3_gn_splits)")
     Ho, Wo = (H - 1) // stride + 1, (W - 1) // stride + 1
-    conv = torch.empty((Nb, Cout, Ho, Wo), dtype=BF16, device=x.device, memory_format=torch.channels_last)
-    out = torch.empty_like(conv)
-    ws = _workspace(Nb * num_groups * splits * 8, x.device)
+    out = torch.empty((Nb, Cout, Ho, Wo), dtype=BF16, device=x.device, memory_format=torch.channels_last)
+    if residual is not None and (residual.shape != out.shape or residual.dtype != BF16
+                                 or not residual.is_contiguous(memory_format=torch.channels_last)):
+        raise ValueError("residual must be a channels_last bfloat16 tensor of the output's shape")
+    partials = torch.empty((Nb, num_groups, splits, 2), dtype=torch.float32, device=x.device)
     if CALL_LOG is not None:
         CALL_LOG.append(("conv3x3", Nb * Ho * Wo, Cout, 9 * Cin, stride))
-        CALL_LOG.append(("group_norm_apply", Nb, Cout, Ho * Wo))
     _weight_prefetch_hint(w_packed)
-    rc = lib.kh_conv3x3_gn_stats_nhwc_bf16(_ptr(x), _ptr(w_packed), _ptr(bias), _ptr(add_nc), _ptr(conv), _ptr(ws), Nb, H, W,
-                                           Cin, Cout, stride, num_groups, _stream())
+    rc = lib.kh_conv3x3_gn_stats_nhwc_bf16(_ptr(x), _ptr(w_packed), _ptr(bias), _ptr(residual), _ptr(add_nc), _ptr(out),
+                                           _ptr(partials), Nb, H, W, Cin, Cout, stride, num_groups, _stream())
     _lib.check(rc, "kh_conv3x3_gn_stats_nhwc_bf16")
-    rc = lib.kh_group_norm_apply_bf16(_ptr(conv), _ptr(out), _ptr(gamma), _ptr(beta), _ptr(add_nc), _ptr(ws), splits, Nb, Cout,
-                                      Ho * Wo, num_groups, float(eps), 1 if activation == "silu" else 0, _stream())
+    return out, partials, splits
+
+
+def group_norm_from_stats(x: torch.Tensor, num_groups: int, weight: Optional[torch.Tensor], bias: Optional[torch.Tensor],
+                          eps: float, activation: str, partials: torch.Tensor, splits: int,
+                          add_nc: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """group_norm(x, ..., add_nc=add_nc) as ONE launch, on the statistics conv3x3_stats left for x (+ the same add_nc):
+    the norm's second pass alone (kh_group_norm_apply_bf16).  x: channels_last bfloat16 [N,C,H,W]."""
+    lib = _lib.load()
+    if not x.is_cuda or x.dtype != BF16 or x.dim() != 4 or not x.is_contiguous(memory_format=torch.channels_last):
+        raise ValueError("x must be a channels_last bfloat16 GPU tensor")
+    if activation not in ("none", "silu"):
+        raise ValueError(f"unknown activation {activation!r}")
+    N, C, H, W = x.shape
+    for t_, name in ((weight, "weight"), (bias, "bias")):
+        if t_ is not None and (t_.shape != (C,) or t_.dtype != BF16 or not t_.is_contiguous()):
+            raise ValueError(f"{name} must be a contiguous bfloat16 [C] tensor")
+    if partials.dtype != torch.float32 or not partials.is_contiguous() or partials.numel() != N * num_groups * splits * 2:
+        raise ValueError("partials must be the float [N, num_groups, splits, 2] tensor conv3x3_stats returned")
+    if add_nc is not None:
+        add_nc = add_nc.reshape(N, C)
+        if add_nc.dtype != BF16 or not add_nc.is_contiguous():
+            raise ValueError("add_nc must be a contiguous bfloat16 [N,C] tensor")
+    out = torch.empty_like(x)
+    if CALL_LOG is not None:
+        CALL_LOG.append(("group_norm_apply", N, C, H * W))
+    rc = lib.kh_group_norm_apply_bf16(_ptr(x), _ptr(out), _ptr(weight), _ptr(bias), _ptr(add_nc), _ptr(partials), splits, N, C,
+                                      H * W, num_groups, float(eps), 1 if activation == "silu" else 0, _stream())
     _lib.check(rc, "kh_group_norm_apply_bf16")
     return out
+
+
+def conv3x3_group_norm(x: torch.Tensor, w_packed: torch.Tensor, bias: Optional[torch.Tensor], num_groups: int,
+                       gamma: Optional[torch.Tensor], beta: Optional[torch.Tensor], eps: float = 1e-5,
+                       activation: str = "none", add_nc: Optional[torch.Tensor] = None, stride: int = 1) -> torch.Tensor:
+    """group_norm(conv3x3(x, w_packed, bias), num_groups, gamma, beta, eps, activation, add_nc=add_nc) in two launches
+    instead of three: conv3x3_stats, then group_norm_from_stats."""
+    y, partials, splits = conv3x3_stats(x, w_packed, bias, num_groups, add_nc=add_nc, stride=stride)
+    return group_norm_from_stats(y, num_groups, gamma, beta, eps, activation, partials, splits, add_nc=add_nc)
 
 
 def cfg_euler_step(noise_pred: torch.Tensor, latents: torch.Tensor, coef: torch.Tensor, guidance_scale: float,

@@ -87,31 +87,53 @@ def test_convolution_that_leaves_the_norm_statistics(Nb, Cin, Cout, H, act, with
 
 
 def test_statistics_against_plain_sums():
-    """The partial sums themselves: folded over the row tiles they equal the sums of the convolution's stored result."""
-    import ctypes
-    from katz_amd import _lib, ops
+    """The partial sums themselves: folded over the row tiles they equal the sums of the convolution's stored result
+    (residual included) plus the per-channel term."""
+    from katz_amd import ops
     say("conv3x3 statistics against torch sums")
     d = dev()
     Nb, Cin, Cout, H, G = 2, 640, 640, 64, 32
     x, w, b, _, _, add = _case(Nb, Cin, Cout, H, seed=3)
+    g = torch.Generator().manual_seed(4)
+    res = randn(g, Nb, Cout, H, H).to(d, BF).contiguous(memory_format=torch.channels_last)
     xd = x.to(d, BF).contiguous(memory_format=torch.channels_last)
     wp = ops.pack_conv3x3_weight(w.to(d, BF))
-    splits = ops.conv3x3_gn_splits(xd, Cout, G)
-    part = torch.full((Nb, G, splits, 2), float("nan"), device=d)
-    conv = torch.empty((Nb, Cout, H, H), dtype=BF, device=d).contiguous(memory_format=torch.channels_last)
     addd = add.to(d, BF)
-    lib = _lib.load()
-    rc = lib.kh_conv3x3_gn_stats_nhwc_bf16(xd.data_ptr(), wp.data_ptr(), b.to(d, BF).data_ptr(), addd.data_ptr(), conv.data_ptr(),
-                                           part.data_ptr(), Nb, H, H, Cin, Cout, 1, G, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
-    assert rc == 0
+    for residual, add_nc in ((None, addd), (res, None), (res, addd)):
+        conv, part, splits = ops.conv3x3_stats(xd, wp, b.to(d, BF), G, add_nc=add_nc, residual=residual)
+        torch.cuda.synchronize()
+        assert torch.equal(conv, ops.conv3x3(xd, wp, b.to(d, BF), residual=residual)), "the convolution's own result is untouched"
+        assert part.shape == (Nb, G, splits, 2) and torch.isfinite(part).all(), "every (image, group, row tile) slot is written"
+        v = conv.float() if add_nc is None else conv.float() + add_nc.float()[:, :, None, None]
+        v = v.double().reshape(Nb, G, Cout // G, H * H)
+        s_ref, q_ref = v.sum(dim=(2, 3)), (v * v).sum(dim=(2, 3))
+        got = part.double().sum(dim=2)
+        assert torch.allclose(got[..., 0], s_ref, rtol=1e-4, atol=2e-2), "sums"
+        assert torch.allclose(got[..., 1], q_ref, rtol=1e-4), "sums of squares"
+
+
+@pytest.mark.parametrize("act", ["none", "silu"])
+def test_norm_behind_a_convolution_with_residual(act):
+    """conv2 + skip, then the next module's GroupNorm (no per-channel term) on the statistics conv2 left."""
+    from katz_amd import ops
+    say("conv3x3 + residual, statistics, group norm", act)
+    d = dev()
+    Nb, Cin, Cout, H, G, eps = 2, 1280, 1280, 32, 32, 1e-6
+    x, w, b, gamma, beta, _ = _case(Nb, Cin, Cout, H, seed=9)
+    g = torch.Generator().manual_seed(10)
+    res = randn(g, Nb, Cout, H, H)
+    xd = x.to(d, BF).contiguous(memory_format=torch.channels_last)
+    resd = res.to(d, BF).contiguous(memory_format=torch.channels_last)
+    wp = ops.pack_conv3x3_weight(w.to(d, BF))
+    y, part, splits = ops.conv3x3_stats(xd, wp, b.to(d, BF), G, residual=resd)
+    n = ops.group_norm_from_stats(y, G, gamma.to(d, BF), beta.to(d, BF), eps, act, part, splits)
+    n2 = ops.group_norm(y, G, gamma.to(d, BF), beta.to(d, BF), eps, act)
     torch.cuda.synchronize()
-    assert torch.equal(conv, ops.conv3x3(xd, wp, b.to(d, BF))), "the convolution's own result is untouched"
-    assert torch.isfinite(part).all(), "every (image, group, row tile) slot is written"
-    v = (conv.float() + addd.float()[:, :, None, None]).double().reshape(Nb, G, Cout // G, H * H)
-    s_ref, q_ref = v.sum(dim=(2, 3)), (v * v).sum(dim=(2, 3))
-    got = part.double().sum(dim=2)
-    assert torch.allclose(got[..., 0], s_ref, rtol=1e-4, atol=1e-2), "sums"
-    assert torch.allclose(got[..., 1], q_ref, rtol=1e-4), "sums of squares"
+    conv = bf16_round(bf16_round(torch.nn.functional.conv2d(x, w, b, padding=1)) + res)   # rounded, residual added, rounded
+    ref = O.group_norm(conv, G, gamma, beta, eps, act)
+    assert_close_rel(n, ref, 2e-2, "norm on the convolution's statistics against the oracle")
+    assert_close_rel(n, n2.float().cpu(), 1e-2, "against kh_group_norm_bf16 on the same tensor")
+    assert (n != n2).float().mean().item() < 0.02
 
 
 def test_shapes_that_are_not_taken():
@@ -176,3 +198,63 @@ def test_resnet_block_with_and_without_the_norm_in_the_convolution(monkeypatch, 
     assert c1 >= 0.9995 and c0 >= 0.9995 and c10 >= 0.9995
     assert_close_rel(y1, ref, 4e-2, "resnet block with norm2's statistics from conv1")
     assert_close_rel(y1, y0.float().cpu(), 2e-2, "statistics from conv1 against the separate kernels")
+
+
+def test_statistics_ride_from_one_block_to_the_next(monkeypatch):
+    """Two residual blocks in a row: the second block's norm1 runs on what the first block's conv2 left (one full
+    GroupNorm in all: the first block's norm1), against the same modules without the hand-over and against the oracle.
+    A tensor modified in place after the convolution loses its statistics."""
+    import katz_amd.layers as L
+    from helpers import cosine, round_module_to_bf16_
+    from katz_amd import ops
+    from oracle import blocks as OB
+
+    say("two resnet blocks, statistics handed from conv2 to the next norm1")
+    d = dev()
+    torch.manual_seed(7)
+    oracle = torch.nn.ModuleList([OB.ResnetBlock2D(in_channels=640, out_channels=640, temb_channels=1280, eps=1e-5) for _ in range(2)])
+    for m in oracle.modules():
+        if isinstance(m, torch.nn.GroupNorm):
+            torch.nn.init.normal_(m.weight, 1.0, 0.2); torch.nn.init.normal_(m.bias, 0.0, 0.2)
+    round_module_to_bf16_(oracle)
+    prod = torch.nn.ModuleList([L.ResnetBlock2D(in_channels=640, out_channels=640, temb_channels=1280, eps=1e-5) for _ in range(2)])
+    prod.load_state_dict(oracle.state_dict(), strict=True)
+    prod = prod.to(d, BF)
+    g = torch.Generator().manual_seed(8)
+    x = bf16_round(torch.randn(2, 640, 64, 64, generator=g))
+    temb = bf16_round(torch.randn(2, 1280, generator=g))
+    xd = x.to(d, BF).contiguous(memory_format=torch.channels_last)
+    temb_act = torch.nn.functional.silu(temb.to(d, BF))
+
+    def run():
+        ops.CALL_LOG = []
+        try:
+            h = xd
+            for blk in prod:
+                h = blk(h, temb_act)
+        finally:
+            log, ops.CALL_LOG = ops.CALL_LOG, None
+        return h, log
+
+    with torch.no_grad():
+        ref = oracle[1](oracle[0](x, temb), temb)
+        y1, log1 = run()
+        assert getattr(y1, "_katz_gn_stats", None) is not None, "the last conv2 leaves statistics for whoever follows"
+        # an in-place change invalidates them: the norm falls back to its own statistics pass
+        y_mod = y1.clone(); y_mod._katz_gn_stats = y1._katz_gn_stats
+        ops.residual_add_(y_mod, [torch.ones_like(y_mod)])
+        ops.CALL_LOG = []
+        n_mod = prod[0].norm_silu1(y_mod)
+        log_mod, ops.CALL_LOG = ops.CALL_LOG, None
+        n_ref = ops.group_norm(y_mod, 32, prod[0].norm_silu1[0].weight, prod[0].norm_silu1[0].bias, 1e-5, "silu")
+        monkeypatch.setattr(L, "CONV_GN_FUSE", False)
+        y0, log0 = run()
+    torch.cuda.synchronize()
+    assert [e[0] for e in log_mod] == ["group_norm"] and torch.equal(n_mod, n_ref)
+    assert sum(1 for e in log1 if e[0] == "group_norm") == 1 and sum(1 for e in log1 if e[0] == "group_norm_apply") == 3
+    assert sum(1 for e in log0 if e[0] == "group_norm") == 4 and not any(e[0] == "group_norm_apply" for e in log0)
+    c1, c0 = cosine(y1, ref), cosine(y0, ref)
+    say(f"  cosine against the oracle: with the hand-over {c1:.6f}, without {c0:.6f}")
+    assert c1 >= 0.9995 and c0 >= 0.9995
+    assert_close_rel(y1, ref, 4e-2, "two blocks with the statistics handed over")
+    assert_close_rel(y1, y0.float().cpu(), 2e-2, "hand-over against separate kernels")
