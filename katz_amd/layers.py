@@ -647,15 +647,18 @@ class Conv1x1(_ConvLoRAFuse, nn.Conv2d):
 
 
 class Downsample2D(nn.Module):
-    def __init__(self, channels, use_conv=True, out_channels=None, padding=1, name="op"):
+    def __init__(self, channels, use_conv=True, out_channels=None, padding=1, name="op", stats_groups=None):
+        """stats_groups: the number of groups of the GroupNorm that reads the result next (the following block's first
+        resnet); its statistics then ride on the output (see Conv3x3.forward)."""
         super().__init__()
         self.padding = padding
+        self.stats_groups = stats_groups
         self.conv = Conv3x3(channels, out_channels or channels, stride=2, padding=padding)
 
     def forward(self, x):
         if self.padding == 0:
             x = F.pad(x, (0, 1, 0, 1))
-        return self.conv(x)
+        return self.conv(x, stats_for=None if self.stats_groups is None else (self.stats_groups, None))
 
 
 class Upsample2D(nn.Module):

@@ -31,7 +31,8 @@ class DownBlock2D(nn.Module):
             ResnetBlock2D(in_channels=in_channels if i == 0 else out_channels, out_channels=out_channels,
                           temb_channels=temb_channels, eps=resnet_eps, groups=resnet_groups)
             for i in range(num_layers)])
-        self.downsamplers = nn.ModuleList([Downsample2D(out_channels, True, out_channels, downsample_padding, "op")]) \
+        self.downsamplers = nn.ModuleList([Downsample2D(out_channels, True, out_channels, downsample_padding, "op",
+                                                        stats_groups=resnet_groups)]) \
             if add_downsample else None
 
     def forward(self, hidden_states, temb_act, encoder_hidden_states=None):
@@ -62,7 +63,8 @@ class CrossAttnDownBlock2D(nn.Module):
                                             norm_num_groups=resnet_groups, use_linear_projection=use_linear_projection))
         self.attentions = nn.ModuleList(attns)
         self.resnets = nn.ModuleList(resnets)
-        self.downsamplers = nn.ModuleList([Downsample2D(out_channels, True, out_channels, downsample_padding, "op")]) \
+        self.downsamplers = nn.ModuleList([Downsample2D(out_channels, True, out_channels, downsample_padding, "op",
+                                                        stats_groups=resnet_groups)]) \
             if add_downsample else None
 
     def forward(self, hidden_states, temb_act, encoder_hidden_states=None):
