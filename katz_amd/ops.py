@@ -7,6 +7,7 @@ CPU: without a GPU (or without the built library) the functions raise.
 """
 from __future__ import annotations
 
+import contextlib
 import ctypes
 import math
 import os
@@ -218,7 +219,8 @@ def lora_linear_pre(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.
 # host's count says nothing about what eager forwards or other graphs have dirtied in between.  The UNet / ControlNet
 # forward resets at its start (inside a captured graph that is one fill node per step and the same slices on every
 # replay); a caller that never resets is served until the arena is full, then it is reset for him.  One stream per
-# device: a reset must not overtake launches that still use their slices.
+# device: a reset must not overtake launches that still use their slices (two models side by side on two streams:
+# clear once before the fork and run both under `split_counters_held`).
 SPLIT_ARENA_INTS = 1 << 16
 _split_arena: dict = {}     # (device type, index) -> [buffer, ints handed out, last slice, ever used]
 
@@ -236,10 +238,27 @@ def _arena(device):
     return st
 
 
+_arena_held: list = [0]
+
+
+@contextlib.contextmanager
+def split_counters_held():
+    """Inside this context `split_counters_reset` does nothing: for a caller that runs two models side by side on two
+    streams (a ControlNet beside the UNet's down blocks), clears the arena ONCE before the fork and must not have one
+    model's reset wipe or re-issue the slices the other's launches are using."""
+    _arena_held[0] += 1
+    try:
+        yield
+    finally:
+        _arena_held[0] -= 1
+
+
 def split_counters_reset(device) -> None:
     """Clear every counter of the device's arena with one fill kernel.  Outside graph capture the fill is skipped
     while no counter has ever been handed out; under capture it is always recorded, because by the time the graph is
     replayed other forwards may have dirtied the arena."""
+    if _arena_held[0]:
+        return
     st = _arena(device)
     if st[3] or torch.cuda.is_current_stream_capturing():
         st[0].zero_()
@@ -280,6 +299,8 @@ def _arena_ints(device, n: int) -> torch.Tensor:
     """n zeroed int32 of the device's counter arena (zero since the last split_counters_reset)."""
     st = _arena(device)
     if st[1] + n > SPLIT_ARENA_INTS:
+        if _arena_held[0]:
+            raise RuntimeError("katz_amd: the LoRA counter arena is full inside split_counters_held()")
         split_counters_reset(device)
     st[2] = st[0][st[1]:st[1] + n]
     st[1] += n
@@ -632,9 +653,23 @@ _gn_workspace: dict = {}
 _gn_retired: list = []     # outgrown workspaces, kept alive for graphs captured while they were current
 
 
+_ws_slot: list = [0]
+
+
+@contextlib.contextmanager
+def side_branch():
+    """Ops called inside this context take their shared scratch (the GroupNorm partial sums) from a second buffer, so
+    that they may run on another stream beside ops called outside it."""
+    _ws_slot[0] += 1
+    try:
+        yield
+    finally:
+        _ws_slot[0] -= 1
+
+
 def _workspace(nbytes: int, device) -> torch.Tensor:
-    """One grow-only fp32 scratch buffer per device (allocated outside graph capture on first use)."""
-    key = (device.type, device.index)
+    """One grow-only fp32 scratch buffer per device and branch (allocated outside graph capture on first use)."""
+    key = (device.type, device.index, _ws_slot[0])
     buf = _gn_workspace.get(key)
     if buf is None or buf.numel() * 4 < nbytes:
         if torch.cuda.is_current_stream_capturing():

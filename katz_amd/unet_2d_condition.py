@@ -534,6 +534,9 @@ class UNet2DConditionModel(nn.Module):
             skips += res
         sample = self.mid_block(sample, temb_act, ctx)
 
+        ready = getattr(self, "before_residuals", None)
+        if ready is not None:   # the residuals come from another stream (a ControlNet run beside the down blocks)
+            ready()
         extra = self._residual_sets(down_block_additional_residuals, len(skips))
         if mid_block_additional_residual is not None:
             mids = mid_block_additional_residual

@@ -135,7 +135,8 @@ def test_controlnet_unet_guided_loop_config5_shape(pair):
 def test_graphed_denoise_step_matches_eager_loop(pair):
     """ControlNet -> UNet -> guidance + Euler as one captured graph per step (GraphedDenoiseStep) against the same
     loop run eagerly, kernel by kernel: identical latents bit for bit, also on a second run with other latents, with
-    the conditioning embedding hoisted out of the loop or recomputed inside the graph."""
+    the conditioning embedding hoisted out of the loop or recomputed inside the graph, and with the ControlNet on a
+    second stream beside the UNet's down blocks (the default) or in front of the UNet on one stream."""
     from katz_amd.graph import GraphedDenoiseStep
     from katz_amd.scheduler import EulerDiscreteScheduler, denoise_loop
 
@@ -155,10 +156,11 @@ def test_graphed_denoise_step_matches_eager_loop(pair):
 
     lats = [bf16_round(x[:1] * psch.init_noise_sigma), bf16_round(x[1:] * psch.init_noise_sigma)]
     eager = [denoise_loop(p_model, psch, l.to(DEV), 7.5) for l in lats]
-    for hoist, fuse_tail in ((True, False), (False, False), (True, True)):
+    for hoist, fuse_tail, overlap in ((True, False, True), (False, False, True), (True, True, True),
+                                      (True, False, False), (False, False, False)):
         step = GraphedDenoiseStep(p_unet, p_cn, lats[0].to(DEV), ctx.to(DEV), added_d, cond.to(DEV), 7.5, 0.5,
-                                  hoist_cond_embedding=hoist, fuse_tail=fuse_tail)
-        assert step.fuse_tail == fuse_tail
+                                  hoist_cond_embedding=hoist, fuse_tail=fuse_tail, overlap=overlap)
+        assert step.fuse_tail == fuse_tail and step.overlap == overlap
         for l, e in zip(lats, eager):
             got = step.run(l.to(DEV), psch)
             torch.cuda.synchronize()
@@ -217,8 +219,11 @@ def test_sdxl_size_controlnet_forward_and_step():
         sch.set_timesteps(2, device=DEV)
         lat0 = (lat.float() * sch.init_noise_sigma).to(BF)
         step = GraphedDenoiseStep(unet, cn, lat0, ctx, added, cond, 7.5, 0.5, fuse_tail=False)
+        assert step.overlap
         got = step.run(lat0, sch)
         fused = GraphedDenoiseStep(unet, cn, lat0, ctx, added, cond, 7.5, 0.5).run(lat0, sch)   # conv_out inside the step kernel
+        one_stream = GraphedDenoiseStep(unet, cn, lat0, ctx, added, cond, 7.5, 0.5, overlap=False).run(lat0, sch)
+        assert torch.equal(fused, one_stream)   # the ControlNet beside the down blocks or in front of them: the same bits
         coef = sch.coef_table(DEV)
         cur = lat0.contiguous(memory_format=torch.channels_last)
         inp = (torch.cat([cur] * 2).float() / coef[0, 3]).to(BF).contiguous(memory_format=torch.channels_last)
