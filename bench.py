@@ -510,11 +510,14 @@ def loop_bench(args):
         "data": "synthetic (random-init SDXL UNet and ControlNet, seeded latents, conditioning image uniform[0,1])",
         "config": {"workload": f"{args.loop_steps}-step SDXL denoise loop at 1024x1024: per step ControlNet (SDXL arch, image "
                                "[2,3,1024,1024], scale 0.5) -> UNet (2 LoRAs r64 s0.8 + r32 s0.6, CFG batch 2) -> guidance 7.5 + "
-                               "Euler discrete; one HIP graph replay per step; conditioning embedding computed once per loop",
+                               "Euler discrete; one HIP graph replay per step" + ("; inside the graph the ControlNet runs on a second stream "
+                               "beside the UNet's down and mid blocks" if step.overlap else "") +
+                               "; conditioning embedding computed once per loop",
                    "global_batch": 2, "parallelism": "single GPU"},
         "loop_ms_all": [round(x, 2) for x in times], "output_finite": finite,
         "kernel_ms_per_step": {k: {"launches": v[0], "ms": round(v[1], 3)} for k, v in sorted(by_kernel.items())},
         "kernel_ms_sum_per_step": round(sum(v[1] for v in by_kernel.values()), 3),
+        "controlnet_beside_unet": bool(step.overlap),
         "cond_embedding_once_per_loop_ms": round(sum(d for _, d in emb_launches), 3),
     }
     print(json.dumps(result))
