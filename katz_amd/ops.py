@@ -48,6 +48,7 @@ def _req(t: torch.Tensor, dtype, name: str) -> None:
 # The table holds weak references only: a hint never keeps a tensor alive, and a dead one is dropped instead of hinted.
 WEIGHT_PREFETCH = os.getenv("KATZ_WEIGHT_PREFETCH", "1") != "0"
 PREFETCH_MIN_K = int(os.getenv("KATZ_PREFETCH_MIN_K", "2560"))
+PREFETCH_SMALL_BYTES = int(os.getenv("KATZ_PREFETCH_SMALL_BYTES", str(4 << 20)))
 _pf_next: dict = {}     # data_ptr of a launch's weights -> weak references to (weights, a_cat, b_cat) of the launch after it
 _pf_last: list = [None]
 _pf_shrink_a: list = [None]   # A_cat of a separate shrink launch, for the hint of the GEMM it belongs to
@@ -80,9 +81,12 @@ def _weight_prefetch_hint(weight: torch.Tensor, a_cat: Optional[torch.Tensor] = 
     # The prefetch is not free for the launch that carries it (its own first operands queue behind it: up to 3.5 us
     # for 26 MB), so weights are only hinted where meeting them in HBM costs more than that: long rows (K >= 2560,
     # the feed-forward output projections and the 3x3 convolutions), whose launches are latency-bound on their
-    # operand stream.  The adapter matrices are small and always hinted.
+    # operand stream -- and small ones (<= 4 MB: the d x d layers), which delay their carrier by well under a microsecond
+    # (measured: 24.19 -> 23.80 ms per step with them, 24.4 with every weight hinted).  The adapter matrices are small
+    # and always hinted.
     k_next = w_next.shape[-1] * (9 if w_next.dim() == 4 else 1)
-    for t in ((w_next if k_next >= PREFETCH_MIN_K else None),) + tuple(live[1:]):
+    small = w_next.numel() * w_next.element_size() <= PREFETCH_SMALL_BYTES
+    for t in ((w_next if (k_next >= PREFETCH_MIN_K or small) else None),) + tuple(live[1:]):
         if t is not None:
             lib.kh_set_weight_prefetch(t.data_ptr(), t.numel() * t.element_size())
 
