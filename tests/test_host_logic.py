@@ -440,8 +440,8 @@ def test_bench_refuses_more_than_one_gpu():
 
 def test_weight_prefetch_hints_are_learned_from_the_previous_pass(monkeypatch):
     """ops._weight_prefetch_hint: the first pass over a sequence of launches gives no hints; the second hints, at launch
-    i, the operands of launch i + 1 - weights only for long rows (K >= 2560 or a 3x3 kernel), adapter matrices always;
-    a tensor that has been freed is dropped instead of hinted."""
+    i, the operands of launch i + 1 - weights only for long rows (K >= 2560 or a 3x3 kernel) or below the size limit,
+    adapter matrices always; a tensor that has been freed is dropped instead of hinted."""
     import gc
 
     from katz_amd import ops
@@ -455,9 +455,10 @@ def test_weight_prefetch_hints_are_learned_from_the_previous_pass(monkeypatch):
 
     monkeypatch.setattr(ops._lib, "load", lambda: FakeLib())
     monkeypatch.setattr(ops, "WEIGHT_PREFETCH", True)
+    monkeypatch.setattr(ops, "PREFETCH_SMALL_BYTES", 16 << 10)
     ops._pf_next.clear()
     ops._pf_last[0] = None
-    w_small = torch.zeros(8, 1280)             # K 1280: not hinted
+    w_small = torch.zeros(8, 1280)             # K 1280 and 40 KB, above the size limit set here: not hinted
     w_long = torch.zeros(8, 5120)              # K 5120: hinted
     w_conv = torch.zeros(4, 3, 3, 320)         # 9 * 320 = 2880: hinted
     a_cat, b_cat = torch.zeros(128, 5120), torch.zeros(8, 128)
@@ -472,6 +473,14 @@ def test_weight_prefetch_hints_are_learned_from_the_previous_pass(monkeypatch):
                       (b_cat.data_ptr(), b_cat.numel() * 4), (w_conv.data_ptr(), w_conv.numel() * 4)]
     # what followed w_conv last time is w_small (the wrap-around), K 1280: its entry exists but hints nothing
     assert ops._pf_next[w_conv.data_ptr()][0]() is w_small
+    # ... until the size limit admits it (the default admits the d x d layers)
+    monkeypatch.setattr(ops, "PREFETCH_SMALL_BYTES", 64 << 10)
+    calls.clear()
+    ops._pf_last[0] = None
+    ops._weight_prefetch_hint(w_conv)
+    assert [c for c in calls if c[0] is not None] == [(w_small.data_ptr(), w_small.numel() * 4)]
+    monkeypatch.setattr(ops, "PREFETCH_SMALL_BYTES", 16 << 10)
+    ops._pf_last[0] = w_conv.data_ptr()
     # a freed successor: dropped
     key = w_small.data_ptr()
     del w_long, seq, w, a, b
