@@ -238,3 +238,29 @@ def test_sdxl_size_controlnet_forward_and_step():
         assert torch.isfinite(got).all() and torch.equal(got, cur)
         assert torch.isfinite(fused).all() and cosine(fused, cur) >= 0.9999, cosine(fused, cur)
     ops.check_split_timeouts(torch.device(DEV))
+
+
+def test_two_stream_helpers_keep_scratch_apart():
+    """What lets two models run side by side on two streams: inside split_counters_held() a reset neither clears the
+    counter arena nor hands its slices out again; inside side_branch() the shared GroupNorm scratch is another buffer."""
+    from katz_amd import ops
+
+    dev = torch.device(DEV)
+    ops.split_counters_reset(dev)
+    a = ops._arena_ints(dev, 4)
+    a.fill_(7)
+    with ops.split_counters_held():
+        ops.split_counters_reset(dev)            # what a model's forward does at its start
+        b = ops._arena_ints(dev, 4)
+        assert a.tolist() == [7, 7, 7, 7] and b.tolist() == [0, 0, 0, 0]
+        assert b.data_ptr() == a.data_ptr() + 16
+    ops.split_counters_reset(dev)
+    c = ops._arena_ints(dev, 4)
+    assert c.data_ptr() == a.data_ptr() and c.tolist() == [0, 0, 0, 0]
+    main_ws = ops._workspace(1024, dev)
+    with ops.side_branch():
+        side_ws = ops._workspace(1024, dev)
+        assert side_ws.data_ptr() != main_ws.data_ptr()
+        assert ops._workspace(1024, dev).data_ptr() == side_ws.data_ptr()
+    assert ops._workspace(1024, dev).data_ptr() == main_ws.data_ptr()
+    ops.split_counters_reset(dev)
