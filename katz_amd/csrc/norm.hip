@@ -141,7 +141,17 @@ __global__ __launch_bounds__(GN_THREADS) void gn_apply_nhwc(const bf16_t* __rest
     double s = 0.0, q = 0.0;
     if (grp < g.G) {
       const float2* pw = reinterpret_cast<const float2*>(ws) + ((size_t)n * g.G + grp) * g.splits;
-      for (int k = part; k < g.splits; k += FT) { const float2 v = pw[k]; s += (double)v.x; q += (double)v.y; }
+      // four loads in flight per thread (a load per addition would pay the memory latency splits / FT times in a row);
+      // the additions keep their order
+      int k = part;
+      for (; k + 3 * FT < g.splits; k += 4 * FT) {
+        const float2 v0 = pw[k], v1 = pw[k + FT], v2 = pw[k + 2 * FT], v3 = pw[k + 3 * FT];
+        s += (double)v0.x; q += (double)v0.y;
+        s += (double)v1.x; q += (double)v1.y;
+        s += (double)v2.x; q += (double)v2.y;
+        s += (double)v3.x; q += (double)v3.y;
+      }
+      for (; k < g.splits; k += FT) { const float2 v = pw[k]; s += (double)v.x; q += (double)v.y; }
     }
     s_ps[tid] = s; s_pq[tid] = q;
     __syncthreads();
