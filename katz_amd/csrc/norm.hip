@@ -498,6 +498,7 @@ KH_EXPORT int kh_group_norm_static_bf16(const void* x, void* y, const void* gamm
   const int64_t need = kh_group_norm_workspace_bytes(N, C, HW, G, channels_last);
   if (need < 0) return (int)need;
   if ((uint64_t)need > GN_STATIC_WS_BYTES) return KH_ERR_TOO_LARGE;
+  if (!x || !y) return KH_ERR_INVALID_ARG;   // before the first device call (the rest is checked by kh_group_norm_bf16)
   float* ws = nullptr;
   const int rc = gn_static_workspace(&ws);
   if (rc != KH_OK) return rc;

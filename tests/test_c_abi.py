@@ -53,3 +53,23 @@ def test_argument_validation_needs_no_gpu():
     assert lib.kh_group_norm_workspace_bytes(2, 30, 64, 4, 1) == -1   # C % G != 0
     assert lib.kh_layer_norm_bf16(16, 16, None, None, 4, 4096, 1e-5, None) == -2  # D > 2048
     assert lib.kh_lora_shrink_bf16(16, 16, 16, 16, 4, 72, 32, None) == -2        # K % 64
+    # the query projection with the text cross-attention in its epilogue
+    assert lib.kh_lora_linear_xattn_ok(2048, 1280, 1280, 128, 1024, 77) == 1
+    assert lib.kh_lora_linear_xattn_ok(2048, 1280, 1280, 128, 1024, 128) == 0      # more than 96 keys
+    assert lib.kh_lora_linear_xattn_ok(2048, 1280, 1280, 128, 1000, 77) == 0       # T % 128
+    assert lib.kh_lora_linear_xattn_bf16(*([None] * 13), 1e-5, *([None] * 3), 2048, 1280, 1280, 128, 1024, 77,
+                                         1280, 1280, 1280, 98560, 98560, 0.125, 0, None) == -1
+    assert lib.kh_lora_linear_xattn_bf16(*([16] * 13), 1e-5, *([16] * 3), 2048, 1280, 1280, 128, 1024, 128,
+                                         1280, 1280, 1280, 163840, 163840, 0.125, 0, None) == -1
+    # convolution with the next GroupNorm's statistics, and the norm's apply pass on them
+    assert lib.kh_conv3x3_gn_splits(2, 32, 32, 1280, 1280, 1, 32) == 16
+    assert lib.kh_conv3x3_gn_splits(2, 64, 64, 640, 640, 1, 32) == 32
+    assert lib.kh_conv3x3_gn_splits(2, 32, 32, 1280, 1280, 1, 7) == 0              # groups do not divide the channels
+    assert lib.kh_conv3x3_gn_splits(2, 128, 128, 320, 4, 1, 2) == 0                # no 160-column tiles
+    assert lib.kh_conv3x3_gn_stats_nhwc_bf16(*([None] * 7), 2, 32, 32, 1280, 1280, 1, 32, None) == -1
+    assert lib.kh_conv3x3_gn_stats_nhwc_bf16(16, 16, None, None, None, 16, 16, 2, 32, 32, 1280, 1280, 1, 7, None) == -1
+    assert lib.kh_group_norm_apply_bf16(None, None, None, None, None, None, 16, 2, 1280, 1024, 32, 1e-5, 1, None) == -1
+    assert lib.kh_group_norm_apply_bf16(16, 16, None, None, None, 16, 16, 2, 1290, 1024, 32, 1e-5, 1, None) == -1
+    # the entry point that allocates nothing: its limit and its arguments are checked before the first device call
+    assert lib.kh_group_norm_static_bf16(16, 16, None, None, None, 4096, 4096, 65536, 32, 1e-5, 0, 1, None) == -4
+    assert lib.kh_group_norm_static_bf16(None, 16, None, None, None, 2, 320, 64, 32, 1e-5, 0, 1, None) == -1
