@@ -12,8 +12,10 @@ Prints ONE JSON line: ms per step (value), the adapter-free step beside it, a `r
 dominant kernel (the fused LoRA GEMM: algorithmic FLOPs of all its launches in a step, counted on the adapters'
 true ranks, / the sum of their durations, each launch timed with its own HIP event pair on the launch stream),
 `rooflines` for the other kernels of the path (attention and convolution against the MFMA peak; GroupNorm,
-LayerNorm, residual injection and the segmented shrink / expand against the HBM peak) and a `cpu_baseline`
-object (the fp32 CPU oracle timed on a bounded sample and extrapolated by FLOPs).
+LayerNorm, residual injection and the segmented shrink / expand against the HBM peak; one summary row each, their
+per-shape tables go to gpurun_out/bench_details.json) and a `cpu_baseline` object (ONE full step of the fp32 CPU oracle on
+the host's cores, with the FLOP-scaled mid-block sample beside it as a cross-check).  The figures the LoRA-cost target
+is stated on (adapter-free step, overhead fraction) sit inside `roofline`.
 """
 from __future__ import annotations
 
@@ -214,9 +216,9 @@ def sgmv_rooflines(dev):
     return out
 
 
-def cpu_baseline(cores):
-    """fp32 CPU oracle on a bounded sample: the UNet mid block (resnet, 10 transformer blocks with both
-    LoRAs, resnet; batch 2, 32x32 latent) -- scaled to a whole step by algorithmic FLOPs."""
+def cpu_baseline_sample(cores, reps=3):
+    """Cross-check of the full-step baseline below: the fp32 CPU oracle's UNet mid block (resnet, 10 transformer blocks
+    with both LoRAs, resnet; batch 2, 32x32 latent), to be scaled to a whole step by algorithmic FLOPs."""
     import torch
     from oracle import blocks as OB
 
@@ -245,12 +247,63 @@ def cpu_baseline(cores):
     with torch.no_grad():
         blk(x, temb, ctx)  # warm-up
         ts = []
-        for _ in range(7):   # ~15 s of CPU work in all
+        for _ in range(reps):
             t0 = time.perf_counter()
             blk(x, temb, ctx)
             ts.append(time.perf_counter() - t0)
     ts.sort()
     return ts[len(ts) // 2], flops
+
+
+def cpu_baseline_full_step(cores):
+    """ONE full step of BASELINE.json configs[2] on the fp32 CPU oracle (oracle/unet_sdxl.py, the restatement of the
+    reference's diffusers path: 2.57 B parameters, both LoRAs unmerged on all 722 linears, the 9 + 1 ControlNet residuals),
+    on `cores` threads.  The weights are random (their values do not change the time): the model is created without
+    torch's initialisers and filled from one pool of normal numbers scaled per tensor, which takes seconds instead of
+    a minute.  Returns the seconds of the one timed step."""
+    import torch
+    from oracle.unet_sdxl import UNet2DConditionModel as OracleUNet, UNetConfig as OracleCfg
+
+    torch.set_num_threads(cores)
+    with torch.device("meta"):
+        model = OracleUNet(OracleCfg.sdxl())
+    model = model.to_empty(device="cpu").eval()
+    g = torch.Generator().manual_seed(0)
+    pool = torch.randn(1 << 24, generator=g)
+
+    def fill(t, std):
+        flat = t.view(-1)
+        for o in range(0, flat.numel(), pool.numel()):
+            n = min(pool.numel(), flat.numel() - o)
+            torch.mul(pool[:n], std, out=flat[o:o + n])
+
+    with torch.no_grad():
+        for name, p in model.named_parameters():
+            if p.dim() > 1:
+                fill(p.data, (3.0 * p[0].numel()) ** -0.5)      # the spread of torch's default Linear / Conv2d init
+            elif name.endswith("weight"):
+                p.fill_(1.0)                                     # norm scales
+            else:
+                p.zero_()
+        for k, m in enumerate(model.lora_linears().values()):
+            for an, r, w in (("r64", 64, 0.8), ("r32", 32, 0.6)):
+                o = (k * 7919 * 64) % (pool.numel() - r * (m.in_features + m.out_features))
+                down = (pool[o:o + r * m.in_features] * 0.02).view(r, m.in_features)
+                up = (pool[o + r * m.in_features:o + r * (m.in_features + m.out_features)] * 0.02).view(m.out_features, r)
+                m.add_adapter(an, down, up, None, w)
+        model.set_adapters(["r64", "r32"], [0.8, 0.6])
+        rn = lambda *s, std=1.0: torch.randn(*s, generator=g) * std
+        x, ctx = rn(2, 4, 128, 128), rn(2, 77, 2048)
+        added = dict(text_embeds=rn(2, 1280), time_ids=torch.tensor([[1024.0, 1024, 0, 0, 1024, 1024]] * 2))
+        shapes = [(320, 128)] * 3 + [(320, 64), (640, 64), (640, 64), (640, 32), (1280, 32), (1280, 32)]
+        down = [rn(2, c, h, h, std=0.1) for c, h in shapes]
+        mid = rn(2, 1280, 32, 32, std=0.1)
+        t0 = time.perf_counter()
+        out = model(x, 500, ctx, added, down, mid)
+        sec = time.perf_counter() - t0
+    if out.shape != (2, 4, 128, 128) or not bool(torch.isfinite(out).all()):
+        raise RuntimeError("cpu_baseline: the oracle step did not produce a finite [2,4,128,128] output")
+    return sec
 
 
 PROFILE_SUMMARY = ROOT / "profiles" / "kernels_at_baseline_shapes_mfma_busy_and_hbm_traffic.txt"
@@ -514,6 +567,8 @@ def loop_bench(args):
                                "beside the UNet's down and mid blocks" if step.overlap else "") +
                                "; conditioning embedding computed once per loop",
                    "global_batch": 2, "parallelism": "single GPU"},
+        "roofline": {"kernel": "whole loop (every kernel of ControlNet + UNet + scheduler step); per-kernel rooflines are in the default mode's line",
+                     "loop_ms": round(med, 2), "ms_per_step": round(med / args.loop_steps, 3), "loop_steps": args.loop_steps},
         "loop_ms_all": [round(x, 2) for x in times], "output_finite": finite,
         "kernel_ms_per_step": {k: {"launches": v[0], "ms": round(v[1], 3)} for k, v in sorted(by_kernel.items())},
         "kernel_ms_sum_per_step": round(sum(v[1] for v in by_kernel.values()), 3),
@@ -692,6 +747,13 @@ def main():
     ]
     rooflines += sgmv_rooflines(dev)
 
+    details = {"rooflines": rooflines, "lora_gemm_by_shape": shape_rows, "shrink_by_shape": shrink_rows,
+               "traffic_note": "HBM-side bytes (read + written) of the largest launch as recorded in "
+                               f"profiles/{PROFILE_SUMMARY.name} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of `bench.py "
+                               f"--kernel-probe`), not measured by this run; row: {traffic_src}"}
+    short = lambda r: {k: r[k] for k in ("M", "N", "K", "launches", "avg_us", "ms_per_step", "frac")} | (
+        {"xattn_keys": r["attention_keys_in_epilogue"]} if "attention_keys_in_epilogue" in r else {}) | (
+        {"layers": r["layers_per_launch"]} if r["layers_per_launch"] > 1 else {})
     result = {
         "metric": "unet_step_ms_1024_2lora_1cn",
         "value": round(ms, 3),
@@ -708,33 +770,50 @@ def main():
         "config": {"workload": "SDXL UNet2DConditionModel step, latent [2,4,128,128] (1024x1024, CFG batch 2), "
                                "2 LoRAs (r64 s0.8 + r32 s0.6) on 722 linears, 1 ControlNet residual set, HIP graph",
                    "global_batch": 2, "parallelism": "single GPU"},
-        "adapter_free_ms_per_step": round(ms_free, 3),
-        "lora_overhead_frac": round(ms / ms_free - 1.0, 4),
-        "step_tflop": round(step_flops / 1e12, 3),
-        "step_tflops_per_s": round(step_flops / (ms * 1e-3) / 1e12, 1),
-        "output_finite": finite,
-        "roofline": {"kernel": "LoRA linear GEMM kernels lora_gemm_pipe / _wide / _ksplit (base GEMM + LoRA delta, all launches of one step, shrink launches included)",
+        "roofline": {"kernel": "LoRA linear GEMMs (lora_gemm_pipe / _wide / _ksplit: base GEMM + LoRA delta), all launches of "
+                               "one step incl. the shrink launches",
                      "bound": "mfma", "achieved": round(achieved_tf, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved_tf / PEAK_BF16_TFLOPS, 4), "traffic": traffic,
-                     "traffic_note": "NOT measured by this run: HBM-side bytes (read + written) of the largest launch as recorded in "
-                                     f"profiles/{PROFILE_SUMMARY.name} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of `bench.py --kernel-probe`); row: {traffic_src}",
+                     "traffic_from": f"profiles/{PROFILE_SUMMARY.name} (largest launch; recorded, not measured by this run)",
+                     "adapter_free_ms_per_step": round(ms_free, 3),
+                     "lora_overhead_frac": round(ms / ms_free - 1.0, 4),
                      "rank_counted": true_rank,
                      "launches_per_step": len(gemm_ms), "shrink_launches_per_step": len(shrink_calls),
-                     "shrink_ms_per_step": round(shrink_ms, 3), "avg_launch_us": round(gemm_total_ms / len(gemm_ms) * 1e3, 2),
-                     "algorithmic_gflop_per_step": round(gemm_flops / 1e9, 1), "by_shape": shape_rows[:10],
-                     "shrink_by_shape": shrink_rows[:6]},
-        "rooflines": rooflines,
-        "kernel_ms_per_step": {k: {"launches": v[0], "ms": round(v[1], 3)} for k, v in sorted(by_kernel.items())},
+                     "shrink_ms_per_step": round(shrink_ms, 3), "gemm_ms_per_step": round(sum(gemm_ms), 3),
+                     "avg_launch_us": round(gemm_total_ms / len(gemm_ms) * 1e3, 2),
+                     "algorithmic_gflop_per_step": round(gemm_flops / 1e9, 1),
+                     "step_tflop": round(step_flops / 1e12, 3), "output_finite": finite,
+                     "by_shape": [short(r) for r in shape_rows[:9]]},
+        "rooflines": [{k: r[k] for k in ("kernel", "bound", "achieved", "unit", "frac") if k in r} |
+                      {k: r[k] for k in ("launches_per_step", "ms_per_step") if k in r} |
+                      {"kernel": r["kernel"].split("(")[0].split(":")[0].strip()[:48]} |
+                      ({"by_shape_frac": {b["shape"].split(",")[0]: b["frac"] for b in r["by_shape"][:3]}} if "by_shape" in r else {})
+                      for r in rooflines],
+        "kernel_ms_per_step": {k: round(v[1], 3) for k, v in sorted(by_kernel.items())},
     }
     if not args.no_cpu_baseline:
         cores = host_cores()
-        sec, sample_flops = cpu_baseline(cores)
+        t0 = time.perf_counter()
+        full_s = cpu_baseline_full_step(cores)
+        build_s = time.perf_counter() - t0 - full_s
+        sec, sample_flops = cpu_baseline_sample(cores)
         est_ms = sec * 1e3 * step_flops / sample_flops
-        result["cpu_baseline"] = {"value": round(est_ms, 1), "unit": "ms", "cores": cores, "kind": "port, extrapolated",
+        print(f"bench.py: cpu baseline: model set-up {build_s:.1f} s, full step {full_s:.2f} s, mid-block sample {sec:.2f} s",
+              file=sys.stderr)
+        result["cpu_baseline"] = {"value": round(full_s * 1e3, 1), "unit": "ms", "cores": cores, "kind": "port",
                                   "cpu": cpu_model(), "host_cpus_visible": os.cpu_count(),
-                                  "sample": f"fp32 oracle, UNet mid block (2 resnets + 10 transformer blocks with both "
-                                            f"LoRAs, batch 2, 32x32) = {sample_flops / 1e12:.3f} TFLOP in {sec:.2f} s "
-                                            f"(median of 7) on {cores} threads, EXTRAPOLATED by FLOPs to the {step_flops / 1e12:.2f} TFLOP step"}
+                                  "sample": f"ONE full step of the same workload on the fp32 oracle (2 LoRAs unmerged, 9 + 1 "
+                                            f"residuals), {cores} threads, timed once without warm-up; cross-check: the UNet mid "
+                                            f"block ({sample_flops / 1e12:.3f} TFLOP in {sec:.2f} s, median of 3) scaled by FLOPs "
+                                            f"to the {step_flops / 1e12:.2f} TFLOP step = {est_ms:.0f} ms"}
+        details["cpu_baseline_cross_check_ms"] = round(est_ms, 1)
+    out_dir = ROOT / "gpurun_out"
+    try:
+        out_dir.mkdir(exist_ok=True)
+        (out_dir / "bench_details.json").write_text(json.dumps(details, indent=1))
+        result["details_file"] = "gpurun_out/bench_details.json"
+    except OSError:
+        pass
     print(json.dumps(result))
 
 

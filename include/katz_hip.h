@@ -164,8 +164,11 @@ int kh_lora_split_timeouts(int32_t* count, int clear);
  * XCD that shares a weight block would fetch it again; measured on the SDXL feed-forward output projection (M 2048,
  * N 1280, K 5120): 53 us with the weights in HBM, 45 us prefetched, 42 us cache-resident.  The hints are consumed by
  * that one launch (also under graph capture, where the pointers are recorded: the ranges must stay allocated while the
- * graph is replayed).  weights == NULL or bytes < 128 clears what is pending.  At most 2 GiB per range.  Wrong hints
- * cost bandwidth, never correctness; the ranges must be readable. */
+ * graph is replayed).  A call of that family drops whatever is pending when it returns, also when it refuses its
+ * arguments before launching: a hint never survives to a later, unrelated launch.  weights == NULL or bytes < 128
+ * clears what is pending.  At most 2 GiB per range.  Wrong hints cost bandwidth, never correctness; the ranges must be
+ * readable.  The Python host issues hints only inside one forward of one model and only at that model's own tensors
+ * (katz_amd/ops.py weight_prefetch_scope), so a captured graph of a model records hinted pointers into that model only. */
 int kh_set_weight_prefetch(const void* weights, int64_t bytes);
 /* How many kernel launches kh_lora_linear_split_bf16 makes for this shape when counters are given (1 or 2; negative:
  * KH_ERR_*).  No counterpart in the reference; for callers that account per launch (benchmarks). */

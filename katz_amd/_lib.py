@@ -85,6 +85,11 @@ def load() -> ctypes.CDLL:
     return lib
 
 
+def is_loaded() -> bool:
+    """True once load() has succeeded in this process (for code that must not trigger the load itself)."""
+    return _lib is not None
+
+
 def check(code: int, what: str) -> None:
     if code != 0:
         msg = load().kh_error_string(int(code)).decode()

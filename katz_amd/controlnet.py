@@ -156,24 +156,25 @@ class ControlNetModel(nn.Module):
         ctx = encoder_hidden_states.to(torch.bfloat16).contiguous()
         if sample.is_cuda:
             ops.split_counters_reset(sample.device)   # one fill per step clears the in-launch shrinks' counters
-        if self._ctx_kv is None:
-            self.prepare()
-        self._ctx_kv.run(ctx)
-        emb = self._embed(sample, timestep, added_cond_kwargs)
-        temb_act = F.silu(emb)
-        self._temb_proj.run(temb_act)   # time_emb_proj of all resnets, batched per width
-        if cond_embedding is None:
-            cond_embedding = self.embed_condition(controlnet_cond)
-        # conv_in(sample) + embedding (:780-783): the add runs in the convolution's epilogue
-        sample = self.conv_in(sample, residual=cond_embedding)
-        skips = (sample,)
-        for blk in self.down_blocks:
-            sample, res = blk(sample, temb_act, ctx)
-            skips += res
-        sample = self.mid_block(sample, temb_act, ctx)
-        zc_cache = self._zero_conv_cache
-        down = [conv1x1_scaled(s, zc, conditioning_scale, zc_cache) for s, zc in zip(skips, self.controlnet_down_blocks)]
-        mid = conv1x1_scaled(sample, self.controlnet_mid_block, conditioning_scale, zc_cache)
+        with ops.weight_prefetch_scope(self):   # hints are learned from, and point into, this model's own last pass
+            if self._ctx_kv is None:
+                self.prepare()
+            self._ctx_kv.run(ctx)
+            emb = self._embed(sample, timestep, added_cond_kwargs)
+            temb_act = F.silu(emb)
+            self._temb_proj.run(temb_act)   # time_emb_proj of all resnets, batched per width
+            if cond_embedding is None:
+                cond_embedding = self.embed_condition(controlnet_cond)
+            # conv_in(sample) + embedding (:780-783): the add runs in the convolution's epilogue
+            sample = self.conv_in(sample, residual=cond_embedding)
+            skips = (sample,)
+            for blk in self.down_blocks:
+                sample, res = blk(sample, temb_act, ctx)
+                skips += res
+            sample = self.mid_block(sample, temb_act, ctx)
+            zc_cache = self._zero_conv_cache
+            down = [conv1x1_scaled(s, zc, conditioning_scale, zc_cache) for s, zc in zip(skips, self.controlnet_down_blocks)]
+            mid = conv1x1_scaled(sample, self.controlnet_mid_block, conditioning_scale, zc_cache)
         if not return_dict:
             return (down, mid)
         return {"down_block_res_samples": down, "mid_block_res_sample": mid}

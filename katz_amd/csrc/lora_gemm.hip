@@ -479,10 +479,19 @@ void kh_take_weight_prefetch(LoraGemmParams& p) {
   g_pf_n = 0;
 }
 
+namespace {
+// Every entry point that can carry the hint holds one of these from its first line: however the call ends -- a refused
+// argument included -- nothing stays pending for an unrelated later launch, by when the hinted range may have been freed.
+struct PendingPrefetchDropped {
+  ~PendingPrefetchDropped() { g_pf_n = 0; }
+};
+}  // namespace
+
 // See include/katz_hip.h for the contract.
 KH_EXPORT int kh_lora_linear_bf16(const void* x, const void* w, const void* bias, const void* a_cat,
                                   const void* b_cat, const float* col_scale, const void* residual, void* y,
                                   int64_t M, int64_t N, int64_t K, int64_t R, int flags, void* stream) {
+  const PendingPrefetchDropped drop_pending_hint;
   if (!x || !w || !y || M <= 0 || N <= 0 || K <= 0 || R < 0) return KH_ERR_INVALID_ARG;
   if (R > 0 && (!a_cat || !b_cat || !col_scale)) return KH_ERR_INVALID_ARG;
   if (K % 8 != 0 || N % 8 != 0 || R % 32 != 0) return KH_ERR_UNSUPPORTED;
@@ -523,6 +532,7 @@ KH_EXPORT int kh_lora_linear_bf16(const void* x, const void* w, const void* bias
 KH_EXPORT int kh_lora_linear_pre_bf16(const void* x, const void* w, const void* bias, const void* t, int64_t ldt,
                                       int64_t n_split, const void* b_cat, const void* residual, void* y, int64_t M,
                                       int64_t N, int64_t K, int64_t R, int flags, void* stream) {
+  const PendingPrefetchDropped drop_pending_hint;
   if (!x || !w || !y || !t || !b_cat || M <= 0 || N <= 0 || K <= 0 || R <= 0 || ldt < R) return KH_ERR_INVALID_ARG;
   if (n_split < 0 || (n_split > 0 && (n_split % 128 != 0 || N % n_split != 0 || ldt < (N / n_split) * R)))
     return KH_ERR_INVALID_ARG;
@@ -588,6 +598,7 @@ KH_EXPORT int kh_lora_linear_split_bf16(const void* x, const void* w, const void
                                         const float* col_scale, const void* b_cat, void* t_scratch, int32_t* counters,
                                         const void* residual, void* y, int64_t M, int64_t N, int64_t K, int64_t R,
                                         int64_t n_split, int flags, void* stream) {
+  const PendingPrefetchDropped drop_pending_hint;
   if (!x || !w || !y || !a_cat || !col_scale || !b_cat || !t_scratch || M <= 0 || N <= 0 || K <= 0 || R <= 0)
     return KH_ERR_INVALID_ARG;
   if (n_split < 0 || (n_split > 0 && (n_split % 128 != 0 || N % n_split != 0))) return KH_ERR_INVALID_ARG;
@@ -628,6 +639,7 @@ static int lora_linear_norm_impl(const void* x, const void* w, const void* bias,
                                  const float* ln_c2, const float* ln_ca1, const float* ln_ca2, float ln_eps,
                                  float* stats_out, int64_t M, int64_t N, int64_t K, int64_t R, int64_t n_split,
                                  int flags, void* stream, const XAttnArgs* xa) {
+  const PendingPrefetchDropped drop_pending_hint;
   if (!x || !w || (!y && !xa) || M <= 0 || N <= 0 || K <= 0 || R < 0) return KH_ERR_INVALID_ARG;
   if (R > 0 && (!a_cat || !col_scale || !b_cat || !t_scratch)) return KH_ERR_INVALID_ARG;
   if (ln_part != nullptr && (!ln_c1 || !ln_c2 || bias != nullptr || (R > 0 && (!ln_ca1 || !ln_ca2)))) return KH_ERR_INVALID_ARG;
@@ -744,6 +756,7 @@ int conv3x3_params(LoraGemmParams& p, const void* x, const void* w, const void* 
 KH_EXPORT int kh_conv3x3_nhwc_bf16(const void* x, const void* w, const void* bias, const void* residual, void* y,
                                    int64_t Nb, int64_t H, int64_t W, int64_t Cin, int64_t Cout, int64_t stride,
                                    void* stream) {
+  const PendingPrefetchDropped drop_pending_hint;
   LoraGemmParams p;
   if (const int rc = conv3x3_params(p, x, w, bias, residual, y, Nb, H, W, Cin, Cout, stride); rc != KH_OK) return rc;
   kh_take_weight_prefetch(p);
@@ -764,6 +777,7 @@ KH_EXPORT int64_t kh_conv3x3_gn_splits(int64_t Nb, int64_t H, int64_t W, int64_t
 KH_EXPORT int kh_conv3x3_gn_stats_nhwc_bf16(const void* x, const void* w, const void* bias, const void* residual,
                                             const void* add_nc, void* y, float* partials, int64_t Nb, int64_t H, int64_t W,
                                             int64_t Cin, int64_t Cout, int64_t stride, int64_t G, void* stream) {
+  const PendingPrefetchDropped drop_pending_hint;
   if (!partials || G <= 0 || Cout % G != 0) return KH_ERR_INVALID_ARG;
   LoraGemmParams p;
   if (const int rc = conv3x3_params(p, x, w, bias, residual, y, Nb, H, W, Cin, Cout, stride); rc != KH_OK) return rc;

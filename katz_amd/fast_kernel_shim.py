@@ -18,8 +18,15 @@ Differences that a caller can see, all on the side of failing loudly:
   * a failed launch raises (the reference drops the cudaError_t, group_norm.cu:167-169);
   * the kernels compute on bf16 storage.  bf16 tensors are used as they are; fp16 tensors (the reference's
     GroupNorm.forward casts to fp16 before the call, normalization.py:88-90) are converted on the way in and out.
-group_norm_fp16 allocates nothing (kh_group_norm_static_bf16 keeps its partial sums in a per-GPU array of the
-library), so unlike the reference's op (two torch::empty per call, group_norm.cu:240-242) it can be captured.
+group_norm_fp16 allocates nothing on bf16 tensors (kh_group_norm_static_bf16 keeps its partial sums in a per-GPU array
+of the library), so unlike the reference's op (two torch::empty per call, group_norm.cu:240-242) it can be captured.
+Limits of that array, and what the shim does about them:
+  * ONE array per GPU: calls that overlap on one GPU (two streams) race on it -- call the op from one stream per GPU;
+  * its device address is looked up on the first call per device, which must not happen under capture: `install()`
+    makes that call for the current device when a GPU is there; on another device run the op once eagerly first;
+  * it holds 256 KiB of partial sums (about N <= 1024 samples at 32 groups, NHWC).  Larger shapes, which the reference's
+    op serves, go through kh_group_norm_bf16 with a torch-allocated workspace instead (that path allocates on first use
+    and when it grows: warm it up before capturing).
 """
 from __future__ import annotations
 
@@ -63,7 +70,14 @@ def group_norm_fp16(x, y, eps, num_groups, activation, weight, bias, affine, cha
                                        None if beta is None else beta.data_ptr(), None,
                                        n, c, h * w, int(num_groups), float(eps), 1 if activation == "silu" else 0,
                                        1 if nhwc else 0, _stream())
-    if rc != 0:
+    if rc == -4:     # KH_ERR_TOO_LARGE: more partial sums than the library's per-GPU array holds
+        from . import ops
+
+        try:
+            ops.group_norm(xb, int(num_groups), gamma, beta, float(eps), activation, out=yb)
+        except (_lib.KatzHipError, ValueError, TypeError) as e:
+            raise RuntimeError(f"group_norm_fp16: {e}") from e
+    elif rc != 0:
         raise RuntimeError(f"group_norm_fp16: {lib.kh_error_string(int(rc)).decode()}")
     if yb is not y:
         y.copy_(yb)
@@ -101,3 +115,7 @@ def install() -> None:
         lib.impl("fast_gelu_mul_fp16", fast_gelu_mul_fp16, "CUDA")
         _registered = lib
     sys.modules.setdefault("fast_kernel", sys.modules[__name__])
+    if torch.cuda.is_available() and not torch.cuda.is_current_stream_capturing():
+        # the first call per device resolves the address of the library's per-GPU array: do it here, outside any capture
+        x = torch.zeros(1, 8, 1, 1, dtype=BF16, device="cuda")
+        group_norm_fp16(x, torch.empty_like(x), 1e-5, 1, "none", None, None, False, True)

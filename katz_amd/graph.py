@@ -26,7 +26,9 @@ class GraphedUNetStep:
     rewritten; adapters on 3x3 convolutions repack on any change).
     After anything that repacks or re-derives buffers -- a different set of active adapters, `load_lora_into_unet` /
     `unload_lora`, `fuse_lora` / `unfuse_lora`, `patch_on_lora`, `load_state_dict`, another batch size or resolution --
-    build a new GraphedUNetStep; replaying the old one would compute with the old buffers."""
+    build a new GraphedUNetStep; replaying the old one would compute with the old buffers.
+    Weight-prefetch hints recorded in the graph point at tensors of this UNet only (they are learned and issued inside
+    one forward of one model, ops.weight_prefetch_scope), so freeing ANOTHER model never invalidates this graph."""
 
     def __init__(self, unet, sample, timestep, encoder_hidden_states, added_cond_kwargs,
                  down_block_additional_residuals: Optional[Sequence[torch.Tensor]] = None,
@@ -102,6 +104,10 @@ class GraphedDenoiseStep:
     beside the UNet's down and mid blocks, which do not read its residuals; the UNet waits for it right after its mid
     block.  Same kernels, same results bit for bit; the 50-step loop at 1024x1024 measured 1769 -> 1610 ms.
 
+    Build it (and call `run`) from a stream that is neither capturing nor itself a fork inside someone else's capture:
+    with overlap on, the capture forks a second stream from the capturing one, and a fork from an already forked stream
+    inside a capture has crashed the runtime at capture end; the constructor refuses to start under a capture.
+
     hoist_cond_embedding: the ControlNet's conditioning embedding depends on the image only, which is the same in every
     step; it is computed once per `run` instead of inside the graph (the reference recomputes it every step,
     controlnet.py:780-783; same value, bit for bit).  Everything the notes on GraphedUNetStep say about rebuilding after
@@ -112,6 +118,9 @@ class GraphedDenoiseStep:
                  warmup: int = 2, fuse_tail: bool = True, overlap: Optional[bool] = None):
         from . import ops
 
+        if latents.is_cuda and torch.cuda.is_current_stream_capturing():
+            raise RuntimeError("GraphedDenoiseStep captures a graph of its own (with a forked stream when overlap is on): "
+                               "build it outside any stream capture")
         self.unet, self.controlnet = unet, controlnet
         self.overlap = (os.getenv("KATZ_CN_OVERLAP", "1") != "0") if overlap is None else bool(overlap)
         self._cn_stream = torch.cuda.Stream(device=latents.device) if self.overlap else None

@@ -44,40 +44,66 @@ def _req(t: torch.Tensor, dtype, name: str) -> None:
 # --------------------------------------------------------------------------------------- K1
 # Weight prefetch: a linear / convolution launch can touch the operands of the launch that follows it (weights, and the
 # packed adapter matrices), so that those wait in the memory-side cache (kh_set_weight_prefetch).  Which operands follow
-# which is learned from the previous pass over the model: a launch with weights W hints at what followed W last time.
-# The table holds weak references only: a hint never keeps a tensor alive, and a dead one is dropped instead of hinted.
+# which is learned from the previous pass over the SAME model: hints are learned and issued only inside
+# `weight_prefetch_scope(model)`, which the UNet / ControlNet forward opens around its body.  Every model has a table of
+# its own and a scope starts with no predecessor, so a pair (launch, next launch) never spans two models or two
+# forwards: a captured graph of a model therefore holds hinted pointers to that model's own tensors only, which it needs
+# alive anyway.  Launches outside any scope (a layer or an op called on its own) neither learn nor hint.
+# The tables hold weak references only: a hint never keeps a tensor alive, and a dead one is dropped instead of hinted.
 WEIGHT_PREFETCH = os.getenv("KATZ_WEIGHT_PREFETCH", "1") != "0"
 PREFETCH_MIN_K = int(os.getenv("KATZ_PREFETCH_MIN_K", "2560"))
 PREFETCH_SMALL_BYTES = int(os.getenv("KATZ_PREFETCH_SMALL_BYTES", str(4 << 20)))
-_pf_next: dict = {}     # data_ptr of a launch's weights -> weak references to (weights, a_cat, b_cat) of the launch after it
+_pf_tables: "weakref.WeakKeyDictionary" = weakref.WeakKeyDictionary()   # model -> its table (below)
+_pf_next: list = [None]  # table of the running scope: data_ptr of a launch's weights -> weak refs to (weights, a_cat, b_cat) of the launch after it
 _pf_last: list = [None]
 _pf_shrink_a: list = [None]   # A_cat of a separate shrink launch, for the hint of the GEMM it belongs to
+
+
+@contextlib.contextmanager
+def weight_prefetch_scope(owner):
+    """One forward of one model: launches inside learn from / hint at `owner`'s own table, starting without a predecessor;
+    on exit the enclosing scope (normally none) is restored and whatever hint is still pending in the library is dropped."""
+    table = _pf_tables.get(owner)
+    if table is None:
+        table = _pf_tables[owner] = {}
+    saved = (_pf_next[0], _pf_last[0], _pf_shrink_a[0])
+    _pf_next[0], _pf_last[0], _pf_shrink_a[0] = table, None, None
+    try:
+        yield table
+    finally:
+        _pf_next[0], _pf_last[0], _pf_shrink_a[0] = saved
+        if WEIGHT_PREFETCH and _lib.is_loaded():
+            _lib.load().kh_set_weight_prefetch(None, 0)
 
 
 def _weight_prefetch_hint(weight: torch.Tensor, a_cat: Optional[torch.Tensor] = None,
                           b_cat: Optional[torch.Tensor] = None) -> None:
     if not WEIGHT_PREFETCH:
         return
+    lib = _lib.load()
+    # whatever an earlier call left pending (its launch was refused before it took the hint) must not reach this launch
+    lib.kh_set_weight_prefetch(None, 0)
+    table = _pf_next[0]
     if a_cat is None and _pf_shrink_a[0] is not None:
         a_cat = _pf_shrink_a[0]()
     _pf_shrink_a[0] = None
+    if table is None:
+        return
     key = weight.data_ptr()
     last = _pf_last[0]
     if last is not None and last != key:
-        _pf_next[last] = tuple(None if t is None else weakref.ref(t) for t in (weight, a_cat, b_cat))
-        if len(_pf_next) > 65536:     # models come and go: forget everything rather than grow without bound
-            _pf_next.clear()
+        table[last] = tuple(None if t is None else weakref.ref(t) for t in (weight, a_cat, b_cat))
+        if len(table) > 65536:     # weights come and go: forget everything rather than grow without bound
+            table.clear()
     _pf_last[0] = key
-    nxt = _pf_next.get(key)
+    nxt = table.get(key)
     if nxt is None:
         return
     live = [None if r is None else r() for r in nxt]
     w_next = live[0]
     if w_next is None:                # the tensor that followed last time is gone
-        del _pf_next[key]
+        del table[key]
         return
-    lib = _lib.load()
-    lib.kh_set_weight_prefetch(None, 0)
     # The prefetch is not free for the launch that carries it (its own first operands queue behind it: up to 3.5 us
     # for 26 MB), so weights are only hinted where meeting them in HBM costs more than that: long rows (K >= 2560,
     # the feed-forward output projections and the 3x3 convolutions), whose launches are latency-bound on their

@@ -521,39 +521,40 @@ class UNet2DConditionModel(nn.Module):
         if sample.is_cuda:
             ops.split_counters_reset(sample.device)   # one fill per step clears the in-launch shrinks' counters
 
-        if self._ctx_kv is None:
-            self.prepare()
-        self._ctx_kv.run(ctx)  # K/V projections of all cross-attentions, grouped
-        emb = self._embed(sample, timestep, added_cond_kwargs)
-        temb_act = F.silu(emb)
-        self._temb_proj.run(temb_act)   # time_emb_proj of all resnets, batched per width
-        sample = self.conv_in(sample)
-        skips = (sample,)
-        for blk in self.down_blocks:
-            sample, res = blk(sample, temb_act, ctx)
-            skips += res
-        sample = self.mid_block(sample, temb_act, ctx)
+        with ops.weight_prefetch_scope(self):   # hints are learned from, and point into, this model's own last pass
+            if self._ctx_kv is None:
+                self.prepare()
+            self._ctx_kv.run(ctx)  # K/V projections of all cross-attentions, grouped
+            emb = self._embed(sample, timestep, added_cond_kwargs)
+            temb_act = F.silu(emb)
+            self._temb_proj.run(temb_act)   # time_emb_proj of all resnets, batched per width
+            sample = self.conv_in(sample)
+            skips = (sample,)
+            for blk in self.down_blocks:
+                sample, res = blk(sample, temb_act, ctx)
+                skips += res
+            sample = self.mid_block(sample, temb_act, ctx)
 
-        ready = getattr(self, "before_residuals", None)
-        if ready is not None:   # the residuals come from another stream (a ControlNet run beside the down blocks)
-            ready()
-        extra = self._residual_sets(down_block_additional_residuals, len(skips))
-        if mid_block_additional_residual is not None:
-            mids = mid_block_additional_residual
-            mids = list(mids) if isinstance(mids, (list, tuple)) else [mids]
-            mids = [m.to(torch.bfloat16).contiguous(memory_format=torch.channels_last) for m in mids]
-            if not sample.is_contiguous(memory_format=torch.channels_last):
-                sample = sample.contiguous(memory_format=torch.channels_last)
-            sample = ops.residual_add_(sample, mids)
+            ready = getattr(self, "before_residuals", None)
+            if ready is not None:   # the residuals come from another stream (a ControlNet run beside the down blocks)
+                ready()
+            extra = self._residual_sets(down_block_additional_residuals, len(skips))
+            if mid_block_additional_residual is not None:
+                mids = mid_block_additional_residual
+                mids = list(mids) if isinstance(mids, (list, tuple)) else [mids]
+                mids = [m.to(torch.bfloat16).contiguous(memory_format=torch.channels_last) for m in mids]
+                if not sample.is_contiguous(memory_format=torch.channels_last):
+                    sample = sample.contiguous(memory_format=torch.channels_last)
+                sample = ops.residual_add_(sample, mids)
 
-        for blk in self.up_blocks:
-            n = len(blk.resnets)
-            res, skips = skips[-n:], skips[:-n]
-            ex, extra = extra[-n:], extra[:-n]
-            sample = blk(sample, res, ex, temb_act, ctx)
-        sample = self.conv_norm_silu(sample)
-        if not getattr(self, "defer_conv_out", False):   # the denoise-loop graph runs conv_out fused with the scheduler step
-            sample = self.conv_out(sample)
+            for blk in self.up_blocks:
+                n = len(blk.resnets)
+                res, skips = skips[-n:], skips[:-n]
+                ex, extra = extra[-n:], extra[:-n]
+                sample = blk(sample, res, ex, temb_act, ctx)
+            sample = self.conv_norm_silu(sample)
+            if not getattr(self, "defer_conv_out", False):   # the denoise-loop graph runs conv_out fused with the scheduler step
+                sample = self.conv_out(sample)
         if cross_attention_kwargs is not None:
             self.scale_lora_layers(1.0)  # unscale_lora_layers, unet_2d_condition.py:1334-1336
         if not return_dict:

@@ -73,3 +73,31 @@ def test_argument_validation_needs_no_gpu():
     # the entry point that allocates nothing: its limit and its arguments are checked before the first device call
     assert lib.kh_group_norm_static_bf16(16, 16, None, None, None, 4096, 4096, 65536, 32, 1e-5, 0, 1, None) == -4
     assert lib.kh_group_norm_static_bf16(None, 16, None, None, None, 2, 320, 64, 32, 1e-5, 0, 1, None) == -1
+
+
+def test_a_refused_call_drops_the_pending_weight_prefetch_hint():
+    """kh_set_weight_prefetch queues up to three ranges for the next launch of the linear / convolution family (a fourth
+    is refused).  A call of that family that refuses its arguments must not leave them pending for an unrelated later
+    launch: afterwards three new ranges can be queued again.  No device call is made."""
+    from katz_amd import _lib
+
+    if not _lib.LIB_PATH.exists():
+        pytest.skip("libkatz_hip.so not built")
+    lib = _lib.load()
+    refused = (
+        lambda: lib.kh_lora_linear_bf16(None, None, None, None, None, None, None, None, 1, 8, 8, 0, 0, None),
+        lambda: lib.kh_lora_linear_pre_bf16(*([None] * 3), None, 0, 0, *([None] * 3), 1, 8, 32, 32, 0, None),
+        lambda: lib.kh_lora_linear_split_bf16(*([None] * 10), 1, 8, 64, 32, 0, 0, None),
+        lambda: lib.kh_lora_linear_norm_bf16(*([None] * 15), 1e-5, None, 1, 8, 64, 0, 0, 0, None),
+        lambda: lib.kh_conv3x3_nhwc_bf16(None, None, None, None, None, 1, 8, 8, 32, 8, 1, None),
+        lambda: lib.kh_conv3x3_gn_stats_nhwc_bf16(*([None] * 7), 2, 32, 32, 1280, 1280, 1, 32, None),
+    )
+    assert lib.kh_set_weight_prefetch(None, 0) == 0
+    for call in refused:
+        for _ in range(3):
+            assert lib.kh_set_weight_prefetch(4096, 1 << 20) == 0
+        assert lib.kh_set_weight_prefetch(4096, 1 << 20) == -4          # three are pending
+        assert call() < 0
+        for _ in range(3):                                               # ... and gone after the refused call
+            assert lib.kh_set_weight_prefetch(4096, 1 << 20) == 0
+        assert lib.kh_set_weight_prefetch(None, 0) == 0

@@ -56,6 +56,27 @@ def test_group_norm_fp16_reference_call(dtype):
 
 
 @pytest.mark.gpu
+def test_group_norm_fp16_serves_shapes_beyond_the_static_scratch():
+    """More partial sums than the library's per-GPU array holds (here 1100 samples x 32 groups: 275 KiB against 256):
+    the reference's op has no such limit, so the drop-in goes through the workspace form instead of refusing."""
+    import katz_amd.fast_kernel_shim as shim
+    from katz_amd import _lib
+    from oracle import ops as O
+
+    shim.install()
+    print("fast_kernel.group_norm_fp16 N=1100", flush=True)
+    assert _lib.load().kh_group_norm_workspace_bytes(1100, 64, 4, 32, 1) > 256 * 1024
+    g = torch.Generator().manual_seed(5)
+    x = bf16_round(torch.randn(1100, 64, 2, 2, generator=g) + 0.2)
+    w, b = bf16_round(1 + 0.1 * torch.randn(64, generator=g)), bf16_round(0.1 * torch.randn(64, generator=g))
+    xd = x.to("cuda:0", BF).contiguous(memory_format=torch.channels_last)
+    y = torch.empty_like(xd)
+    torch.ops.fast_kernel.group_norm_fp16(xd, y, 1e-5, 32, "silu", w.to("cuda:0", BF), b.to("cuda:0", BF), True, False)
+    torch.cuda.synchronize()
+    assert_close_rel(y, O.group_norm(x, 32, w, b, 1e-5, "silu"), 2e-2, "fast_kernel.group_norm_fp16 beyond the scratch")
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_fast_gelu_mul_fp16_reference_call(dtype):
     """activations.py:145: fast_gelu_mul_fp16(proj_2(h), proj_1(h)) = gelu_tanh(x) * m, callee-allocated."""

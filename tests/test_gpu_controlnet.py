@@ -172,10 +172,100 @@ def test_graphed_denoise_step_matches_eager_loop(pair):
                 assert cosine(got, e) >= 0.9995, cosine(got, e)
 
 
+def test_config5_loop_with_two_loras_against_the_oracle_loop():
+    """Configuration 5 with its adapters at tiny widths: ControlNet -> UNet carrying TWO active LoRAs (weights 0.8 / 0.6)
+    -> guidance 7.5 -> Euler, 6 steps, against oracle.euler.denoise_loop over the oracle models with the same adapters:
+    the eager loop, and GraphedDenoiseStep (one graph per step, conv_out + guidance + Euler fused) with the ControlNet
+    beside the UNet's down blocks on a second stream and in front of it on one stream.  Cosine >= 0.999 each; the two
+    graph forms agree bit for bit, and the unfused graph equals the eager loop bit for bit."""
+    import katz_amd.layers as L
+    from katz_amd import ops
+    from katz_amd.controlnet import ControlNetModel
+    from katz_amd.graph import GraphedDenoiseStep
+    from katz_amd.scheduler import EulerDiscreteScheduler, denoise_loop
+    from katz_amd.unet_2d_condition import UNet2DConditionModel, UNetConfig
+
+    say("config-5 loop with two LoRAs")
+    torch.manual_seed(4)
+    cfg = OracleCfg.tiny()
+    o_cn = OracleControlNet(cfg).eval()
+    _randomise_zero_convs(o_cn, 2)
+    round_module_to_bf16_(o_cn)
+    o_unet = round_module_to_bf16_(OracleUNet(cfg).eval())
+    L.SKIP_INIT = True
+    try:
+        p_cn, p_unet = ControlNetModel(UNetConfig.tiny()), UNet2DConditionModel(UNetConfig.tiny())
+    finally:
+        L.SKIP_INIT = False
+    p_cn.load_state_dict(o_cn.state_dict(), strict=True)
+    p_unet.load_state_dict(o_unet.state_dict(), strict=True)
+    p_cn, p_unet = p_cn.to_runtime(DEV, BF), p_unet.to_runtime(DEV, BF)
+    g = torch.Generator().manual_seed(11)
+    lora = {}
+    for name, m in o_unet.lora_linears().items():
+        for an, r in (("r16", 16), ("r8", 8)):
+            d = bf16_round(torch.randn(r, m.in_features, generator=g) * 0.05)
+            u = bf16_round(torch.randn(m.out_features, r, generator=g) * 0.05)
+            m.add_adapter(an, d, u)
+            lora.setdefault(an, {})[f"unet.{name}.lora.down.weight"] = d
+            lora[an][f"unet.{name}.lora.up.weight"] = u
+    o_unet.set_adapters(["r16", "r8"], [0.8, 0.6])
+    for an in ("r16", "r8"):
+        p_unet.load_lora_into_unet(lora[an], adapter_name=an)
+    p_unet.set_adapters(["r16", "r8"], [0.8, 0.6])
+
+    x, ctx, added, cond = _inputs(cfg, 16, 77, 12)
+    sd = dict(beta_start=0.00085, beta_end=0.012, beta_schedule="scaled_linear", timestep_spacing="leading", steps_offset=1)
+    osch, psch = OracleScheduler(**sd), EulerDiscreteScheduler(**sd)
+    osch.set_timesteps(6)
+    psch.set_timesteps(6, device=DEV)
+    lat0 = bf16_round(x[:1] * osch.init_noise_sigma)
+    added_d = {k: v.to(DEV) for k, v in added.items()}
+
+    def o_model(inp, t):
+        with torch.no_grad():
+            inp = bf16_round(inp)
+            d, m = o_cn(inp, t, ctx, cond, 0.5, added)
+            return bf16_round(o_unet(inp, t, ctx, added, [bf16_round(v) for v in d], bf16_round(m)))
+
+    def p_model(inp, t):
+        with torch.no_grad():
+            d, m = p_cn(inp, t.reshape(1), ctx.to(DEV), cond.to(DEV), 0.5, added_cond_kwargs=added_d)
+            return p_unet(inp, t.reshape(1), ctx.to(DEV), added_cond_kwargs=added_d, down_block_additional_residuals=d,
+                          mid_block_additional_residual=m, return_dict=False)[0]
+
+    ref = oracle_loop(o_model, osch, lat0.float(), 7.5)
+    # the adapters matter: without them the oracle loop ends somewhere else
+    o_unet.set_adapters([], [])
+    ref_free = oracle_loop(o_model, osch, lat0.float(), 7.5)
+    o_unet.set_adapters(["r16", "r8"], [0.8, 0.6])
+    assert cosine(ref_free, ref) < 0.9999, cosine(ref_free, ref)
+    eager = denoise_loop(p_model, psch, lat0.to(DEV), 7.5)
+    torch.cuda.synchronize()
+    assert torch.isfinite(eager).all() and cosine(eager, ref) >= 0.999, cosine(eager, ref)
+    got = {}
+    for overlap in (True, False):
+        for fuse_tail in (True, False):
+            step = GraphedDenoiseStep(p_unet, p_cn, lat0.to(DEV), ctx.to(DEV), added_d, cond.to(DEV), 7.5, 0.5,
+                                      fuse_tail=fuse_tail, overlap=overlap)
+            assert step.overlap == overlap and step.fuse_tail == fuse_tail
+            out = step.run(lat0.to(DEV), psch)          # raises if an in-launch shrink wait ran out
+            again = step.run(lat0.to(DEV), psch)
+            torch.cuda.synchronize()
+            assert torch.isfinite(out).all() and torch.equal(out, again)
+            assert cosine(out, ref) >= 0.999, (overlap, fuse_tail, cosine(out, ref))
+            got[(overlap, fuse_tail)] = out
+    assert torch.equal(got[(True, True)], got[(False, True)]) and torch.equal(got[(True, False)], got[(False, False)])
+    assert torch.equal(got[(True, False)].contiguous(), eager.contiguous())
+    ops.check_split_timeouts(torch.device(DEV))
+
+
 def test_sdxl_size_controlnet_forward_and_step():
     """ONE full-size ControlNet forward (SDXL widths, conditioning image [2,3,1024,1024], latents [2,4,128,128]) feeding
-    one full-size UNet step: residual shapes of unet_2d_condition.py:539-563, finite values, bit-reproducible, and the
-    captured ControlNet -> UNet -> guidance + Euler graph equal to the eager sequence.  Random-init weights, the
+    one full-size UNet step WITH configuration 5's two adapters (rank 64 weight 0.8 + rank 32 weight 0.6 on all 722
+    linears): residual shapes of unet_2d_condition.py:539-563, finite values, bit-reproducible, the adapters change the
+    result, and the captured ControlNet -> UNet -> guidance + Euler graph equal to the eager sequence (the ControlNet
+    beside the UNet's in-launch-shrink kernels on a second stream, or in front of them).  Random-init weights, the
     ControlNet built with from_unet and non-zero "zero" convolutions; no oracle at this size (the CPU model needs
     minutes), parity of the same code is checked at small widths above and against the reference's own outputs in
     test_gpu_reference_fixture.py."""
@@ -197,6 +287,12 @@ def test_sdxl_size_controlnet_forward_and_step():
                 m.weight.copy_(torch.randn(m.weight.shape, generator=g, device=DEV) * (0.5 / m.weight[0].numel() ** 0.5))
     unet, cn = unet.to_runtime(DEV, BF), cn.to_runtime(DEV, BF)
     rn = lambda *s: torch.randn(*s, generator=g, device=DEV).to(BF)
+    lins = unet.lora_linears()
+    assert len(lins) == 722
+    for name, rank in (("r64", 64), ("r32", 32)):
+        for lin in lins.values():
+            lin.add_adapter(name, (rn(rank, lin.in_features).float() * 0.02).to(BF),
+                            (rn(lin.out_features, rank).float() * 0.02).to(BF), alpha=None)
     lat = rn(1, 4, 128, 128)
     x = torch.cat([lat, lat])
     ctx = rn(2, 77, 2048)
@@ -211,8 +307,11 @@ def test_sdxl_size_controlnet_forward_and_step():
         for a, b in zip(list(d) + [m], list(d2) + [m2]):
             assert torch.isfinite(a).all() and torch.equal(a, b)
             assert a.float().abs().max() > 0
+        eps_free = unet(x, t, ctx, added_cond_kwargs=added, down_block_additional_residuals=d, mid_block_additional_residual=m).sample
+        unet.set_adapters(["r64", "r32"], [0.8, 0.6])
         eps = unet(x, t, ctx, added_cond_kwargs=added, down_block_additional_residuals=d, mid_block_additional_residual=m).sample
-        assert eps.shape == (2, 4, 128, 128) and torch.isfinite(eps).all()
+        assert eps.shape == (2, 4, 128, 128) and torch.isfinite(eps).all() and torch.isfinite(eps_free).all()
+        assert not torch.equal(eps, eps_free) and cosine(eps, eps_free) > 0.5     # the adapters are in the step
         # one step of the loop: eager sequence against the captured graph
         sch = EulerDiscreteScheduler(beta_start=0.00085, beta_end=0.012, beta_schedule="scaled_linear",
                                      timestep_spacing="leading", steps_offset=1)

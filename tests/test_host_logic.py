@@ -438,15 +438,8 @@ def test_bench_refuses_more_than_one_gpu():
     assert r.returncode == 2 and "ONE GPU" in r.stderr
 
 
-def test_weight_prefetch_hints_are_learned_from_the_previous_pass(monkeypatch):
-    """ops._weight_prefetch_hint: the first pass over a sequence of launches gives no hints; the second hints, at launch
-    i, the operands of launch i + 1 - weights only for long rows (K >= 2560 or a 3x3 kernel) or below the size limit,
-    adapter matrices always; a tensor that has been freed is dropped instead of hinted."""
-    import gc
-
+def _fake_prefetch_lib(monkeypatch, calls):
     from katz_amd import ops
-
-    calls = []
 
     class FakeLib:
         def kh_set_weight_prefetch(self, ptr, nbytes):
@@ -454,39 +447,108 @@ def test_weight_prefetch_hints_are_learned_from_the_previous_pass(monkeypatch):
             return 0
 
     monkeypatch.setattr(ops._lib, "load", lambda: FakeLib())
+    monkeypatch.setattr(ops._lib, "is_loaded", lambda: True)
     monkeypatch.setattr(ops, "WEIGHT_PREFETCH", True)
+
+
+def test_weight_prefetch_hints_are_learned_from_the_previous_pass(monkeypatch):
+    """ops._weight_prefetch_hint inside one model's scope: the first pass over a sequence of launches gives no hints; the
+    second hints, at launch i, the operands of launch i + 1 - weights only for long rows (K >= 2560 or a 3x3 kernel) or
+    below the size limit, adapter matrices always; a tensor that has been freed is dropped instead of hinted."""
+    import gc
+
+    from katz_amd import ops
+
+    calls = []
+    _fake_prefetch_lib(monkeypatch, calls)
     monkeypatch.setattr(ops, "PREFETCH_SMALL_BYTES", 16 << 10)
-    ops._pf_next.clear()
-    ops._pf_last[0] = None
+    model = torch.nn.Identity()
     w_small = torch.zeros(8, 1280)             # K 1280 and 40 KB, above the size limit set here: not hinted
     w_long = torch.zeros(8, 5120)              # K 5120: hinted
     w_conv = torch.zeros(4, 3, 3, 320)         # 9 * 320 = 2880: hinted
     a_cat, b_cat = torch.zeros(128, 5120), torch.zeros(8, 128)
     seq = [(w_small, None, None), (w_long, a_cat, b_cat), (w_conv, None, None)]
-    for w, a, b in seq:
-        ops._weight_prefetch_hint(w, a, b)
-    assert calls == []                          # nothing known on the first pass
-    for w, a, b in seq:
-        ops._weight_prefetch_hint(w, a, b)
-    hinted = [c for c in calls if c[0] is not None]
-    assert hinted == [(w_long.data_ptr(), w_long.numel() * 4), (a_cat.data_ptr(), a_cat.numel() * 4),
-                      (b_cat.data_ptr(), b_cat.numel() * 4), (w_conv.data_ptr(), w_conv.numel() * 4)]
-    # what followed w_conv last time is w_small (the wrap-around), K 1280: its entry exists but hints nothing
-    assert ops._pf_next[w_conv.data_ptr()][0]() is w_small
-    # ... until the size limit admits it (the default admits the d x d layers)
+    hinted = lambda: [c for c in calls if c[0] is not None]
+    with ops.weight_prefetch_scope(model) as table:
+        for w, a, b in seq:
+            ops._weight_prefetch_hint(w, a, b)
+    assert hinted() == []                       # nothing known on the first pass
+    with ops.weight_prefetch_scope(model) as table2:
+        assert table2 is table                  # the same model: the same table
+        for w, a, b in seq:
+            ops._weight_prefetch_hint(w, a, b)
+    assert hinted() == [(w_long.data_ptr(), w_long.numel() * 4), (a_cat.data_ptr(), a_cat.numel() * 4),
+                        (b_cat.data_ptr(), b_cat.numel() * 4), (w_conv.data_ptr(), w_conv.numel() * 4)]
+    # a forward starts without a predecessor: the last launch of a pass learns nothing about the next pass's first
+    assert w_conv.data_ptr() not in table and set(table) == {w_small.data_ptr(), w_long.data_ptr()}
+    # the size limit admits small weights whatever their K (the default admits the d x d layers)
     monkeypatch.setattr(ops, "PREFETCH_SMALL_BYTES", 64 << 10)
     calls.clear()
-    ops._pf_last[0] = None
-    ops._weight_prefetch_hint(w_conv)
-    assert [c for c in calls if c[0] is not None] == [(w_small.data_ptr(), w_small.numel() * 4)]
-    monkeypatch.setattr(ops, "PREFETCH_SMALL_BYTES", 16 << 10)
-    ops._pf_last[0] = w_conv.data_ptr()
+    with ops.weight_prefetch_scope(model):
+        ops._weight_prefetch_hint(w_conv)
+        ops._weight_prefetch_hint(w_small)      # learned: w_small follows w_conv
+    calls.clear()
+    with ops.weight_prefetch_scope(model):
+        ops._weight_prefetch_hint(w_conv)
+    assert hinted() == [(w_small.data_ptr(), w_small.numel() * 4)]
     # a freed successor: dropped
     key = w_small.data_ptr()
     del w_long, seq, w, a, b
     gc.collect()
     calls.clear()
-    ops._weight_prefetch_hint(w_small)
-    assert [c for c in calls if c[0] is not None] == [] and key not in ops._pf_next
-    ops._pf_next.clear()
-    ops._pf_last[0] = None
+    with ops.weight_prefetch_scope(model):
+        ops._weight_prefetch_hint(w_small)
+    assert hinted() == [] and key not in table
+
+
+def test_weight_prefetch_hints_never_cross_models_or_forwards(monkeypatch):
+    """A hinted pointer is baked into a captured graph, so it must belong to the model whose forward issues it: every
+    model learns into a table of its own, a launch outside any model's forward neither learns nor hints, whatever is
+    still pending in the library is cleared before every new hint and at the end of a scope, and a model that is freed
+    takes its table with it."""
+    import gc
+
+    from katz_amd import ops
+
+    calls = []
+    _fake_prefetch_lib(monkeypatch, calls)
+    monkeypatch.setattr(ops, "PREFETCH_SMALL_BYTES", 1 << 30)
+    unet, cnet = torch.nn.Identity(), torch.nn.Identity()
+    wu = [torch.zeros(8, 64) for _ in range(3)]
+    wc = [torch.zeros(8, 64) for _ in range(2)]
+    stray = torch.zeros(8, 64)
+    hinted = lambda: [c[0] for c in calls if c[0] is not None]
+
+    def loop():                     # ControlNet -> UNet -> a stand-alone launch, as an eager denoise loop issues them
+        with ops.weight_prefetch_scope(cnet):
+            for w in wc:
+                ops._weight_prefetch_hint(w)
+        with ops.weight_prefetch_scope(unet):
+            for w in wu:
+                ops._weight_prefetch_hint(w)
+        ops._weight_prefetch_hint(stray)
+
+    loop()
+    assert hinted() == []
+    calls.clear()
+    loop()
+    # inside the ControlNet only its own second weight is hinted, inside the UNet only its own second and third:
+    # nothing of the other model, nothing of the stand-alone launch, and the last launch of a model hints nothing
+    assert hinted() == [wc[1].data_ptr(), wu[1].data_ptr(), wu[2].data_ptr()]
+    tu, tc = ops._pf_tables[unet], ops._pf_tables[cnet]
+    assert set(tu) == {wu[0].data_ptr(), wu[1].data_ptr()} and set(tc) == {wc[0].data_ptr()}
+    assert ops._pf_next[0] is None and ops._pf_last[0] is None
+    # every hint call first clears what may be pending (a launch that was refused never consumed its hint) ...
+    calls.clear()
+    ops._weight_prefetch_hint(stray)
+    assert calls == [(None, 0)]
+    # ... and so does the end of a scope
+    calls.clear()
+    with ops.weight_prefetch_scope(unet):
+        ops._weight_prefetch_hint(wu[0])
+    assert calls[-1] == (None, 0) and hinted() == [wu[1].data_ptr()]
+    # a freed model: its table goes with it
+    n = len(ops._pf_tables)
+    del cnet, tc
+    gc.collect()
+    assert len(ops._pf_tables) == n - 1
