@@ -109,6 +109,27 @@ __device__ __forceinline__ void kh_prefetch_lines(const void* const (&pf)[3], co
 #endif
 }
 
+// The same from waves that have nothing else to do (the idle half of an in-launch shrink workgroup): as many rounds as
+// the ranges need, up to 16 (the first range) / 4 (the others), in a loop.
+__device__ __forceinline__ void kh_prefetch_lines_idle(const void* const (&pf)[3], const uint32_t (&lines)[3], char* wave_lds, int wg, int n_wg,
+                                                       int tid, int nt) {
+#if __HIP_DEVICE_COMPILE__
+  if (pf[0] == nullptr) return;
+  const uint32_t first = ((uint32_t)wg * (uint32_t)nt + (uint32_t)tid) << 7, step = ((uint32_t)n_wg * (uint32_t)nt) << 7;
+#pragma unroll
+  for (int k = 0; k < 3; ++k) {
+    if (pf[k] == nullptr) continue;
+    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(pf[k]), 0, (int)(lines[k] << 7), 0x00020000);
+    const uint32_t bytes = lines[k] << 7;                       // at most 2 GiB
+    uint32_t rounds = (bytes + step - 1) / step;
+    const uint32_t cap = k == 0 ? 16u : 4u;
+    rounds = rounds < cap ? rounds : cap;
+    for (uint32_t r = 0; r < rounds; ++r)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)wave_lds, 4, first + r * step, 0, 0, 0);
+  }
+#endif
+}
+
 // a column tile's pair for one output row, and (from tile 0) zeros in the slots no tile writes
 __device__ __forceinline__ void kh_ln_store_stats(float* part, int row, int M, int tile, int n_tiles, float s, float q) {
   u32x2* dst = reinterpret_cast<u32x2*>(part) + row;

@@ -591,6 +591,24 @@ struct XAttnTile {
   }
 };
 
+using ILTileWide = SCfg<4, 2, 2>;               // in-launch shrink tiles: 64 x 64 ...
+using ILTileNarrow = SCfg<4, 2, 1>;             // ... and 64 x 32 (see il_narrow; a ring of three stages measured no faster)
+constexpr int IL_SHRINK_LDS = ILTileWide::LDS > ILTileNarrow::LDS ? ILTileWide::LDS : ILTileNarrow::LDS;
+constexpr int IL_PF_OFF = IL_SHRINK_LDS;        // in-launch shrink workgroups: LDS offset of their prefetch landing zone (1 KB)
+
+// Weight prefetch of a launch with its own shrink: by the idle waves of the shrink workgroups when the first range is short
+__host__ __device__ inline bool il_prefetch_by_idle_waves(const LoraGemmParams& p) { return p.pf_lines[0] <= ((8u << 20) >> 7); }
+
+// In-launch shrink on 64 x 32 tiles: a single layer (T has R = 128 columns) of which at most the first 96 rank columns are
+// in use (two adapters of ranks 64 + 32, say), short enough in K that its GEMM tiles would otherwise wait for T, and
+// small enough in M that the three tiles per 64 rows fit beside the GEMM tiles.  The GEMM tiles never multiply the
+// columns the shrink leaves unwritten (r_used bounds their K loop).
+__host__ __device__ inline bool il_narrow(const LoraGemmParams& p) {
+  return p.R == 128 && p.ldt == 128 && p.r_used > 0 && p.r_used <= 96 && p.K <= 2560 &&
+         (long)((p.M + 127) / 128) * ((p.N + 127) / 128) + (long)((p.M + 63) / 64) * 3 <= 256;
+}
+__host__ __device__ inline int il_col_tiles(const LoraGemmParams& p) { return il_narrow(p) ? 3 : p.ldt / 64; }
+
 // LNF bit 0: the instantiation can fold a LayerNorm in front of the layer into its epilogue (ln_part); bit 1: it can write
 // the row statistics for one behind it (st_part).  The plain one (0) carries none of that code.
 // XA: the output tile is an attention's queries and the epilogue runs the cross-attention on it (XAttnTile).
@@ -603,14 +621,35 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
     // then one arrival per tile on the counter of the GEMM row block the tile belongs to.  They have the lowest
     // block ids, so they are resident before any workgroup that waits for them.
     if ((int)blockIdx.x < pin.il_blocks) {
-      const int gx = (pin.M + 63) / 64, gy = pin.ldt / 64;   // T has ldt columns (several layers' ranks side by side)
+      // T has ldt columns (several layers' ranks side by side, R each).  Tiles are 64 rows x 64 columns, or -- for a single
+      // layer of which only the first 96 of the 128 rank columns are in use -- 64 x 32: three tiles per 64 rows instead of
+      // two, each with 3/4 of the operand bytes of a 64 x 64 one.  The GEMM workgroups wait for T at the end of their K
+      // loop, and a short layer's shrink tile is not done by then: what a tile streams through its 160 KB of LDS sets
+      // when T arrives, and 96 tiles still find a CU each beside 160 GEMM tiles
+      const bool narrow = il_narrow(pin);
+      const int gx = (pin.M + 63) / 64, gy = il_col_tiles(pin);
       if ((int)blockIdx.x >= gx * gy) return;               // padding to a multiple of 8 (the XCD map of the rest)
       const int bx = blockIdx.x % gx, by = blockIdx.x / gx;
       ShrinkParams sp;
       sp.x = pin.x; sp.a_cat = pin.a_cat; sp.col_scale = pin.col_scale; sp.t = const_cast<bf16_t*>(pin.t_ext);
       sp.M = pin.M; sp.K = pin.K; sp.R = pin.ldt;
       if (LNF & 1) { sp.ln_part = pin.ln_part; sp.ln_ca1 = pin.ln_ca1; sp.ln_ca2 = pin.ln_ca2; sp.ln_eps = pin.ln_eps; }
-      lora_shrink_tile<SCfg<4, 2, 2>, true, C::NT>(sp, bx, by, smem);
+      // The tile is the work of waves 0..3.  Waves 4..7 touch the next launch's weights instead (towards the memory-side
+      // cache, see LoraGemmParams::pf), so that no GEMM wave's first operands queue behind that duty, and end: a barrier
+      // waits for the surviving waves only.  They start when most of the tile's own loads are out (T's arrival is what the
+      // GEMM workgroups of a short layer wait for: nothing may queue in front of it), and wait for their own loads (into
+      // 256 bytes each behind the tile's rings) before they end, so that this workgroup's LDS is not handed on with loads
+      // still landing in it.
+      if (threadIdx.x >= 256) {
+        if (!il_prefetch_by_idle_waves(pin)) return;
+        __builtin_amdgcn_s_sleep(127);   // 8128 clocks: measured against 1, 40, 160 and 254 (23.87 / 24.0 / 24.06 / 24.1 / 25.4 ms per step)
+        kh_prefetch_lines_idle(pin.pf, pin.pf_lines, smem + IL_PF_OFF + (__builtin_amdgcn_readfirstlane(threadIdx.x >> 6) - 4) * 256,
+                               (int)blockIdx.x, gx * gy, (int)threadIdx.x - 256, 256);
+        __builtin_amdgcn_s_waitcnt(0);
+        return;
+      }
+      if (narrow) lora_shrink_tile<ILTileNarrow, true, 256>(sp, bx * 64, by * 32, smem);
+      else lora_shrink_tile<ILTileWide, true, 256>(sp, bx * 64, by * 64, smem);
       __builtin_amdgcn_s_waitcnt(0);                          // this thread's write-through stores have completed
       __syncthreads();
       if (threadIdx.x == 0)
@@ -619,9 +658,11 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
     }
   }
   const int bid = IL ? (int)blockIdx.x - pin.il_blocks : (int)blockIdx.x;
-  // the next launch's weights, towards the memory-side cache (see LoraGemmParams::pf); not from the 256x128 tiles that run
-  // beside their shrink: with a folded LayerNorm they have no register to spare, and a kernel with scratch loses more
-  if (!(IL && C::BM == 256) && blockIdx.y == 0)
+  // the next launch's weights, towards the memory-side cache (see LoraGemmParams::pf); in a launch that carries its own
+  // shrink the idle waves of the shrink workgroups do that (above) unless the range is long: a CU keeps only so many
+  // missing lines in flight, and 29 MB of convolution weights from 64 CUs took 25 us.  (Not from the 256x128 tiles that run
+  // beside their shrink: with a folded LayerNorm they have no register to spare, and a kernel with scratch loses more.)
+  if ((!IL || (C::BM != 256 && !il_prefetch_by_idle_waves(pin))) && blockIdx.y == 0)
     kh_prefetch_lines(pin.pf, pin.pf_lines, smem + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) * (C::UX / C::NW) * 1024, bid,
                       (int)gridDim.x - (IL ? pin.il_blocks : 0), threadIdx.x, C::NT);
   if (pin.grp != nullptr) {  // grouped launch: this workgroup's layer
@@ -891,7 +932,7 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
         constexpr int TPB = BM / 64;                                                   // 64-row shrink tiles per row block
         const int gx = (M + 63) / 64, rt = gx - TPB * m_blk < TPB ? gx - TPB * m_blk : TPB;
         k_loop2<C, CONV, true>(smem, d, rs, KT, KT1, lane, wave, wm, wn, l32, lh, sw, acc, ConvGeom{0, 0},
-                               p.il_cnt + m_blk, rt * (p.ldt / 64), p.il_cnt + (p.M + 127) / 128, half_last);
+                               p.il_cnt + m_blk, rt * il_col_tiles(p), p.il_cnt + (p.M + 127) / 128, half_last);
       } else {
         k_loop2<C, CONV, false>(smem, d, rs, KT, KT1, lane, wave, wm, wn, l32, lh, sw, acc, ConvGeom{p.conv_w, p.conv_cin},
                                 nullptr, 0, nullptr, half_last);
@@ -1164,7 +1205,7 @@ bool plain_ok(const LoraGemmParams& p) { return p.R == 0 || p.t_ext != nullptr; 
 // tiles take a round of CUs first, the GEMM tiles follow as they free up: still shorter than two launches)
 static int il_form(const LoraGemmParams& p) {
   const long tiles = (long)((p.M + 127) / 128) * ((p.N + 127) / 128);
-  const long shr = (long)((p.M + 63) / 64) * (p.ldt / 64);
+  const long shr = (long)((p.M + 63) / 64) * il_col_tiles(p);
   const bool t_ok = p.t_nsplit == 0 ? p.ldt == p.R : (p.N % p.t_nsplit == 0 && p.ldt == (p.N / p.t_nsplit) * p.R && p.t_nsplit % 128 == 0);
   const bool ok = p.R > 0 && p.R % 64 == 0 && p.ldt % 64 == 0 && p.K % 64 == 0 && p.t_ext != nullptr && p.a_cat != nullptr &&
                   p.col_scale != nullptr && p.il_cnt != nullptr && t_ok && p.grp == nullptr && p.sg_mode == 0 && p.conv_cin == 0 &&
@@ -1194,14 +1235,18 @@ KH_EXPORT int kh_lora_split_timeouts(int32_t* count, int clear) {
 
 template <class C>
 static int launch_il(const LoraGemmParams& pin, hipStream_t stream) {
-  using S = SCfg<4, 2, 2>;
   LoraGemmParams p = pin;
   p.m_tiles = (p.M + C::BM - 1) / C::BM;
   p.n_tiles = (p.N + C::BN - 1) / C::BN;
   p.n_chunk = 1;
   p.n_chunks = p.n_tiles;
-  constexpr int LDS = (int)C::LDS_BYTES > S::LDS ? (int)C::LDS_BYTES : S::LDS;
-  p.ln_lds = LDS;
+  // dynamic LDS: the GEMM workgroups' ring and, behind it, their LayerNorm terms (KH_LN_LDS); the shrink workgroups' rings
+  // start at 0 as well and carry their own row statistics inside
+  constexpr int SL = IL_SHRINK_LDS + 1024;    // the shrink workgroups' rings and, behind them, their prefetch landing zone
+  constexpr int LDS = (int)C::LDS_BYTES > SL ? (int)C::LDS_BYTES : SL;
+  constexpr int LDS_LN = (int)C::LDS_BYTES + KH_LN_LDS > SL ? (int)C::LDS_BYTES + KH_LN_LDS : SL;
+  static_assert(LDS_LN <= 160 * 1024, "LDS of one workgroup");
+  p.ln_lds = (int)C::LDS_BYTES;
   double best = 0;
   p.xg_n = 0;
   for (int gm = 1; gm <= 8; gm *= 2) {
@@ -1210,7 +1255,7 @@ static int launch_il(const LoraGemmParams& pin, hipStream_t stream) {
     const double cost = ((double)rm * C::BM + (double)rn * C::BN) * (8.0 * rm * rn) / ((double)p.m_tiles * p.n_tiles);
     if (p.xg_n == 0 || cost < best) { best = cost; p.xg_n = gn; p.xr_m = rm; p.xr_n = rn; }
   }
-  const int shr = ((p.M + 63) / 64) * (p.ldt / 64);
+  const int shr = ((p.M + 63) / 64) * il_col_tiles(p);
   p.il_blocks = (shr + 7) / 8 * 8;
   const unsigned grid = (unsigned)p.il_blocks + 8u * (unsigned)p.xr_m * (unsigned)p.xr_n;
   if (p.xa_k != nullptr) {
@@ -1218,8 +1263,8 @@ static int launch_il(const LoraGemmParams& pin, hipStream_t stream) {
       if (p.res != nullptr || p.st_part != nullptr || p.M % 128 != 0 || p.N % 128 != 0) return KH_ERR_UNSUPPORTED;
       auto go = [&](auto lnf) {
         constexpr int L = decltype(lnf)::value;
-        if (hipError_t e = kh_allow_lds<lora_gemm_pipe_kernel<C, false, true, L, true>>(LDS + KH_LN_LDS); e != hipSuccess) return (int)e;
-        kh_launch(KH_TAG_LORA_GEMM, lora_gemm_pipe_kernel<C, false, true, L, true>, dim3(grid), dim3(C::NT), (size_t)LDS + KH_LN_LDS, stream, p);
+        if (hipError_t e = kh_allow_lds<lora_gemm_pipe_kernel<C, false, true, L, true>>(LDS_LN); e != hipSuccess) return (int)e;
+        kh_launch(KH_TAG_LORA_GEMM, lora_gemm_pipe_kernel<C, false, true, L, true>, dim3(grid), dim3(C::NT), (size_t)LDS_LN, stream, p);
         KH_RETURN_LAST_ERROR();
       };
       return p.ln_part != nullptr ? go(std::integral_constant<int, 1>{}) : go(std::integral_constant<int, 0>{});
@@ -1231,8 +1276,8 @@ static int launch_il(const LoraGemmParams& pin, hipStream_t stream) {
     if (p.st_part != nullptr && p.n_tiles > KH_LN_SLOTS) return KH_ERR_UNSUPPORTED;
     auto go = [&](auto lnf) {
       constexpr int L = decltype(lnf)::value;
-      if (hipError_t e = kh_allow_lds<lora_gemm_pipe_kernel<C, false, true, L>>(LDS + KH_LN_LDS); e != hipSuccess) return (int)e;
-      kh_launch(KH_TAG_LORA_GEMM, lora_gemm_pipe_kernel<C, false, true, L>, dim3(grid), dim3(C::NT), (size_t)LDS + KH_LN_LDS, stream, p);
+      if (hipError_t e = kh_allow_lds<lora_gemm_pipe_kernel<C, false, true, L>>(LDS_LN); e != hipSuccess) return (int)e;
+      kh_launch(KH_TAG_LORA_GEMM, lora_gemm_pipe_kernel<C, false, true, L>, dim3(grid), dim3(C::NT), (size_t)LDS_LN, stream, p);
       KH_RETURN_LAST_ERROR();
     };
     if (p.ln_part != nullptr && p.st_part != nullptr) return go(std::integral_constant<int, 3>{});

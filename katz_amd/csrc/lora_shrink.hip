@@ -27,7 +27,7 @@ namespace {
 template <class C>
 __global__ __launch_bounds__(C::NW * 64) void lora_shrink_kernel(const ShrinkParams p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  lora_shrink_tile<C, false, C::NW * 64>(p, blockIdx.x, blockIdx.y, smem);
+  lora_shrink_tile<C, false, C::NW * 64>(p, (int)blockIdx.x * C::TR * 32, (int)blockIdx.y * C::TC * 32, smem);
 }
 
 template <class C>

@@ -24,54 +24,60 @@ __device__ __forceinline__ void wait_vm() {  // vmcnt = VM, other counters uncon
 }
 __device__ __forceinline__ void wait_lgkm0() { __builtin_amdgcn_s_waitcnt(15 | (7 << 4) | (0 << 8) | (3 << 14)); }
 
-template <int NW_, int TR_, int TC_>
+template <int NW_, int TR_, int TC_, int NS_ = 2>
 struct SCfg {
   static constexpr int NW = NW_, TR = TR_, TC = TC_;
-  static constexpr int NS = 2;                       // stages per wave
+  static constexpr int NS = NS_;                     // stages per wave (2 or 3)
   static constexpr int UNITS = (TR + TC) * 4;        // 8-row DMA units per stage (x rows, then A_cat rows)
   static constexpr int STAGE = UNITS * 1024;         // 64 K-columns: 128-byte rows (whole cache lines), XOR-swizzled
   static constexpr int RING = NW * NS * STAGE;
   static constexpr int LD = TC * 32 + 4;             // padded fp32 row of the partial-sum tile
   static constexpr int PART = NW * TR * 32 * LD * 4;
   static constexpr int LDS = RING > PART ? RING : PART;
-  static_assert(LDS <= 160 * 1024 && UNITS < 64, "LDS / vmcnt budget");
+  static_assert(LDS <= 160 * 1024 && UNITS * (NS - 1) < 64 && (NS == 2 || NS == 3), "LDS / vmcnt budget");
 };
 
-// One output tile (bx, by) of t = bf16((x . A_cat^T) * col_scale).  The block may have more waves than C::NW: the extra
-// ones only join the barriers and the final fold.  WT: the results are stored write-through at agent scope (for
-// readers on other XCDs inside the same launch).
+// One output tile of t = bf16((x . A_cat^T) * col_scale): rows m0 .. m0 + TR*32, rank columns r0 .. r0 + TC*32, by the NTB
+// threads that call it (all live waves of the block: its barriers are workgroup barriers).  NTB may exceed C::NW waves: the
+// extra ones only join the barriers and the final fold.  WT: the results are
+// stored write-through at agent scope (for readers on other XCDs inside the same launch).
+// Operands are read with buffer loads: a byte offset per lane and unit that never changes (row inside the tile, swizzled
+// piece, this wave's first chunk) plus a scalar offset per chunk, so the loop carries no vector address arithmetic.
 template <class C, bool WT, int NTB>   // NTB: threads of the block
-__device__ __forceinline__ void lora_shrink_tile(const ShrinkParams& p, int bx, int by, char* smem) {
+__device__ __forceinline__ void lora_shrink_tile(const ShrinkParams& p, int m0, int r0, char* smem) {
+#if __HIP_DEVICE_COMPILE__
   constexpr int NW = C::NW, TR = C::TR, TC = C::TC, NS = C::NS, UNITS = C::UNITS, STAGE = C::STAGE, LD = C::LD;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31, lh = lane >> 5;
   const bool active = wave < NW;
-  const int m0 = bx * TR * 32, r0 = by * TC * 32;
   const int K = p.K, KC = K / 64;                    // 64-column chunks, dealt to the waves round-robin
   const int n = active ? (KC - wave + NW - 1) / NW : 0;   // chunks wave, wave + NW, ... of this wave
   char* ring = smem + (active ? wave : 0) * (NS * STAGE);
 
   // DMA: lane i of a unit lands in LDS slot i = row i/8, physical piece i%8, which holds logical piece
   // (i%8) ^ ((row/2)%8); the swizzle is applied to the address the lane fetches
-  const bf16_t* src[UNITS];
+  auto clamp32 = [](size_t bytes) { return (int)(uint32_t)(bytes < 0xFFFFFFFFull ? bytes : 0xFFFFFFFFull); };
+  const __amdgpu_buffer_rsrc_t rsx = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(p.x + (size_t)m0 * K), 0,
+                                                                       clamp32((size_t)(p.M - m0) * K * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsa = __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(p.a_cat + (size_t)r0 * K), 0,
+                                                                       clamp32((size_t)(p.R - r0) * K * 2), 0x00020000);
+  uint32_t voff[UNITS];
 #pragma unroll
   for (int u = 0; u < UNITS; ++u) {
     const int ru = u * 8 + (lane >> 3);                // row inside the stacked [x rows | A_cat rows] stage
-    const int pc = ((lane & 7) ^ ((ru >> 1) & 7)) * 8;
-    if (u < TR * 4) {
-      int row = m0 + ru; row = row < p.M ? row : p.M - 1;
-      src[u] = p.x + (size_t)row * K + wave * 64 + pc;
-    } else {
-      int row = r0 + ru - TR * 32; row = row < p.R ? row : p.R - 1;
-      src[u] = p.a_cat + (size_t)row * K + wave * 64 + pc;
-    }
+    const uint32_t pcb = (uint32_t)(((lane & 7) ^ ((ru >> 1) & 7)) * 16);
+    int row = u < TR * 4 ? ru : ru - TR * 32;
+    const int last = u < TR * 4 ? p.M - 1 - m0 : p.R - 1 - r0;
+    row = row < last ? row : last;
+    voff[u] = (uint32_t)row * (uint32_t)K * 2u + (uint32_t)wave * 128u + pcb;
   }
   auto issue = [&](int i) {                            // this wave's i-th chunk
     char* st = ring + (i % NS) * STAGE;
+    const int so = i * (NW * 128);
 #pragma unroll
     for (int u = 0; u < UNITS; ++u)
-      __builtin_amdgcn_global_load_lds((gptr_t)(src[u] + (size_t)i * (NW * 64)), (lptr_t)(st + u * 1024), 16, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(u < TR * 4 ? rsx : rsa, (lptr_t)(st + u * 1024), 16, voff[u], so, 0, 0);
   };
   f32x16 acc[TR][TC];
 #pragma unroll
@@ -88,9 +94,11 @@ __device__ __forceinline__ void lora_shrink_tile(const ShrinkParams& p, int bx, 
   if (p.ln_part != nullptr) ln_stats.load(p.ln_part, m0, p.M, tid);
   if (n > 0) issue(0);
   if (n > 1) issue(1);
+  if (NS > 2 && n > 2) issue(2);
 
   for (int i = 0; i < n; ++i) {
-    if (i + 1 < n) wait_vm<UNITS>(); else wait_vm<0>();   // chunk i has landed; chunk i+1 may be in flight
+    // chunk i has landed; the chunks behind it (at most NS - 1) may be in flight
+    if (NS > 2 && i + 2 < n) wait_vm<2 * UNITS>(); else if (i + 1 < n) wait_vm<UNITS>(); else wait_vm<0>();
     const char* st = ring + (i % NS) * STAGE;
     bf16x8 a[4][TR], b[4][TC];
 #pragma unroll
@@ -128,7 +136,7 @@ __device__ __forceinline__ void lora_shrink_tile(const ShrinkParams& p, int bx, 
   }
   __syncthreads();
   constexpr int COLS = TC * 32, ROWS = TR * 32;
-  for (int i = tid; i < ROWS * COLS / 2; i += (int)blockDim.x) {   // two neighbouring columns per thread
+  for (int i = tid; i < ROWS * COLS / 2; i += NTB) {   // two neighbouring columns per thread
     const int rr = (2 * i) / COLS, c = (2 * i) % COLS;
     float s0 = part[rr * LD + c], s1 = part[rr * LD + c + 1];
 #pragma unroll
@@ -148,6 +156,7 @@ __device__ __forceinline__ void lora_shrink_tile(const ShrinkParams& p, int bx, 
       else *dst = v;
     }
   }
+#endif
 }
 
 }  // namespace

@@ -456,7 +456,7 @@ def lora_linear_norm(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch
     if CALL_LOG is not None:   # one entry per kernel launch
         if R and lib.kh_lora_linear_split_launches(M, N, K, R, n_split, flags) == 2:
             CALL_LOG.append(("lora_shrink", M, K, RT))
-        CALL_LOG.append(("lora_linear", M, N, K, R, bool(geglu), residual is not None))
+        CALL_LOG.append(("lora_linear", M, N, K, R, bool(geglu), residual is not None, ln is not None, stats_out is not None))
     _weight_prefetch_hint(weight, a_cat, b_cat)
     rc = lib.kh_lora_linear_norm_bf16(_ptr(x), _ptr(weight), _ptr(bias), _ptr(a_cat), _ptr(col_scale), _ptr(b_cat), _ptr(t),
                                       _ptr(cnt), _ptr(residual), _ptr(out), _ptr(part), _ptr(c1), _ptr(c2), _ptr(ca1), _ptr(ca2),

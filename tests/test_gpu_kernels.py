@@ -894,6 +894,61 @@ def test_wide_tile_geglu_gate_range():
 
 
 @pytest.mark.parametrize("case", [
+    # (M, N, K, residual, n_split)
+    (2048, 1280, 1280, True, 0),       # the d x d layers: 160 GEMM + 32 shrink workgroups
+    (2048, 1280, 5120, True, 0),       # ff.net.2
+    (1990, 1280, 1280, False, 0),      # ragged rows: the last shrink tile is partly out of range
+    (2048, 3840, 1280, False, 1280),   # stacked q / k / v: T = [M, 3 x 128], one 64 x 96 tile per layer and 64 rows
+])
+def test_lora_linear_split_rank_96_of_128(case):
+    """Two adapters of ranks 64 + 32 packed into 128 rank columns of which the last 32 are padding (r_used = 96): the
+    in-launch shrink then runs on 64 x 96 tiles and leaves T's padding columns unwritten, which the GEMM tiles never
+    multiply.  T is poisoned with NaNs first; results against the oracle, against the two-launch form and (bit for bit)
+    against the call that does not know about the padding."""
+    from katz_amd import ops
+
+    M, N, K, has_res, n_split = case
+    R, RU = 128, 96
+    say("lora_linear_split r_used 96", case)
+    d = dev()
+    g = torch.Generator().manual_seed(M + N + K + 96)
+    parts = N // n_split if n_split else 1
+    x, w, b = randn(g, M, K), randn(g, N, K, std=0.03), randn(g, N)
+    A, B = randn(g, parts * R, K, std=0.05), randn(g, N, R, std=0.05)
+    for j in range(parts):
+        A[j * R + RU:(j + 1) * R] = 0
+    B[:, RU:] = 0
+    res = randn(g, M, N) if has_res else None
+    xd, wd, bd, Ad, Bd = (t.to(d, BF) for t in (x, w, b, A, B))
+    rd = None if res is None else res.to(d, BF)
+    cs = torch.full((parts * R,), 0.7, device=d)
+    assert ops._lib.load().kh_lora_linear_split_launches(M, N, K, R, n_split, (RU // 16) << 16) == 1
+    # every scratch buffer torch hands out next is full of NaNs: what the shrink does not write must never be read
+    for _ in range(3):
+        junk = torch.full((M, parts * R), float("nan"), device=d, dtype=BF)
+        del junk
+    ops.split_counters_reset(d)
+    y = ops.lora_linear_split(xd, wd, bd, Ad, cs, Bd, residual=rd, n_split=n_split, r_used=RU)
+    flag = ops.split_counters_last(d)[-1:].clone()
+    y_again = ops.lora_linear_split(xd, wd, bd, Ad, cs, Bd, residual=rd, n_split=n_split, r_used=RU)
+    y_two = ops.lora_linear_split(xd, wd, bd, Ad, cs, Bd, residual=rd, n_split=n_split, r_used=RU, two_launches=True)
+    y_full = ops.lora_linear_split(xd, wd, bd, Ad, cs, Bd, residual=rd, n_split=n_split)
+    torch.cuda.synchronize()
+    assert int(flag) == 0 and torch.isfinite(y.float()).all()
+    assert torch.equal(y, y_again) and torch.equal(y, y_full)
+    # the two-launch form differs only by the fp32 summation order inside the shrink: a handful of last-bit differences
+    assert (y != y_two).float().mean().item() < 5e-3
+    xf, wf, bfl, Af, Bf = (t.float().cpu() for t in (xd, wd, bd, Ad, Bd))
+    step = n_split if n_split else N
+    for j in range(parts):
+        rows = slice(j * step, (j + 1) * step)
+        ref = O.lora_linear(xf, wf[rows], bfl[rows], [(Af[j * R:(j + 1) * R], Bf[rows], 0.7)],
+                            residual=None if rd is None else rd.float().cpu()[:, rows])
+        assert_close_rel(y[:, rows], ref, REL_BF16, f"split r_used 96 {case} part {j}")
+    ops.check_split_timeouts(d)
+
+
+@pytest.mark.parametrize("case", [
     # (M, N, K, R, residual, n_split)
     (2048, 1280, 1280, 128, True, 0),      # to_out / attn2.to_q at 32x32: 160 GEMM + 64 shrink workgroups in one launch
     (2048, 1280, 1280, 64, False, 0),

@@ -251,7 +251,8 @@ def test_transformer_with_and_without_the_fold(monkeypatch):
         log0, ops.CALL_LOG = ops.CALL_LOG, None
     torch.cuda.synchronize()
     assert sum(1 for e in log0 if e[0] == "layer_norm") == 6 and not any(e[0] == "layer_norm" for e in log1)
-    assert [e for e in log0 if e[0] != "layer_norm"] == log1, "the same GEMM launches either way"
+    # (a folded launch logs two more fields: whether it folds a norm in front, whether it leaves row statistics)
+    assert [e[:7] for e in log0 if e[0] != "layer_norm"] == [e[:7] for e in log1], "the same GEMM launches either way"
     c1, c0, c10 = cosine(y1, ref), cosine(y0, ref), cosine(y1, y0)
     say(f"  cosine against the oracle: folded {c1:.6f}, separate norms {c0:.6f}; folded against separate {c10:.6f}")
     assert c1 >= 0.9995 and c0 >= 0.9995 and c10 >= 0.9995
