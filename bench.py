@@ -206,6 +206,34 @@ def sgmv_rooflines(dev):
             rows[kind].append({"shape": f"8 requests x {T} rows, K{K} N{N}, ranks {ranks}", "avg_us": round(med * 1e3, 2),
                                "achieved": round(nbytes / (med * 1e-3) / 1e9, 1),
                                "frac": round(nbytes / (med * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)})
+    # the 77-row class (cross-attention to_k / to_v read the text context) as ONE launch over all layers of a width: 120
+    # layers at 1280 (60 blocks x to_k, to_v), x shared, per-layer A / B / y from a pointer table
+    T, K, N, L = 77, 2048, 1280, 120
+    x = rn(8 * T, K)
+    a_alls = [torch.zeros(8, 128, K, device=dev, dtype=bf) for _ in range(L)]
+    b_alls = [torch.zeros(8, N, 128, device=dev, dtype=bf) for _ in range(L)]
+    for a, b in zip(a_alls, b_alls):
+        for i, r in enumerate(ranks):
+            a[i, :r].normal_(0, 0.02, generator=g)
+            b[i, :, :r].normal_(0, 0.02, generator=g)
+    ys = [rn(8 * T, N) for _ in range(L)]
+    ss = torch.arange(0, 9 * T, T, dtype=torch.int32, device=dev)
+    table = ops.sgmv_fused_grouped_table(ys, a_alls, b_alls)
+    for _ in range(2):
+        ops.sgmv_fused_grouped_(ys, x, a_alls, b_alls, ss, sa, rp, sc, T, table=table)
+    torch.cuda.synchronize()
+    ops.profile_begin()
+    for _ in range(5):
+        ops.sgmv_fused_grouped_(ys, x, a_alls, b_alls, ss, sa, rp, sc, T, table=table)
+    lg = sorted(d for _, d in ops.profile_end())
+    assert len(lg) == 5, len(lg)
+    sr = float(sum(ranks))
+    nbytes = 2.0 * (8 * T * K + L * (sr * (K + N) + 2 * 8 * T * N))
+    med = lg[len(lg) // 2]
+    rows["fused"].append({"shape": f"8 requests x {T} rows, K{K} N{N}, {L} layers in one launch (grouped), ranks {ranks}",
+                          "avg_us": round(med * 1e3, 2), "achieved": round(nbytes / (med * 1e-3) / 1e9, 1),
+                          "frac": round(nbytes / (med * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)})
+    del a_alls, b_alls, ys
     out = []
     for kind in ("shrink", "expand", "fused"):
         best = rows[kind][0]
@@ -787,7 +815,7 @@ def main():
         "rooflines": [{k: r[k] for k in ("kernel", "bound", "achieved", "unit", "frac") if k in r} |
                       {k: r[k] for k in ("launches_per_step", "ms_per_step") if k in r} |
                       {"kernel": r["kernel"].split("(")[0].split(":")[0].strip()[:48]} |
-                      ({"by_shape_frac": {b["shape"].split(",")[0]: b["frac"] for b in r["by_shape"][:3]}} if "by_shape" in r else {})
+                      ({"by_shape_frac": {(b["shape"].split(",")[0] + (" grouped" if "grouped" in b["shape"] else "")): b["frac"] for b in r["by_shape"][:4]}} if "by_shape" in r else {})
                       for r in rooflines],
         "kernel_ms_per_step": {k: round(v[1], 3) for k, v in sorted(by_kernel.items())},
     }

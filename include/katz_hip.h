@@ -223,6 +223,15 @@ int kh_sgmv_expand_bf16(const void* t, const void* b_all, void* y, const int32_t
 int kh_sgmv_fused_bf16(const void* x, const void* a_all, const void* b_all, void* y, const int32_t* seg_start,
                        const int32_t* seg_adapter, const int32_t* adapter_rank, const float* adapter_scale,
                        int64_t n_segments, int64_t max_seg_rows, int64_t N, int64_t K, int64_t RP, void* stream);
+/* The same for n_layers layers that read the SAME x with the SAME segments (the to_k / to_v projections of all
+ * cross-attentions of one width read the one text context, diffusers-hf/src/diffusers/models/attention_processor.py:1246-1251)
+ * in one launch: table = n_layers rows of three device pointers {a_all_l, b_all_l, y_l} (8-byte aligned device memory; the
+ * pointed-to arrays as in kh_sgmv_fused_bf16, 16-byte aligned, all layers with the same N, K, RP and adapter table).
+ * A 77-row request gives one layer's launch a few microseconds of traffic; all layers of a width together are bound by
+ * the memory system instead of by the launch.  No counterpart in the reference. */
+int kh_sgmv_fused_grouped_bf16(const void* x, const uint64_t* table, int64_t n_layers, const int32_t* seg_start,
+                               const int32_t* seg_adapter, const int32_t* adapter_rank, const float* adapter_scale,
+                               int64_t n_segments, int64_t max_seg_rows, int64_t N, int64_t K, int64_t RP, void* stream);
 
 /* ---- K3: attention ----------------------------------------------------------------------------
  * o = softmax(q k^T * scale) v per (batch, head); replaces F.scaled_dot_product_attention in

@@ -29,6 +29,7 @@ SIGNATURES = {
     "kh_sgmv_shrink_bf16": (c_int, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
     "kh_sgmv_expand_bf16": (c_int, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P]),
     "kh_sgmv_fused_bf16": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
+    "kh_sgmv_fused_grouped_bf16": (c_int, [_P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
     "kh_attention_bf16": (c_int, [_P, _P, _P, _P] + [_I] * 13 + [c_float, _P]),
     "kh_group_norm_workspace_bytes": (c_int64, [_I, _I, _I, _I, c_int]),
     "kh_group_norm_bf16": (c_int, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, c_float, c_int, c_int, _P]),

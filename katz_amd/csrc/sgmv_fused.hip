@@ -16,6 +16,10 @@
 // Rows / columns of A_a / B_a beyond the adapter's rank are zero by contract, so the padded rank only saves work.
 // Batches with few row blocks deal the column tiles of y to several workgroups (blockIdx.z), each of which repeats
 // phase 1 for its rows: x is then read from L2 more than once, which such small batches do not notice.
+// Grouped form (kh_sgmv_fused_grouped_bf16): several layers that read the same x with the same segments (the to_k / to_v
+// projections of every cross-attention read the one text context) in one launch, blockIdx.z = (layer, column range),
+// per-layer A / B / y from a device table: 77-row requests give a single layer's launch a few microseconds of traffic,
+// 120 layers fill the chip.
 #include "kh_common.h"
 
 namespace {
@@ -33,6 +37,8 @@ struct FusedParams {
   const int* seg_start; const int* seg_adapter; const int* adapter_rank; const float* adapter_scale;
   int K, N, RP;
   int tiles_per_z;   // 128-column tiles of y per workgroup: blockIdx.z selects the range (T is recomputed per range)
+  int z_per_layer;   // column ranges per layer (grid.z = layers x z_per_layer)
+  const uint64_t* table;   // grouped form: rows {a_all, b_all, y} of device pointers, one per layer; null: the fields above
 };
 
 constexpr int BM = 128, BR = 128;                 // rows of a workgroup, rank columns (RP <= 128)
@@ -57,10 +63,16 @@ __global__ __launch_bounds__(512, 2) void sgmv_fused_kernel(const FusedParams p)
   const int rank = p.adapter_rank[ad];            // multiple of 32, <= RP
   const float scale = p.adapter_scale[ad];
   const int K = p.K, N = p.N, RP = p.RP;
+  const int layer = (int)blockIdx.z / p.z_per_layer, zz = (int)blockIdx.z % p.z_per_layer;
+  const bf16_t* a_all = p.a_all; const bf16_t* b_all = p.b_all; bf16_t* y_all = p.y;
+  if (p.table != nullptr) {
+    const uint64_t* row = p.table + (size_t)layer * 3;
+    a_all = reinterpret_cast<const bf16_t*>(row[0]); b_all = reinterpret_cast<const bf16_t*>(row[1]); y_all = reinterpret_cast<bf16_t*>(row[2]);
+  }
   const bf16_t* x = p.x + (size_t)r0 * K;
-  bf16_t* y = p.y + (size_t)r0 * N;
-  const bf16_t* A = p.a_all + (size_t)ad * RP * K;
-  const bf16_t* B = p.b_all + (size_t)ad * N * RP;
+  bf16_t* y = y_all + (size_t)r0 * N;
+  const bf16_t* A = a_all + (size_t)ad * RP * K;
+  const bf16_t* B = b_all + (size_t)ad * N * RP;
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -149,7 +161,7 @@ __global__ __launch_bounds__(512, 2) void sgmv_fused_kernel(const FusedParams p)
   }
 
   // ---- phase 2: y tile += scale * T . B_tile^T for every 128-column tile ----
-  const int j0 = blockIdx.z * p.tiles_per_z;
+  const int j0 = zz * p.tiles_per_z;
   const int n_tiles = (N / 128 - j0) < p.tiles_per_z ? (N / 128 - j0) : p.tiles_per_z;   // tiles j0 .. j0 + n_tiles - 1
   const int ks_total = rank / 16;                 // MFMA steps over the padded rank (2, 4, 6 or 8)
   const int nstage = (rank + 63) / 64;            // B stages per tile (1 or 2)
@@ -235,28 +247,53 @@ __global__ __launch_bounds__(512, 2) void sgmv_fused_kernel(const FusedParams p)
 
 }  // namespace
 
-// See include/katz_hip.h.
-KH_EXPORT int kh_sgmv_fused_bf16(const void* x, const void* a_all, const void* b_all, void* y, const int32_t* seg_start,
-                                 const int32_t* seg_adapter, const int32_t* adapter_rank, const float* adapter_scale,
-                                 int64_t n_segments, int64_t max_seg_rows, int64_t N, int64_t K, int64_t RP, void* stream) {
-  if (!x || !a_all || !b_all || !y || !seg_start || !seg_adapter || !adapter_rank || !adapter_scale) return KH_ERR_INVALID_ARG;
-  if (n_segments <= 0 || max_seg_rows <= 0 || N <= 0 || K <= 0 || RP <= 0) return KH_ERR_INVALID_ARG;
+namespace {
+
+int sgmv_fused_impl(const void* x, const void* a_all, const void* b_all, void* y, const uint64_t* table, int64_t n_layers,
+                    const int32_t* seg_start, const int32_t* seg_adapter, const int32_t* adapter_rank, const float* adapter_scale,
+                    int64_t n_segments, int64_t max_seg_rows, int64_t N, int64_t K, int64_t RP, void* stream) {
+  if (!x || !seg_start || !seg_adapter || !adapter_rank || !adapter_scale) return KH_ERR_INVALID_ARG;
+  if (table == nullptr && (!a_all || !b_all || !y)) return KH_ERR_INVALID_ARG;
+  if (n_segments <= 0 || max_seg_rows <= 0 || N <= 0 || K <= 0 || RP <= 0 || n_layers <= 0) return KH_ERR_INVALID_ARG;
   if (RP > 128) return KH_ERR_TOO_LARGE;
   if (K % 64 != 0 || N % 128 != 0 || RP % 32 != 0) return KH_ERR_UNSUPPORTED;
   if (n_segments > 65535 || max_seg_rows > (1 << 24) || N > (1 << 24) || K > (1 << 24)) return KH_ERR_TOO_LARGE;
-  if (!kh_aligned16(x) || !kh_aligned16(a_all) || !kh_aligned16(b_all) || !kh_aligned16(y)) return KH_ERR_ALIGNMENT;
+  if (!kh_aligned16(x) || (table == nullptr && (!kh_aligned16(a_all) || !kh_aligned16(b_all) || !kh_aligned16(y))) ||
+      (table != nullptr && ((uintptr_t)table & 7) != 0))
+    return KH_ERR_ALIGNMENT;
   FusedParams p;
   p.x = (const bf16_t*)x; p.a_all = (const bf16_t*)a_all; p.b_all = (const bf16_t*)b_all; p.y = (bf16_t*)y;
   p.seg_start = seg_start; p.seg_adapter = seg_adapter; p.adapter_rank = adapter_rank; p.adapter_scale = adapter_scale;
-  p.K = (int)K; p.N = (int)N; p.RP = (int)RP;
+  p.K = (int)K; p.N = (int)N; p.RP = (int)RP; p.table = table;
   if (hipError_t e = kh_allow_lds<sgmv_fused_kernel>(LDS_BYTES); e != hipSuccess) return (int)e;
   // few row blocks: the column tiles of y are dealt to several workgroups (each recomputes its rows' T) until the chip is covered
-  const int64_t row_wgs = ((max_seg_rows + BM - 1) / BM) * n_segments, n_tiles = N / 128;
+  const int64_t row_wgs = ((max_seg_rows + BM - 1) / BM) * n_segments * n_layers, n_tiles = N / 128;
   int64_t z = row_wgs >= 256 ? 1 : (256 + row_wgs - 1) / row_wgs;
   z = z < n_tiles ? z : n_tiles;
   p.tiles_per_z = (int)((n_tiles + z - 1) / z);
   z = (n_tiles + p.tiles_per_z - 1) / p.tiles_per_z;
-  dim3 grid((unsigned)((max_seg_rows + BM - 1) / BM), (unsigned)n_segments, (unsigned)z);
+  p.z_per_layer = (int)z;
+  if (z * n_layers > 65535) return KH_ERR_TOO_LARGE;
+  dim3 grid((unsigned)((max_seg_rows + BM - 1) / BM), (unsigned)n_segments, (unsigned)(z * n_layers));
   kh_launch(KH_TAG_SGMV_FUSED, sgmv_fused_kernel, grid, dim3(512), LDS_BYTES, (hipStream_t)stream, p);
   KH_RETURN_LAST_ERROR();
+}
+
+}  // namespace
+
+// See include/katz_hip.h.
+KH_EXPORT int kh_sgmv_fused_bf16(const void* x, const void* a_all, const void* b_all, void* y, const int32_t* seg_start,
+                                 const int32_t* seg_adapter, const int32_t* adapter_rank, const float* adapter_scale,
+                                 int64_t n_segments, int64_t max_seg_rows, int64_t N, int64_t K, int64_t RP, void* stream) {
+  return sgmv_fused_impl(x, a_all, b_all, y, nullptr, 1, seg_start, seg_adapter, adapter_rank, adapter_scale, n_segments, max_seg_rows,
+                         N, K, RP, stream);
+}
+
+// See include/katz_hip.h.
+KH_EXPORT int kh_sgmv_fused_grouped_bf16(const void* x, const uint64_t* table, int64_t n_layers, const int32_t* seg_start,
+                                         const int32_t* seg_adapter, const int32_t* adapter_rank, const float* adapter_scale,
+                                         int64_t n_segments, int64_t max_seg_rows, int64_t N, int64_t K, int64_t RP, void* stream) {
+  if (!table) return KH_ERR_INVALID_ARG;
+  return sgmv_fused_impl(x, nullptr, nullptr, nullptr, table, n_layers, seg_start, seg_adapter, adapter_rank, adapter_scale, n_segments,
+                         max_seg_rows, N, K, RP, stream);
 }

@@ -650,6 +650,44 @@ def sgmv_fused_(y, x, a_all, b_all, seg_start, seg_adapter, adapter_rank, adapte
     return y
 
 
+def sgmv_fused_grouped_table(ys, a_alls, b_alls) -> torch.Tensor:
+    """The device table of sgmv_fused_grouped_: one row {a_all_l, b_all_l, y_l} of pointers per layer.  Build it once per
+    set of layers; it holds addresses, so the tensors must stay where they are (and alive) while it is used."""
+    if not (len(ys) == len(a_alls) == len(b_alls)) or not ys:
+        raise ValueError("one y, a_all and b_all per layer")
+    rows = []
+    for y, a, b in zip(ys, a_alls, b_alls):
+        _req(y, BF16, "y"); _req(a, BF16, "a_all"); _req(b, BF16, "b_all")
+        if y.shape != ys[0].shape or a.shape != a_alls[0].shape or b.shape != b_alls[0].shape:
+            raise ValueError("all layers of a grouped launch have the same shapes")
+        rows.append([a.data_ptr(), b.data_ptr(), y.data_ptr()])
+    return torch.tensor(rows, dtype=torch.int64, device=ys[0].device)
+
+
+def sgmv_fused_grouped_(ys, x, a_alls, b_alls, seg_start, seg_adapter, adapter_rank, adapter_scale, max_seg_rows: int,
+                        table: Optional[torch.Tensor] = None):
+    """sgmv_fused_ for several layers that read the same x with the same segments (the to_k / to_v projections of all
+    cross-attentions of one width) in ONE launch: ys[l][rows] += scale_a * bf16(x[rows] A_{l,a}^T) B_{l,a}^T.
+    table: the result of sgmv_fused_grouped_table(ys, a_alls, b_alls) when the caller keeps it between calls."""
+    lib = _lib.load()
+    _req(x, BF16, "x"); _req(adapter_scale, torch.float32, "adapter_scale")
+    for n, t in (("seg_start", seg_start), ("seg_adapter", seg_adapter), ("adapter_rank", adapter_rank)):
+        _req(t, torch.int32, n)
+    if table is None:
+        table = sgmv_fused_grouped_table(ys, a_alls, b_alls)
+    rows, K = x.shape
+    N = ys[0].shape[1]
+    RP = a_alls[0].shape[1]
+    if (ys[0].shape[0] != rows or a_alls[0].shape[2] != K or b_alls[0].shape[1:] != (N, RP) or b_alls[0].shape[0] != a_alls[0].shape[0]
+            or table.shape != (len(ys), 3) or table.dtype != torch.int64 or not table.is_cuda or not table.is_contiguous()):
+        raise ValueError("x [rows, K], ys[l] [rows, N], a_alls[l] [n_adapters, RP, K], b_alls[l] [n_adapters, N, RP], table [layers, 3]")
+    nseg = seg_adapter.numel()
+    rc = lib.kh_sgmv_fused_grouped_bf16(_ptr(x), _ptr(table), len(ys), _ptr(seg_start), _ptr(seg_adapter), _ptr(adapter_rank),
+                                        _ptr(adapter_scale), nseg, max_seg_rows, N, K, RP, _stream())
+    _lib.check(rc, "kh_sgmv_fused_grouped_bf16")
+    return ys
+
+
 # --------------------------------------------------------------------------------------- K3
 def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, heads: int, scale: Optional[float] = None,
               out: Optional[torch.Tensor] = None) -> torch.Tensor:

@@ -70,6 +70,10 @@ def test_argument_validation_needs_no_gpu():
     assert lib.kh_conv3x3_gn_stats_nhwc_bf16(16, 16, None, None, None, 16, 16, 2, 32, 32, 1280, 1280, 1, 7, None) == -1
     assert lib.kh_group_norm_apply_bf16(None, None, None, None, None, None, 16, 2, 1280, 1024, 32, 1e-5, 1, None) == -1
     assert lib.kh_group_norm_apply_bf16(16, 16, None, None, None, 16, 16, 2, 1290, 1024, 32, 1e-5, 1, None) == -1
+    # several layers' segmented shrink + expand in one launch: the table is required, shapes as for the single layer
+    assert lib.kh_sgmv_fused_grouped_bf16(16, None, 4, 16, 16, 16, 16, 8, 77, 1280, 2048, 128, None) == -1
+    assert lib.kh_sgmv_fused_grouped_bf16(16, 16, 4, 16, 16, 16, 16, 8, 77, 1280, 2048, 160, None) == -4     # RP > 128
+    assert lib.kh_sgmv_fused_grouped_bf16(16, 16, 4, 16, 16, 16, 16, 8, 77, 1200, 2048, 128, None) == -2     # N % 128
     # the entry point that allocates nothing: its limit and its arguments are checked before the first device call
     assert lib.kh_group_norm_static_bf16(16, 16, None, None, None, 4096, 4096, 65536, 32, 1e-5, 0, 1, None) == -4
     assert lib.kh_group_norm_static_bf16(None, 16, None, None, None, 2, 320, 64, 32, 1e-5, 0, 1, None) == -1

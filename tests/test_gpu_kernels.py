@@ -536,6 +536,78 @@ def test_sgmv_fused_ragged_segments_and_small_rank_pad():
     assert torch.equal(y[seg_start[2]:seg_start[3]], guard[seg_start[2]:seg_start[3]])   # the request without an adapter
 
 
+def test_sgmv_fused_grouped_layers_share_the_context():
+    """kh_sgmv_fused_grouped_bf16: the to_k / to_v projections of several cross-attentions read the same 77-token text
+    context per request (8 requests, each with its own adapter; one without), every layer with its own A / B / y, all in
+    ONE launch: against the oracle per layer, and bit for bit against one kh_sgmv_fused_bf16 launch per layer."""
+    from katz_amd import ops
+
+    say("sgmv fused grouped")
+    g = torch.Generator().manual_seed(23)
+    n_req, T, K, N, RP, L = 8, 77, 2048, 1280, 128, 5
+    ranks = [8, 128, 32, 64, 16, 128, 64, 32]
+    seg_adapter = [3, 1, -1, 0, 7, 5, 2, 6]
+    seg_start = [i * T for i in range(n_req + 1)]
+    x = randn(g, n_req * T, K)
+    d = dev()
+    rank_pad = torch.tensor([(r + 31) // 32 * 32 for r in ranks], dtype=torch.int32, device=d)
+    ss = torch.tensor(seg_start, dtype=torch.int32, device=d)
+    sa = torch.tensor(seg_adapter, dtype=torch.int32, device=d)
+    xd = x.to(d, BF)
+    layers = []
+    for l in range(L):
+        adapters = [(randn(g, r, K, std=0.02), randn(g, N, r, std=0.02), 0.4 + 0.1 * i) for i, r in enumerate(ranks)]
+        a_all = torch.zeros(n_req, RP, K); b_all = torch.zeros(n_req, N, RP)
+        for i, (A, B, _) in enumerate(adapters):
+            a_all[i, : A.shape[0]] = A
+            b_all[i, :, : B.shape[1]] = B
+        base = randn(g, n_req * T, N)
+        layers.append((adapters, a_all.to(d, BF), b_all.to(d, BF), base))
+    scales = torch.tensor([0.4 + 0.1 * i for i in range(n_req)], dtype=torch.float32, device=d)
+    ys = [base.to(d, BF).clone() for (_, _, _, base) in layers]
+    singles = [y.clone() for y in ys]
+    table = ops.sgmv_fused_grouped_table(ys, [l[1] for l in layers], [l[2] for l in layers])
+    ops.profile_begin()
+    ops.sgmv_fused_grouped_(ys, xd, [l[1] for l in layers], [l[2] for l in layers], ss, sa, rank_pad, scales, T, table=table)
+    launches = ops.profile_end()
+    assert len(launches) == 1, launches                      # one launch for all layers
+    for y1, (_, a_all, b_all, _) in zip(singles, layers):
+        ops.sgmv_fused_(y1, xd, a_all, b_all, ss, sa, rank_pad, scales, T)
+    torch.cuda.synchronize()
+    for l, (adapters, _, _, base) in enumerate(layers):
+        ref = O.sgmv(x.to(BF).float(), seg_start, seg_adapter, adapters, base.to(BF).float())
+        assert_close_rel(ys[l], ref, REL_BF16, f"sgmv fused grouped, layer {l}")
+        assert torch.equal(ys[l], singles[l]), f"layer {l}: grouped and single launches differ"
+        assert torch.equal(ys[l][2 * T:3 * T], base.to(d, BF)[2 * T:3 * T])    # the request without an adapter
+
+
+def test_sgmv_fused_many_column_tiles():
+    """N = 5120 (40 column tiles): a workgroup takes at most five, whatever the row count; 4 requests x 200 rows."""
+    from katz_amd import ops
+
+    say("sgmv fused wide N")
+    g = torch.Generator().manual_seed(29)
+    n_req, T, K, N, RP = 4, 200, 640, 5120, 64
+    ranks = [64, 16, 32, 8]
+    seg_adapter = [1, 3, 0, 2]
+    seg_start = [i * T for i in range(n_req + 1)]
+    x, base = randn(g, n_req * T, K), randn(g, n_req * T, N)
+    adapters = [(randn(g, r, K, std=0.02), randn(g, N, r, std=0.02), 0.5 + 0.1 * i) for i, r in enumerate(ranks)]
+    a_all = torch.zeros(n_req, RP, K); b_all = torch.zeros(n_req, N, RP)
+    for i, (A, B, _) in enumerate(adapters):
+        a_all[i, : A.shape[0]] = A
+        b_all[i, :, : B.shape[1]] = B
+    d = dev()
+    rank_pad = torch.tensor([(r + 31) // 32 * 32 for r in ranks], dtype=torch.int32, device=d)
+    scales = torch.tensor([a[2] for a in adapters], dtype=torch.float32, device=d)
+    y = base.to(d, BF).clone()
+    ops.sgmv_fused_(y, x.to(d, BF), a_all.to(d, BF), b_all.to(d, BF), torch.tensor(seg_start, dtype=torch.int32, device=d),
+                    torch.tensor(seg_adapter, dtype=torch.int32, device=d), rank_pad, scales, T)
+    torch.cuda.synchronize()
+    ref = O.sgmv(x.to(BF).float(), seg_start, seg_adapter, adapters, base.to(BF).float())
+    assert_close_rel(y, ref, REL_BF16, "sgmv fused wide N")
+
+
 def test_fused_qkv_matches_separate_projections():
     """Stacked to_q/to_k/to_v (n_split) with a shared shrink == three separate LoRA linears."""
     from katz_amd import ops
