@@ -543,7 +543,7 @@ def loop_bench(args):
     sch.set_timesteps(args.loop_steps, device=dev)
     lat0 = (torch.randn(1, 4, 128, 128, generator=g, device=dev) * sch.init_noise_sigma).to(bf)
     with torch.no_grad():
-        step = GraphedDenoiseStep(unet, cn, lat0, ctx, added, cond, 7.5, 0.5)
+        step = GraphedDenoiseStep(unet, cn, lat0, ctx, added, cond, 7.5, 0.5, hoist_context_kv=not args.context_kv_per_step)
         for _ in range(args.warmup_loops):
             out = step.run(lat0, sch)
         torch.cuda.synchronize()
@@ -593,7 +593,8 @@ def loop_bench(args):
                                "[2,3,1024,1024], scale 0.5) -> UNet (2 LoRAs r64 s0.8 + r32 s0.6, CFG batch 2) -> guidance 7.5 + "
                                "Euler discrete; one HIP graph replay per step" + ("; inside the graph the ControlNet runs on a second stream "
                                "beside the UNet's down and mid blocks" if step.overlap else "") +
-                               "; conditioning embedding computed once per loop",
+                               "; conditioning embedding" + (" and the text context's K / V projections" if step.hoist_kv else "") +
+                               " computed once per loop",
                    "global_batch": 2, "parallelism": "single GPU"},
         "roofline": {"kernel": "whole loop (every kernel of ControlNet + UNet + scheduler step); per-kernel rooflines are in the default mode's line",
                      "loop_ms": round(med, 2), "ms_per_step": round(med / args.loop_steps, 3), "loop_steps": args.loop_steps},
@@ -619,6 +620,8 @@ def main():
     ap.add_argument("--loop-steps", type=int, default=50)
     ap.add_argument("--loops", type=int, default=3)
     ap.add_argument("--warmup-loops", type=int, default=1)
+    ap.add_argument("--context-kv-per-step", action="store_true",
+                    help="--loop: project the text context's K / V inside every step (as the reference does) instead of once per loop")
     ap.add_argument("--kernel-probe", action="store_true",
                     help="run only a 64 MiB copy and each kernel at its BASELINE shapes three times (for rocprofv3)")
     args = ap.parse_args()

@@ -108,6 +108,12 @@ class GraphedDenoiseStep:
     with overlap on, the capture forks a second stream from the capturing one, and a fork from an already forked stream
     inside a capture has crashed the runtime at capture end; the constructor refuses to start under a capture.
 
+    hoist_context_kv (default on): the to_k / to_v projections of all cross-attentions (with their adapters) read the text
+    context only, which does not change during a loop; they run once per `run` (for both models) instead of in every step
+    (the reference projects the context again in every step, attention_processor.py:1246-1251; same values, bit for bit:
+    the same kernels on the same inputs).  The graph then reads their result buffers, so a change of the adapters' scales
+    takes effect for these layers at the next `run`.
+
     hoist_cond_embedding: the ControlNet's conditioning embedding depends on the image only, which is the same in every
     step; it is computed once per `run` instead of inside the graph (the reference recomputes it every step,
     controlnet.py:780-783; same value, bit for bit).  Everything the notes on GraphedUNetStep say about rebuilding after
@@ -115,7 +121,7 @@ class GraphedDenoiseStep:
 
     def __init__(self, unet, controlnet, latents, encoder_hidden_states, added_cond_kwargs, controlnet_cond,
                  guidance_scale: float, conditioning_scale: float = 0.5, hoist_cond_embedding: bool = True,
-                 warmup: int = 2, fuse_tail: bool = True, overlap: Optional[bool] = None):
+                 warmup: int = 2, fuse_tail: bool = True, overlap: Optional[bool] = None, hoist_context_kv: bool = True):
         from . import ops
 
         if latents.is_cuda and torch.cuda.is_current_stream_capturing():
@@ -137,6 +143,7 @@ class GraphedDenoiseStep:
         self.row[:4] = torch.tensor([1.0, 0.5, 1.0, 1.0])     # harmless values for the warm-up runs
         self.row[4] = 500.0
         self.hoist = hoist_cond_embedding
+        self.hoist_kv = bool(hoist_context_kv)
         self.cond_emb = None
         co = unet.conv_out
         self.fuse_tail = bool(fuse_tail and co.in_channels % 16 == 0 and co.out_channels == 4 and not co.adapters)
@@ -149,6 +156,7 @@ class GraphedDenoiseStep:
         with torch.cuda.stream(side), torch.no_grad():
             if self.hoist:
                 self.cond_emb = controlnet.embed_condition(self.cond)
+            self._project_context()
             for _ in range(warmup):
                 self._step()
         torch.cuda.current_stream().wait_stream(side)
@@ -160,10 +168,25 @@ class GraphedDenoiseStep:
         self.latents.copy_(keep[0]); self.model_input.copy_(keep[1])
         self._ops = ops
 
+    def _project_context(self):
+        """The context K / V of both models from the static context tensor (hoist_context_kv)."""
+        if self.hoist_kv:
+            for m in (self.controlnet, self.unet):
+                m._ctx_kv.run(self.ctx)
+
     def _step(self):
         from . import ops
 
         t = self.row[4:5]
+        self.unet.context_kv_ready = self.controlnet.context_kv_ready = self.hoist_kv
+        try:
+            self._step_models(t)
+        finally:
+            self.unet.context_kv_ready = self.controlnet.context_kv_ready = False
+
+    def _step_models(self, t):
+        from . import ops
+
         if self.overlap:
             eps = self._models_side_by_side(t)
         else:
@@ -209,7 +232,7 @@ class GraphedDenoiseStep:
         return eps
 
     def run(self, latents: torch.Tensor, scheduler, controlnet_cond: Optional[torch.Tensor] = None,
-            check: bool = True) -> torch.Tensor:
+            check: bool = True, encoder_hidden_states: Optional[torch.Tensor] = None) -> torch.Tensor:
         """The whole loop: `latents` already scaled by init_noise_sigma (prepare_latents, pipeline :872-887);
         scheduler.set_timesteps(...) done.  Returns the final latents (a copy, in the model dtype like the reference's
         scheduler output, scheduling_euler_discrete.py:530)."""
@@ -220,6 +243,9 @@ class GraphedDenoiseStep:
                 self.cond.copy_(controlnet_cond)
                 if self.hoist:
                     self.cond_emb.copy_(self.controlnet.embed_condition(self.cond))
+            if encoder_hidden_states is not None:
+                self.ctx.copy_(encoder_hidden_states)
+            self._project_context()
             self.latents.copy_(latents)
             self.model_input.copy_((torch.cat([latents] * 2).float() / table[0, 3]).to(torch.bfloat16))
             for i in range(table.shape[0]):

@@ -524,7 +524,8 @@ class UNet2DConditionModel(nn.Module):
         with ops.weight_prefetch_scope(self):   # hints are learned from, and point into, this model's own last pass
             if self._ctx_kv is None:
                 self.prepare()
-            self._ctx_kv.run(ctx)  # K/V projections of all cross-attentions, grouped
+            if not getattr(self, "context_kv_ready", False):   # (a denoise loop projects its one text context once, not per step)
+                self._ctx_kv.run(ctx)  # K/V projections of all cross-attentions, grouped
             emb = self._embed(sample, timestep, added_cond_kwargs)
             temb_act = F.silu(emb)
             self._temb_proj.run(temb_act)   # time_emb_proj of all resnets, batched per width

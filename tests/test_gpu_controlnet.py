@@ -257,6 +257,10 @@ def test_config5_loop_with_two_loras_against_the_oracle_loop():
             assert cosine(out, ref) >= 0.999, (overlap, fuse_tail, cosine(out, ref))
             got[(overlap, fuse_tail)] = out
     assert torch.equal(got[(True, True)], got[(False, True)]) and torch.equal(got[(True, False)], got[(False, False)])
+    # the context K / V projected inside every step (as the reference does) instead of once per loop: the same bits
+    in_step = GraphedDenoiseStep(p_unet, p_cn, lat0.to(DEV), ctx.to(DEV), added_d, cond.to(DEV), 7.5, 0.5,
+                                 hoist_context_kv=False).run(lat0.to(DEV), psch)
+    assert torch.equal(in_step, got[(True, True)])
     assert torch.equal(got[(True, False)].contiguous(), eager.contiguous())
     ops.check_split_timeouts(torch.device(DEV))
 
