@@ -397,6 +397,14 @@ def kernel_probe():
     add(f"lora_linear_split M{M} K{K} N{N} R{R} (shrink in launch)",
         lambda x=x, w=w, b=b, a=a_cat, s=scale, bc=b_cat: ops.lora_linear_split(x, w, b, a, s, bc),
         2.0 * M * N * (K + R) + 2.0 * M * K * R, 2.0 * (M * K + K * N + M * N + R * N + R * K))
+    # ... and as the step runs it: ranks 64 + 32 in 128 packed columns (r_used = 96), the in-launch shrink on 64 x 32 tiles
+    Rt = 96
+    a96, b96 = a_cat.clone(), b_cat.clone()
+    a96[Rt:] = 0
+    b96[:, Rt:] = 0
+    add(f"lora_linear_split M{M} K{K} N{N} R{R} r_used {Rt} (shrink in launch, 64x32 tiles)",
+        lambda x=x, w=w, b=b, a=a96, s=scale, bc=b96: ops.lora_linear_split(x, w, b, a, s, bc, r_used=96),
+        2.0 * M * N * (K + Rt) + 2.0 * M * K * Rt, 2.0 * (M * K + K * N + M * N + Rt * N + Rt * K))
     # K3: attention at the three SDXL shapes
     for (B, H, T, S) in ((2, 10, 4096, 4096), (2, 20, 1024, 1024), (2, 20, 1024, 77)):
         q, k, v = rn(B, T, H * 64), rn(B, S, H * 64), rn(B, S, H * 64)
