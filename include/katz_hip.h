@@ -98,7 +98,14 @@ int kh_lora_linear_pre_bf16(const void* x, const void* w, const void* bias, cons
  * call is then undefined).  n_split > 0: w / bias / b_cat stack N / n_split layers of n_split rows each (q, k, v of a
  * self-attention), a_cat / col_scale stack their A matrices ([N / n_split * R, K]) and t_scratch is [M, N / n_split * R],
  * as for kh_lora_linear_pre_bf16.  K % 64 == 0, R % 32 == 0, R <= 128.  flags: bit 0 GEGLU, bits 8..15: 1 = always two
- * launches, bits 16..23: r_used / 16 as above. */
+ * launches, bits 16..23: r_used / 16 as above, bit 24: never the cooperative form (below).
+ * Cooperative form: where the GEMM's 128x160 tiles give every CU exactly one workgroup (N = 640 at M = 8192), R = 128 and
+ * 0 < r_used <= 96, no CU is idle, and EVERY workgroup first computes a 32-row x 96-column piece of its row block's
+ * t_scratch, counts itself into `counters` and only then runs its tile, waiting (bounded, as above) for the four pieces
+ * of its row block before the last K tiles.  No workgroup waits before its own piece is out, so one such launch always
+ * completes; TWO of them running at the same time on different streams can each hold the CUs the other's not yet
+ * started workgroups need, and then both only end through the bounded wait.  A caller that enqueues these calls on
+ * streams that may overlap sets bit 24 on all but one of the streams. */
 #define KH_SPLIT_COUNTER_INTS(M) (((M) + 127) / 128 + 1)
 int kh_lora_linear_split_bf16(const void* x, const void* w, const void* bias, const void* a_cat, const float* col_scale,
                               const void* b_cat, void* t_scratch, int32_t* counters, const void* residual, void* y,
@@ -150,7 +157,8 @@ int kh_lora_linear_xattn_ok(int64_t M, int64_t N, int64_t K, int64_t R, int64_t 
 /* Bounded waits of kh_lora_linear_split_bf16's in-launch shrink that have run out on the current device since the
  * process started (or since the last call with clear != 0): writes the number to *count (HOST pointer).  A GEMM workgroup
  * of that launch waits for the shrink workgroups of the same launch, which have lower workgroup ids and are therefore
- * dispatched first; the wait gives up after 2^20 polls (about a quarter of a second) and the result of that call is then
+ * dispatched first (in the cooperative form: for the other workgroups of its row block, each of which delivers its piece
+ * before it waits); the wait gives up after 2^20 polls (about a quarter of a second) and the result of that call is then
  * undefined.  The flag word in `counters` says so per call but is wiped by the caller's next reset; this count is not.
  * A non-zero value means results since the last check cannot be trusted.  Blocks until the device's earlier work is
  * done (a 4-byte copy on the null stream); not under graph capture.  No counterpart in the reference. */

@@ -79,6 +79,9 @@ struct LoraGemmParams {
   uint32_t pf_lines[3] = {0, 0, 0};
 };
 
+// bit 24 of the `flags` of kh_lora_linear_split_bf16 / _norm_bf16: do not use the cooperative in-launch shrink (see include/katz_hip.h)
+constexpr int KH_FLAG_NO_COOP = 1 << 24;
+
 // The pending weight prefetch of this host thread (kh_set_weight_prefetch), handed to the next launch.
 void kh_take_weight_prefetch(LoraGemmParams& p);
 
@@ -224,6 +227,11 @@ int lora_gemm_pipe_launch_xattn(const LoraGemmParams& p, hipStream_t stream);
 // plain or K-extended GEMM with bias / residual, K % 64 == 0.  row_groups 2 or 4.
 bool lora_gemm_ksplit_ok(const LoraGemmParams& p);
 int lora_gemm_ksplit_launch(const LoraGemmParams& p, int row_groups, hipStream_t stream);
+// Shrink and GEMM in one launch on the 128 x 160 tiles, every workgroup computing a piece of T first (p.a_cat / col_scale /
+// b_cat set, p.t_ext = scratch for the shrink result, p.il_cnt = counters, p.r_used <= 96 of R = 128).
+bool lora_gemm_ksplit_coop_ok(const LoraGemmParams& p);
+int lora_gemm_ksplit_launch_coop(const LoraGemmParams& p, hipStream_t stream);
+int lora_gemm_ksplit_coop_timeouts(int* count, int clear);
 bool lora_gemm_ksplit_conv_ok(const LoraGemmParams& p);
 int lora_gemm_ksplit_launch_conv(const LoraGemmParams& p, int row_groups, hipStream_t stream);
 // the convolution that also leaves GroupNorm statistics (gn_cg / gn_hw set): row groups of the 160-column tiles it would run

@@ -588,9 +588,11 @@ KH_EXPORT int kh_lora_linear_split_launches(int64_t M, int64_t N, int64_t K, int
   if (((flags >> 8) & 0xff) != 0) return 2;
   static int32_t dummy_counter;                  // the rule only asks whether counters were given
   static const char dummy = 0;
-  const LoraGemmParams p = split_params(&dummy, &dummy, nullptr, &dummy, reinterpret_cast<const float*>(&dummy), &dummy,
-                                        const_cast<char*>(&dummy), &dummy_counter, nullptr, const_cast<char*>(&dummy), M, N, K, R,
-                                        n_split, (flags & 1) != 0);
+  LoraGemmParams p = split_params(&dummy, &dummy, nullptr, &dummy, reinterpret_cast<const float*>(&dummy), &dummy,
+                                  const_cast<char*>(&dummy), &dummy_counter, nullptr, const_cast<char*>(&dummy), M, N, K, R,
+                                  n_split, (flags & 1) != 0);
+  p.r_used = ((flags >> 16) & 0xff) * 16;
+  if ((flags & KH_FLAG_NO_COOP) == 0 && lora_gemm_ksplit_coop_ok(p)) return 1;
   return lora_gemm_pipe_il_ok(p) ? 1 : 2;
 }
 
@@ -616,6 +618,7 @@ KH_EXPORT int kh_lora_linear_split_bf16(const void* x, const void* w, const void
     LoraGemmParams p = split_params(x, w, bias, a_cat, col_scale, b_cat, t_scratch, counters, residual, y, M, N, K, R, n_split, geglu);
     p.r_used = ((flags >> 16) & 0xff) * 16;
     kh_take_weight_prefetch(p);
+    if ((flags & KH_FLAG_NO_COOP) == 0 && lora_gemm_ksplit_coop_ok(p)) return lora_gemm_ksplit_launch_coop(p, (hipStream_t)stream);
     return lora_gemm_pipe_launch_il(p, (hipStream_t)stream);
   }
   const int rc = kh_lora_shrink_bf16(x, a_cat, col_scale, t_scratch, M, K, RT, stream);
@@ -689,6 +692,8 @@ static int lora_linear_norm_impl(const void* x, const void* w, const void* bias,
     p.ldt = 0; p.t_nsplit = 0; p.il_cnt = nullptr;
     return lora_gemm_pipe_launch(p, tile_sel, (hipStream_t)stream);
   }
+  if (counters != nullptr && tile_sel == 0 && (flags & KH_FLAG_NO_COOP) == 0 && lora_gemm_ksplit_coop_ok(p))
+    return lora_gemm_ksplit_launch_coop(p, (hipStream_t)stream);
   if (counters != nullptr && tile_sel == 0 && lora_gemm_pipe_il_ok(p)) return lora_gemm_pipe_launch_il(p, (hipStream_t)stream);
   const int rc = lora_shrink_ln_launch(x, a_cat, col_scale, t_scratch, M, K, RT, ln_part, ln_ca1, ln_ca2, ln_eps, (hipStream_t)stream);
   if (rc != KH_OK) return rc;

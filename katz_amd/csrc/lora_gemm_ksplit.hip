@@ -19,6 +19,11 @@
 // waves below N_HI issue one more than the others, and every wait picks its count by a wave-uniform branch.
 #include "kh_common.h"
 #include "lora_gemm.h"
+#include "lora_shrink_tile.h"
+
+// Bounded waits of the cooperative shrink that have run out on this GPU; read (and cleared) by kh_lora_split_timeouts
+// together with the count of the in-launch shrink of lora_gemm_pipe.hip.
+static __device__ int kh_coop_timeout_count;
 
 namespace {
 
@@ -59,8 +64,17 @@ __device__ __attribute__((aligned(256))) const uint32_t ks_zero_page[64] = {0};
 // (kh, kw) sit (kh * W + kw) * Cin elements after the row's base (the pixel above-left of its window), and rows
 // whose tap falls outside the image read zeros.
 // GNF: the epilogue also leaves the GroupNorm statistics of the result (LoraGemmParams::gn_part).
-template <class C, bool CONV, bool GNF = false>
-__global__ __launch_bounds__(512, 2) void lora_gemm_ksplit_kernel(const LoraGemmParams p) {
+// COOP: the launch computes its own shrink, cooperatively.  These tiles fill every CU, so there is no idle CU for shrink
+// workgroups beside the GEMM ones; instead EVERY workgroup first computes one piece of T -- 32 rows x 96 rank columns: the
+// n_tiles = 4 x (ldt / 128) workgroups of a row block of 128 rows share that block's 4 row quarters x ldt / 128 column
+// groups of T, workgroup n_blk takes quarter n_blk % 4 of group n_blk / 4 --, stores it write-through, zeroes the 32
+// padding columns of its group, counts itself into the row block's counter and then runs its GEMM tile; before its first
+// request for T (the last K tiles) it waits, bounded, for the row block's count and reads T past the L2.  A workgroup
+// never waits before its own piece is out, so the launch makes progress in whatever order its workgroups become
+// resident, as long as no OTHER launch whose workgroups wait for each other shares the device with it (the binding does
+// not use this form on a second stream).
+template <class C, bool CONV, bool GNF = false, bool COOP = false>
+__global__ __launch_bounds__(512, COOP ? 1 : 2) void lora_gemm_ksplit_kernel(const LoraGemmParams p) {
 #if __HIP_DEVICE_COMPILE__   // the host pass only needs the kernel's symbol (it cannot lower the buffer-resource type)
   extern __shared__ __attribute__((aligned(16))) char smem[];
   constexpr int BM = C::BM, BN = C::BN, TN = C::TN, KSW = C::KSW, NST = C::NST, STAGE = C::STAGE;
@@ -70,7 +84,8 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_ksplit_kernel(const LoraGemm
   const int wm = wave / C::WK, wk = wave % C::WK;
   const int l32 = lane & 31, lh = lane >> 5;
 
-  kh_prefetch_lines(p.pf, p.pf_lines, smem + wave * 1024, blockIdx.x, gridDim.x, tid, 512);   // the next launch's weights
+  // the next launch's weights (a cooperative launch issues this after its shrink piece, whose rings use the same LDS)
+  if (!COOP) kh_prefetch_lines(p.pf, p.pf_lines, smem + wave * 1024, blockIdx.x, gridDim.x, tid, 512);
   // tile of this workgroup: XCD b % 8 owns a block of xr_m x xr_n tiles (its W rows stay in its L2)
   const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
   const int m_blk = (xcd / p.xg_n) * p.xr_m + local / p.xr_n;
@@ -81,6 +96,29 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_ksplit_kernel(const LoraGemm
   const int KT1 = K / 64;
   const int KT = KT1 + (p.t_ext != nullptr ? p.R / 64 : 0);
   const bool has_hi = wave < N_HI;
+  if constexpr (COOP) {
+    // this workgroup's piece of T = bf16((x . A_cat^T) * col_scale) (with a folded LayerNorm in front: the form documented at
+    // ShrinkParams), then the padding columns, then the arrival
+    const int q4 = n_blk & 3, grp = n_blk >> 2;
+    ShrinkParams sp;
+    sp.x = p.x; sp.a_cat = p.a_cat; sp.col_scale = p.col_scale; sp.t = const_cast<bf16_t*>(p.t_ext);
+    sp.M = M; sp.K = K; sp.R = p.ldt;
+    sp.ln_part = p.ln_part; sp.ln_ca1 = p.ln_ca1; sp.ln_ca2 = p.ln_ca2; sp.ln_eps = p.ln_eps;
+    // (a quarter that starts past the last row has nothing to compute: the tile's addressing assumes m0 < M)
+    if (m0 + 32 * q4 < M) lora_shrink_tile<SCfg<4, 1, 3>, true, 512>(sp, m0 + 32 * q4, grp * 128, smem);
+    if (tid < 128) {   // columns 96 .. 127 of the group: 32 rows x 4 pieces of 16 bytes
+      const int row = m0 + 32 * q4 + (tid >> 2);
+      if (row < M) {
+        uint32_t* dst = reinterpret_cast<uint32_t*>(const_cast<bf16_t*>(p.t_ext) + (size_t)row * p.ldt + grp * 128 + 96 + (tid & 3) * 8);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) __hip_atomic_store(dst + e, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    __builtin_amdgcn_s_waitcnt(0);                          // this thread's write-through stores have completed
+    __syncthreads();
+    if (tid == 0) __hip_atomic_fetch_add(p.il_cnt + m_blk, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    kh_prefetch_lines(p.pf, p.pf_lines, smem + wave * 1024, blockIdx.x, gridDim.x, tid, 512);
+  }
   // folded LayerNorm: mean and 1/std of this tile's x rows, read in the epilogue (the barriers of the K loop lie between)
   // and the two per-column terms of this column tile; requested here, finished once the bias loads are under way
   float* sMu = reinterpret_cast<float*>(smem + p.ln_lds);
@@ -166,11 +204,26 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_ksplit_kernel(const LoraGemm
         }
       }
     } else {
+      if (COOP && t == KT1) {
+        // first request for T: wait (bounded) until every workgroup of this row block has delivered its piece
+        if (lane == 0) {
+          int it = 0;
+          while (__hip_atomic_load(p.il_cnt + m_blk, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < p.n_tiles && ++it < (1 << 20))
+            __builtin_amdgcn_s_sleep(8);
+          if (it >= (1 << 20)) {
+            __hip_atomic_store(p.il_cnt + (p.M + 127) / 128, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_fetch_add(&kh_coop_timeout_count, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
+        }
+      }
       const int so = (t - KT1) * 128;
 #pragma unroll
       for (int q = 0; q < LPS_HI; ++q)
-        if (q < LPS_LO || has_hi)
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(q < XQ ? rs_t : rs_b, (lptr_t)(stage + (wave + 8 * q) * 1024), 16, voff2[q], so, 0, 0);
+        if (q < LPS_LO || has_hi) {
+          // (COOP) T was written inside this launch, maybe on another XCD: read past the (non-coherent) L2
+          if (COOP && q < XQ) __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_t, (lptr_t)(stage + (wave + 8 * q) * 1024), 16, voff2[q], so, 0, 17 /* sc0 sc1 */);
+          else __builtin_amdgcn_raw_ptr_buffer_load_lds(q < XQ ? rs_t : rs_b, (lptr_t)(stage + (wave + 8 * q) * 1024), 16, voff2[q], so, 0, 0);
+        }
     }
     if (CONV) {
       cv_c0 += 64;
@@ -467,12 +520,13 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_ksplit_kernel(const LoraGemm
 #endif
 }
 
-template <class C, bool CONV = false, bool GNF = false>
+template <class C, bool CONV = false, bool GNF = false, bool COOP = false>
 int launch_ksplit(LoraGemmParams p, hipStream_t stream) {
   p.m_tiles = (p.M + C::BM - 1) / C::BM;
   p.n_tiles = (p.N + C::BN - 1) / C::BN;
   static_assert(C::LDS + KH_LN_LDS <= 160 * 1024, "LDS budget with the row statistics");
-  if (hipError_t e = kh_allow_lds<lora_gemm_ksplit_kernel<C, CONV, GNF>>(C::LDS + KH_LN_LDS); e != hipSuccess) return (int)e;
+  static_assert(!COOP || (SCfg<4, 1, 3>::LDS <= C::LDS && C::BM == 128), "the shrink piece's rings fit the GEMM ring; four quarters per row block");
+  if (hipError_t e = kh_allow_lds<lora_gemm_ksplit_kernel<C, CONV, GNF, COOP>>(C::LDS + KH_LN_LDS); e != hipSuccess) return (int)e;
   if ((p.ln_part != nullptr || p.st_part != nullptr) && CONV) return KH_ERR_UNSUPPORTED;
   if (p.st_part != nullptr && p.n_tiles > KH_LN_SLOTS) return KH_ERR_UNSUPPORTED;
   p.ln_lds = C::LDS;
@@ -493,7 +547,7 @@ int launch_ksplit(LoraGemmParams p, hipStream_t stream) {
         p.M % p.gn_hw != 0)
       return KH_ERR_UNSUPPORTED;
   }
-  kh_launch(CONV ? KH_TAG_CONV : KH_TAG_LORA_GEMM, lora_gemm_ksplit_kernel<C, CONV, GNF>, dim3(grid), dim3(512), lds, stream, p);
+  kh_launch(CONV ? KH_TAG_CONV : KH_TAG_LORA_GEMM, lora_gemm_ksplit_kernel<C, CONV, GNF, COOP>, dim3(grid), dim3(512), lds, stream, p);
   KH_RETURN_LAST_ERROR();
 }
 
@@ -512,6 +566,37 @@ bool lora_gemm_ksplit_ok(const LoraGemmParams& p) {
   return plain && ks_fits_buffers(p) && p.grp == nullptr && p.sg_mode == 0 && p.conv_cin == 0 && !p.geglu && p.K % 64 == 0 && p.K >= 64 &&
          (p.t_ext == nullptr || (p.R % 64 == 0 && p.ldt % 8 == 0)) && (p.t_nsplit == 0 || p.t_nsplit % 160 == 0) &&
          p.N % 8 == 0;
+}
+
+// The cooperative form (see the kernel): the layers whose 128 x 160 tiles fill the chip -- exactly the shapes the rule in
+// lora_gemm_pipe_launch gives these tiles --, T of one or several stacked layers with 128 packed rank columns each of which
+// at most 96 are in use, four column tiles per 128 rank columns of T.
+bool lora_gemm_ksplit_coop_ok(const LoraGemmParams& p) {
+  if (!(p.t_ext != nullptr && p.a_cat != nullptr && p.col_scale != nullptr && p.il_cnt != nullptr)) return false;
+  if (!lora_gemm_ksplit_ok(p) || p.N % 160 != 0 || p.R != 128 || p.r_used <= 0 || p.r_used > 96 || p.ldt % 128 != 0) return false;
+  const long tiles = (long)((p.M + 127) / 128) * ((p.N + 127) / 128), m128 = (p.M + 127) / 128, n160 = p.N / 160;
+  if (!(tiles > 256 && tiles <= 384 && m128 * n160 <= 256)) return false;
+  const bool t_ok = p.t_nsplit == 0 ? p.ldt == p.R : (p.N % p.t_nsplit == 0 && p.ldt == (p.N / p.t_nsplit) * p.R);
+  return t_ok && n160 == 4 * (p.ldt / 128) && n160 <= KH_LN_SLOTS;
+}
+
+// this file's share of kh_lora_split_timeouts (synchronous)
+int lora_gemm_ksplit_coop_timeouts(int* count, int clear) {
+  int v = 0;
+  hipError_t e = hipMemcpyFromSymbol(&v, HIP_SYMBOL(kh_coop_timeout_count), sizeof(int), 0, hipMemcpyDeviceToHost);
+  if (e != hipSuccess) return (int)e;
+  *count = v;
+  if (clear && v != 0) {
+    const int zero = 0;
+    e = hipMemcpyToSymbol(HIP_SYMBOL(kh_coop_timeout_count), &zero, sizeof(int), 0, hipMemcpyHostToDevice);
+    if (e != hipSuccess) return (int)e;
+  }
+  return KH_OK;
+}
+
+int lora_gemm_ksplit_launch_coop(const LoraGemmParams& p, hipStream_t stream) {
+  if (!lora_gemm_ksplit_coop_ok(p)) return KH_ERR_UNSUPPORTED;
+  return launch_ksplit<KCfg<4>, false, false, true>(p, stream);
 }
 
 int lora_gemm_ksplit_launch(const LoraGemmParams& p, int row_groups, hipStream_t stream) {

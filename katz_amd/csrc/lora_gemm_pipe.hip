@@ -1224,12 +1224,14 @@ KH_EXPORT int kh_lora_split_timeouts(int32_t* count, int clear) {
   int v = 0;
   hipError_t e = hipMemcpyFromSymbol(&v, HIP_SYMBOL(kh_split_timeout_count), sizeof(int), 0, hipMemcpyDeviceToHost);
   if (e != hipSuccess) return (int)e;
-  *count = v;
   if (clear && v != 0) {
     const int zero = 0;
     e = hipMemcpyToSymbol(HIP_SYMBOL(kh_split_timeout_count), &zero, sizeof(int), 0, hipMemcpyHostToDevice);
     if (e != hipSuccess) return (int)e;
   }
+  int v2 = 0;   // the cooperative form's waits (lora_gemm_ksplit.hip)
+  if (const int rc = lora_gemm_ksplit_coop_timeouts(&v2, clear); rc != KH_OK) return rc;
+  *count = v + v2;
   return KH_OK;
 }
 

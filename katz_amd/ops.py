@@ -200,6 +200,13 @@ def lora_shrink(x: torch.Tensor, a_cat: torch.Tensor, col_scale: torch.Tensor, o
     return out
 
 
+def _no_coop_bit() -> int:
+    """Flag bit 24 of the split / norm entry points: inside side_branch() the cooperative in-launch shrink is off.  Its
+    workgroups wait for each other, and two such launches running side by side on two streams could each hold the CUs
+    the other one's last workgroups need."""
+    return (1 << 24) if _ws_slot[0] > 0 else 0
+
+
 def _r_used_bits(r_used: int, R: int) -> int:
     if r_used < 0 or r_used > R or r_used % 16:
         raise ValueError(f"r_used must be a multiple of 16 in [0, {R}], got {r_used}")
@@ -374,7 +381,7 @@ def lora_linear_split(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torc
     out = torch.empty(tuple(x.shape[:-1]) + (n_out,), dtype=BF16, device=x.device)
     t = torch.empty((M, RT), dtype=BF16, device=x.device)
     cnt = _split_counters(x.device, M)
-    flags = (1 if geglu else 0) | ((1 if two_launches else 0) << 8) | (_r_used_bits(r_used, R) << 16)
+    flags = (1 if geglu else 0) | ((1 if two_launches else 0) << 8) | (_r_used_bits(r_used, R) << 16) | _no_coop_bit()
     if CALL_LOG is not None:   # one entry per kernel launch
         if lib.kh_lora_linear_split_launches(M, N, K, R, n_split, flags) == 2:
             CALL_LOG.append(("lora_shrink", M, K, RT))
@@ -452,7 +459,7 @@ def lora_linear_norm(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch
     if R:
         t = torch.empty((M, RT), dtype=BF16, device=x.device)
         cnt = _split_counters(x.device, M)
-    flags = (1 if geglu else 0) | ((1 if two_launches else 0) << 8) | (_r_used_bits(r_used, R) << 16 if R else 0)
+    flags = (1 if geglu else 0) | ((1 if two_launches else 0) << 8) | (_r_used_bits(r_used, R) << 16 if R else 0) | _no_coop_bit()
     if CALL_LOG is not None:   # one entry per kernel launch
         if R and lib.kh_lora_linear_split_launches(M, N, K, R, n_split, flags) == 2:
             CALL_LOG.append(("lora_shrink", M, K, RT))
@@ -521,7 +528,8 @@ def lora_linear_xattn(x: torch.Tensor, weight: torch.Tensor, k: torch.Tensor, v:
     if R:
         t = torch.empty((M, R), dtype=BF16, device=x.device)
         cnt = _split_counters(x.device, M)
-    flags = ((1 if two_launches else 0) << 8) | (_r_used_bits(r_used, R) << 16 if R else 0)
+    # bit 24: the cooperative shrink belongs to another kernel family (the launch count below must not count on it)
+    flags = ((1 if two_launches else 0) << 8) | (_r_used_bits(r_used, R) << 16 if R else 0) | (1 << 24)
     if CALL_LOG is not None:   # one entry per kernel launch
         if R and lib.kh_lora_linear_split_launches(M, N, K, R, 0, flags) == 2:
             CALL_LOG.append(("lora_shrink", M, K, R))

@@ -182,6 +182,70 @@ def test_layer_norm_folded_into_the_linear(M, N, K, R, n_split, geglu):
         assert_close_rel(y2, exact.float(), 4e-2 if geglu else 2e-2, "folded LayerNorm + linear, two launches")
 
 
+@pytest.mark.parametrize("M,N,K,n_split,res,stats", [
+    (8192, 640, 640, 0, False, False),      # a folded LayerNorm in front
+    (8192, 640, 2560, 0, True, True),       # ff.net.2: residual, statistics for the next block's norm1
+    (8192, 640, 640, 0, True, True),        # to_out
+    (8000, 640, 640, 0, False, True),       # ragged rows
+])
+def test_cooperative_shrink_with_fold_and_statistics(M, N, K, n_split, res, stats):
+    """Ranks 64 + 32 in 128 packed columns (r_used = 96) on the layers whose 128 x 160 tiles fill the chip: every GEMM
+    workgroup first computes a 32 x 96 piece of T, with the folded LayerNorm's correction where there is one.  Against
+    float64, against the two-launch form, and the row statistics of the result."""
+    from katz_amd import ops
+    from katz_amd.lora import fold_layer_norm
+    say("cooperative shrink + fold / statistics", M, N, K, n_split, res, stats)
+    d = dev()
+    R, RU = 128, 96
+    fold = not res
+    h, gamma, beta, w, b, A, B = _fold_case(M, N, K, R, seed=M + N + K + 96, n_split=n_split)
+    parts = N // n_split if n_split else 1
+    for j in range(parts):
+        A[j * R + RU:(j + 1) * R] = 0
+    B[:, RU:] = 0
+    scale = 0.8
+    assert ops._lib.load().kh_lora_linear_split_launches(M, N, K, R, n_split, (RU // 16) << 16) == 1
+    assert ops._lib.load().kh_lora_linear_split_launches(M, N, K, R, n_split, 0) == 2
+    s = torch.full((A.shape[0],), scale, device=d)
+    r = None
+    if res:
+        g = torch.Generator().manual_seed(M + 1)
+        r = bf16_round(randn(g, M, N))
+    st_out = None
+    if stats:
+        st_out = ops.row_stats_buffer(M, d)
+        st_out.fill_(float("nan"))
+    ops.split_counters_reset(d)
+    if fold:
+        wp, c1, c2, ap, ca1, ca2 = fold_layer_norm(w.to(d, BF), b.to(d, BF), gamma.to(d, BF), beta.to(d, BF), A.to(d, BF))
+        ln = (_stats_from(h, d), c1, c2, ca1, ca2, 1e-5)
+        run = lambda **kw: ops.lora_linear_norm(h.to(d, BF), wp, None, ap, s, B.to(d, BF), n_split=n_split, r_used=RU, ln=ln,
+                                                stats_out=st_out, **kw)
+        exact = _ref_fold(h, gamma, beta, w, b, A, B, scale, n_split, exact=True)
+        e_ref = _rms_err(bf16_round(_ref_fold(h, gamma, beta, w, b, A, B, scale, n_split)), exact)
+    else:
+        run = lambda **kw: ops.lora_linear_norm(h.to(d, BF), w.to(d, BF), b.to(d, BF), A.to(d, BF), s, B.to(d, BF),
+                                                residual=r.to(d, BF), n_split=n_split, r_used=RU, stats_out=st_out, **kw)
+        exact = O.lora_linear(h.double(), w.double(), b.double(), [(A.double(), B.double(), scale)], residual=r.double())
+        e_ref = 0.0
+    y = run()
+    flag = ops.split_counters_last(d)[-1:].clone()
+    got = None if st_out is None else st_out.double().sum(0).cpu()
+    y2 = run(two_launches=True)
+    torch.cuda.synchronize()
+    assert int(flag) == 0
+    assert_close_rel(y, exact.float(), 2e-2, "cooperative shrink")
+    if fold:
+        assert _rms_err(y, exact) <= 1.25 * e_ref + 1e-4
+    assert (y != y2).float().mean().item() < 5e-3          # the shrink's fp32 summation order differs
+    if stats:
+        s1, s2 = _stats_of(y)
+        assert torch.isfinite(got).all()
+        assert torch.allclose(got[:, 0], s1.double().cpu(), rtol=1e-3, atol=1e-2 * float(s2.max().sqrt()))
+        assert torch.allclose(got[:, 1], s2.double().cpu(), rtol=1e-3)
+    ops.check_split_timeouts(d)
+
+
 def test_producer_feeds_consumer():
     """to_out (residual, statistics out) -> norm -> to_q with the norm folded: against the unfused chain."""
     from katz_amd import ops
