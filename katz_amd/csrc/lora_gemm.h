@@ -244,7 +244,7 @@ int lora_gemm_wide_launch(LoraGemmParams p, hipStream_t stream);
 
 // The shrink of a layer, optionally with a folded LayerNorm in front (ln_part != nullptr; lora_shrink.hip).
 int lora_shrink_ln_launch(const void* x, const void* a_cat, const float* col_scale, void* t, int64_t M, int64_t K, int64_t R,
-                          const float* ln_part, const float* ln_ca1, const float* ln_ca2, float ln_eps, hipStream_t stream);
+                          const float* ln_part, const float* ln_ca1, const float* ln_ca2, float ln_eps, hipStream_t stream, int group, int r_used);
 
 extern "C" int kh_lora_shrink_bf16(const void* x, const void* a_cat, const float* col_scale, void* t, int64_t M, int64_t K,
                                    int64_t R, void* stream);

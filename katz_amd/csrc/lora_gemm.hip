@@ -621,7 +621,8 @@ KH_EXPORT int kh_lora_linear_split_bf16(const void* x, const void* w, const void
     if ((flags & KH_FLAG_NO_COOP) == 0 && lora_gemm_ksplit_coop_ok(p)) return lora_gemm_ksplit_launch_coop(p, (hipStream_t)stream);
     return lora_gemm_pipe_launch_il(p, (hipStream_t)stream);
   }
-  const int rc = kh_lora_shrink_bf16(x, a_cat, col_scale, t_scratch, M, K, RT, stream);
+  const int rc = lora_shrink_ln_launch(x, a_cat, col_scale, t_scratch, M, K, RT, nullptr, nullptr, nullptr, 0.f, (hipStream_t)stream,
+                                       (int)R, ((flags >> 16) & 0xff) * 16);
   if (rc != KH_OK) return rc;
   return kh_lora_linear_pre_bf16(x, w, bias, t_scratch, RT, n_split, b_cat, residual, y, M, N, K, R, flags & 0xff00ff, stream);
 }
@@ -682,7 +683,7 @@ static int lora_linear_norm_impl(const void* x, const void* w, const void* bias,
     kh_take_weight_prefetch(p);
     if (R == 0) return lora_gemm_pipe_launch_xattn(p, (hipStream_t)stream);
     if (counters != nullptr && tile_sel == 0 && lora_gemm_pipe_il_ok(p)) return lora_gemm_pipe_launch_xattn(p, (hipStream_t)stream);
-    const int rc = lora_shrink_ln_launch(x, a_cat, col_scale, t_scratch, M, K, RT, ln_part, ln_ca1, ln_ca2, ln_eps, (hipStream_t)stream);
+    const int rc = lora_shrink_ln_launch(x, a_cat, col_scale, t_scratch, M, K, RT, ln_part, ln_ca1, ln_ca2, ln_eps, (hipStream_t)stream, (int)R, p.r_used);
     if (rc != KH_OK) return rc;
     p.a_cat = nullptr; p.col_scale = nullptr; p.il_cnt = nullptr;
     return lora_gemm_pipe_launch_xattn(p, (hipStream_t)stream);
@@ -695,7 +696,7 @@ static int lora_linear_norm_impl(const void* x, const void* w, const void* bias,
   if (counters != nullptr && tile_sel == 0 && (flags & KH_FLAG_NO_COOP) == 0 && lora_gemm_ksplit_coop_ok(p))
     return lora_gemm_ksplit_launch_coop(p, (hipStream_t)stream);
   if (counters != nullptr && tile_sel == 0 && lora_gemm_pipe_il_ok(p)) return lora_gemm_pipe_launch_il(p, (hipStream_t)stream);
-  const int rc = lora_shrink_ln_launch(x, a_cat, col_scale, t_scratch, M, K, RT, ln_part, ln_ca1, ln_ca2, ln_eps, (hipStream_t)stream);
+  const int rc = lora_shrink_ln_launch(x, a_cat, col_scale, t_scratch, M, K, RT, ln_part, ln_ca1, ln_ca2, ln_eps, (hipStream_t)stream, (int)R, p.r_used);
   if (rc != KH_OK) return rc;
   p.a_cat = nullptr; p.col_scale = nullptr; p.il_cnt = nullptr;
   return lora_gemm_pipe_launch(p, tile_sel == 1 ? 0 : tile_sel, (hipStream_t)stream);

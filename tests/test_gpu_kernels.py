@@ -1029,6 +1029,55 @@ def test_lora_linear_split_rank_96_of_128(case):
     ops.check_split_timeouts(d)
 
 
+@pytest.mark.parametrize("M", [8192, 8100, 4096])
+@pytest.mark.parametrize("fold", [False, True], ids=["plain", "ln-fold"])
+def test_stacked_layers_rank_96_shrink_as_its_own_launch(M, fold):
+    """q / k / v of the 64 x 64 level: three stacked layers, rank 96 of 128 each, on GEMM tiles that fill the chip in several
+    rounds, so the shrink stays a launch of its own -- on 128-row x 96-column tiles, one per layer and 128 rows, that skip
+    the padding columns and zero them in T.  T is poisoned with NaNs first.  Against the oracle and against the call
+    without the promise (64 x 64 tiles over all 384 columns: another summation order)."""
+    from katz_amd import ops
+    from katz_amd.lora import fold_layer_norm
+
+    N, K, n_split, R, RU = 1920, 640, 640, 128, 96
+    say("stacked rank-96 shrink", M, fold)
+    d = dev()
+    g = torch.Generator().manual_seed(M + 17)
+    x, w, b = randn(g, M, K), randn(g, N, K, std=0.03), randn(g, N, std=0.1)
+    A, B = randn(g, 3 * R, K, std=0.05), randn(g, N, R, std=0.05)
+    for j in range(3):
+        A[j * R + RU:(j + 1) * R] = 0
+    B[:, RU:] = 0
+    cs = torch.full((3 * R,), 0.7, device=d)
+    assert ops._lib.load().kh_lora_linear_split_launches(M, N, K, R, n_split, (RU // 16) << 16) == 2
+    xd, wd, bd, Ad, Bd = (t.to(d, BF) for t in (x, w, b, A, B))
+    if fold:
+        gamma, beta = randn(g, K, std=0.2) + 1.0, randn(g, K, std=0.2)
+        wp, c1, c2, ap, ca1, ca2 = fold_layer_norm(wd, bd, gamma.to(d, BF), beta.to(d, BF), Ad)
+        st = torch.zeros((ops.LN_SLOTS, M, 2), dtype=torch.float32, device=d)
+        st[0, :, 0] = xd.float().sum(-1)
+        st[0, :, 1] = (xd.float() ** 2).sum(-1)
+        run = lambda ru: ops.lora_linear_norm(xd, wp, None, ap, cs, Bd, n_split=n_split, r_used=ru, ln=(st, c1, c2, ca1, ca2, 1e-5))
+        xn = O.layer_norm(xd.float().cpu(), gamma.to(BF).float(), beta.to(BF).float(), 1e-5)
+    else:
+        run = lambda ru: ops.lora_linear_split(xd, wd, bd, Ad, cs, Bd, n_split=n_split, r_used=ru)
+        xn = xd.float().cpu()
+    for _ in range(3):   # what torch hands out next is full of NaNs
+        junk = torch.full((M, 3 * R), float("nan"), device=d, dtype=BF)
+        del junk
+    y = run(RU)
+    y_again = run(RU)
+    y_full = run(0)
+    torch.cuda.synchronize()
+    assert torch.isfinite(y.float()).all() and torch.equal(y, y_again)
+    assert (y != y_full).float().mean().item() < 5e-3
+    wf, bfl, Af, Bf = (t.float().cpu() for t in (wd, bd, Ad, Bd))
+    for j in range(3):
+        rows = slice(j * n_split, (j + 1) * n_split)
+        ref = O.lora_linear(xn, wf[rows], bfl[rows], [(Af[j * R:(j + 1) * R], Bf[rows], 0.7)])
+        assert_close_rel(y[:, rows], ref, REL_BF16, f"stacked rank-96 shrink part {j}")
+
+
 @pytest.mark.parametrize("case", [
     # (M, N, K, R, residual, n_split)
     (2048, 1280, 1280, 128, True, 0),      # to_out / attn2.to_q at 32x32: 160 GEMM + 64 shrink workgroups in one launch
