@@ -405,6 +405,15 @@ def kernel_probe():
     add(f"lora_linear_split M{M} K{K} N{N} R{R} r_used {Rt} (shrink in launch, 64x32 tiles)",
         lambda x=x, w=w, b=b, a=a96, s=scale, bc=b96: ops.lora_linear_split(x, w, b, a, s, bc, r_used=96),
         2.0 * M * N * (K + Rt) + 2.0 * M * K * Rt, 2.0 * (M * K + K * N + M * N + Rt * N + Rt * K))
+    # the N 640 layer of the 64 x 64 level as ONE launch: every workgroup of the 128 x 160 tiles computes a piece of T first
+    M, K, N = 8192, 640, 640
+    x8, w8, b8 = rn(M, K), rn(N, K, std=0.02), rn(N)
+    a8, bc8 = rn(R, K, std=0.02), rn(N, R, std=0.02)
+    a8[Rt:] = 0
+    bc8[:, Rt:] = 0
+    add(f"lora_linear_split M{M} K{K} N{N} R{R} r_used {Rt} (cooperative shrink in launch)",
+        lambda: ops.lora_linear_split(x8, w8, b8, a8, scale, bc8, r_used=96),
+        2.0 * M * N * (K + Rt) + 2.0 * M * K * Rt, 2.0 * (M * K + K * N + M * N + Rt * N + Rt * K))
     # K3: attention at the three SDXL shapes
     for (B, H, T, S) in ((2, 10, 4096, 4096), (2, 20, 1024, 1024), (2, 20, 1024, 77)):
         q, k, v = rn(B, T, H * 64), rn(B, S, H * 64), rn(B, S, H * 64)
