@@ -131,6 +131,24 @@ __global__ __launch_bounds__(GN_THREADS) void gn_apply_nhwc(const bf16_t* __rest
   const int n = blockIdx.y, split = blockIdx.x;
   const int tid = threadIdx.x;
   const double cnt = (double)g.Cg * (double)g.HW;
+  // What does not depend on the statistics is requested first: this thread's channel constants of its first chunk and
+  // its first (at most) GN_UNROLL pixels.  Their latency then runs beside the fold of the partial sums below instead of behind it
+  // (a kernel this short is a chain of memory round trips: partial sums, constants, first pixels).
+  const int per = (g.HW + g.asplits - 1) / g.asplits;
+  const int p0 = split * per, p1 = min(g.HW, p0 + per);
+  const int tx = tid % g.NTX, ty = tid / g.NTX;
+  const bool active = ty < g.PL;
+  const u32x4 z4 = {0, 0, 0, 0};
+  u32x4 pre[GN_UNROLL], cg0 = z4, cb0 = z4, ca0 = z4;
+  if (active) {
+    const int c0 = tx * 8;
+    if (gamma) cg0 = *reinterpret_cast<const u32x4*>(gamma + c0);
+    if (beta) cb0 = *reinterpret_cast<const u32x4*>(beta + c0);
+    if (add_nc) ca0 = *reinterpret_cast<const u32x4*>(add_nc + (size_t)n * g.C + c0);
+  }
+#pragma unroll
+  for (int u = 0; u < GN_UNROLL; ++u)
+    pre[u] = (active && p0 + ty + u * g.PL < p1) ? *reinterpret_cast<const u32x4*>(x + ((size_t)n * g.HW + p0 + ty + u * g.PL) * g.C + tx * 8) : z4;
   // Fold the statistics pass's partial sums of every group (a workgroup needs all groups: a pixel has all channels).
   // FT threads share a group, each summing every FT-th partial in fp64; their FT sums are then added in a fixed
   // order, so the result does not depend on scheduling.
@@ -165,20 +183,23 @@ __global__ __launch_bounds__(GN_THREADS) void gn_apply_nhwc(const bf16_t* __rest
     }
     __syncthreads();
   }
-  const int per = (g.HW + g.asplits - 1) / g.asplits;
-  const int p0 = split * per, p1 = min(g.HW, p0 + per);
-  const int tx = tid % g.NTX, ty = tid / g.NTX;
-  if (ty >= g.PL) return;
+  if (!active) return;
   for (int k = 0; k < g.CPT; ++k) {
     const int c0 = (tx + k * g.NTX) * 8;
-    float sc[8], sh[8];
+    u32x4 cg = cg0, cb = cb0, ca = ca0;
+    if (k > 0) {
+      cg = gamma ? *reinterpret_cast<const u32x4*>(gamma + c0) : z4;
+      cb = beta ? *reinterpret_cast<const u32x4*>(beta + c0) : z4;
+      ca = add_nc ? *reinterpret_cast<const u32x4*>(add_nc + (size_t)n * g.C + c0) : z4;
+    }
+    float gaf[8], bef[8], adf[8], sc[8], sh[8];
+    unpack8(cg, gaf); unpack8(cb, bef); unpack8(ca, adf);
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      const int c = c0 + e, grp = c / g.Cg;
-      const float ga = gamma ? (float)gamma[c] : 1.f, be = beta ? (float)beta[c] : 0.f;
-      const float ad = add_nc ? (float)add_nc[(size_t)n * g.C + c] : 0.f;
+      const int grp = (c0 + e) / g.Cg;
+      const float ga = gamma ? gaf[e] : 1.f;
       sc[e] = ga * s_rstd[grp];
-      sh[e] = be + (ad - s_mean[grp]) * sc[e];
+      sh[e] = bef[e] + (adf[e] - s_mean[grp]) * sc[e];
     }
     const size_t off = ((size_t)n * g.HW) * g.C + c0;
     const bf16_t* xb = x + off;
@@ -197,6 +218,12 @@ __global__ __launch_bounds__(GN_THREADS) void gn_apply_nhwc(const bf16_t* __rest
       *reinterpret_cast<u32x4*>(yb + (size_t)p * g.C) = o;
     };
     int p = p0 + ty;
+    if (k == 0) {   // the pixels requested at the top
+#pragma unroll
+      for (int u = 0; u < GN_UNROLL; ++u)
+        if (p + u * g.PL < p1) emit(pre[u], p + u * g.PL);
+      p += GN_UNROLL * g.PL;
+    }
     for (; p + (GN_UNROLL - 1) * g.PL < p1; p += GN_UNROLL * g.PL) {
       u32x4 v[GN_UNROLL];
 #pragma unroll
