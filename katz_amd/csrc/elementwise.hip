@@ -112,6 +112,7 @@ __global__ __launch_bounds__(EW_THREADS) void concat_residual_kernel(const bf16_
                                                                      int C2) {
   const int cp1 = C1 / 8, cp = (C1 + C2) / 8;
   const long total = rows * cp;
+  const KhOut yout(out, (size_t)rows * (C1 + C2) * 2);
   for (long i = (long)blockIdx.x * EW_THREADS + threadIdx.x; i < total; i += (long)gridDim.x * EW_THREADS) {
     const long row = i / cp;
     const int c = (int)(i % cp);
@@ -128,7 +129,7 @@ __global__ __launch_bounds__(EW_THREADS) void concat_residual_kernel(const bf16_
         for (int e = 0; e < 4; ++e) o[e] = pack_bf16x2(bf16_lo(o[e]) + acc[2 * e], bf16_hi(o[e]) + acc[2 * e + 1]);
       }
     }
-    *reinterpret_cast<u32x4*>(out + row * (C1 + C2) + c * 8) = o;
+    yout.store16((size_t)(row * (C1 + C2) + c * 8) * 2, o);
   }
 }
 

@@ -72,6 +72,40 @@ typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
+// A kernel's results, stored THROUGH the L2 at agent scope (`sc1`: the line stays in the L2 and the data moves on to the
+// memory side at once).  With plain stores a launch's dirty lines leave the eight L2s when the launch ends, all at the same
+// moment and with nothing to overlap them; written through, they leave while other waves still compute.  Only for 16-byte
+// pieces that fill whole rows (8-byte pieces that complete a line over several instructions got slower).  The store is the
+// compiler's own buffer store with a cache-policy operand, NOT inline assembly: a hand-written `global_store_dwordx4` is
+// invisible to the compiler's hazard recogniser, which otherwise keeps the next vector instruction from overwriting the
+// data registers of a store wider than 8 bytes during its first two wait states -- such stores wrote garbage now and then.
+// Offsets are 32 bits: outputs of 4 GiB and more take plain stores.
+#if __HIP_DEVICE_COMPILE__
+struct KhOut {
+  __amdgpu_buffer_rsrc_t rs;
+  char* base;
+  bool wt;
+  __device__ __forceinline__ KhOut(void* y, size_t bytes)
+      : rs(__builtin_amdgcn_make_buffer_rsrc(y, 0, (int)(uint32_t)(bytes < 0xFFFFFFFFull ? bytes : 0), 0x00020000)),
+        base(reinterpret_cast<char*>(y)),
+#if defined(KH_PLAIN_STORES)   // build-time switch back to plain stores (python -m katz_amd.build with -DKH_PLAIN_STORES in HIPCC_FLAGS)
+        wt(false) {}
+#else
+        wt(bytes < 0xFFFFFFFFull) {}
+#endif
+  __device__ __forceinline__ void store16(size_t byte_off, const u32x4 v) const {
+    if (wt) __builtin_amdgcn_raw_buffer_store_b128(v, rs, (int)(uint32_t)byte_off, 0, 16 /* sc1 */);
+    else *reinterpret_cast<u32x4*>(base + byte_off) = v;
+  }
+};
+#else
+struct KhOut {   // the host pass only parses the kernels
+  char* base;
+  __host__ __device__ KhOut(void* y, size_t) : base(reinterpret_cast<char*>(y)) {}
+  __host__ __device__ void store16(size_t byte_off, const u32x4 v) const { *reinterpret_cast<u32x4*>(base + byte_off) = v; }
+};
+#endif
+
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t lo16) {
   return __uint_as_float(lo16 << 16);
 }

@@ -473,6 +473,7 @@ __global__ __launch_bounds__(512, COOP ? 1 : 2) void lora_gemm_ksplit_kernel(con
       *reinterpret_cast<f32x2*>(p.gn_part + (((size_t)n_img * G + n0 / cg + tid) * splits + split) * 2) = f32x2{s, q};
     }
   }
+  const KhOut yout(p.y, (size_t)M * N * 2);
   if (p.st_part != nullptr) {
     // as below, and every row's (sum, sum of squares) over this tile's columns for a following folded LayerNorm: the 20
     // pieces of a row meet in LDS (the partial strips are dead) and are added in a fixed order
@@ -489,7 +490,7 @@ __global__ __launch_bounds__(512, COOP ? 1 : 2) void lora_gemm_ksplit_kernel(con
         for (int e = 0; e < 4; ++e)
           o[e] = pack_bf16x2(bf16_lo(o[e]) + bf16_lo(rr[q][e]), bf16_hi(o[e]) + bf16_hi(rr[q][e]));
       }
-      if (ok) *reinterpret_cast<u32x4*>(p.y + (size_t)grow * N + gcol) = o;
+      if (ok) yout.store16(((size_t)grow * N + gcol) * 2, o);
       float ps, pq;
       kh_piece_sums(o, ps, pq);
       if (c < C::OPC) *reinterpret_cast<u32x2*>(sp + 2 * c) = u32x2{__float_as_uint(ps), __float_as_uint(pq)};
@@ -514,7 +515,7 @@ __global__ __launch_bounds__(512, COOP ? 1 : 2) void lora_gemm_ksplit_kernel(con
         for (int e = 0; e < 4; ++e)
           o[e] = pack_bf16x2(bf16_lo(o[e]) + bf16_lo(rr[q][e]), bf16_hi(o[e]) + bf16_hi(rr[q][e]));
       }
-      *reinterpret_cast<u32x4*>(p.y + (size_t)grow * N + gcol) = o;
+      yout.store16(((size_t)grow * N + gcol) * 2, o);
     }
   }
 #endif

@@ -986,6 +986,7 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
     // writes so their latency hides behind the transpose.
     stamp(4);
     const int out_ld = p.geglu ? (N >> 1) : N;
+    const KhOut yout(p.y, (size_t)M * out_ld * 2);
     constexpr int CPR = BN / 8;                                   // 16-byte pieces per staged row
     constexpr int ECH = C::WAVES_M * 32 * CPR / C::NT;            // pieces per thread per pass
     constexpr int OPR = BN / 16;                                  // GEGLU: output pieces per staged row
@@ -1054,7 +1055,7 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
             for (int e = 0; e < 4; ++e)
               o[e] = pack_bf16x2(bf16_lo(o[e]) + bf16_lo(rr[q][e]), bf16_hi(o[e]) + bf16_hi(rr[q][e]));
           }
-          if (ok) *reinterpret_cast<u32x4*>(p.y + (size_t)grow * N + gcol) = o;
+          if (ok) yout.store16(((size_t)grow * N + gcol) * 2, o);
           float ps, pq;
           kh_piece_sums(o, ps, pq);
           static_assert(CPR == 16 || CPR == 32, "a row's pieces fill one or two DPP rows");
@@ -1078,7 +1079,7 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
               for (int e = 0; e < 4; ++e)
                 o[e] = pack_bf16x2(bf16_lo(o[e]) + bf16_lo(rr[q][e]), bf16_hi(o[e]) + bf16_hi(rr[q][e]));
             }
-            *reinterpret_cast<u32x4*>(p.y + (size_t)grow * N + gcol) = o;
+            yout.store16(((size_t)grow * N + gcol) * 2, o);
           }
         }
       } else {
@@ -1101,7 +1102,7 @@ __global__ __launch_bounds__(C::NT, C::OCC) void lora_gemm_pipe_kernel(const Lor
               const uint32_t ar = pack_bf16x2(a0, a1);  // gelu(gate) rounded to bf16 before the product
               o[e] = pack_bf16x2(bf16_lo(hv[e]) * bf16_lo(ar), bf16_hi(hv[e]) * bf16_hi(ar));
             }
-            *reinterpret_cast<u32x4*>(p.y + (size_t)grow * out_ld + gcol) = o;
+            yout.store16(((size_t)grow * out_ld + gcol) * 2, o);
           }
         }
       }

@@ -248,6 +248,7 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_wide_kernel(const LoraGemmPa
   // a contiguous output row; two passes of 128 rows (the waves' upper / lower 32-row MFMA tiles).
   bf16_t* sC = reinterpret_cast<bf16_t*>(smem);
   const int out_ld = p.geglu ? (N >> 1) : N;
+  const KhOut yout(p.y, (size_t)p.M * out_ld * 2);
   constexpr int CPR = WBN / 8, ECH = 128 * CPR / 512;        // plain: pieces per staged row, per thread
   constexpr int OPR = WBN / 16, GCH = 128 * OPR / 512;       // GEGLU: output pieces per staged row, per thread
 #pragma unroll
@@ -296,7 +297,7 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_wide_kernel(const LoraGemmPa
 #pragma unroll
           for (int e = 0; e < 4; ++e) o[e] = pack_bf16x2(bf16_lo(o[e]) + bf16_lo(rr[e]), bf16_hi(o[e]) + bf16_hi(rr[e]));
         }
-        *reinterpret_cast<u32x4*>(p.y + g) = o;
+        yout.store16(g * 2, o);
       }
     } else {
       // staged columns come in groups of 64 = 32 value columns then their 32 gate columns
@@ -325,7 +326,7 @@ __global__ __launch_bounds__(512, 2) void lora_gemm_wide_kernel(const LoraGemmPa
         u32x4 o;
 #pragma unroll
         for (int e = 0; e < 4; ++e) o[e] = pack_bf16x2(bf16_lo(hv[e]) * bf16_lo(ar[e]), bf16_hi(hv[e]) * bf16_hi(ar[e]));
-        *reinterpret_cast<u32x4*>(p.y + g) = o;
+        yout.store16(g * 2, o);
       }
     }
     __syncthreads();

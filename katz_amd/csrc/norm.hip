@@ -184,6 +184,7 @@ __global__ __launch_bounds__(GN_THREADS) void gn_apply_nhwc(const bf16_t* __rest
     __syncthreads();
   }
   if (!active) return;
+  const KhOut yout(y, (size_t)g.N * g.HW * g.C * 2);
   for (int k = 0; k < g.CPT; ++k) {
     const int c0 = (tx + k * g.NTX) * 8;
     u32x4 cg = cg0, cb = cb0, ca = ca0;
@@ -203,7 +204,6 @@ __global__ __launch_bounds__(GN_THREADS) void gn_apply_nhwc(const bf16_t* __rest
     }
     const size_t off = ((size_t)n * g.HW) * g.C + c0;
     const bf16_t* xb = x + off;
-    bf16_t* yb = y + off;
     auto emit = [&](const u32x4 v, int p) {
       float f[8];
       unpack8(v, f);
@@ -215,7 +215,7 @@ __global__ __launch_bounds__(GN_THREADS) void gn_apply_nhwc(const bf16_t* __rest
         if (SILU) { a = silu_f(a); b = silu_f(b); }
         o[e] = pack_bf16x2(a, b);
       }
-      *reinterpret_cast<u32x4*>(yb + (size_t)p * g.C) = o;
+      yout.store16((off + (size_t)p * g.C) * 2, o);
     };
     int p = p0 + ty;
     if (k == 0) {   // the pixels requested at the top
