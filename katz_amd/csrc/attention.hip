@@ -237,17 +237,28 @@ __global__ __launch_bounds__(NW * 64, 2) void attention_kernel(const AttnParams 
   if (full_tiles < n_tiles) tile_step(full_tiles, std::true_type{});
 
   const float inv = 1.0f / l_run;   // the MFMA row sums already cover the keys of both lane halves
-  if (qrow < p.T) {
+  // A lane holds runs of 4 dims (8 bytes); lanes l and l + 32 hold the two halves of every 16-byte piece of their query's
+  // row.  Two pieces at a time, the pair trades halves (v_permlane32_swap: the upper half of the first register against the
+  // lower half of the second), after which lane l owns the even piece and lane l + 32 the odd one: 16-byte stores.
+#if __HIP_DEVICE_COMPILE__
 #pragma unroll
-    for (int dt = 0; dt < 2; ++dt)
+  for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        u32x2 o2;
-        o2[0] = pack_bf16x2(oacc[dt][4 * g + 0] * inv, oacc[dt][4 * g + 1] * inv);
-        o2[1] = pack_bf16x2(oacc[dt][4 * g + 2] * inv, oacc[dt][4 * g + 3] * inv);
-        *reinterpret_cast<u32x2*>(op + (size_t)qrow * p.ldo + dt * 32 + 8 * g + 4 * lh) = o2;
+    for (int gp = 0; gp < 2; ++gp) {
+      const int ge = 2 * gp, go = 2 * gp + 1;
+      const uint32_t e0 = pack_bf16x2(oacc[dt][4 * ge + 0] * inv, oacc[dt][4 * ge + 1] * inv);
+      const uint32_t e1 = pack_bf16x2(oacc[dt][4 * ge + 2] * inv, oacc[dt][4 * ge + 3] * inv);
+      const uint32_t o0 = pack_bf16x2(oacc[dt][4 * go + 0] * inv, oacc[dt][4 * go + 1] * inv);
+      const uint32_t o1 = pack_bf16x2(oacc[dt][4 * go + 2] * inv, oacc[dt][4 * go + 3] * inv);
+      const auto s0 = __builtin_amdgcn_permlane32_swap(e0, o0, false, false);
+      const auto s1 = __builtin_amdgcn_permlane32_swap(e1, o1, false, false);
+      const u32x4 piece = {s0[0], s1[0], s0[1], s1[1]};
+      if (qrow < p.T) {
+        const size_t off = (size_t)qrow * p.ldo + dt * 32 + 8 * (2 * gp + lh);
+        *reinterpret_cast<u32x4*>(op + off) = piece;   // (plain: written through the L2, 32 bytes of a row at a time gained nothing)
       }
-  }
+    }
+#endif
 }
 
 }  // namespace
