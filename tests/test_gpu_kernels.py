@@ -126,6 +126,31 @@ def test_lora_shrink_then_pre_gemm(case):
     assert torch.equal(y, y2)
 
 
+def test_output_of_four_gib_takes_the_plain_store_path():
+    """The GEMM epilogues store through a buffer descriptor with 32-bit offsets; an output of 4 GiB or more cannot be
+    addressed that way and takes plain stores with 64-bit addresses.  M = 2^21 + 200 rows of 1024 columns (4.0 GiB):
+    rows at the start, across the 4 GiB boundary and at the ragged end against the oracle, and the smaller problem made
+    of the same rows bit for bit."""
+    from katz_amd import ops
+
+    say("4 GiB output")
+    d = dev()
+    M, N, K = (1 << 21) + 200, 1024, 64
+    g = torch.Generator(device=d).manual_seed(12)
+    x = (torch.randn(M, K, device=d, generator=g)).to(BF)
+    w = (torch.randn(N, K, device=d, generator=g) * 0.1).to(BF)
+    b = torch.randn(N, device=d, generator=g).to(BF)
+    y = ops.lora_linear(x, w, b)
+    assert y.numel() * 2 >= 1 << 32
+    torch.cuda.synchronize()
+    for r0 in (0, (1 << 21) - 300, M - 333):
+        rows = slice(r0, r0 + 333)
+        ref = O.lora_linear(x[rows].float().cpu(), w.float().cpu(), b.float().cpu(), [])
+        assert_close_rel(y[rows], ref, REL_BF16, f"4 GiB output rows {r0}")
+        assert torch.equal(y[rows][:128], ops.lora_linear(x[rows][:128].contiguous(), w, b))
+    del y, x
+
+
 def test_lora_linear_bf16_scale_zero_is_base():
     say("lora_linear_bf16 scale 0")
     x, w, b, adapters, _ = _lora_case(512, 640, 640, (64,), (0.0,), True, False, seed=3)
